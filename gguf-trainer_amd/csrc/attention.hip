@@ -1,0 +1,282 @@
+// Causal / sliding-window GQA attention, forward and backward, softmax recomputed in backward
+// from a saved per-row log-sum-exp (srcAttnFwd / BwdD / BwdDq / BwdDkv, src/backend/wgsl.ts:657-918;
+// dispatch src/backend/webgpu.ts:1142-1174). Layout: q,out [B*T, Hq*hd], k,v [B*T, Hkv*hd], row-major,
+// head-major inside a row; query head h reads kv head h / (Hq/Hkv); query t attends keys
+// [max(0, t-window+1), t], window 0 = full causal (src/model/autograd.ts:651-661).
+//
+// The saved statistic is lse2 = m*c + log2(sum exp2(s*c - m*c)) with c = log2(e)/sqrt(hd): scores
+// live in the log2 domain so p = exp2(s*c - lse2) is one v_exp_f32, as in wgsl.ts:460-464.
+//
+// This file holds the shape-generic kernels (any hd, any T): one wavefront per query row (forward,
+// dQ) or per key row (dK/dV). A 64-key (or 64-query) tile is scored with lanes across keys, the
+// probabilities go through LDS, and the value/key accumulation runs with lanes across head dims,
+// so global reads of K/V/Q/dO rows in that phase are contiguous. dK/dV sums over the query heads
+// of the group and over queries in a fixed order; nothing is atomic.
+// The MFMA kernels for hd = 64 / 128 live in attention_mfma.hip and take over when they apply.
+#include <algorithm>
+#include "common.h"
+
+#define MAXD 4          // head dims per lane in the lanes-across-dims phase: hd <= 64*MAXD
+
+struct AttnP {
+  int B, T, Hq, Hkv, hd, window;
+  float c2;              // log2(e)/sqrt(hd)
+  float scale;           // 1/sqrt(hd)
+};
+
+__device__ __forceinline__ int win_lo(int t, int window) { return (window > 0 && t + 1 > window) ? t + 1 - window : 0; }
+
+// dot of q-row (in LDS, broadcast reads) with a key row in global memory
+__device__ __forceinline__ float dot_row(const float *__restrict__ qs, const float *__restrict__ kr, int hd) {
+  float s = 0;
+  if ((hd & 3) == 0) {
+    for (int d = 0; d < hd; d += 4) {
+      float4 kv = *reinterpret_cast<const float4 *>(kr + d);
+      s += qs[d] * kv.x + qs[d + 1] * kv.y + qs[d + 2] * kv.z + qs[d + 3] * kv.w;
+    }
+  } else {
+    for (int d = 0; d < hd; d++) s += qs[d] * kr[d];
+  }
+  return s;
+}
+
+// ---- forward ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void attn_fwd_gen(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+                                                    const float *__restrict__ v, float *__restrict__ out,
+                                                    float *__restrict__ lse) {
+  extern __shared__ float sm[];                       // per wave: q[hd] + p[64]
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  float *qs = sm + wave * (p.hd + WAVE), *ps = qs + p.hd;
+  int64_t rid = (int64_t)blockIdx.x * 4 + wave;       // (b, h, t), t fastest
+  if (rid >= (int64_t)p.B * p.Hq * p.T) return;
+  const int t = (int)(rid % p.T), h = (int)((rid / p.T) % p.Hq), b = (int)(rid / ((int64_t)p.T * p.Hq));
+  const int kvh = h / (p.Hq / p.Hkv);
+  const size_t qstr = (size_t)p.Hq * p.hd, kstr = (size_t)p.Hkv * p.hd;
+  const float *qr = q + ((size_t)b * p.T + t) * qstr + (size_t)h * p.hd;
+  const float *kb = k + (size_t)b * p.T * kstr + (size_t)kvh * p.hd;
+  const float *vb = v + (size_t)b * p.T * kstr + (size_t)kvh * p.hd;
+  for (int d = lane; d < p.hd; d += WAVE) qs[d] = qr[d] * p.c2;
+  __builtin_amdgcn_wave_barrier();
+  const int s0 = win_lo(t, p.window);
+  // pass 1: row max and sum in the log2 domain, lane-local online then combined
+  float m = -INFINITY, l = 0;
+  for (int s = s0 + lane; s <= t; s += WAVE) {
+    float sc = dot_row(qs, kb + (size_t)s * kstr, p.hd);
+    float mn = fmaxf(m, sc);
+    l = l * exp2f(m - mn) + exp2f(sc - mn);
+    m = mn;
+  }
+  float M = wave_max(m);
+  l = wave_sum(l * exp2f(m - M));                     // lanes with no key: l = 0, exp2(-inf) = 0
+  const float L2 = M + log2f(l);
+  if (lane == 0) lse[rid] = L2;
+  // pass 2: probabilities through LDS, output with lanes across head dims
+  float acc[MAXD] = {0, 0, 0, 0};
+  for (int base = s0; base <= t; base += WAVE) {
+    int s = base + lane;
+    float pr = 0;
+    if (s <= t) pr = exp2f(dot_row(qs, kb + (size_t)s * kstr, p.hd) - L2);
+    __builtin_amdgcn_wave_barrier();
+    ps[lane] = pr;
+    __builtin_amdgcn_wave_barrier();
+    int cnt = min(WAVE, t - base + 1);
+    for (int j = 0; j < cnt; j++) {
+      float pj = ps[j];
+      const float *vr = vb + (size_t)(base + j) * kstr;
+#pragma unroll
+      for (int i = 0; i < MAXD; i++) { int d = lane + i * WAVE; if (d < p.hd) acc[i] += pj * vr[d]; }
+    }
+  }
+  float *orow = out + ((size_t)b * p.T + t) * qstr + (size_t)h * p.hd;
+#pragma unroll
+  for (int i = 0; i < MAXD; i++) { int d = lane + i * WAVE; if (d < p.hd) orow[d] = acc[i]; }
+}
+
+// D[b,h,t] = sum_d dO*O  (srcAttnBwdD, wgsl.ts:711-730)
+__global__ __launch_bounds__(256) void attn_bwd_d(AttnP p, const float *__restrict__ o, const float *__restrict__ go,
+                                                  float *__restrict__ Dr) {
+  const int lane = threadIdx.x % WAVE;
+  int64_t rid = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  if (rid >= (int64_t)p.B * p.Hq * p.T) return;
+  const int t = (int)(rid % p.T), h = (int)((rid / p.T) % p.Hq), b = (int)(rid / ((int64_t)p.T * p.Hq));
+  size_t off = ((size_t)b * p.T + t) * p.Hq * p.hd + (size_t)h * p.hd;
+  float s = 0;
+  for (int d = lane; d < p.hd; d += WAVE) s += o[off + d] * go[off + d];
+  s = wave_sum(s);
+  if (lane == 0) Dr[rid] = s;
+}
+
+// ---- dQ: one wavefront per query row (srcAttnBwdDq, wgsl.ts:741-784) -----------------------------
+__global__ __launch_bounds__(256) void attn_bwd_dq_gen(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+                                                       const float *__restrict__ v, const float *__restrict__ go,
+                                                       const float *__restrict__ lse, const float *__restrict__ Dr,
+                                                       float *dq, int acc_q) {
+  extern __shared__ float sm[];                       // per wave: q[hd] + dO[hd] + ds[64]
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  float *qs = sm + wave * (2 * p.hd + WAVE), *gs = qs + p.hd, *ds = gs + p.hd;
+  int64_t rid = (int64_t)blockIdx.x * 4 + wave;
+  if (rid >= (int64_t)p.B * p.Hq * p.T) return;
+  const int t = (int)(rid % p.T), h = (int)((rid / p.T) % p.Hq), b = (int)(rid / ((int64_t)p.T * p.Hq));
+  const int kvh = h / (p.Hq / p.Hkv);
+  const size_t qstr = (size_t)p.Hq * p.hd, kstr = (size_t)p.Hkv * p.hd;
+  const size_t qoff = ((size_t)b * p.T + t) * qstr + (size_t)h * p.hd;
+  const float *kb = k + (size_t)b * p.T * kstr + (size_t)kvh * p.hd;
+  const float *vb = v + (size_t)b * p.T * kstr + (size_t)kvh * p.hd;
+  for (int d = lane; d < p.hd; d += WAVE) { qs[d] = q[qoff + d] * p.c2; gs[d] = go[qoff + d]; }
+  __builtin_amdgcn_wave_barrier();
+  const float L2 = lse[rid], Dt = Dr[rid];
+  const int s0 = win_lo(t, p.window);
+  float acc[MAXD] = {0, 0, 0, 0};
+  for (int base = s0; base <= t; base += WAVE) {
+    int s = base + lane;
+    float dsv = 0;
+    if (s <= t) {
+      float pr = exp2f(dot_row(qs, kb + (size_t)s * kstr, p.hd) - L2);
+      float dp = dot_row(gs, vb + (size_t)s * kstr, p.hd);
+      dsv = pr * (dp - Dt) * p.scale;
+    }
+    __builtin_amdgcn_wave_barrier();
+    ds[lane] = dsv;
+    __builtin_amdgcn_wave_barrier();
+    int cnt = min(WAVE, t - base + 1);
+    for (int j = 0; j < cnt; j++) {
+      float dj = ds[j];
+      const float *kr = kb + (size_t)(base + j) * kstr;
+#pragma unroll
+      for (int i = 0; i < MAXD; i++) { int d = lane + i * WAVE; if (d < p.hd) acc[i] += dj * kr[d]; }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MAXD; i++) {
+    int d = lane + i * WAVE;
+    if (d < p.hd) dq[qoff + d] = acc_q ? dq[qoff + d] + acc[i] : acc[i];
+  }
+}
+
+// ---- dK, dV: one wavefront per key row, summed over the group's query heads
+// (srcAttnBwdDkv, wgsl.ts:804-918) ---------------------------------------------------------------
+__global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+                                                        const float *__restrict__ v, const float *__restrict__ go,
+                                                        const float *__restrict__ lse, const float *__restrict__ Dr,
+                                                        float *dk, int acc_k, float *dv, int acc_v) {
+  extern __shared__ float sm[];                       // per wave: k[hd] + v[hd] + p[64] + ds[64]
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  float *ks = sm + wave * (2 * p.hd + 2 * WAVE), *vs = ks + p.hd, *ps = vs + p.hd, *ds = ps + WAVE;
+  int64_t rid = (int64_t)blockIdx.x * 4 + wave;       // (b, kvh, s), s fastest
+  if (rid >= (int64_t)p.B * p.Hkv * p.T) return;
+  const int s = (int)(rid % p.T), kvh = (int)((rid / p.T) % p.Hkv), b = (int)(rid / ((int64_t)p.T * p.Hkv));
+  const int group = p.Hq / p.Hkv;
+  const size_t qstr = (size_t)p.Hq * p.hd, kstr = (size_t)p.Hkv * p.hd;
+  const size_t koff = ((size_t)b * p.T + s) * kstr + (size_t)kvh * p.hd;
+  for (int d = lane; d < p.hd; d += WAVE) { ks[d] = k[koff + d] * p.c2; vs[d] = v[koff + d]; }
+  __builtin_amdgcn_wave_barrier();
+  // queries that see key s: t in [s, min(T-1, s+window-1)]
+  const int t1 = p.window > 0 ? min(p.T - 1, s + p.window - 1) : p.T - 1;
+  float ak[MAXD] = {0, 0, 0, 0}, av[MAXD] = {0, 0, 0, 0};
+  for (int hh = 0; hh < group; hh++) {
+    const int h = kvh * group + hh;
+    const float *qb = q + (size_t)b * p.T * qstr + (size_t)h * p.hd;
+    const float *gb = go + (size_t)b * p.T * qstr + (size_t)h * p.hd;
+    const float *lb = lse + ((size_t)b * p.Hq + h) * p.T, *db = Dr + ((size_t)b * p.Hq + h) * p.T;
+    for (int base = s; base <= t1; base += WAVE) {
+      int t = base + lane;
+      float pr = 0, dsv = 0;
+      if (t <= t1) {
+        pr = exp2f(dot_row(ks, qb + (size_t)t * qstr, p.hd) - lb[t]);
+        float dp = dot_row(vs, gb + (size_t)t * qstr, p.hd);
+        dsv = pr * (dp - db[t]) * p.scale;
+      }
+      __builtin_amdgcn_wave_barrier();
+      ps[lane] = pr;
+      ds[lane] = dsv;
+      __builtin_amdgcn_wave_barrier();
+      int cnt = min(WAVE, t1 - base + 1);
+      for (int j = 0; j < cnt; j++) {
+        float pj = ps[j], dj = ds[j];
+        const float *gr = gb + (size_t)(base + j) * qstr, *qr = qb + (size_t)(base + j) * qstr;
+#pragma unroll
+        for (int i = 0; i < MAXD; i++) {
+          int d = lane + i * WAVE;
+          if (d < p.hd) { av[i] += pj * gr[d]; ak[i] += dj * qr[d]; }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MAXD; i++) {
+    int d = lane + i * WAVE;
+    if (d < p.hd) {
+      dk[koff + d] = acc_k ? dk[koff + d] + ak[i] : ak[i];
+      dv[koff + d] = acc_v ? dv[koff + d] + av[i] : av[i];
+    }
+  }
+}
+
+int attn_mfma_supported(int hd);
+int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
+int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
+                  gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+
+static int check(gt_ctx *ctx, const char *who, int B, int T, int Hq, int Hkv, int hd, int window) {
+  GT_REQUIRE(ctx, B >= 1 && T >= 1 && Hq >= 1 && Hkv >= 1 && hd >= 1 && window >= 0, "%s: bad shape", who);
+  GT_REQUIRE(ctx, Hq % Hkv == 0, "%s: %d query heads do not group over %d kv heads", who, Hq, Hkv);
+  GT_REQUIRE(ctx, hd <= WAVE * MAXD, "%s: head dim %d exceeds %d", who, hd, WAVE * MAXD);
+  return 0;
+}
+
+static bool g_no_mfma = false;
+
+extern "C" {
+int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                gt_buf lse) {
+  GT_ENTER(ctx);
+  if (check(ctx, "gt_attn_fwd", B, T, Hq, Hkv, hd, window)) return 1;
+  GT_REQUIRE(ctx, q && k && v && out && lse, "gt_attn_fwd: null operand");
+  AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd)};
+  ProfScope ps(ctx, "attention");
+  static bool env = (g_no_mfma = getenv("GGUFHIP_ATTN_GENERIC") != nullptr, true);
+  (void)env;
+  if (!g_no_mfma && attn_mfma_supported(hd)) return attn_fwd_mfma(ctx, p, q, k, v, out, lse);
+  int64_t rows = (int64_t)B * Hq * T;
+  size_t smem = 4 * (size_t)(hd + WAVE) * sizeof(float);
+  hipLaunchKernelGGL(attn_fwd_gen, dim3((unsigned)cdiv(rows, 4)), dim3(256), smem, ctx->stream, p, P<const float>(q),
+                     P<const float>(k), P<const float>(v), P<float>(out), P<float>(lse));
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                gt_buf dout, gt_buf lse, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+  GT_ENTER(ctx);
+  if (check(ctx, "gt_attn_bwd", B, T, Hq, Hkv, hd, window)) return 1;
+  GT_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, "gt_attn_bwd: null operand");
+  AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd)};
+  int64_t rows = (int64_t)B * Hq * T, krows = (int64_t)B * Hkv * T;
+  void *ws;
+  if (gt_ws_reserve(ctx, (size_t)rows * sizeof(float), &ws)) return 1;
+  float *Dr = static_cast<float *>(ws);
+  {
+    ProfScope ps(ctx, "attention.bwdD");
+    hipLaunchKernelGGL(attn_bwd_d, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, p, P<const float>(out),
+                       P<const float>(dout), Dr);
+    GT_LAUNCHED(ctx);
+  }
+  if (!g_no_mfma && attn_mfma_supported(hd)) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, dq, acc_q, dk, acc_k, dv, acc_v);
+  {
+    ProfScope ps(ctx, "attention.bwdDq");
+    size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);
+    hipLaunchKernelGGL(attn_bwd_dq_gen, dim3((unsigned)cdiv(rows, 4)), dim3(256), smem, ctx->stream, p, P<const float>(q),
+                       P<const float>(k), P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q);
+    GT_LAUNCHED(ctx);
+  }
+  {
+    ProfScope ps(ctx, "attention.bwdDkv");
+    size_t smem = 4 * (size_t)(2 * hd + 2 * WAVE) * sizeof(float);
+    hipLaunchKernelGGL(attn_bwd_dkv_gen, dim3((unsigned)cdiv(krows, 4)), dim3(256), smem, ctx->stream, p, P<const float>(q),
+                       P<const float>(k), P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k,
+                       P<float>(dv), acc_v);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
+}

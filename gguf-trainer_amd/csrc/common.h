@@ -1,0 +1,98 @@
+// Shared by every translation unit of libggufhip: the context, error plumbing, launch helpers
+// and wavefront (64-lane) reductions. gfx950 only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/ggufhip.h"
+
+#define WAVE 64
+
+struct ProfEvent { std::string label; hipEvent_t a, b; };
+
+struct gt_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  char err[512] = {0};
+  char name[256] = {0};
+  int num_cu = 256;
+  uint64_t live_bytes = 0;
+  std::map<uint64_t, size_t> allocs;
+  // grow-only scratch for kernels that need more than inputs and outputs (split-K partials,
+  // per-block dw partials, embedding sort keys). One stream => one user at a time.
+  void *ws = nullptr; size_t ws_bytes = 0;
+  // RoPE cos/sin tables keyed by (T, hd, base, pos): computed once in f64, kept as f32.
+  struct RopeKey { int T, hd, pos; double base; bool operator<(const RopeKey &o) const {
+    if (T != o.T) return T < o.T; if (hd != o.hd) return hd < o.hd; if (pos != o.pos) return pos < o.pos; return base < o.base; } };
+  std::map<RopeKey, float *> rope_tables;
+  bool prof_on = false;
+  std::vector<ProfEvent> prof;
+};
+
+extern thread_local char g_create_err[512];
+
+#define GT_FAIL(ctx, ...) do { snprintf((ctx)->err, sizeof((ctx)->err), __VA_ARGS__); return 1; } while (0)
+#define GT_HIP(ctx, call) do { hipError_t e_ = (call); if (e_ != hipSuccess) { \
+  snprintf((ctx)->err, sizeof((ctx)->err), "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+  return 1; } } while (0)
+// after a launch: a bad configuration shows here, a fault inside the kernel at the next sync
+#define GT_LAUNCHED(ctx) GT_HIP(ctx, hipGetLastError())
+#define GT_ENTER(ctx) do { if (!(ctx)) return 1; GT_HIP(ctx, hipSetDevice((ctx)->device)); } while (0)
+#define GT_REQUIRE(ctx, cond, ...) do { if (!(cond)) GT_FAIL(ctx, __VA_ARGS__); } while (0)
+
+int gt_ws_reserve(gt_ctx *ctx, size_t bytes, void **out);
+
+// Brackets the launches made during its lifetime with a pair of events when profiling is on.
+struct ProfScope {
+  gt_ctx *c; bool on;
+  ProfScope(gt_ctx *ctx, const char *label) : c(ctx), on(ctx->prof_on) {
+    if (!on) return;
+    ProfEvent e; e.label = label;
+    (void)hipEventCreate(&e.a); (void)hipEventCreate(&e.b);
+    (void)hipEventRecord(e.a, c->stream);
+    c->prof.push_back(e);
+  }
+  ~ProfScope() { if (on) (void)hipEventRecord(c->prof.back().b, c->stream); }
+};
+
+template <typename T> static inline T *P(gt_buf b) { return reinterpret_cast<T *>(b); }
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+// Sum over a block of NW wavefronts; every thread gets the result. `sm` holds NW floats.
+template <int NW> __device__ __forceinline__ float block_sum(float v, float *sm) {
+  v = wave_sum(v);
+  int w = threadIdx.x / WAVE, l = threadIdx.x % WAVE;
+  __syncthreads();
+  if (l == 0) sm[w] = v;
+  __syncthreads();
+  float r = 0;
+#pragma unroll
+  for (int i = 0; i < NW; i++) r += sm[i];
+  return r;
+}
+template <int NW> __device__ __forceinline__ float block_max(float v, float *sm) {
+  v = wave_max(v);
+  int w = threadIdx.x / WAVE, l = threadIdx.x % WAVE;
+  __syncthreads();
+  if (l == 0) sm[w] = v;
+  __syncthreads();
+  float r = sm[0];
+#pragma unroll
+  for (int i = 1; i < NW; i++) r = fmaxf(r, sm[i]);
+  return r;
+}

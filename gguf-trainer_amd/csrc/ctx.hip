@@ -1,0 +1,171 @@
+// Context, device memory, transfers, profiling records.
+#include "common.h"
+
+thread_local char g_create_err[512] = {0};
+
+extern "C" {
+
+int gt_ctx_create(int device, gt_ctx **out) {
+  if (!out) return 1;
+  *out = nullptr;
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n <= 0) {
+    snprintf(g_create_err, sizeof g_create_err, "no HIP device available (%s)", hipGetErrorString(e));
+    return 1;
+  }
+  if (device < 0 || device >= n) {
+    snprintf(g_create_err, sizeof g_create_err, "device %d out of range (%d visible)", device, n);
+    return 1;
+  }
+  gt_ctx *c = new gt_ctx();
+  c->device = device;
+  hipDeviceProp_t p;
+  if ((e = hipSetDevice(device)) != hipSuccess || (e = hipGetDeviceProperties(&p, device)) != hipSuccess ||
+      (e = hipStreamCreate(&c->stream)) != hipSuccess) {
+    snprintf(g_create_err, sizeof g_create_err, "context setup failed: %s", hipGetErrorString(e));
+    delete c;
+    return 1;
+  }
+  snprintf(c->name, sizeof c->name, "%s (%s, %d CUs)", p.name, p.gcnArchName, p.multiProcessorCount);
+  c->num_cu = p.multiProcessorCount;
+  if (strncmp(p.gcnArchName, "gfx950", 6) != 0) {
+    snprintf(g_create_err, sizeof g_create_err, "libggufhip is built for gfx950 only; device is %s", p.gcnArchName);
+    hipStreamDestroy(c->stream);
+    delete c;
+    return 1;
+  }
+  *out = c;
+  return 0;
+}
+
+int gt_ctx_destroy(gt_ctx *ctx) {
+  if (!ctx) return 0;
+  hipSetDevice(ctx->device);
+  hipStreamSynchronize(ctx->stream);
+  for (auto &kv : ctx->allocs) hipFree(reinterpret_cast<void *>(kv.first));
+  for (auto &kv : ctx->rope_tables) hipFree(kv.second);
+  if (ctx->ws) hipFree(ctx->ws);
+  for (auto &e : ctx->prof) { hipEventDestroy(e.a); hipEventDestroy(e.b); }
+  hipStreamDestroy(ctx->stream);
+  delete ctx;
+  return 0;
+}
+
+const char *gt_last_error(gt_ctx *ctx) { return ctx ? ctx->err : g_create_err; }
+const char *gt_device_name(gt_ctx *ctx) { return ctx ? ctx->name : ""; }
+
+int gt_alloc(gt_ctx *ctx, size_t bytes, int zero, gt_buf *out) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, out, "gt_alloc: out is NULL");
+  void *p = nullptr;
+  size_t sz = bytes ? bytes : 4;
+  GT_HIP(ctx, hipMalloc(&p, sz));
+  if (zero) GT_HIP(ctx, hipMemsetAsync(p, 0, sz, ctx->stream));
+  ctx->allocs[reinterpret_cast<uint64_t>(p)] = sz;
+  ctx->live_bytes += sz;
+  *out = reinterpret_cast<uint64_t>(p);
+  return 0;
+}
+
+int gt_free(gt_ctx *ctx, gt_buf buf) {
+  GT_ENTER(ctx);
+  auto it = ctx->allocs.find(buf);
+  GT_REQUIRE(ctx, it != ctx->allocs.end(), "gt_free: %llx was not returned by gt_alloc", (unsigned long long)buf);
+  GT_HIP(ctx, hipStreamSynchronize(ctx->stream));      // nothing queued may still touch it
+  GT_HIP(ctx, hipFree(reinterpret_cast<void *>(buf)));
+  ctx->live_bytes -= it->second;
+  ctx->allocs.erase(it);
+  return 0;
+}
+
+int gt_memset0(gt_ctx *ctx, gt_buf buf, size_t bytes) {
+  GT_ENTER(ctx);
+  ProfScope ps(ctx, "clear");
+  if (bytes) GT_HIP(ctx, hipMemsetAsync(P<void>(buf), 0, bytes, ctx->stream));
+  return 0;
+}
+
+int gt_h2d(gt_ctx *ctx, gt_buf dst, const void *src, size_t bytes) {
+  GT_ENTER(ctx);
+  // pageable source: the runtime stages it before returning, so the caller may reuse src at once
+  if (bytes) GT_HIP(ctx, hipMemcpyAsync(P<void>(dst), src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  return 0;
+}
+
+int gt_d2h(gt_ctx *ctx, void *dst, gt_buf src, size_t bytes) {
+  GT_ENTER(ctx);
+  if (bytes) GT_HIP(ctx, hipMemcpyAsync(dst, P<void>(src), bytes, hipMemcpyDeviceToHost, ctx->stream));
+  GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return 0;
+}
+
+int gt_d2d(gt_ctx *ctx, gt_buf dst, gt_buf src, size_t bytes) {
+  GT_ENTER(ctx);
+  ProfScope ps(ctx, "copy");
+  if (bytes) GT_HIP(ctx, hipMemcpyAsync(P<void>(dst), P<void>(src), bytes, hipMemcpyDeviceToDevice, ctx->stream));
+  return 0;
+}
+
+int gt_sync(gt_ctx *ctx) {
+  GT_ENTER(ctx);
+  GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return 0;
+}
+
+int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes) {
+  if (!ctx || !bytes) return 1;
+  *bytes = ctx->live_bytes + ctx->ws_bytes;
+  return 0;
+}
+
+int gt_prof_begin(gt_ctx *ctx) {
+  GT_ENTER(ctx);
+  for (auto &e : ctx->prof) { hipEventDestroy(e.a); hipEventDestroy(e.b); }
+  ctx->prof.clear();
+  ctx->prof_on = true;
+  return 0;
+}
+
+int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n) {
+  GT_ENTER(ctx);
+  ctx->prof_on = false;
+  GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  std::map<std::string, std::pair<double, int64_t>> sum;
+  std::vector<std::string> order;
+  for (auto &e : ctx->prof) {
+    float ms = 0;
+    GT_HIP(ctx, hipEventElapsedTime(&ms, e.a, e.b));
+    if (!sum.count(e.label)) order.push_back(e.label);
+    sum[e.label].first += ms;
+    sum[e.label].second += 1;
+    hipEventDestroy(e.a); hipEventDestroy(e.b);
+  }
+  ctx->prof.clear();
+  int k = 0;
+  for (auto &l : order) {
+    if (k >= cap) break;
+    snprintf(out[k].label, sizeof out[k].label, "%s", l.c_str());
+    out[k].ms = sum[l].first;
+    out[k].count = sum[l].second;
+    k++;
+  }
+  if (n) *n = k;
+  return 0;
+}
+
+}  // extern "C"
+
+int gt_ws_reserve(gt_ctx *ctx, size_t bytes, void **out) {
+  if (bytes > ctx->ws_bytes) {
+    // queued kernels may still read the old block
+    GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->ws) GT_HIP(ctx, hipFree(ctx->ws));
+    ctx->ws = nullptr; ctx->ws_bytes = 0;
+    size_t sz = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    GT_HIP(ctx, hipMalloc(&ctx->ws, sz));
+    ctx->ws_bytes = sz;
+  }
+  *out = ctx->ws;
+  return 0;
+}

@@ -1,0 +1,162 @@
+// Embedding gather / scatter-add (srcEmbeddingFwd / Bwd, src/backend/wgsl.ts:305-344) and RoPE
+// (srcRope, wgsl.ts:346-384).
+//
+// Embedding backward. The reference gives one thread to every (vocab row, column) and scans all T
+// ids: V*d*T work. Here the ids are ranked on the device (a stable counting rank, O(T^2) integer
+// compares over LDS-staged tiles), which yields the tokens grouped by id in position order; one
+// workgroup per distinct id then sums that id's gradient rows in that fixed order and adds the
+// sum to its dW row. No atomics, no dependence on launch timing, repeated ids (Zipf) included.
+//
+// RoPE. cos/sin per (position, pair) are computed once per (T, hd, base, pos) in f64 and kept as
+// an f32 table in the context, like the reference CPU op's precomputed Float32Array tables
+// (src/model/autograd.ts:590-601); evaluating pow/cos/sin in f32 per element, as the WGSL does,
+// loses ~1e-4 at position 2047.
+#include <algorithm>
+#include "common.h"
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void embedding_fwd_k(int rows, int d, const int *__restrict__ ids,
+                                                       const float *__restrict__ W, float *__restrict__ out) {
+  // one wavefront per row, float4 when d % 4 == 0
+  const int lane = threadIdx.x % WAVE;
+  int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  if (row >= rows) return;
+  const float *src = W + (size_t)ids[row] * d;
+  float *dst = out + row * d;
+  if (d % 4 == 0) {
+    for (int j = lane; j < d / 4; j += WAVE) reinterpret_cast<v4f *>(dst)[j] = reinterpret_cast<const v4f *>(src)[j];
+  } else {
+    for (int j = lane; j < d; j += WAVE) dst[j] = src[j];
+  }
+}
+
+// pos[t] = #{t' : id[t'] < id[t]} + #{t' < t : id[t'] == id[t]}: the stable sorted position.
+__global__ __launch_bounds__(256) void rank_ids_k(int n, const int *__restrict__ ids, int *__restrict__ order,
+                                                  int *__restrict__ sorted) {
+  __shared__ int tile[256];
+  int t = blockIdx.x * 256 + threadIdx.x;
+  int mine = t < n ? ids[t] : 0x7fffffff;
+  int pos = 0;
+  for (int base = 0; base < n; base += 256) {
+    int j = base + threadIdx.x;
+    __syncthreads();
+    tile[threadIdx.x] = j < n ? ids[j] : 0x7fffffff;
+    __syncthreads();
+    int lim = min(256, n - base);
+    for (int q = 0; q < lim; q++) {
+      int o = tile[q];
+      pos += (o < mine) || (o == mine && base + q < t);
+    }
+  }
+  if (t < n) { order[pos] = t; sorted[pos] = mine; }
+}
+
+// one workgroup per sorted slot; only the first slot of each id does work
+__global__ __launch_bounds__(256) void embedding_bwd_k(int n, int d, const int *__restrict__ order,
+                                                       const int *__restrict__ sorted, const float *__restrict__ g,
+                                                       float *dW) {
+  int p = blockIdx.x;
+  int id = sorted[p];
+  if (p > 0 && sorted[p - 1] == id) return;
+  int e = p + 1;
+  while (e < n && sorted[e] == id) e++;
+  float *dst = dW + (size_t)id * d;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    float s = 0;
+    for (int q = p; q < e; q++) s += g[(size_t)order[q] * d + c];
+    dst[c] += s;
+  }
+}
+
+// ---- RoPE ------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void rope_table_k(int T, int hd, double base, int pos, float *__restrict__ tab) {
+  int half = hd / 2;
+  int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= T * half) return;
+  int t = i / half, j = i % half;
+  double freq = pow(base, (-2.0 * j) / hd);
+  double ang = (double)(t + pos) * freq;
+  tab[2 * i] = (float)cos(ang);
+  tab[2 * i + 1] = (float)sin(ang);
+}
+
+template <bool BWD>
+__global__ __launch_bounds__(256) void rope_k(int64_t npairs, int T, int H, int hd, const float2 *__restrict__ tab,
+                                              const float *__restrict__ in, float *out, int acc) {
+  int half = hd / 2;
+  int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < npairs; i += stride) {
+    int j = (int)(i % half);
+    int64_t rh = i / half;                        // row*H + h
+    int64_t row = rh / H;
+    int t = (int)(row % T);
+    float2 cs = tab[(size_t)t * half + j];
+    int64_t b = rh * hd + j;
+    float a0 = in[b], a1 = in[b + half], o0, o1;
+    if (!BWD) { o0 = a0 * cs.x - a1 * cs.y; o1 = a0 * cs.y + a1 * cs.x; }
+    else { o0 = cs.x * a0 + cs.y * a1; o1 = -cs.y * a0 + cs.x * a1; }
+    if (acc) { o0 += out[b]; o1 += out[b + half]; }
+    out[b] = o0;
+    out[b + half] = o1;
+  }
+}
+
+extern "C" {
+int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, gt_buf ids, gt_buf W, gt_buf out) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && ids && W && out, "gt_embedding_fwd: bad arguments");
+  if (rows == 0) return 0;
+  ProfScope ps(ctx, "embedding");
+  hipLaunchKernelGGL(embedding_fwd_k, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, rows, d, P<const int>(ids),
+                     P<const float>(W), P<float>(out));
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, gt_buf dW, int acc) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && V >= 1 && ids && g && dW, "gt_embedding_bwd: bad arguments");
+  ProfScope ps(ctx, "embedding.bwd");
+  if (!acc) GT_HIP(ctx, hipMemsetAsync(P<void>(dW), 0, (size_t)V * d * sizeof(float), ctx->stream));
+  if (rows == 0) return 0;
+  void *ws;
+  if (gt_ws_reserve(ctx, (size_t)rows * 2 * sizeof(int), &ws)) return 1;
+  int *order = static_cast<int *>(ws), *sorted = order + rows;
+  hipLaunchKernelGGL(rank_ids_k, dim3((unsigned)cdiv(rows, 256)), dim3(256), 0, ctx->stream, rows, P<const int>(ids), order, sorted);
+  GT_LAUNCHED(ctx);
+  hipLaunchKernelGGL(embedding_bwd_k, dim3((unsigned)rows), dim3(256), 0, ctx->stream, rows, d, order, sorted,
+                     P<const float>(g), P<float>(dW));
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, int backward, gt_buf in, gt_buf out, int acc) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && T >= 1 && H >= 1 && hd >= 2 && hd % 2 == 0 && in && out, "gt_rope: bad arguments (hd %d)", hd);
+  GT_REQUIRE(ctx, rows % T == 0, "gt_rope: rows %d is not a whole number of sequences of %d", rows, T);
+  if (rows == 0) return 0;
+  ProfScope ps(ctx, backward ? "rope.bwd" : "rope");
+  gt_ctx::RopeKey key{T, hd, pos, base};
+  auto it = ctx->rope_tables.find(key);
+  float *tab;
+  if (it == ctx->rope_tables.end()) {
+    int n = T * (hd / 2);
+    GT_HIP(ctx, hipMalloc(reinterpret_cast<void **>(&tab), (size_t)n * 2 * sizeof(float)));
+    hipLaunchKernelGGL(rope_table_k, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, T, hd, base, pos, tab);
+    GT_LAUNCHED(ctx);
+    ctx->rope_tables[key] = tab;
+  } else tab = it->second;
+  int64_t npairs = (int64_t)rows * H * (hd / 2);
+  unsigned nb = (unsigned)std::min<int64_t>(cdiv(npairs, 256), (int64_t)ctx->num_cu * 16);
+  if (backward)
+    hipLaunchKernelGGL((rope_k<true>), dim3(nb), dim3(256), 0, ctx->stream, npairs, T, H, hd, reinterpret_cast<const float2 *>(tab),
+                       P<const float>(in), P<float>(out), acc);
+  else
+    hipLaunchKernelGGL((rope_k<false>), dim3(nb), dim3(256), 0, ctx->stream, npairs, T, H, hd, reinterpret_cast<const float2 *>(tab),
+                       P<const float>(in), P<float>(out), acc);
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+}

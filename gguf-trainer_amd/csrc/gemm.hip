@@ -1,0 +1,299 @@
+// FP32 GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32), the contraction behind
+// linear forward (NT), dX = dY.W (NN) and dW = dY^T.X (TN), the chunked-CE readout and the
+// Newton-Schulz products. Replaces srcGemm (src/backend/wgsl.ts:87-196).
+//
+// Shape of the kernel. A workgroup of WM x WN wavefronts owns a BM x BN tile of C and walks K in
+// steps of 16. Each wavefront owns a (BM/WM) x (BN/WN) sub-tile as TM x TN MFMA tiles of 32x32,
+// 16 accumulator VGPRs each. Global loads for step i+1 are issued into registers before the
+// MFMAs of step i and stored to LDS after them, so HBM/L2 latency hides under 32+ MFMAs.
+//
+// LDS layouts. An operand whose K index is contiguous in memory (A of NT/NN, B of NT) is kept as
+// [row][16+4]: the float4 read from global is written as one ds_write_b128 and a lane fetches its
+// MFMA inputs for four consecutive steps with one ds_read_b128 (row stride 20 words makes every
+// 8-lane group of a b128 read touch all 32 banks). An operand whose row index is contiguous
+// (A of TN, B of NN/TN) is kept as [k][rows] and fetched with ds_read_b32, consecutive lanes on
+// consecutive banks. Because an MFMA step consumes K pairs (lane/32 selects which), the order in
+// which K is consumed is free as long as A and B agree: inside every run of 8, lane group g takes
+// k = 4g + i at step i, which is what lets the b128 fetch feed four steps.
+//
+// dW has a small output and a long K (rows of the batch), so it is split along K over blockIdx.z
+// into per-split partial tiles in the workspace, summed in split order by a second kernel: no
+// atomics, bit-identical from run to run.
+#include <algorithm>
+#include "common.h"
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+#define BK 16
+#define KS 20   // LDS row stride (words) of a k-contiguous operand tile
+
+struct GemmArgs {
+  const float *A, *B;
+  float *C;
+  int M, N, K;
+  int lda, ldb, ldc;
+  int acc;
+  int kchunk;              // K range per blockIdx.z when splitting (multiple of BK), else K
+  int splits;              // >1: write partials to P[z][M][N]
+  float *Pp;
+  int64_t sA, sB, sC;      // batch strides (elements); batch index = blockIdx.z when splits == 1
+  int nbm, nbn;
+};
+
+// One operand tile of R rows x 16 k. KC: k contiguous in memory (element (r,k) at p[r*ld + k]);
+// otherwise row contiguous (element (r,k) at p[k*ld + r]).
+template <int R, bool KC, bool VEC, int NT>
+struct Tile {
+  static constexpr int UNITS = R * 4;          // float4 units per tile
+  static constexpr int PER = UNITS / NT;       // per thread
+  static_assert(UNITS % NT == 0, "tile rows must be a multiple of threads/4");
+  static constexpr int LDS_WORDS = KC ? R * KS : BK * R;
+
+  // registers <- global, zero outside [0,Rtot) x [k0,kend)
+  __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ p, int ld, int r0, int Rtot,
+                                              int k0, int kend, int tid) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      int u = tid + i * NT;
+      v4f v = {0.f, 0.f, 0.f, 0.f};
+      if (KC) {
+        int r = r0 + u / 4, k = k0 + (u % 4) * 4;
+        if (r < Rtot) {
+          const float *q = p + (size_t)r * ld + k;
+          if (VEC) { if (k < kend) v = *reinterpret_cast<const v4f *>(q); }
+          else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) if (k + j < kend) v[j] = q[j];
+          }
+        }
+      } else {
+        int k = k0 + u / (R / 4), r = r0 + (u % (R / 4)) * 4;
+        if (k < kend) {
+          const float *q = p + (size_t)k * ld + r;
+          if (VEC) { if (r < Rtot) v = *reinterpret_cast<const v4f *>(q); }
+          else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) if (r + j < Rtot) v[j] = q[j];
+          }
+        }
+      }
+      reg[i] = v;
+    }
+  }
+  __device__ static __forceinline__ void store(const v4f (&reg)[PER], float *lds, int tid) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      int u = tid + i * NT;
+      if (KC) *reinterpret_cast<v4f *>(lds + (u / 4) * KS + (u % 4) * 4) = reg[i];
+      else *reinterpret_cast<v4f *>(lds + (u / (R / 4)) * R + (u % (R / 4)) * 4) = reg[i];
+    }
+  }
+  // MFMA inputs of this lane for the four steps of K-run c (0 or 1): row = tile row, g = lane/32
+  __device__ static __forceinline__ v4f fetch(const float *lds, int row, int c, int g) {
+    if (KC) return *reinterpret_cast<const v4f *>(lds + row * KS + c * 8 + g * 4);
+    v4f v;
+    const float *q = lds + (c * 8 + g * 4) * R + row;
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = q[j * R];
+    return v;
+  }
+};
+
+template <int BM, int BN, int WM, int WN, int KIND, bool VEC>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be whole MFMA tiles");
+  constexpr bool AKC = (KIND != GT_TN), BKC = (KIND == GT_NT);
+  using TA = Tile<BM, AKC, VEC, NT>;
+  using TB = Tile<BN, BKC, VEC, NT>;
+  __shared__ __attribute__((aligned(16))) float sA[TA::LDS_WORDS];
+  __shared__ __attribute__((aligned(16))) float sB[TB::LDS_WORDS];
+
+  // Workgroup i runs on XCD i mod 8, each XCD with its own L2. Renumber so that one XCD walks a
+  // contiguous range of tiles (N fastest): neighbours then share their A row panel in that L2.
+  int nblk = a.nbm * a.nbn;
+  int pid = blockIdx.x;
+  {
+    int xcd = pid % 8, idx = pid / 8, base = nblk / 8, rem = nblk % 8;
+    pid = xcd * base + (xcd < rem ? xcd : rem) + idx;
+  }
+  const int pm = pid / a.nbn, pn = pid % a.nbn;
+  const int m0 = pm * BM, n0 = pn * BN;
+  const int z = blockIdx.z;
+  const float *A = a.A, *B = a.B;
+  int k0 = 0, kend = a.K;
+  if (a.splits > 1) { k0 = z * a.kchunk; kend = min(a.K, k0 + a.kchunk); }
+  else { A += z * a.sA; B += z * a.sB; }
+
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int wm = wave / WN, wn = wave % WN;
+  const int g = lane / 32, l32 = lane % 32;
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  v4f ra[TA::PER], rb[TB::PER];
+  TA::load(ra, A, a.lda, m0, a.M, k0, kend, tid);
+  TB::load(rb, B, a.ldb, n0, a.N, k0, kend, tid);
+
+  for (int k = k0; k < kend; k += BK) {
+    __syncthreads();                       // previous step's LDS reads are done
+    TA::store(ra, sA, tid);
+    TB::store(rb, sB, tid);
+    __syncthreads();
+    if (k + BK < kend) {
+      TA::load(ra, A, a.lda, m0, a.M, k + BK, kend, tid);
+      TB::load(rb, B, a.ldb, n0, a.N, k + BK, kend, tid);
+    }
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      v4f fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[i] = TA::fetch(sA, wm * (TM * 32) + i * 32 + l32, c, g);
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[j] = TB::fetch(sB, wn * (TN * 32) + j * 32 + l32, c, g);
+#pragma unroll
+      for (int s = 0; s < 4; s++)
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // accumulator register r of lane (g,l32) is C[8*(r/4) + 4*g + r%4][l32] of its 32x32 tile
+  float *C;
+  int ldc;
+  bool add;
+  if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
+  else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0; }
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      int col = n0 + wn * (TN * 32) + j * 32 + l32;
+      if (col >= a.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int row = m0 + wm * (TM * 32) + i * 32 + 8 * (r / 4) + 4 * g + (r % 4);
+        if (row < a.M) {
+          float *q = C + (size_t)row * ldc + col;
+          *q = add ? *q + acc[i][j][r] : acc[i][j][r];
+        }
+      }
+    }
+}
+
+// C (+)= sum over splits, in split order
+__global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ Pp, float *__restrict__ C, int64_t n,
+                                                     int splits, int acc) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = Pp[i];
+  for (int z = 1; z < splits; z++) s += Pp[(size_t)z * n + i];
+  C[i] = acc ? C[i] + s : s;
+}
+
+template <int BM, int BN, int WM, int WN>
+static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
+  a.nbm = (int)cdiv(a.M, BM);
+  a.nbn = (int)cdiv(a.N, BN);
+  dim3 grid(a.nbm * a.nbn, 1, zdim), block(WM * WN * 64);
+#define GO(KIND, VEC) hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, KIND, VEC>), grid, block, 0, ctx->stream, a)
+  if (kind == GT_NT) { if (vec) GO(GT_NT, true); else GO(GT_NT, false); }
+  else if (kind == GT_NN) { if (vec) GO(GT_NN, true); else GO(GT_NN, false); }
+  else { if (vec) GO(GT_TN, true); else GO(GT_TN, false); }
+#undef GO
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+static int g_force_cfg = -1;     // tuning hook: GGUFHIP_GEMM_CFG=0..3 pins the tile shape
+
+static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
+                     gt_buf C, int64_t sC, int count) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, kind >= 0 && kind <= 2, "gt_gemm: kind %d is not NT(0)/NN(1)/TN(2)", kind);
+  GT_REQUIRE(ctx, M >= 1 && N >= 1 && K >= 1 && count >= 1, "gt_gemm: M,N,K,count must be >= 1 (got %d,%d,%d,%d)", M, N, K, count);
+  GT_REQUIRE(ctx, A && B && C, "gt_gemm: null operand");
+  ProfScope ps(ctx, kind == GT_NT ? "gemm.nt" : kind == GT_NN ? "gemm.nn" : "gemm.tn");
+  GemmArgs a;
+  a.A = P<const float>(A); a.B = P<const float>(B); a.C = P<float>(C);
+  a.M = M; a.N = N; a.K = K;
+  a.lda = (kind == GT_TN) ? M : K;
+  a.ldb = (kind == GT_NT) ? K : N;
+  a.ldc = N;
+  a.acc = acc; a.kchunk = K; a.splits = 1; a.Pp = nullptr;
+  a.sA = sA; a.sB = sB; a.sC = sC;
+  bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
+             (sA % 4 == 0) && (sB % 4 == 0);
+
+  static bool env_read = false;
+  if (!env_read) { env_read = true; const char *e = getenv("GGUFHIP_GEMM_CFG"); if (e) g_force_cfg = atoi(e); }
+
+  // Tile choice: the largest tile that still gives every CU a few workgroups; narrow N (heads,
+  // LoRA rank) takes the 64-wide tile so columns are not wasted.
+  int cfg;
+  auto blocks = [&](int bm, int bn) { return cdiv(M, bm) * cdiv(N, bn) * count; };
+  if (N <= 64 || M <= 64) cfg = 0;
+  else if (N % 192 == 0 && N % 128 != 0 && blocks(128, 192) >= ctx->num_cu) cfg = 3;
+  else if (blocks(128, 128) >= 2 * ctx->num_cu) cfg = 2;
+  else cfg = 1;
+  if (g_force_cfg >= 0) cfg = g_force_cfg;
+  int bm = cfg == 0 ? 64 : 128, bn = cfg == 0 ? 64 : cfg == 1 ? 64 : cfg == 2 ? 128 : 192;
+
+  // split K when the output alone cannot fill the chip (dW: K = rows of the batch)
+  int splits = 1;
+  if (count == 1) {
+    int64_t nb = blocks(bm, bn);
+    int64_t ksteps = cdiv(K, BK);
+    if (nb < 2 * ctx->num_cu && ksteps >= 16) {
+      splits = (int)std::min<int64_t>(cdiv(3 * ctx->num_cu, nb), ksteps / 8);
+      if (splits < 1) splits = 1;
+      if (splits > 64) splits = 64;
+    }
+  }
+  if (splits > 1) {
+    int64_t kc = cdiv(cdiv(K, splits), BK) * BK;
+    splits = (int)cdiv(K, kc);
+    a.kchunk = (int)kc;
+  }
+  if (splits > 1) {
+    void *ws;
+    if (gt_ws_reserve(ctx, (size_t)splits * M * N * sizeof(float), &ws)) return 1;
+    a.splits = splits; a.Pp = static_cast<float *>(ws);
+  }
+  int zdim = splits > 1 ? splits : count;
+  int rc;
+  switch (cfg) {
+    case 0: rc = launch_cfg<64, 64, 2, 2>(ctx, kind, vec, a, zdim); break;
+    case 1: rc = launch_cfg<128, 64, 2, 2>(ctx, kind, vec, a, zdim); break;
+    case 2: rc = launch_cfg<128, 128, 2, 2>(ctx, kind, vec, a, zdim); break;
+    default: rc = launch_cfg<128, 192, 2, 2>(ctx, kind, vec, a, zdim); break;
+  }
+  if (rc) return rc;
+  if (splits > 1) {
+    int64_t n = (int64_t)M * N;
+    hipLaunchKernelGGL(splitk_reduce, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, a.Pp, a.C, n, splits, acc);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
+
+extern "C" {
+int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_buf B, gt_buf C) {
+  return gemm_impl(ctx, kind, acc, M, N, K, A, 0, B, 0, C, 0, 1);
+}
+int gt_gemm_batched(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t strideA, gt_buf B,
+                    int64_t strideB, gt_buf C, int64_t strideC, int count) {
+  return gemm_impl(ctx, kind, acc, M, N, K, A, strideA, B, strideB, C, strideC, count);
+}
+}

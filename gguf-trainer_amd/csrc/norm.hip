@@ -1,0 +1,263 @@
+// RMSNorm forward and backward (srcRmsNormFwd / BwdX / BwdW, src/backend/wgsl.ts:217-303), also
+// serving per-head QK-norm as rows = T*H, d = hd (src/backend/webgpu.ts:1085-1088).
+//
+// A row is handled by LPR lanes of one wavefront (LPR = 16, 32 or 64, the smallest that keeps
+// float4 per lane useful), so hd = 64 packs four rows per wavefront instead of idling 48 lanes.
+// Backward makes ONE pass over x and g: the row sum S and dx for the row, and per-lane column
+// partials of dw = sum_rows g*x*r kept in registers across the rows a workgroup owns. The
+// partials are reduced across the workgroup in LDS, written as one row per workgroup and summed
+// in workgroup order by a second small kernel: the reference's one-thread-per-column scan
+// (wgsl.ts:286-303) without its strided re-reads, and still deterministic.
+#include <algorithm>
+#include "common.h"
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int LPR> __device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = LPR / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+
+// NJ = float4 chunks per lane: d <= LPR*4*NJ. d % 4 == 0.
+template <int LPR, int NJ>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_k(int rows, int d, float eps, const float *__restrict__ x,
+                                                     const float *__restrict__ w, float *__restrict__ y,
+                                                     float *__restrict__ rinv) {
+  constexpr int RPW = WAVE / LPR;                // rows per wavefront
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int sub = lane / LPR, li = lane % LPR;
+  const int d4 = d / 4;
+  v4f wv[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    int c = li + j * LPR;
+    wv[j] = c < d4 ? reinterpret_cast<const v4f *>(w)[c] : v4f{0, 0, 0, 0};
+  }
+  for (int64_t row = ((int64_t)blockIdx.x * 4 + wave) * RPW + sub; row < rows; row += (int64_t)gridDim.x * 4 * RPW) {
+    const v4f *xr = reinterpret_cast<const v4f *>(x + row * d);
+    v4f xv[NJ];
+    float ss = 0;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+      int c = li + j * LPR;
+      xv[j] = c < d4 ? xr[c] : v4f{0, 0, 0, 0};
+      ss += xv[j][0] * xv[j][0] + xv[j][1] * xv[j][1] + xv[j][2] * xv[j][2] + xv[j][3] * xv[j][3];
+    }
+    ss = group_sum<LPR>(ss);
+    float r = 1.0f / sqrtf(ss / (float)d + eps);
+    if (li == 0) rinv[row] = r;
+    v4f *yr = reinterpret_cast<v4f *>(y + row * d);
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+      int c = li + j * LPR;
+      if (c < d4) yr[c] = xv[j] * r * wv[j];
+    }
+  }
+}
+
+template <int LPR, int NJ>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const float *__restrict__ x,
+                                                     const float *__restrict__ w, const float *__restrict__ g,
+                                                     const float *__restrict__ rinv, float *dx, int acc_dx,
+                                                     float *__restrict__ dw_part) {
+  constexpr int RPW = WAVE / LPR;
+  constexpr int NG = 4 * RPW;                    // row groups per workgroup
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int sub = lane / LPR, li = lane % LPR;
+  const int d4 = d / 4;
+  const float invd = 1.0f / (float)d;
+  v4f wv[NJ], dwv[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    int c = li + j * LPR;
+    wv[j] = c < d4 ? reinterpret_cast<const v4f *>(w)[c] : v4f{0, 0, 0, 0};
+    dwv[j] = v4f{0, 0, 0, 0};
+  }
+  for (int64_t row = ((int64_t)blockIdx.x * 4 + wave) * RPW + sub; row < rows; row += (int64_t)gridDim.x * 4 * RPW) {
+    const v4f *xr = reinterpret_cast<const v4f *>(x + row * d);
+    const v4f *gr = reinterpret_cast<const v4f *>(g + row * d);
+    v4f xv[NJ], gv[NJ];
+    float S = 0;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+      int c = li + j * LPR;
+      bool in = c < d4;
+      xv[j] = in ? xr[c] : v4f{0, 0, 0, 0};
+      gv[j] = in ? gr[c] : v4f{0, 0, 0, 0};
+      v4f t = gv[j] * wv[j] * xv[j];
+      S += t[0] + t[1] + t[2] + t[3];
+    }
+    S = group_sum<LPR>(S);
+    const float r = rinv[row];
+    const float k2 = r * r * r * S * invd;
+    v4f *dxr = reinterpret_cast<v4f *>(dx + row * d);
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+      int c = li + j * LPR;
+      if (c < d4) {
+        v4f o = wv[j] * gv[j] * r - xv[j] * k2;
+        if (acc_dx) o += dxr[c];
+        dxr[c] = o;
+      }
+      dwv[j] += gv[j] * xv[j] * r;
+    }
+  }
+  if (!dw_part) return;
+  // workgroup reduction of the NG row groups' column partials, fixed order
+  extern __shared__ float sm[];                  // [NG][d]
+  const int grp = wave * RPW + sub;
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    int c = li + j * LPR;
+    if (c < d4) reinterpret_cast<v4f *>(sm + (size_t)grp * d)[c] = dwv[j];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < d; c += 256) {
+    float s = 0;
+#pragma unroll
+    for (int q = 0; q < NG; q++) s += sm[(size_t)q * d + c];
+    dw_part[(size_t)blockIdx.x * d + c] = s;
+  }
+}
+
+__global__ __launch_bounds__(256) void colsum_reduce(const float *__restrict__ part, int nparts, int d, float *dw, int acc) {
+  int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= d) return;
+  float s = 0;
+  for (int p = 0; p < nparts; p++) s += part[(size_t)p * d + c];
+  dw[c] = acc ? dw[c] + s : s;
+}
+
+// scalar fallback for d % 4 != 0 or very wide rows: one wavefront per row
+__global__ __launch_bounds__(256) void rmsnorm_fwd_gen(int rows, int d, float eps, const float *__restrict__ x,
+                                                       const float *__restrict__ w, float *__restrict__ y,
+                                                       float *__restrict__ rinv) {
+  const int lane = threadIdx.x % WAVE;
+  int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  if (row >= rows) return;
+  const float *xr = x + row * d;
+  float ss = 0;
+  for (int j = lane; j < d; j += WAVE) ss += xr[j] * xr[j];
+  ss = wave_sum(ss);
+  float r = 1.0f / sqrtf(ss / (float)d + eps);
+  if (lane == 0) rinv[row] = r;
+  for (int j = lane; j < d; j += WAVE) y[row * d + j] = xr[j] * r * w[j];
+}
+__global__ __launch_bounds__(256) void rmsnorm_bwd_gen(int rows, int d, const float *__restrict__ x,
+                                                       const float *__restrict__ w, const float *__restrict__ g,
+                                                       const float *__restrict__ rinv, float *dx, int acc_dx) {
+  const int lane = threadIdx.x % WAVE;
+  int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  if (row >= rows) return;
+  const float *xr = x + row * d, *gr = g + row * d;
+  float S = 0;
+  for (int j = lane; j < d; j += WAVE) S += gr[j] * w[j] * xr[j];
+  S = wave_sum(S);
+  float r = rinv[row], k2 = r * r * r * S / (float)d;
+  for (int j = lane; j < d; j += WAVE) {
+    float o = w[j] * r * gr[j] - xr[j] * k2;
+    dx[row * d + j] = acc_dx ? dx[row * d + j] + o : o;
+  }
+}
+// dw for the fallback: one thread per column over a slab of rows, partials per slab
+__global__ __launch_bounds__(256) void rmsnorm_dw_gen(int rows, int d, int slab, const float *__restrict__ x,
+                                                      const float *__restrict__ g, const float *__restrict__ rinv,
+                                                      float *__restrict__ part) {
+  int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= d) return;
+  int64_t r0 = (int64_t)blockIdx.y * slab, r1 = std::min<int64_t>(rows, r0 + slab);
+  float s = 0;
+  for (int64_t r = r0; r < r1; r++) s += g[r * d + c] * x[r * d + c] * rinv[r];
+  part[(size_t)blockIdx.y * d + c] = s;
+}
+
+template <int LPR, int NJ>
+static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
+                       gt_buf dx, int acc_dx, gt_buf dw, int acc_dw) {
+  constexpr int RPB = 4 * (WAVE / LPR);
+  int64_t nb = std::min<int64_t>(cdiv(rows, RPB), (int64_t)ctx->num_cu * 4);
+  if (!bwd) {
+    hipLaunchKernelGGL((rmsnorm_fwd_k<LPR, NJ>), dim3((unsigned)nb), dim3(256), 0, ctx->stream, rows, d, eps,
+                       P<const float>(x), P<const float>(w), P<float>(y_or_g), P<float>(rinv));
+    GT_LAUNCHED(ctx);
+    return 0;
+  }
+  float *part = nullptr;
+  if (dw) {
+    void *ws;
+    if (gt_ws_reserve(ctx, (size_t)nb * d * sizeof(float), &ws)) return 1;
+    part = static_cast<float *>(ws);
+  }
+  size_t smem = dw ? (size_t)RPB * d * sizeof(float) : 0;
+  hipLaunchKernelGGL((rmsnorm_bwd_k<LPR, NJ>), dim3((unsigned)nb), dim3(256), smem, ctx->stream, rows, d,
+                     P<const float>(x), P<const float>(w), P<const float>(y_or_g), P<const float>(rinv), P<float>(dx),
+                     acc_dx, part);
+  GT_LAUNCHED(ctx);
+  if (dw) {
+    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 256)), dim3(256), 0, ctx->stream, part, (int)nb, d,
+                       P<float>(dw), acc_dw);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
+
+static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
+                    gt_buf dx, int acc_dx, gt_buf dw, int acc_dw) {
+  bool aligned = (x | w | y_or_g | dx) % 16 == 0;
+  int d4 = d / 4;
+#define FAST(LPR, NJ) return launch_fast<LPR, NJ>(ctx, bwd, rows, d, eps, x, w, y_or_g, rinv, dx, acc_dx, dw, acc_dw)
+  if (d % 4 == 0 && aligned && d <= 2048) {
+    if (d4 <= 16) FAST(16, 1);
+    if (d4 <= 32) FAST(32, 1);
+    if (d4 <= 64) FAST(64, 1);
+    if (d4 <= 128) FAST(64, 2);
+    if (d4 <= 192) FAST(64, 3);
+    if (d4 <= 256) FAST(64, 4);
+    FAST(64, 8);
+  }
+#undef FAST
+  unsigned nb = (unsigned)cdiv(rows, 4);
+  if (!bwd) {
+    hipLaunchKernelGGL(rmsnorm_fwd_gen, dim3(nb), dim3(256), 0, ctx->stream, rows, d, eps, P<const float>(x),
+                       P<const float>(w), P<float>(y_or_g), P<float>(rinv));
+    GT_LAUNCHED(ctx);
+    return 0;
+  }
+  hipLaunchKernelGGL(rmsnorm_bwd_gen, dim3(nb), dim3(256), 0, ctx->stream, rows, d, P<const float>(x), P<const float>(w),
+                     P<const float>(y_or_g), P<const float>(rinv), P<float>(dx), acc_dx);
+  GT_LAUNCHED(ctx);
+  if (dw) {
+    int slab = 256, ns = (int)cdiv(rows, slab);
+    void *ws;
+    if (gt_ws_reserve(ctx, (size_t)ns * d * sizeof(float), &ws)) return 1;
+    hipLaunchKernelGGL(rmsnorm_dw_gen, dim3((unsigned)cdiv(d, 256), ns), dim3(256), 0, ctx->stream, rows, d, slab,
+                       P<const float>(x), P<const float>(y_or_g), P<const float>(rinv), static_cast<float *>(ws));
+    GT_LAUNCHED(ctx);
+    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 256)), dim3(256), 0, ctx->stream, static_cast<float *>(ws), ns,
+                       d, P<float>(dw), acc_dw);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
+
+extern "C" {
+int gt_rmsnorm_fwd(gt_ctx *ctx, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y, gt_buf rinv) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && x && w && y && rinv, "gt_rmsnorm_fwd: bad arguments (rows %d, d %d)", rows, d);
+  if (rows == 0) return 0;
+  ProfScope ps(ctx, "rmsnorm");
+  return dispatch(ctx, false, rows, d, eps, x, w, y, rinv, 0, 0, 0, 0);
+}
+int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx, int acc_dx,
+                   gt_buf dw, int acc_dw) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && x && w && g && rinv && dx, "gt_rmsnorm_bwd: bad arguments (rows %d, d %d)", rows, d);
+  if (rows == 0) {
+    if (dw && !acc_dw) GT_HIP(ctx, hipMemsetAsync(P<void>(dw), 0, (size_t)d * 4, ctx->stream));
+    return 0;
+  }
+  ProfScope ps(ctx, "rmsnorm.bwd");
+  return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dw, acc_dw);
+}
+}

@@ -1,0 +1,342 @@
+// Device-resident AdamW and Muon (src/backend/adamw-gpu.ts, src/backend/muon-gpu.ts; the CPU
+// specs are src/train/adam.ts:46-82 and src/train/muon.ts:69-158).
+//
+// AdamW. The reference issues two reduction dispatches and one update dispatch per tensor (816
+// launches for a 272-tensor model). Here the group is described once by a chunk table on the
+// device (tensor index, offset, length per 64K-element chunk) and a step is three launches for any
+// number of tensors: per-chunk sum of squares, a single-workgroup fold of the chunk sums into the
+// clip scale, and the fused element update. The fold runs in chunk order, so the norm and
+// everything downstream is identical from run to run.
+//
+// Muon. Per matrix: momentum + Nesterov + sum of squares, normalise (transposing tall matrices so
+// the Gram matrix is the small one), five quintic Newton-Schulz iterations as three MFMA GEMMs and
+// two fused elementwise combines each, then the scaled descent. Matrices are processed one after
+// another on the context's stream.
+#include <algorithm>
+#include <vector>
+#include "common.h"
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+#define CHUNK 65536
+
+struct Chunk { int tensor; int len; int64_t off; };
+struct TensorPtrs { float *w, *g, *m, *v; };
+
+struct gt_adamw {
+  int n = 0, nchunks = 0;
+  float beta1, beta2, eps, wd, clip;
+  Chunk *chunks = nullptr;
+  TensorPtrs *ptrs = nullptr;
+  float *partial = nullptr;     // [nchunks]
+  float *scale = nullptr;       // [2]: clip scale, grad norm
+};
+
+__global__ __launch_bounds__(256) void adamw_ssq_k(const Chunk *__restrict__ chunks, const TensorPtrs *__restrict__ ptrs,
+                                                   float *__restrict__ partial) {
+  __shared__ float sm[4];
+  Chunk c = chunks[blockIdx.x];
+  const float *g = ptrs[c.tensor].g + c.off;
+  float s = 0;
+  if ((reinterpret_cast<uintptr_t>(g) & 15) == 0) {
+    int n4 = c.len / 4;
+    for (int i = threadIdx.x; i < n4; i += 256) {
+      v4f x = reinterpret_cast<const v4f *>(g)[i];
+      s += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+    }
+    for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) s += g[i] * g[i];
+  } else {
+    for (int i = threadIdx.x; i < c.len; i += 256) s += g[i] * g[i];
+  }
+  s = block_sum<4>(s, sm);
+  if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
+// scale = norm > clip ? clip/(norm + 1e-12) : 1   (adam.ts:56-62, adamw-gpu.ts:84-95)
+__global__ __launch_bounds__(256) void adamw_scale_k(int nchunks, const float *__restrict__ partial, float clip,
+                                                     float *__restrict__ scale) {
+  __shared__ float sm[4];
+  float s = 0;
+  for (int i = threadIdx.x; i < nchunks; i += 256) s += partial[i];
+  s = block_sum<4>(s, sm);
+  if (threadIdx.x == 0) {
+    float norm = sqrtf(s);
+    scale[0] = norm > clip ? clip / (norm + 1e-12f) : 1.0f;
+    scale[1] = norm;
+  }
+}
+__device__ __forceinline__ void adam1(float g, float &m, float &v, float &w, float b1, float b2, float eps, float wd,
+                                      float lr, float ibc1, float ibc2) {
+  m = b1 * m + (1.f - b1) * g;
+  v = b2 * v + (1.f - b2) * g * g;
+  float upd = (m * ibc1) / (sqrtf(v * ibc2) + eps);
+  if (wd > 0.f) upd += wd * w;
+  w -= lr * upd;
+}
+__global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ chunks, const TensorPtrs *__restrict__ ptrs,
+                                                      const float *__restrict__ scale, float b1, float b2, float eps,
+                                                      float wd, float lr, float bc1, float bc2) {
+  Chunk c = chunks[blockIdx.x];
+  TensorPtrs p = ptrs[c.tensor];
+  const float sc = scale[0];
+  const float ibc1 = 1.0f / bc1, ibc2 = 1.0f / bc2;
+  float *w = p.w + c.off, *m = p.m + c.off, *v = p.v + c.off;
+  const float *g = p.g + c.off;
+  bool vec = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(m) | reinterpret_cast<uintptr_t>(v) |
+               reinterpret_cast<uintptr_t>(g)) & 15) == 0;
+  int n4 = vec ? c.len / 4 : 0;
+  for (int i = threadIdx.x; i < n4; i += 256) {
+    v4f gg = reinterpret_cast<const v4f *>(g)[i] * sc;
+    v4f mm = reinterpret_cast<v4f *>(m)[i], vv = reinterpret_cast<v4f *>(v)[i], ww = reinterpret_cast<v4f *>(w)[i];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      float tm = mm[j], tv = vv[j], tw = ww[j];
+      adam1(gg[j], tm, tv, tw, b1, b2, eps, wd, lr, ibc1, ibc2);
+      mm[j] = tm; vv[j] = tv; ww[j] = tw;
+    }
+    reinterpret_cast<v4f *>(m)[i] = mm;
+    reinterpret_cast<v4f *>(v)[i] = vv;
+    reinterpret_cast<v4f *>(w)[i] = ww;
+  }
+  for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) adam1(g[i] * sc, m[i], v[i], w[i], b1, b2, eps, wd, lr, ibc1, ibc2);
+}
+
+// ---- Muon -------------------------------------------------------------------------------------------
+
+struct MuonMat { float *w, *g, *buf; int rows, cols; };
+struct gt_muon {
+  std::vector<MuonMat> mats;
+  float momentum; int nesterov, ns_steps;
+  float *U = nullptr, *X = nullptr, *A = nullptr, *AA = nullptr, *BX = nullptr, *part = nullptr;   // sized for the largest matrix
+  size_t max_elems = 0, max_r = 0;
+};
+
+#define NS_A 3.4445f
+#define NS_B (-4.7750f)
+#define NS_C 2.0315f
+#define RED_BLOCKS 256
+
+// buf = mu*buf + g; U = nesterov ? g + mu*buf : buf; per-workgroup sum of U^2 (muon-gpu.ts:51-92)
+__global__ __launch_bounds__(256) void muon_momentum_k(int64_t n, const float *__restrict__ g, float *buf, float *__restrict__ U,
+                                                       float mu, int nesterov, float *__restrict__ part) {
+  __shared__ float sm[4];
+  float s = 0;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    float gi = g ? g[i] : 0.f;
+    float b = buf ? mu * buf[i] + gi : gi;
+    if (buf) buf[i] = b;
+    float u = (buf && nesterov) ? gi + mu * b : b;
+    if (!buf) u = U[i];
+    else U[i] = u;
+    s += u * u;
+  }
+  s = block_sum<4>(s, sm);
+  if (threadIdx.x == 0) part[blockIdx.x] = s;
+}
+// X = (flip ? U^T : U) / (sqrt(sum part) + 1e-7); U is [m,n], X is [r,c] with r = min(m,n)
+__global__ __launch_bounds__(256) void muon_normalize_k(int m, int n, int flip, const float *__restrict__ U,
+                                                        const float *__restrict__ part, int nparts, float *__restrict__ X) {
+  __shared__ float sm[4];
+  float s = 0;
+  for (int i = threadIdx.x; i < nparts; i += 256) s += part[i];
+  s = block_sum<4>(s, sm);
+  const float inv = 1.0f / (sqrtf(s) + 1e-7f);
+  int64_t total = (int64_t)m * n;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    // i indexes X row-major [r,c]
+    float u;
+    if (flip) { int64_t xr = i / m, xc = i % m; u = U[xc * n + xr]; }   // X[xr,xc] = U[xc,xr], X is [n,m]
+    else u = U[i];
+    X[i] = u * inv;
+  }
+}
+__global__ __launch_bounds__(256) void muon_combine_a_k(int64_t n, float *A, const float *__restrict__ AA) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) A[i] = NS_B * A[i] + NS_C * AA[i];
+}
+__global__ __launch_bounds__(256) void muon_combine_x_k(int64_t n, float *X, const float *__restrict__ BX) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) X[i] = NS_A * X[i] + BX[i];
+}
+// W[m,n] -= f * (flip ? X^T : X)
+__global__ __launch_bounds__(256) void muon_apply_k(int m, int n, int flip, float *W, const float *__restrict__ X, float f) {
+  int64_t total = (int64_t)m * n;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    float x;
+    if (flip) { int64_t wr = i / n, wc = i % n; x = X[wc * m + wr]; }    // X is [n,m]
+    else x = X[i];
+    W[i] -= f * x;
+  }
+}
+
+static inline unsigned sgrid(gt_ctx *ctx, int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>(cdiv(n, 256), (int64_t)ctx->num_cu * 8)); }
+
+// Leaves NS(U) in X ([r,c]); U already holds the input, part its per-workgroup sums of squares.
+static int newton_schulz_run(gt_ctx *ctx, int m, int n, int steps, float *U, float *X, float *A, float *AA, float *BX,
+                             float *part, int nparts) {
+  int flip = m > n;
+  int r = flip ? n : m, c = flip ? m : n;
+  int64_t size = (int64_t)m * n;
+  hipLaunchKernelGGL(muon_normalize_k, dim3(sgrid(ctx, size)), dim3(256), 0, ctx->stream, m, n, flip, U, part, nparts, X);
+  GT_LAUNCHED(ctx);
+  gt_buf bX = reinterpret_cast<gt_buf>(X), bA = reinterpret_cast<gt_buf>(A), bAA = reinterpret_cast<gt_buf>(AA), bBX = reinterpret_cast<gt_buf>(BX);
+  for (int s = 0; s < steps; s++) {
+    if (gt_gemm(ctx, GT_NT, 0, r, r, c, bX, bX, bA)) return 1;          // A = X X^T
+    if (gt_gemm(ctx, GT_NN, 0, r, r, r, bA, bA, bAA)) return 1;         // AA = A^2
+    hipLaunchKernelGGL(muon_combine_a_k, dim3(sgrid(ctx, (int64_t)r * r)), dim3(256), 0, ctx->stream, (int64_t)r * r, A, AA);
+    GT_LAUNCHED(ctx);
+    if (gt_gemm(ctx, GT_NN, 0, r, c, r, bA, bX, bBX)) return 1;         // BX = (bA + cA^2) X
+    hipLaunchKernelGGL(muon_combine_x_k, dim3(sgrid(ctx, size)), dim3(256), 0, ctx->stream, size, X, BX);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
+
+static int muon_alloc(gt_ctx *ctx, gt_muon *o, size_t elems, size_t r) {
+  GT_HIP(ctx, hipMalloc((void **)&o->U, elems * 4));
+  GT_HIP(ctx, hipMalloc((void **)&o->X, elems * 4));
+  GT_HIP(ctx, hipMalloc((void **)&o->BX, elems * 4));
+  GT_HIP(ctx, hipMalloc((void **)&o->A, r * r * 4));
+  GT_HIP(ctx, hipMalloc((void **)&o->AA, r * r * 4));
+  GT_HIP(ctx, hipMalloc((void **)&o->part, RED_BLOCKS * 4));
+  ctx->live_bytes += elems * 12 + r * r * 8 + RED_BLOCKS * 4;
+  o->max_elems = elems; o->max_r = r;
+  return 0;
+}
+static void muon_release(gt_ctx *ctx, gt_muon *o) {
+  hipStreamSynchronize(ctx->stream);
+  hipFree(o->U); hipFree(o->X); hipFree(o->BX); hipFree(o->A); hipFree(o->AA); hipFree(o->part);
+  ctx->live_bytes -= o->max_elems * 12 + o->max_r * o->max_r * 8 + RED_BLOCKS * 4;
+}
+
+extern "C" {
+
+int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *m, const gt_buf *v,
+                    const int64_t *sizes, float beta1, float beta2, float eps, float weight_decay, float clip, gt_adamw **out) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, n >= 0 && out && (n == 0 || (w && g && m && v && sizes)), "gt_adamw_create: bad arguments");
+  gt_adamw *o = new gt_adamw();
+  o->n = n; o->beta1 = beta1; o->beta2 = beta2; o->eps = eps; o->wd = weight_decay; o->clip = clip;
+  std::vector<Chunk> ch;
+  std::vector<TensorPtrs> tp(n);
+  for (int i = 0; i < n; i++) {
+    if (!(w[i] && g[i] && m[i] && v[i] && sizes[i] >= 0)) { delete o; GT_FAIL(ctx, "gt_adamw_create: tensor %d has a null buffer", i); }
+    tp[i] = {P<float>(w[i]), P<float>(g[i]), P<float>(m[i]), P<float>(v[i])};
+    for (int64_t off = 0; off < sizes[i]; off += CHUNK) ch.push_back({i, (int)std::min<int64_t>(CHUNK, sizes[i] - off), off});
+  }
+  o->nchunks = (int)ch.size();
+  size_t cb = std::max<size_t>(1, ch.size()) * sizeof(Chunk), pb = std::max<size_t>(1, tp.size()) * sizeof(TensorPtrs);
+  GT_HIP(ctx, hipMalloc((void **)&o->chunks, cb));
+  GT_HIP(ctx, hipMalloc((void **)&o->ptrs, pb));
+  GT_HIP(ctx, hipMalloc((void **)&o->partial, std::max<size_t>(1, ch.size()) * 4));
+  GT_HIP(ctx, hipMalloc((void **)&o->scale, 8));
+  if (!ch.empty()) GT_HIP(ctx, hipMemcpy(o->chunks, ch.data(), ch.size() * sizeof(Chunk), hipMemcpyHostToDevice));
+  if (!tp.empty()) GT_HIP(ctx, hipMemcpy(o->ptrs, tp.data(), tp.size() * sizeof(TensorPtrs), hipMemcpyHostToDevice));
+  float one[2] = {1.0f, 0.0f};
+  GT_HIP(ctx, hipMemcpy(o->scale, one, 8, hipMemcpyHostToDevice));
+  *out = o;
+  return 0;
+}
+
+int gt_adamw_step(gt_ctx *ctx, gt_adamw *o, float lr, float bc1, float bc2) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, o, "gt_adamw_step: null optimizer");
+  GT_REQUIRE(ctx, bc1 > 0 && bc2 > 0, "gt_adamw_step: bias corrections must be positive");
+  if (o->nchunks == 0) return 0;
+  ProfScope ps(ctx, "adamw");
+  if (o->clip > 0) {
+    hipLaunchKernelGGL(adamw_ssq_k, dim3(o->nchunks), dim3(256), 0, ctx->stream, o->chunks, o->ptrs, o->partial);
+    GT_LAUNCHED(ctx);
+    hipLaunchKernelGGL(adamw_scale_k, dim3(1), dim3(256), 0, ctx->stream, o->nchunks, o->partial, o->clip, o->scale);
+    GT_LAUNCHED(ctx);
+  }
+  hipLaunchKernelGGL(adamw_update_k, dim3(o->nchunks), dim3(256), 0, ctx->stream, o->chunks, o->ptrs, o->scale, o->beta1,
+                     o->beta2, o->eps, o->wd, lr, bc1, bc2);
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+int gt_adamw_grad_norm(gt_ctx *ctx, gt_adamw *o, float *norm) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, o && norm, "gt_adamw_grad_norm: null argument");
+  float s[2];
+  GT_HIP(ctx, hipMemcpyAsync(s, o->scale, 8, hipMemcpyDeviceToHost, ctx->stream));
+  GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  *norm = s[1];
+  return 0;
+}
+
+int gt_adamw_destroy(gt_ctx *ctx, gt_adamw *o) {
+  GT_ENTER(ctx);
+  if (!o) return 0;
+  hipStreamSynchronize(ctx->stream);
+  hipFree(o->chunks); hipFree(o->ptrs); hipFree(o->partial); hipFree(o->scale);
+  delete o;
+  return 0;
+}
+
+int gt_muon_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *buf, const int *rows, const int *cols,
+                   float momentum, int nesterov, int ns_steps, gt_muon **out) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, n >= 0 && out && ns_steps >= 0 && (n == 0 || (w && g && buf && rows && cols)), "gt_muon_create: bad arguments");
+  gt_muon *o = new gt_muon();
+  o->momentum = momentum; o->nesterov = nesterov; o->ns_steps = ns_steps;
+  size_t me = 1, mr = 1;
+  for (int i = 0; i < n; i++) {
+    if (!(w[i] && g[i] && buf[i] && rows[i] >= 1 && cols[i] >= 1)) { delete o; GT_FAIL(ctx, "gt_muon_create: matrix %d is malformed", i); }
+    o->mats.push_back({P<float>(w[i]), P<float>(g[i]), P<float>(buf[i]), rows[i], cols[i]});
+    me = std::max(me, (size_t)rows[i] * cols[i]);
+    mr = std::max(mr, (size_t)std::min(rows[i], cols[i]));
+  }
+  if (muon_alloc(ctx, o, me, mr)) { delete o; return 1; }
+  *out = o;
+  return 0;
+}
+
+int gt_muon_step(gt_ctx *ctx, gt_muon *o, float lr) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, o, "gt_muon_step: null optimizer");
+  ProfScope ps(ctx, "muon");
+  for (auto &mt : o->mats) {
+    int64_t size = (int64_t)mt.rows * mt.cols;
+    unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv(size, 256));
+    hipLaunchKernelGGL(muon_momentum_k, dim3(nb), dim3(256), 0, ctx->stream, size, mt.g, mt.buf, o->U, o->momentum, o->nesterov, o->part);
+    GT_LAUNCHED(ctx);
+    if (newton_schulz_run(ctx, mt.rows, mt.cols, o->ns_steps, o->U, o->X, o->A, o->AA, o->BX, o->part, (int)nb)) return 1;
+    float f = lr * sqrtf(std::max(1.0f, (float)mt.rows / (float)mt.cols));
+    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, size)), dim3(256), 0, ctx->stream, mt.rows, mt.cols, mt.rows > mt.cols ? 1 : 0,
+                       mt.w, o->X, f);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
+
+int gt_muon_destroy(gt_ctx *ctx, gt_muon *o) {
+  GT_ENTER(ctx);
+  if (!o) return 0;
+  muon_release(ctx, o);
+  delete o;
+  return 0;
+}
+
+int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, m >= 1 && n >= 1 && steps >= 0 && G && out, "gt_newton_schulz: bad arguments");
+  ProfScope ps(ctx, "muon");
+  gt_muon tmp;
+  size_t size = (size_t)m * n;
+  if (muon_alloc(ctx, &tmp, size, (size_t)std::min(m, n))) return 1;
+  GT_HIP(ctx, hipMemcpyAsync(tmp.U, P<void>(G), size * 4, hipMemcpyDeviceToDevice, ctx->stream));
+  unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv((int64_t)size, 256));
+  // sums of squares of U only (no momentum buffer, no gradient)
+  hipLaunchKernelGGL(muon_momentum_k, dim3(nb), dim3(256), 0, ctx->stream, (int64_t)size, (const float *)nullptr, (float *)nullptr,
+                     tmp.U, 0.f, 0, tmp.part);
+  GT_LAUNCHED(ctx);
+  int rc = newton_schulz_run(ctx, m, n, steps, tmp.U, tmp.X, tmp.A, tmp.AA, tmp.BX, tmp.part, (int)nb);
+  if (!rc) {
+    // out = 0 - (-1) * X(^T): reuse the apply kernel on a cleared destination
+    hipMemsetAsync(P<void>(out), 0, size * 4, ctx->stream);
+    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, (int64_t)size)), dim3(256), 0, ctx->stream, m, n, m > n ? 1 : 0, P<float>(out),
+                       tmp.X, -1.0f);
+  }
+  muon_release(ctx, &tmp);
+  return rc;
+}
+}

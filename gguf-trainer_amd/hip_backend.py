@@ -1,0 +1,658 @@
+"""HipBackend: the device backend behind the autograd op set, on one MI355X.
+
+Mirrors the public surface of WebGPUBackend (src/backend/webgpu.ts:290-1888): it implements
+OpsBackend (every op records device work, installs `out._backward`, returns at once) and
+RegionBackend (begin_region / end_region / seed_grad_from for `checkpoint`), plus the buffer
+surface the device optimizers and the trainer use (buffers_for, keep_grad_on_device,
+create/write/read_state_buffer, upload_params, sync, reclaim_step_transients, resident_bytes,
+region_count, start/stop_profile). All work goes to the one HIP stream the library context owns.
+
+What differs from the reference, on purpose:
+  * Gradient buffers are not cleared and then added to. Each backward kernel is told whether it is
+    the first writer of its destination in this accumulation window (store) or a later one (add),
+    so an intermediate's gradient costs one write instead of clear + read + write, and
+    `grad_clears_issued` stays near zero. Parameter accumulators follow the same rule across the
+    micro-batches of a step and are re-armed when the optimizer has consumed them.
+  * Intermediate gradient buffers are allocated at their first write in backward, not at forward.
+  * silu/gelu outputs are lazy: when their only use is the gate of `mul`, forward and backward run
+    the fused gated-activation kernels on the pre-activation and the activation tensor never
+    exists in memory. Any other consumer materialises it and the unfused kernels run.
+  * Host arrays of intermediates are never allocated unless sync() is asked to read them.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+import weakref
+
+import numpy as np
+
+from . import autograd as ag
+from .autograd import Tensor
+from .lib import NN, NT, TN, HipError, ProfRec, buf as c_buf, check, lib
+
+_ALIGN = 256
+
+
+class _Entry:
+    __slots__ = ("data", "grad", "nbytes", "external", "grad_init", "lazy_act", "consumers", "fused_uses",
+                 "region", "keep_grad")
+
+    def __init__(self, nbytes, external):
+        self.data = 0
+        self.grad = 0
+        self.nbytes = nbytes
+        self.external = external
+        self.grad_init = False
+        self.lazy_act = None        # (x tensor, act id) while a silu/gelu output has not been computed
+        self.consumers = 0
+        self.fused_uses = 0
+        self.region = 0
+        self.keep_grad = False
+
+
+class HipBackend:
+    def __init__(self, device: int = 0):
+        self._ctx = C.c_void_p()
+        rc = lib.gt_ctx_create(device, C.byref(self._ctx))
+        if rc != 0:
+            raise HipError("gt_ctx_create: " + (lib.gt_last_error(None) or b"").decode())
+        self.adapter_name = lib.gt_device_name(self._ctx).decode()
+        self.attn_flash_min_t = 2048      # kept for interface parity; one kernel family serves every T here
+        self.last_sync_readback_bytes = 0
+        self.grad_clears_issued = 0
+        self.fuse_glu = True
+        self._pool: dict[int, list[int]] = {}
+        self._pool_bytes = 0
+        self._state_bytes = 0
+        self._entries: "weakref.WeakKeyDictionary[Tensor, _Entry]" = weakref.WeakKeyDictionary()
+        self._externals: "weakref.WeakSet[Tensor]" = weakref.WeakSet()
+        self._touched: list = []
+        self._touched_ids: set = set()
+        self._transients: list = []       # (tensor weakref-free strong ref, entry) in creation order
+        self._scratch: list = []          # (buf, nbytes) raw transients: id uploads, saved statistics
+        self._regions_opened = 0
+        self._profiling = False
+        self._destroyed = False
+
+    # ---- install (webgpu.ts:393-399) ---------------------------------------------------------------
+    def install(self):
+        ag.set_ops_backend(self)
+
+    def uninstall(self):
+        ag.set_ops_backend(None)
+
+    # ---- raw memory ------------------------------------------------------------------------------------
+    def _acquire(self, nbytes: int) -> int:
+        size = max(_ALIGN, (nbytes + _ALIGN - 1) // _ALIGN * _ALIGN)
+        free = self._pool.get(size)
+        if free:
+            return free.pop()
+        out = c_buf()
+        check(self._ctx, lib.gt_alloc(self._ctx, size, 0, C.byref(out)), "gt_alloc")
+        self._pool_bytes += size
+        return out.value
+
+    def _recycle(self, b: int, nbytes: int):
+        size = max(_ALIGN, (nbytes + _ALIGN - 1) // _ALIGN * _ALIGN)
+        self._pool.setdefault(size, []).append(b)
+
+    def _scratch_buf(self, nbytes: int) -> int:
+        b = self._acquire(nbytes)
+        self._scratch.append((b, nbytes))
+        return b
+
+    def _upload(self, arr: np.ndarray) -> int:
+        arr = np.ascontiguousarray(arr)
+        b = self._scratch_buf(arr.nbytes)
+        check(self._ctx, lib.gt_h2d(self._ctx, b, arr.ctypes.data_as(C.c_void_p), arr.nbytes), "gt_h2d")
+        return b
+
+    # ---- entries (webgpu.ts:1539-1593) -----------------------------------------------------------------
+    def _entry_for(self, t: Tensor) -> _Entry:
+        """Device buffers of an existing tensor; a tensor never seen before is external (a parameter):
+        it gets a persistent data buffer, uploaded once."""
+        e = self._entries.get(t)
+        if e is None:
+            if t._prev:
+                raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's buffers")
+            e = _Entry(t.size * 4, True)
+            e.data = self._acquire(e.nbytes)
+            check(self._ctx, lib.gt_h2d(self._ctx, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
+            self._entries[t] = e
+            self._externals.add(t)
+        if e.external and t.requires_grad and id(t) not in self._touched_ids:
+            self._touched_ids.add(id(t))
+            self._touched.append(t)
+        return e
+
+    def _make_out(self, shape, prev, alloc=True) -> tuple:
+        out = Tensor(None, shape)
+        out._prev = list(prev)
+        e = _Entry(out.size * 4, False)
+        if alloc:
+            e.data = self._acquire(e.nbytes)
+        e.region = self._regions_opened
+        self._entries[out] = e
+        self._transients.append((out, e))
+        return out, e
+
+    def _data(self, t: Tensor) -> int:
+        """Device address of t's values, as an op input."""
+        e = self._entry_for(t)
+        e.consumers += 1
+        if e.lazy_act is not None:
+            self._materialise(t, e)
+        return e.data
+
+    def _materialise(self, t: Tensor, e: _Entry):
+        x, act = e.lazy_act
+        e.lazy_act = None
+        e.data = self._acquire(e.nbytes)
+        xe = self._entry_for(x)
+        fn = lib.gt_silu_fwd if act == 0 else lib.gt_gelu_fwd
+        check(self._ctx, fn(self._ctx, t.size, xe.data, e.data), "act.fwd")
+
+    def _gdst(self, t: Tensor) -> tuple:
+        """(gradient buffer, acc) for a backward kernel about to contribute to t's gradient;
+        (0, 0) when t takes no gradient (a frozen parameter)."""
+        e = self._entries.get(t)
+        if e is None:
+            e = self._entry_for(t)
+        if e.external and not t.requires_grad:
+            return 0, 0
+        if e.grad == 0:
+            e.grad = self._acquire(e.nbytes)
+        acc = 1 if e.grad_init else 0
+        e.grad_init = True
+        return e.grad, acc
+
+    def _gsrc(self, t: Tensor) -> int:
+        """Gradient buffer of an op output inside its backward closure."""
+        e = self._entries.get(t)
+        if e is None:
+            raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
+                               "gradient buffers, so this backward would read pool garbage")
+        if e.grad == 0 or not e.grad_init:
+            # nothing downstream wrote it (an output the loss does not depend on): its gradient is zero
+            if e.grad == 0:
+                e.grad = self._acquire(e.nbytes)
+            check(self._ctx, lib.gt_memset0(self._ctx, e.grad, e.nbytes), "gt_memset0")
+            self.grad_clears_issued += 1
+            e.grad_init = True
+        return e.grad
+
+    # ---- public buffer surface (webgpu.ts:1432-1537) ----------------------------------------------------
+    def upload_params(self, tensors):
+        for t in tensors:
+            e = self._entry_for(t)
+            check(self._ctx, lib.gt_h2d(self._ctx, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
+
+    def buffers_for(self, t: Tensor) -> dict:
+        e = self._entry_for(t)
+        if t.requires_grad and e.grad == 0:
+            e.grad = self._acquire(e.nbytes)
+            check(self._ctx, lib.gt_memset0(self._ctx, e.grad, e.nbytes), "gt_memset0")
+            self.grad_clears_issued += 1
+        return {"data": e.data, "grad": e.grad}
+
+    def keep_grad_on_device(self, t: Tensor):
+        self._entry_for(t).keep_grad = True
+
+    def grads_consumed(self, tensors):
+        """The optimizer has read these accumulators: the next backward write stores instead of adding
+        (the reference's deferred per-step clear, src/backend/muon-gpu.ts:8-16)."""
+        for t in tensors:
+            e = self._entries.get(t)
+            if e is not None:
+                e.grad_init = False
+
+    def ensure_grads_defined(self, tensors):
+        """An accumulator no kernel wrote since it was last consumed holds zero, as a cleared one would."""
+        for t in tensors:
+            e = self._entry_for(t)
+            if e.grad == 0:
+                e.grad = self._acquire(e.nbytes)
+            if not e.grad_init:
+                check(self._ctx, lib.gt_memset0(self._ctx, e.grad, e.nbytes), "gt_memset0")
+                self.grad_clears_issued += 1
+                e.grad_init = True
+
+    def seed_grad_from_host(self, t: Tensor):
+        e = self._entries.get(t)
+        if e is None:
+            raise RuntimeError("seed_grad_from_host: tensor has no device buffers")
+        if e.grad == 0:
+            e.grad = self._acquire(e.nbytes)
+        check(self._ctx, lib.gt_h2d(self._ctx, e.grad, t.grad.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
+        e.grad_init = True
+
+    def create_state_buffer(self, nbytes: int) -> int:
+        out = c_buf()
+        check(self._ctx, lib.gt_alloc(self._ctx, max(4, nbytes), 1, C.byref(out)), "gt_alloc")
+        self._state_bytes += max(4, nbytes)
+        return out.value
+
+    def write_state_buffer(self, b: int, arr: np.ndarray):
+        arr = np.ascontiguousarray(arr)
+        check(self._ctx, lib.gt_h2d(self._ctx, b, arr.ctypes.data_as(C.c_void_p), arr.nbytes), "gt_h2d")
+
+    def read_state_buffer(self, b: int, n: int, dtype=np.float32) -> np.ndarray:
+        out = np.empty(n, dtype=dtype)
+        check(self._ctx, lib.gt_d2h(self._ctx, out.ctypes.data_as(C.c_void_p), b, out.nbytes), "gt_d2h")
+        return out
+
+    def resident_bytes(self) -> int:
+        v = C.c_uint64()
+        lib.gt_resident_bytes(self._ctx, C.byref(v))
+        return int(v.value)
+
+    def region_count(self) -> int:
+        return self._regions_opened
+
+    @property
+    def ctx(self):
+        return self._ctx
+
+    # ---- sync / reclaim (webgpu.ts:419-636) -------------------------------------------------------------
+    def _release_transients(self, keep=()):
+        keep_ids = {id(t) for t in keep}
+        kept = []
+        for t, e in self._transients:
+            if id(t) in keep_ids:
+                kept.append((t, e))
+                continue
+            if e.data:
+                self._recycle(e.data, e.nbytes)
+            if e.grad:
+                self._recycle(e.grad, e.nbytes)
+            e.data = e.grad = 0
+            self._entries.pop(t, None)
+        self._transients = kept
+        for b, n in self._scratch:
+            self._recycle(b, n)
+        self._scratch = []
+
+    def sync(self, reads=()):
+        """Wait for the stream; read back `reads` (values) and the accumulated gradients of every
+        trainable external tensor touched since the last sync that is not kept on the device; recycle
+        all intermediates. The graph is unusable for backward afterwards."""
+        nbytes = 0
+        for t in reads:
+            e = self._entries.get(t)
+            if e is None:
+                raise RuntimeError("sync: tensor has no device buffers")
+            if e.lazy_act is not None:
+                self._materialise(t, e)
+            check(self._ctx, lib.gt_d2h(self._ctx, t.data.ctypes.data_as(C.c_void_p), e.data, e.nbytes), "gt_d2h")
+            nbytes += e.nbytes
+        for t in self._touched:
+            e = self._entries.get(t)
+            if e is None or e.keep_grad or not t.requires_grad:
+                continue
+            if e.grad and e.grad_init:
+                check(self._ctx, lib.gt_d2h(self._ctx, t.grad.ctypes.data_as(C.c_void_p), e.grad, e.nbytes), "gt_d2h")
+                nbytes += e.nbytes
+            else:
+                t.grad.fill(0)
+            e.grad_init = False            # read back: the next step starts from zero
+        self._touched = []
+        self._touched_ids = set()
+        check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")
+        self.last_sync_readback_bytes = nbytes
+        self._release_transients()
+
+    def reclaim_step_transients(self, keep=()):
+        """Free a finished micro-batch's intermediates mid-step; parameter gradients keep accumulating."""
+        check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")
+        self._release_transients(keep)
+
+    def destroy(self):
+        if not self._destroyed:
+            self._destroyed = True
+            lib.gt_ctx_destroy(self._ctx)
+
+    # ---- profiling (webgpu.ts:830-880) -----------------------------------------------------------------------
+    def start_profile(self):
+        check(self._ctx, lib.gt_prof_begin(self._ctx), "gt_prof_begin")
+
+    def stop_profile(self) -> dict:
+        recs = (ProfRec * 64)()
+        n = C.c_int()
+        check(self._ctx, lib.gt_prof_end(self._ctx, recs, 64, C.byref(n)), "gt_prof_end")
+        return {recs[i].label.decode(): (recs[i].ms, recs[i].count) for i in range(n.value)}
+
+    # ---- RegionBackend (webgpu.ts:639-761) ------------------------------------------------------------------------
+    def begin_region(self) -> int:
+        self._regions_opened += 1
+        return len(self._transients)
+
+    def end_region(self, mark: int, keep):
+        keep_ids = {id(t) for t in keep}
+        tail = self._transients[mark:]
+        del self._transients[mark:]
+        for t, e in tail:
+            if id(t) in keep_ids:
+                self._transients.append((t, e))
+                continue
+            if e.data:
+                self._recycle(e.data, e.nbytes)
+            if e.grad:
+                self._recycle(e.grad, e.nbytes)
+            e.data = e.grad = 0
+            self._entries.pop(t, None)
+
+    def seed_grad_from(self, dst: Tensor, src: Tensor):
+        if dst.size != src.size:
+            raise ValueError(f"seed_grad_from: size mismatch {dst.size} vs {src.size}")
+        g = self._gsrc(src)
+        d, _ = self._gdst(dst)
+        check(self._ctx, lib.gt_d2d(self._ctx, d, g, dst.size * 4), "gt_d2d")
+
+    # ---- ops --------------------------------------------------------------------------------------------------------
+    def linear(self, x: Tensor, w: Tensor) -> Tensor:
+        T, ind = x.shape
+        outd = w.shape[0]
+        xd, wd = self._data(x), self._data(w)
+        out, e = self._make_out([T, outd], [x, w])
+        check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, T, outd, ind, xd, wd, e.data), "linear")
+        wants_dw = w.requires_grad
+
+        def bw():
+            g = self._gsrc(out)
+            dx, acc = self._gdst(x)
+            if dx:
+                check(self._ctx, lib.gt_gemm(self._ctx, NN, acc, T, ind, outd, g, wd, dx), "linear.dx")
+            if wants_dw:
+                dw, accw = self._gdst(w)
+                if dw:
+                    check(self._ctx, lib.gt_gemm(self._ctx, TN, accw, outd, ind, T, g, xd, dw), "linear.dw")
+
+        out._backward = bw
+        return out
+
+    def add(self, a: Tensor, b: Tensor) -> Tensor:
+        ad, bd = self._data(a), self._data(b)
+        out, e = self._make_out(a.shape, [a, b])
+        check(self._ctx, lib.gt_add_fwd(self._ctx, out.size, ad, bd, e.data), "add")
+
+        def bw():
+            g = self._gsrc(out)
+            if a is b:
+                da, acc = self._gdst(a)
+                check(self._ctx, lib.gt_add_bwd(self._ctx, out.size, g, da, acc, da, acc), "add.bwd")
+                return
+            da, acca = self._gdst(a)
+            db, accb = self._gdst(b)
+            check(self._ctx, lib.gt_add_bwd(self._ctx, out.size, g, da, acca, db, accb), "add.bwd")
+
+        out._backward = bw
+        return out
+
+    def mul(self, a: Tensor, b: Tensor) -> Tensor:
+        ea, eb = self._entry_for(a), self._entry_for(b)
+        if self.fuse_glu and a is not b:
+            # gate * up with a lazy activation on one side: run the fused kernels on the pre-activation
+            lazy, other = (a, b) if ea.lazy_act is not None else ((b, a) if eb.lazy_act is not None else (None, None))
+            if lazy is not None and self._entries[other].lazy_act is None:
+                le = self._entries[lazy]
+                gate, act = le.lazy_act
+                le.consumers += 1
+                le.fused_uses += 1
+                gd, ud = self._data(gate), self._data(other)
+                out, e = self._make_out(a.shape, [a, b])
+                check(self._ctx, lib.gt_glu_fwd(self._ctx, act, out.size, gd, ud, e.data), "glu")
+
+                def bw_fused():
+                    g = self._gsrc(out)
+                    dg, accg = self._gdst(gate)
+                    du, accu = self._gdst(other)
+                    check(self._ctx, lib.gt_glu_bwd(self._ctx, act, out.size, g, gd, ud, dg, accg, du, accu), "glu.bwd")
+
+                out._backward = bw_fused
+                return out
+        ad, bd = self._data(a), self._data(b)
+        out, e = self._make_out(a.shape, [a, b])
+        check(self._ctx, lib.gt_mul_fwd(self._ctx, out.size, ad, bd, e.data), "mul")
+
+        def bw():
+            g = self._gsrc(out)
+            if a is b:
+                da, acc = self._gdst(a)
+                check(self._ctx, lib.gt_mul_bwd(self._ctx, out.size, g, ad, ad, da, acc, da, acc), "mul.bwd")
+                return
+            da, acca = self._gdst(a)
+            db, accb = self._gdst(b)
+            check(self._ctx, lib.gt_mul_bwd(self._ctx, out.size, g, ad, bd, da, acca, db, accb), "mul.bwd")
+
+        out._backward = bw
+        return out
+
+    def _activation(self, x: Tensor, act: int) -> Tensor:
+        xd = self._data(x)
+        out, e = self._make_out(x.shape, [x], alloc=not self.fuse_glu)
+        if self.fuse_glu:
+            e.lazy_act = (x, act)
+        else:
+            fn = lib.gt_silu_fwd if act == 0 else lib.gt_gelu_fwd
+            check(self._ctx, fn(self._ctx, out.size, xd, e.data), "act")
+
+        def bw():
+            oe = self._entries.get(out)
+            if oe is None:
+                raise RuntimeError("backward over a graph built before a sync()")
+            if oe.fused_uses and oe.fused_uses == oe.consumers:
+                return                       # every use was a fused gate*up, which already wrote x's gradient
+            if oe.grad == 0 and oe.fused_uses:
+                return                       # its other consumers contributed nothing
+            g = self._gsrc(out)
+            dx, acc = self._gdst(x)
+            fn = lib.gt_silu_bwd if act == 0 else lib.gt_gelu_bwd
+            check(self._ctx, fn(self._ctx, out.size, g, xd, dx, acc), "act.bwd")
+
+        out._backward = bw
+        return out
+
+    def silu(self, x: Tensor) -> Tensor:
+        return self._activation(x, 0)
+
+    def gelu(self, x: Tensor) -> Tensor:
+        return self._activation(x, 1)
+
+    def scale(self, x: Tensor, c: float) -> Tensor:
+        xd = self._data(x)
+        out, e = self._make_out(x.shape, [x])
+        check(self._ctx, lib.gt_scale_fwd(self._ctx, out.size, xd, c, e.data), "scale")
+
+        def bw():
+            g = self._gsrc(out)
+            dx, acc = self._gdst(x)
+            if dx:
+                check(self._ctx, lib.gt_scale_bwd(self._ctx, out.size, g, c, dx, acc), "scale.bwd")
+
+        out._backward = bw
+        return out
+
+    def _rms_rows(self, x, weight, rows, d, eps, shape):
+        xd, wd = self._data(x), self._data(weight)
+        out, e = self._make_out(shape, [x, weight])
+        rinv = self._scratch_buf(rows * 4)
+        check(self._ctx, lib.gt_rmsnorm_fwd(self._ctx, rows, d, eps, xd, wd, e.data, rinv), "rmsnorm")
+        wants_dw = weight.requires_grad
+
+        def bw():
+            g = self._gsrc(out)
+            dx, acc = self._gdst(x)
+            dw, accw = self._gdst(weight) if wants_dw else (0, 0)
+            check(self._ctx, lib.gt_rmsnorm_bwd(self._ctx, rows, d, xd, wd, g, rinv, dx, acc, dw, accw), "rmsnorm.bwd")
+
+        out._backward = bw
+        return out
+
+    def rms_norm(self, x, weight, eps):
+        T, d = x.shape
+        return self._rms_rows(x, weight, T, d, eps, [T, d])
+
+    def rms_norm_heads(self, x, weight, T, H, hd, eps):
+        return self._rms_rows(x, weight, T * H, hd, eps, [T, H * hd])
+
+    def embedding(self, weight: Tensor, ids) -> Tensor:
+        V, d = weight.shape
+        ids32 = np.ascontiguousarray(ids, dtype=np.int32)
+        T = ids32.size
+        wd = self._data(weight)
+        idb = self._upload(ids32)
+        out, e = self._make_out([T, d], [weight])
+        check(self._ctx, lib.gt_embedding_fwd(self._ctx, T, d, idb, wd, e.data), "embedding")
+        wants_dw = weight.requires_grad
+
+        def bw():
+            if not wants_dw:
+                return
+            g = self._gsrc(out)
+            dw, acc = self._gdst(weight)
+            check(self._ctx, lib.gt_embedding_bwd(self._ctx, T, d, V, idb, g, dw, acc), "embedding.bwd")
+
+        out._backward = bw
+        return out
+
+    def rope(self, x, T, H, hd, base, pos_offset=0):
+        rows = x.shape[0]
+        xd = self._data(x)
+        out, e = self._make_out([rows, H * hd], [x])
+        check(self._ctx, lib.gt_rope(self._ctx, rows, T, H, hd, base, pos_offset, 0, xd, e.data, 0), "rope")
+
+        def bw():
+            g = self._gsrc(out)
+            dx, acc = self._gdst(x)
+            check(self._ctx, lib.gt_rope(self._ctx, rows, T, H, hd, base, pos_offset, 1, g, dx, acc), "rope.bwd")
+
+        out._backward = bw
+        return out
+
+    def attention(self, q, k, v, T, Hq, Hkv, hd, window=0):
+        rows = q.shape[0]
+        if rows % T:
+            raise ValueError(f"attention: {rows} rows are not a whole number of sequences of {T}")
+        B = rows // T
+        qd, kd, vd = self._data(q), self._data(k), self._data(v)
+        out, e = self._make_out([rows, Hq * hd], [q, k, v])
+        lse = self._scratch_buf(B * Hq * T * 4)
+        check(self._ctx, lib.gt_attn_fwd(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, e.data, lse), "attention")
+        od = e.data
+
+        def bw():
+            g = self._gsrc(out)
+            dq, aq = self._gdst(q)
+            dk, ak = self._gdst(k)
+            dv, av = self._gdst(v)
+            check(self._ctx, lib.gt_attn_bwd(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, od, g, lse,
+                                             dq, aq, dk, ak, dv, av), "attention.bwd")
+
+        out._backward = bw
+        return out
+
+    @staticmethod
+    def _inv_denoms(kept):
+        kept = np.atleast_1d(np.asarray(kept, dtype=np.int64))
+        return (1.0 / np.maximum(kept, 1)).astype(np.float32)
+
+    def cross_entropy(self, logits, targets, kept) -> Tensor:
+        rows, V = logits.shape
+        inv = self._inv_denoms(kept)
+        nseq = inv.size
+        T = rows // nseq
+        zd = self._data(logits)
+        tg = self._upload(np.ascontiguousarray(targets, dtype=np.int32))
+        invb = self._upload(inv)
+        lse = self._scratch_buf(rows * 4)
+        loss, e = self._make_out([nseq], [logits])
+        check(self._ctx, lib.gt_ce_fwd(self._ctx, rows, V, T, zd, tg, invb, e.data, lse), "crossEntropy")
+
+        def bw():
+            if self._entries.get(loss) is None:
+                raise RuntimeError("backward over a graph built before a sync()")
+            seed = float(loss.grad[0])
+            dz, acc = self._gdst(logits)
+            check(self._ctx, lib.gt_ce_bwd(self._ctx, rows, V, T, zd, tg, invb, lse, seed, dz, acc), "crossEntropy.bwd")
+
+        loss._backward = bw
+        return loss
+
+    def fused_cross_entropy(self, hidden, w, targets, chunk, kept) -> Tensor:
+        rows, H = hidden.shape
+        V = w.shape[0]
+        inv = self._inv_denoms(kept)
+        nseq = inv.size
+        T = rows // nseq
+        hd_, wd = self._data(hidden), self._data(w)
+        tg = self._upload(np.ascontiguousarray(targets, dtype=np.int32))
+        invb = self._upload(inv)
+        rmax, rsum, tl = (self._scratch_buf(rows * 4) for _ in range(3))
+        width = min(chunk, V)
+        cb = self._scratch_buf(rows * width * 4)
+        spans = [(v0, min(v0 + chunk, V) - v0) for v0 in range(0, V, chunk)]
+        for i, (v0, vc) in enumerate(spans):
+            check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, rows, vc, H, hd_, wd + v0 * H * 4, cb), "fusedCE.logits")
+            check(self._ctx, lib.gt_ce_chunk_stats(self._ctx, rows, vc, v0, 1 if i == 0 else 0, cb, tg, rmax, rsum, tl), "fusedCE.stats")
+        loss, e = self._make_out([nseq], [hidden, w])
+        check(self._ctx, lib.gt_ce_loss_from_stats(self._ctx, rows, T, tg, invb, rmax, rsum, tl, e.data), "fusedCE.loss")
+        wants_dw = w.requires_grad
+
+        def bw():
+            if self._entries.get(loss) is None:
+                raise RuntimeError("backward over a graph built before a sync()")
+            seed = float(loss.grad[0])
+            dh, acch = self._gdst(hidden)
+            dw, accw = self._gdst(w) if wants_dw else (0, 0)
+            for v0, vc in spans:
+                check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, rows, vc, H, hd_, wd + v0 * H * 4, cb), "fusedCE.logits")
+                check(self._ctx, lib.gt_ce_chunk_grad(self._ctx, rows, vc, v0, T, cb, tg, invb, rmax, rsum, seed), "fusedCE.grad")
+                check(self._ctx, lib.gt_gemm(self._ctx, NN, acch, rows, H, vc, cb, wd + v0 * H * 4, dh), "fusedCE.dh")
+                acch = 1
+                if dw:
+                    # rows [v0, v0+vc) of dW are written by this span only
+                    check(self._ctx, lib.gt_gemm(self._ctx, TN, accw, vc, H, rows, cb, hd_, dw + v0 * H * 4), "fusedCE.dw")
+
+        loss._backward = bw
+        return loss
+
+    def soft_cross_entropy(self, logits, teacher_ids, teacher_probs, k, kept) -> Tensor:
+        rows, V = logits.shape
+        inv = 1.0 / max(int(kept), 1)
+        zd = self._data(logits)
+        ti = self._upload(np.ascontiguousarray(teacher_ids, dtype=np.int32))
+        tp = self._upload(np.ascontiguousarray(teacher_probs, dtype=np.float32))
+        lse, mass = self._scratch_buf(rows * 4), self._scratch_buf(rows * 4)
+        loss, e = self._make_out([1], [logits])
+        check(self._ctx, lib.gt_soft_ce_fwd(self._ctx, rows, V, k, zd, ti, tp, inv, e.data, lse, mass), "softCE")
+
+        def bw():
+            if self._entries.get(loss) is None:
+                raise RuntimeError("backward over a graph built before a sync()")
+            seed = float(loss.grad[0])
+            dz, acc = self._gdst(logits)
+            check(self._ctx, lib.gt_soft_ce_bwd(self._ctx, rows, V, k, zd, ti, tp, inv, lse, mass, seed, dz, acc), "softCE.bwd")
+
+        loss._backward = bw
+        return loss
+
+    # ---- raw GEMM for tests and benches (webgpu.ts:1654) --------------------------------------------------------------
+    def gemm(self, kind: int, acc: int, M: int, N: int, K: int, a: int, b: int, c: int):
+        check(self._ctx, lib.gt_gemm(self._ctx, kind, acc, M, N, K, a, b, c), "gemm")
+
+
+def init_hip(device: int = 0):
+    """initWebGPU analogue (webgpu.ts:1823): a backend, or None when no MI355X is visible."""
+    try:
+        return HipBackend(device)
+    except HipError:
+        return None
+
+
+def require_gpu(purpose: str, device: int = 0) -> HipBackend:
+    """requireGPU analogue (webgpu.ts:1812)."""
+    try:
+        return HipBackend(device)
+    except HipError as e:
+        raise RuntimeError(f"{purpose} needs an MI355X: {e}") from e

@@ -1,0 +1,171 @@
+/*
+ * libggufhip: C ABI of the MI355X (gfx950) device backend for gguf-trainer's training hot path:
+ * backward pass, fused gradient kernels, optimizer step, and the forward producers the backward
+ * reads. A host binds these symbols (Deno.dlopen, ctypes) and keeps its own tape; the library owns
+ * one HIP stream per context and every call below only enqueues work on it, except gt_sync,
+ * gt_d2h and gt_prof_end, which wait.
+ *
+ * Conventions
+ *   - every function returns 0 on success, non-zero on error; gt_last_error() gives the message.
+ *     Asynchronous HIP errors are sticky: the next call (or gt_sync) reports them.
+ *   - gt_buf is a device address (64-bit). Offsets into a buffer are plain additions, which is how
+ *     a vocab span of the readout matrix or one sequence of a batch is addressed.
+ *   - tensors are f32, row-major; ids / targets are int32 with -1 as the ignore marker.
+ *   - "acc" arguments: 0 = the kernel stores its result (the destination need not be cleared),
+ *     1 = it adds to what the destination holds. The reference zeroes every gradient buffer and
+ *     always adds (src/backend/webgpu.ts:21-26, 1397-1429); a host that knows a gradient's first
+ *     writer can skip both the clear and the read. No kernel uses atomics: one thread owns one
+ *     output element and every reduction has a fixed order, so results are run-to-run identical.
+ *   - rows-batched extension: where the reference runs one sequence of T rows per call, these take
+ *     `rows` (= B*T, sequences stacked) plus what per-sequence structure the op needs (T for
+ *     positions, B for attention, one denominator per sequence for the loss). B = 1 is the
+ *     reference call.
+ *
+ * Reference interface replaced: OpsBackend (src/model/autograd.ts:103-151), RegionBackend
+ * (:160-164), WebGPUBackend's buffer surface (src/backend/webgpu.ts:1446-1537), AdamWGpu
+ * (src/backend/adamw-gpu.ts:131-251) and MuonGpu (src/backend/muon-gpu.ts:351-470).
+ */
+#ifndef GGUFHIP_H
+#define GGUFHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct gt_ctx gt_ctx;
+typedef struct gt_adamw gt_adamw;
+typedef struct gt_muon gt_muon;
+typedef uint64_t gt_buf;
+
+/* ---- context, memory, transfers ------------------------------------------------------------
+ * Replaces initWebGPU / GpuDevice+queue (webgpu.ts:129-141, 1823), createStateBuffer (:1465),
+ * writeStateBuffer (:1482), readStateBuffer (:1492), clearBuffer (:1421-1427),
+ * copyBufferToBuffer in seedGradFrom (:742-761), sync (:419-576), residentBytes (:774). */
+int gt_ctx_create(int device, gt_ctx **out);
+int gt_ctx_destroy(gt_ctx *ctx);
+const char *gt_last_error(gt_ctx *ctx);            /* ctx may be NULL: error of a failed create */
+const char *gt_device_name(gt_ctx *ctx);
+int gt_alloc(gt_ctx *ctx, size_t bytes, int zero, gt_buf *out);
+int gt_free(gt_ctx *ctx, gt_buf buf);
+int gt_memset0(gt_ctx *ctx, gt_buf buf, size_t bytes);
+int gt_h2d(gt_ctx *ctx, gt_buf dst, const void *src, size_t bytes);   /* enqueued; src is copied before return */
+int gt_d2h(gt_ctx *ctx, void *dst, gt_buf src, size_t bytes);         /* waits for the stream */
+int gt_d2d(gt_ctx *ctx, gt_buf dst, gt_buf src, size_t bytes);
+int gt_sync(gt_ctx *ctx);
+int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt_alloc bytes + workspace */
+
+/* ---- GEMM: srcGemm (src/backend/wgsl.ts:87-196), WebGPUBackend.gemm (webgpu.ts:1654) ---------
+ * kind 0 "NT": C[M,N] = A[M,K] . B[N,K]^T      forward y = x W^T           (webgpu.ts:892)
+ * kind 1 "NN": C[M,N] = A[M,K] . B[K,N]        dX = dY W                   (webgpu.ts:896)
+ * kind 2 "TN": C[M,N] = A[K,M]^T . B[K,N]      dW = dY^T X                 (webgpu.ts:900)
+ * FP32 MFMA, f32 accumulate. Any M, N, K >= 1. */
+enum { GT_NT = 0, GT_NN = 1, GT_TN = 2 };
+int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_buf B, gt_buf C);
+/* batch of `count` independent products with element strides between consecutive problems
+ * (Newton-Schulz over same-shaped matrices; no counterpart call in the reference, which loops). */
+int gt_gemm_batched(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t strideA,
+                    gt_buf B, int64_t strideB, gt_buf C, int64_t strideC, int count);
+
+/* ---- elementwise: srcElementwise (wgsl.ts:199-209) with the bodies of webgpu.ts:905-1078 ------ */
+int gt_add_fwd(gt_ctx *ctx, int64_t n, gt_buf a, gt_buf b, gt_buf out);
+int gt_mul_fwd(gt_ctx *ctx, int64_t n, gt_buf a, gt_buf b, gt_buf out);
+int gt_silu_fwd(gt_ctx *ctx, int64_t n, gt_buf x, gt_buf out);
+int gt_gelu_fwd(gt_ctx *ctx, int64_t n, gt_buf x, gt_buf out);       /* tanh form, K=0.7978845608028654, A=0.044715 */
+int gt_scale_fwd(gt_ctx *ctx, int64_t n, gt_buf x, float c, gt_buf out);
+/* a destination of 0 is skipped; da == db (add(t,t), mul(t,t)) is allowed and receives both terms */
+int gt_add_bwd(gt_ctx *ctx, int64_t n, gt_buf g, gt_buf da, int acc_a, gt_buf db, int acc_b);
+int gt_mul_bwd(gt_ctx *ctx, int64_t n, gt_buf g, gt_buf a, gt_buf b, gt_buf da, int acc_a, gt_buf db, int acc_b);
+int gt_silu_bwd(gt_ctx *ctx, int64_t n, gt_buf g, gt_buf x, gt_buf dx, int acc);
+int gt_gelu_bwd(gt_ctx *ctx, int64_t n, gt_buf g, gt_buf x, gt_buf dx, int acc);
+int gt_scale_bwd(gt_ctx *ctx, int64_t n, gt_buf g, float c, gt_buf dx, int acc);
+/* out = act(gate) * up and its backward in one pass each (act 0 = silu, 1 = gelu-tanh): the
+ * mul(silu(gate), up) / mul(gelu(gate), up) pair of src/arch/llama.ts:207-209, gemma3.ts:205-207
+ * fused; backward reads g, gate, up and writes dgate, dup (20 B per element). */
+int gt_glu_fwd(gt_ctx *ctx, int act, int64_t n, gt_buf gate, gt_buf up, gt_buf out);
+int gt_glu_bwd(gt_ctx *ctx, int act, int64_t n, gt_buf g, gt_buf gate, gt_buf up,
+               gt_buf dgate, int acc_gate, gt_buf dup, int acc_up);
+
+/* ---- RMSNorm: srcRmsNormFwd / BwdX / BwdW (wgsl.ts:217-303), rmsNormRows (webgpu.ts:1680-1699) -
+ * Serves rmsNorm (rows = T, d = hidden) and rmsNormHeads (rows = T*H, d = hd; webgpu.ts:1085-1088).
+ * Backward computes dx and the per-column dw sums in one pass over x and g; dw == 0 skips it. */
+int gt_rmsnorm_fwd(gt_ctx *ctx, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y, gt_buf rinv);
+int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv,
+                   gt_buf dx, int acc_dx, gt_buf dw, int acc_dw);
+
+/* ---- embedding: srcEmbeddingFwd / Bwd (wgsl.ts:305-344) ------------------------------------- */
+int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, gt_buf ids, gt_buf W, gt_buf out);
+int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, gt_buf dW, int acc);
+
+/* ---- RoPE: srcRope (wgsl.ts:346-384), NeoX pairing (j, j+hd/2); position of row r is
+ * (r mod T) + pos. backward = 1 applies the transposed rotation. */
+int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, int backward,
+            gt_buf in, gt_buf out, int acc);
+
+/* ---- attention: srcAttnFwd / BwdD / BwdDq / BwdDkv (wgsl.ts:657-918), webgpu.ts:1142-1189 -----
+ * q[B*T, Hq*hd], k,v[B*T, Hkv*hd], causal, window > 0 keeps keys [t-window+1, t]; GQA head h reads
+ * kv head h / (Hq/Hkv). lse[B*Hq*T] is the saved softmax statistic (log2 domain). */
+int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
+                gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
+int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
+                gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf dout, gt_buf lse,
+                gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+
+/* ---- cross-entropy: srcCeFwd / CeReduce / CeBwd (wgsl.ts:936-1133), webgpu.ts:1281-1327 ------
+ * rows = n_seq * T. Sequence s owns rows [s*T, (s+1)*T) and its own denominator
+ * max(kept_s, 1) (autograd.ts:938), passed as inv_denom[s] = 1/denominator (f32, device).
+ * fwd writes loss[s] = inv_denom[s] * sum over kept rows of (logsumexp - z_target) and lse[rows].
+ * bwd: dlogits[r,:] (+)= seed * inv_denom[s] * (softmax - onehot); ignored rows get 0 (acc = 0)
+ * or are left alone (acc = 1). */
+int gt_ce_fwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets, gt_buf inv_denom,
+              gt_buf loss, gt_buf lse);
+int gt_ce_bwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets, gt_buf inv_denom,
+              gt_buf lse, float seed, gt_buf dlogits, int acc);
+/* chunked path: srcCeChunkStats / CeLossFromStats / CeChunkGrad (wgsl.ts:1153-1247),
+ * fusedCrossEntropy (webgpu.ts:1214-1278). `chunk` holds logits of vocab span [v0, v0+vc). */
+int gt_ce_chunk_stats(gt_ctx *ctx, int rows, int vc, int v0, int first, gt_buf chunk, gt_buf targets,
+                      gt_buf row_max, gt_buf row_sum, gt_buf tgt_logit);
+int gt_ce_loss_from_stats(gt_ctx *ctx, int rows, int T, gt_buf targets, gt_buf inv_denom,
+                          gt_buf row_max, gt_buf row_sum, gt_buf tgt_logit, gt_buf loss);
+int gt_ce_chunk_grad(gt_ctx *ctx, int rows, int vc, int v0, int T, gt_buf chunk, gt_buf targets,
+                     gt_buf inv_denom, gt_buf row_max, gt_buf row_sum, float seed);
+/* sparse-teacher soft CE: srcSoftCeFwd / BwdP / BwdQ (wgsl.ts:1004-1110), webgpu.ts:1331-1378 */
+int gt_soft_ce_fwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf teacher_ids, gt_buf teacher_probs,
+                   float inv_denom, gt_buf loss, gt_buf lse, gt_buf row_mass);
+int gt_soft_ce_bwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf teacher_ids, gt_buf teacher_probs,
+                   float inv_denom, gt_buf lse, gt_buf row_mass, float seed, gt_buf dlogits, int acc);
+
+/* ---- AdamW: AdamWGpu (adamw-gpu.ts:131-251), spec src/train/adam.ts:46-82 --------------------
+ * One object per parameter group; step() = global grad-norm clip over the whole group (when
+ * clip > 0) followed by the fused element update, two launches for any number of tensors.
+ * bc1 = 1 - beta1^t and bc2 = 1 - beta2^t come from the host, as in adamw-gpu.ts:211-218. */
+int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *m, const gt_buf *v,
+                    const int64_t *sizes, float beta1, float beta2, float eps, float weight_decay, float clip,
+                    gt_adamw **out);
+int gt_adamw_step(gt_ctx *ctx, gt_adamw *opt, float lr, float bc1, float bc2);
+int gt_adamw_grad_norm(gt_ctx *ctx, gt_adamw *opt, float *norm);   /* last step's global norm; waits */
+int gt_adamw_destroy(gt_ctx *ctx, gt_adamw *opt);
+
+/* ---- Muon: MuonGpu (muon-gpu.ts:351-470), buildNewtonSchulz (:224-252), spec src/train/muon.ts -
+ * Matrices w[i] are [rows[i], cols[i]]; buf[i] is the momentum. step(): buf = mu*buf + g;
+ * U = nesterov ? g + mu*buf : buf; X = NS(U); w -= lr*sqrt(max(1, rows/cols))*X. */
+int gt_muon_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *buf,
+                   const int *rows, const int *cols, float momentum, int nesterov, int ns_steps, gt_muon **out);
+int gt_muon_step(gt_ctx *ctx, gt_muon *opt, float lr);
+int gt_muon_destroy(gt_ctx *ctx, gt_muon *opt);
+/* newtonSchulzGpu (muon-gpu.ts:259-283): out[m,n] = NS(G[m,n]) */
+int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out);
+
+/* ---- profiling: startProfile / stopProfile (webgpu.ts:830-880) --------------------------------
+ * Between begin and end every launch is bracketed by HIP events on the context's stream and
+ * summed per label. gt_prof_end waits, then fills up to `cap` records. */
+typedef struct gt_prof_rec { char label[32]; double ms; int64_t count; } gt_prof_rec;
+int gt_prof_begin(gt_ctx *ctx);
+int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,286 @@
+"""Per-op parity, HIP backend (through the C ABI) against the CPU oracle on identical seeded inputs:
+the op cases of tests/gpu-parity.ts:654-930 and the edge cases it names."""
+import math
+
+import numpy as np
+import pytest
+
+from gpu_common import assert_close, backward_from, mod, op_case
+
+pytestmark = pytest.mark.gpu
+
+
+def R(ref, seed):
+    rng = ref.Mulberry32(seed)
+    return lambda *s, sc=0.8: rng.fill_randn(list(s), sc)
+
+
+@pytest.mark.parametrize("T,ind,outd", [(70, 83, 75), (64, 64, 64), (1, 5, 3), (257, 128, 192), (128, 576, 1536),
+                                        (130, 1536, 576), (33, 16, 200), (512, 40, 16), (300, 1000, 7)])
+def test_linear(gpu, ref, T, ind, outd):
+    """GEMM NT forward, NN dX, TN dW; 70x83 . (75x83)^T is the ragged case of gpu-parity.ts:654-672."""
+    r = R(ref, T * 7 + ind)
+    op_case(gpu, ref, [r(T, ind), r(outd, ind)], lambda ag, x, w: ag.linear(x, w), lambda rf, x, w: rf.linear(x, w),
+            f"linear {T}x{ind}x{outd}")
+
+
+def test_linear_frozen_weight_and_split_k(gpu, ref):
+    """dW with a long K (rows) and a small output takes the split-K path; a frozen weight gets no dW."""
+    r = R(ref, 5)
+    op_case(gpu, ref, [r(4096, 48), r(40, 48)], lambda ag, x, w: ag.linear(x, w), lambda rf, x, w: rf.linear(x, w), "linear split-K")
+    op_case(gpu, ref, [r(96, 48), r(40, 48)], lambda ag, x, w: ag.linear(x, w), lambda rf, x, w: rf.linear(x, w),
+            "linear frozen", frozen=(1,))
+
+
+def test_elementwise(gpu, ref):
+    r = R(ref, 11)
+    for n in [(4, 6), (5, 7), (129, 33), (64, 1024)]:
+        op_case(gpu, ref, [r(*n), r(*n)], lambda ag, a, b: ag.add(a, b), lambda rf, a, b: rf.add(a, b), f"add {n}")
+        op_case(gpu, ref, [r(*n), r(*n)], lambda ag, a, b: ag.mul(a, b), lambda rf, a, b: rf.mul(a, b), f"mul {n}")
+        op_case(gpu, ref, [r(*n, sc=1.5)], lambda ag, x: ag.silu(x), lambda rf, x: rf.silu(x), f"silu {n}")
+        op_case(gpu, ref, [r(*n, sc=1.5)], lambda ag, x: ag.gelu(x), lambda rf, x: rf.gelu(x), f"gelu {n}")
+        op_case(gpu, ref, [r(*n)], lambda ag, x: ag.scale(x, 2.5), lambda rf, x: rf.scale(x, 2.5), f"scale {n}")
+
+
+def test_aliasing_add_mul_same_tensor(gpu, ref):
+    """gpu-parity.ts:2166-2173: add(t,t) and mul(t,t) accumulate both contributions into one gradient."""
+    r = R(ref, 12)
+    op_case(gpu, ref, [r(9, 13)], lambda ag, t: ag.add(t, t), lambda rf, t: rf.add(t, t), "add(t,t)")
+    op_case(gpu, ref, [r(9, 13)], lambda ag, t: ag.mul(t, t), lambda rf, t: rf.mul(t, t), "mul(t,t)")
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_gated_activation_fused_and_unfused(gpu, ref, act, fuse):
+    """mul(act(gate), up): the fused kernels and the unfused pair give the oracle's result; with a second
+    consumer of the activation the fused path must still propagate that consumer's gradient."""
+    r = R(ref, 13)
+    old = gpu.fuse_glu
+    gpu.fuse_glu = fuse
+    try:
+        op_case(gpu, ref, [r(37, 52, sc=1.5), r(37, 52)],
+                lambda ag, g, u: ag.mul(getattr(ag, act)(g), u), lambda rf, g, u: rf.mul(getattr(rf, act)(g), u), f"glu {act}")
+        op_case(gpu, ref, [r(37, 52, sc=1.5), r(37, 52)],
+                lambda ag, g, u: ag.mul(u, getattr(ag, act)(g)), lambda rf, g, u: rf.mul(u, getattr(rf, act)(g)), f"glu swapped {act}")
+
+        def two_uses(m, g, u):
+            a = getattr(m, act)(g)
+            return m.add(m.mul(a, u), a)
+        op_case(gpu, ref, [r(21, 40, sc=1.5), r(21, 40)], lambda ag, g, u: two_uses(ag, g, u),
+                lambda rf, g, u: two_uses(rf, g, u), f"glu + second consumer {act}")
+    finally:
+        gpu.fuse_glu = old
+
+
+@pytest.mark.parametrize("rows,d", [(4, 6), (9, 64), (33, 128), (70, 576), (16, 640), (5, 1024), (3, 2048), (7, 2500), (12, 30)])
+def test_rms_norm(gpu, ref, rows, d):
+    r = R(ref, rows + d)
+    w = 1 + 0.3 * r(d)
+    op_case(gpu, ref, [r(rows, d), w], lambda ag, x, g: ag.rms_norm(x, g, 1e-5), lambda rf, x, g: rf.rms_norm(x, g, 1e-5), f"rmsNorm {rows}x{d}")
+    op_case(gpu, ref, [r(rows, d), w], lambda ag, x, g: ag.rms_norm(x, g, 1e-5), lambda rf, x, g: rf.rms_norm(x, g, 1e-5),
+            f"rmsNorm frozen gain {rows}x{d}", frozen=(1,))
+
+
+@pytest.mark.parametrize("T,H,hd", [(3, 2, 4), (17, 9, 64), (20, 16, 128), (11, 3, 32), (5, 2, 6)])
+def test_rms_norm_heads(gpu, ref, T, H, hd):
+    r = R(ref, T + hd)
+    w = 1 + 0.3 * r(hd)
+    op_case(gpu, ref, [r(T, H * hd), w], lambda ag, x, g: ag.rms_norm_heads(x, g, T, H, hd, 1e-6),
+            lambda rf, x, g: rf.rms_norm_heads(x, g, T, H, hd, 1e-6), f"rmsNormHeads {T},{H},{hd}")
+
+
+def test_embedding_repeated_ids(gpu, ref):
+    r = R(ref, 3)
+    ids = [0, 3, 3, 6, 1, 3]
+    op_case(gpu, ref, [r(7, 4)], lambda ag, w: ag.embedding(w, ids), lambda rf, w: rf.embedding(w, ids), "embedding")
+    rng = ref.Mulberry32(8)
+    ids = [min(511, int(512 * rng() ** 3)) for _ in range(700)]       # skewed: many repeats of small ids
+    op_case(gpu, ref, [r(512, 96)], lambda ag, w: ag.embedding(w, ids), lambda rf, w: rf.embedding(w, ids), "embedding skewed")
+    ids = [5] * 300
+    op_case(gpu, ref, [r(9, 33)], lambda ag, w: ag.embedding(w, ids), lambda rf, w: rf.embedding(w, ids), "embedding one id")
+
+
+@pytest.mark.parametrize("T,H,hd,base,pos", [(4, 2, 6, 1e4, 0), (4, 2, 6, 1e4, 5), (130, 9, 64, 1e5, 0), (64, 3, 128, 1e6, 17)])
+def test_rope(gpu, ref, T, H, hd, base, pos):
+    r = R(ref, T + hd)
+    op_case(gpu, ref, [r(T, H * hd)], lambda ag, x: ag.rope(x, T, H, hd, base, pos), lambda rf, x: rf.rope(x, T, H, hd, base, pos), "rope")
+
+
+def test_rope_far_positions(gpu, ref):
+    """Position 2047 at pair 0 is where per-element f32 angles lose ~1e-4; the f64-built table must not."""
+    r = R(ref, 99)
+    T, H, hd = 2048, 1, 64
+    op_case(gpu, ref, [r(T, H * hd)], lambda ag, x: ag.rope(x, T, H, hd, 1e5, 0), lambda rf, x: rf.rope(x, T, H, hd, 1e5, 0), "rope T=2048")
+
+
+ATTN = [(5, 4, 2, 6, 0), (67, 4, 2, 16, 0), (130, 6, 2, 32, 0), (193, 9, 3, 64, 0), (64, 2, 2, 64, 0), (256, 4, 1, 64, 0),
+        (96, 16, 8, 128, 0), (6, 4, 2, 6, 3), (130, 4, 2, 16, 17), (200, 10, 2, 64, 64), (150, 2, 1, 64, 1)]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,hd,window", ATTN)
+def test_attention(gpu, ref, T, Hq, Hkv, hd, window):
+    """gpu-parity.ts:872-930: GQA, head dims 6..128, full causal and sliding windows (1, smaller and larger than a tile)."""
+    r = R(ref, T * 3 + hd + window)
+    op_case(gpu, ref, [r(T, Hq * hd), r(T, Hkv * hd), r(T, Hkv * hd)],
+            lambda ag, q, k, v: ag.attention(q, k, v, T, Hq, Hkv, hd, window),
+            lambda rf, q, k, v: rf.attention(q, k, v, T, Hq, Hkv, hd, window), f"attention {T},{Hq},{Hkv},{hd},w{window}")
+
+
+def test_attention_stacked_sequences(gpu, ref):
+    """rows = B*T: each sequence attends only to itself, positions restart per sequence."""
+    ag = mod("autograd")
+    B, T, Hq, Hkv, hd = 3, 40, 4, 2, 16
+    r = R(ref, 77)
+    q, k, v = r(B * T, Hq * hd), r(B * T, Hkv * hd), r(B * T, Hkv * hd)
+    up = ref.Mulberry32(1).fill_uniform([B * T * Hq * hd])
+    hq, hk, hv = (ag.Tensor(a, list(a.shape), True) for a in (q, k, v))
+    gpu.install()
+    try:
+        out = ag.attention(ag.rope(hq, T, Hq, hd, 1e4), ag.rope(hk, T, Hkv, hd, 1e4), hv, T, Hq, Hkv, hd, 0)
+        backward_from(gpu, ag, out, up)
+        gpu.sync([out])
+    finally:
+        gpu.uninstall()
+    for b in range(B):
+        s = slice(b * T, (b + 1) * T)
+        rq, rk, rv = (ref.Tensor(a[s], [T, a.shape[1]], True) for a in (q, k, v))
+        o = ref.attention(ref.rope(rq, T, Hq, hd, 1e4), ref.rope(rk, T, Hkv, hd, 1e4), rv, T, Hq, Hkv, hd, 0)
+        ref.backward_from(o, up.reshape(B, -1)[b])
+        assert_close(out.data.reshape(B, -1)[b], o.data, f"stacked attention out[{b}]")
+        for h, rr, nm in ((hq, rq, "q"), (hk, rk, "k"), (hv, rv, "v")):
+            assert_close(h.grad.reshape(B, -1)[b], rr.grad, f"stacked attention d{nm}[{b}]")
+
+
+def test_cross_entropy_cases(gpu, ref):
+    """gpu-parity.ts:762-829: ignore-index rows, V > 256, a target far behind the maximum, closed-form rows."""
+    r = R(ref, 21)
+    tg = [2, 7, -1, 0, 8, -1, 3]
+    op_case(gpu, ref, [r(7, 9)], lambda ag, z: ag.cross_entropy(z, tg), lambda rf, z: rf.cross_entropy(z, tg), "CE ignore")
+    rng = ref.Mulberry32(4)
+    tg = [int(rng() * 1000) for _ in range(33)]
+    tg[5] = tg[20] = -1
+    op_case(gpu, ref, [r(33, 1000, sc=2.0)], lambda ag, z: ag.cross_entropy(z, tg), lambda rf, z: rf.cross_entropy(z, tg), "CE V=1000")
+    tg = [int(rng() * 1003) for _ in range(10)]
+    op_case(gpu, ref, [r(10, 1003, sc=2.0)], lambda ag, z: ag.cross_entropy(z, tg), lambda rf, z: rf.cross_entropy(z, tg), "CE V=1003 (unaligned rows)")
+    z = np.array([[90, 0, 0, -3], [60, 1, 0, 0]], dtype=np.float32)
+    out_h, _ = op_case(gpu, ref, [z], lambda ag, x: ag.cross_entropy(x, [3, 2]), lambda rf, x: rf.cross_entropy(x, [3, 2]), "CE far-behind target")
+    exact = (math.log(math.exp(90) + 2 + math.exp(-3)) + 3 + math.log(math.exp(60) + math.e + 2)) / 2
+    assert abs(out_h.data[0] - exact) < 1e-4
+    for gap in [1, 10, 30, 60, 90]:
+        row = np.array([[gap, 0, 0, -3]], dtype=np.float32)
+        out_h, _ = op_case(gpu, ref, [row], lambda ag, x: ag.cross_entropy(x, [3]), lambda rf, x: rf.cross_entropy(x, [3]), f"CE gap {gap}")
+        assert abs(out_h.data[0] - (math.log(math.exp(gap) + 2 + math.exp(-3)) + 3)) < 1e-4
+
+
+def test_cross_entropy_all_ignored_is_exactly_zero(gpu, ref):
+    """gpu-parity.ts:2419-2502."""
+    ag = mod("autograd")
+    z = ag.Tensor(ref.Mulberry32(2).fill_randn([6, 50]), [6, 50], True)
+    h = ag.Tensor(ref.Mulberry32(3).fill_randn([6, 8]), [6, 8], True)
+    w = ag.Tensor(ref.Mulberry32(4).fill_randn([50, 8]), [50, 8], True)
+    gpu.install()
+    try:
+        l1 = ag.cross_entropy(z, [-1] * 6)
+        ag.backward(l1, 1.0)
+        l2 = ag.fused_cross_entropy(h, w, [-1] * 6, 16)
+        ag.backward(l2, 1.0)
+        gpu.sync([l1, l2])
+    finally:
+        gpu.uninstall()
+    assert l1.data[0] == 0.0 and l2.data[0] == 0.0
+    assert not np.any(z.grad) and not np.any(h.grad) and not np.any(w.grad)
+
+
+def test_cross_entropy_per_sequence_denominators(gpu, ref):
+    """Stacked sequences: one loss per sequence over its own kept count, equal to separate calls."""
+    ag = mod("autograd")
+    B, T, V = 3, 11, 40
+    z = ref.Mulberry32(6).fill_randn([B * T, V], 2.0)
+    rng = ref.Mulberry32(7)
+    tg = [int(rng() * V) if rng() > 0.4 else -1 for _ in range(B * T)]
+    hz = ag.Tensor(z, [B * T, V], True)
+    gpu.install()
+    try:
+        loss = ag.cross_entropy(hz, tg, seq_len=T)
+        ag.backward(loss, 1.0 / B)
+        gpu.sync([loss])
+    finally:
+        gpu.uninstall()
+    for b in range(B):
+        rz = ref.Tensor(z[b * T:(b + 1) * T], [T, V], True)
+        rl = ref.cross_entropy(rz, tg[b * T:(b + 1) * T])
+        ref.backward(rl, 1.0 / B)
+        assert abs(loss.data[b] - rl.data[0]) <= 1e-5 * abs(rl.data[0])
+        assert_close(hz.grad.reshape(B, -1)[b], rz.grad, f"stacked CE dz[{b}]")
+
+
+@pytest.mark.parametrize("chunk", [1, 7, 16, 64, 100])
+def test_fused_cross_entropy_equals_dense(gpu, ref, chunk):
+    """gpu-parity.ts:166-208 / gradcheck.ts:854-877."""
+    r = R(ref, 31)
+    tg = [3, -1, 36, 0, 7, -1, 7, 20, 1]
+    op_case(gpu, ref, [r(9, 24), r(37, 24)], lambda ag, h, w: ag.fused_cross_entropy(h, w, tg, chunk),
+            lambda rf, h, w: rf.cross_entropy(rf.linear(h, w), tg), f"fusedCE chunk {chunk}")
+    op_case(gpu, ref, [r(9, 24), r(37, 24)], lambda ag, h, w: ag.fused_cross_entropy(h, w, tg, chunk),
+            lambda rf, h, w: rf.fused_cross_entropy(h, w, tg, chunk), f"fusedCE frozen readout {chunk}", frozen=(1,))
+
+
+def test_soft_cross_entropy(gpu, ref):
+    r = R(ref, 41)
+    T, V, k = 6, 50, 3
+    rng = ref.Mulberry32(9)
+    tids, tp = [], []
+    for t in range(T):
+        row = [int(rng() * V) for _ in range(k)]
+        pr = [0.5, 0.3, 0.0] if t % 2 else [0.4, 0.25, 0.1]
+        if t == 2:
+            row[0] = -1
+        if t == 4:
+            row[1] = row[0]           # duplicate id inside a row
+        tids += row
+        tp += pr
+    op_case(gpu, ref, [r(T, V, sc=2.0)], lambda ag, z: ag.soft_cross_entropy(z, tids, tp, k),
+            lambda rf, z: rf.soft_cross_entropy(z, tids, tp, k), "softCE")
+
+
+def test_validators_refuse_above_the_dispatch(gpu, ref):
+    """gpu-parity.ts:2203-2290: malformed inputs raise before any device work."""
+    ag = mod("autograd")
+    gpu.install()
+    try:
+        x = ag.Tensor(np.zeros((3, 5), np.float32), [3, 5], True)
+        w = ag.Tensor(np.zeros((4, 6), np.float32), [4, 6], True)
+        with pytest.raises(ValueError, match="linear dim mismatch"):
+            ag.linear(x, w)
+        e = ag.Tensor(np.zeros((4, 3), np.float32), [4, 3], True)
+        with pytest.raises(ValueError, match="not an integer in"):
+            ag.embedding(e, [0, 6])
+        z = ag.Tensor(np.zeros((3, 6), np.float32), [3, 6], True)
+        with pytest.raises(ValueError, match="not -1"):
+            ag.cross_entropy(z, [0, 6, 1])
+        with pytest.raises(ValueError, match="not -1"):
+            ag.cross_entropy(z, [0, -2, 1])
+        with pytest.raises(ValueError, match="targets for"):
+            ag.cross_entropy(z, [0, 1])
+        with pytest.raises(ValueError, match="chunk must be positive"):
+            ag.fused_cross_entropy(x, ag.Tensor(np.zeros((7, 5), np.float32), [7, 5], True), [0, 1, 2], 0)
+        with pytest.raises(ValueError, match="teacher id"):
+            ag.soft_cross_entropy(z, [0, 9, 1], [1.0, 1.0, 1.0], 1)
+    finally:
+        gpu.uninstall()
+
+
+def test_late_backward_after_sync_is_refused(gpu, ref):
+    """webgpu.ts:1412-1418 (test gpu-parity.ts:1842-1850): a backward over a graph whose buffers a sync recycled throws."""
+    ag = mod("autograd")
+    x = ag.Tensor(np.ones((4, 8), np.float32), [4, 8], True)
+    w = ag.Tensor(np.ones((8, 8), np.float32), [8, 8], True)
+    gpu.install()
+    try:
+        loss = ag.cross_entropy(ag.linear(x, w), [1, 2, 3, 4])
+        gpu.sync([loss])
+        with pytest.raises(RuntimeError, match="before a sync"):
+            ag.backward(loss, 1.0)
+    finally:
+        gpu.uninstall()
+        gpu.sync([])
