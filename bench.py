@@ -1,0 +1,202 @@
+#!/usr/bin/env python3
+"""Headline benchmark: train tokens/s of one full training step (forward + backward + AdamW, loss read
+back every step) at the SmolLM2-135M shape, seq 2048 x batch 8, fp32, on one MI355X, plus the roofline of the
+dominant kernel (the backward GEMMs, against the FP32 MFMA peak) and a CPU baseline beside it.
+
+    python bench.py [--gpus 1] [--steps 20] [--warmup 3]
+
+One JSON line on stdout. `value` is tokens/s with every input already resident in HBM at the start of the timed
+region (weights, optimizer state and the token batches' ids are uploaded by the step itself: 128 KiB per step).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+PKG = "gguf-trainer_amd"
+
+PEAK_FP32_MFMA = 157.3e12      # MI355X dense FP32 matrix peak, FLOP/s
+PEAK_HBM = 8.0e12              # B/s
+
+SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
+               rope_base=100000.0, rms_eps=1e-5, tie=True)
+SEQ, BATCH = 2048, 8
+
+
+def synth_weights(arch, cfg, seed=0):
+    """Random-init weights of the named architecture: matrices N(0, 0.02), norm gains 1."""
+    rs = np.random.RandomState(seed)
+    w = {}
+    for n in arch.param_names(cfg):
+        shp = arch.param_shape(cfg, n)
+        w[n] = np.ones(shp, np.float32) if len(shp) == 1 else (0.02 * rs.standard_normal(shp)).astype(np.float32)
+    return w
+
+
+def zipf_tokens(vocab, n, seed, s=1.1):
+    """Zipf(1.1) over the vocabulary by inverse CDF, on a fixed permutation of the ids."""
+    rs = np.random.RandomState(seed)
+    p = 1.0 / np.arange(1, vocab + 1, dtype=np.float64) ** s
+    cdf = np.cumsum(p / p.sum())
+    perm = np.random.RandomState(12345).permutation(vocab)
+    return perm[np.minimum(np.searchsorted(cdf, rs.rand(n)), vocab - 1)].astype(np.int64)
+
+
+def cpu_baseline(seconds_hint=20.0):
+    """The CPU oracle (a C restatement of the reference's CPU ops) on a bounded sample of the same workload:
+    one 256-token sequence through 2 of the 30 layers (forward + backward), the full tied readout + cross-entropy,
+    and AdamW over those parameters; the per-token time is extrapolated to 30 layers. OpenMP over the host cores
+    where the loops write disjoint outputs (dW/dX as per-output dot products). Reported, never a target."""
+    from oracle import ref
+    cores = max(1, min(ref.max_threads(), len(os.sched_getaffinity(0))))
+    ref.set_threads(cores)
+    T, L = 256, 2
+    kw = dict(SMOLLM2)
+    kw["layers"] = L
+    rs = np.random.RandomState(0)
+    cfg = ref.ModelConfig(**kw)
+    weights = {}
+    for n, shp in [("tokenEmbd", [cfg.vocab, cfg.hidden]), ("outputNorm", [cfg.hidden])] + \
+                  [(f"L{l}.{k}", s) for l in range(L) for k, s in ref.layer_shapes(cfg).items()]:
+        weights[n] = np.ones(shp, np.float32) if len(shp) == 1 else (0.02 * rs.standard_normal(shp)).astype(np.float32)
+    model = ref.Model(cfg, weights=weights)
+    ids = zipf_tokens(cfg.vocab, T + 1, 1)
+    ref.PARALLEL_BWD = True
+    try:
+        t0 = time.perf_counter()
+        loss = ref.sequence_loss(model, ids[:-1].tolist(), ids[1:].tolist())
+        ref.backward(loss, 1.0)
+        t_all = time.perf_counter() - t0
+        # split: time the two layers alone (no embedding / readout / loss)
+        h0 = ref.Tensor(0.02 * rs.standard_normal((T, cfg.hidden)).astype(np.float32), [T, cfg.hidden], True)
+        t0 = time.perf_counter()
+        h = h0
+        for il, Lw in enumerate(model.layers):
+            h = model._block(h, Lw, il, T)()
+        ref.backward_from(h, np.ones(h.size, np.float32))
+        t_layers = time.perf_counter() - t0
+        opt = ref.AdamW(model.params(), lr=1e-3, beta2=0.95, weight_decay=0.1)
+        t0 = time.perf_counter()
+        opt.step()
+        t_opt = time.perf_counter() - t0
+    finally:
+        ref.PARALLEL_BWD = False
+        ref.set_threads(1)
+    t_head = max(t_all - t_layers, 0.0)
+    n_layer_params = sum(p.size for Lw in model.layers for p in Lw.values())
+    n_head_params = model.tokenEmbd.size + model.outputNorm.size
+    t_opt_full = t_opt * (n_head_params + n_layer_params / L * 30) / (n_head_params + n_layer_params)
+    # one optimizer step serves BATCH*SEQ tokens
+    per_token = (t_layers / L * 30 + t_head) / T + t_opt_full / (BATCH * SEQ)
+    return {"value": round(1.0 / per_token, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"oracle (C restatement of the reference's CPU ops), 1 sequence x {T} tokens through {L} of 30 layers "
+                      f"fwd+bwd ({t_layers:.1f}s) + full readout and cross-entropy ({t_head:.1f}s) + AdamW ({t_opt:.1f}s); "
+                      f"per-token time extrapolated to 30 layers; attention is O(T) per token so T=2048 would be slower"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+              "(no collectives are part of it, see DESIGN.md on sharding)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch  # device plumbing only: make sure a GPU is there before touching the library
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    ag = importlib.import_module(f"{PKG}.autograd")
+    hb = importlib.import_module(f"{PKG}.hip_backend")
+    arch = importlib.import_module(f"{PKG}.arch")
+    optim = importlib.import_module(f"{PKG}.optim")
+
+    cfg = arch.ModelConfig(**SMOLLM2)
+    model = arch.Model(cfg, synth_weights(arch, cfg))
+    n_params = sum(p.size for p in model.params())
+    gpu = hb.require_gpu("bench.py")
+    opt = optim.AdamWHip(gpu, model.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
+    total = a.steps + a.warmup
+    toks = [zipf_tokens(cfg.vocab, BATCH * (SEQ + 1), 100 + i).reshape(BATCH, SEQ + 1) for i in range(total)]
+
+    def step(i):
+        t = toks[i]
+        if a.sequential:
+            losses = []
+            for b in range(BATCH):
+                loss = arch.sequence_loss(model, t[b, :-1], t[b, 1:], 0)
+                ag.backward(loss, 1.0 / BATCH)
+                losses.append(loss)
+        else:
+            loss = arch.sequence_loss(model, t[:, :-1].reshape(-1), t[:, 1:].reshape(-1), 0, SEQ)
+            ag.backward(loss, 1.0 / BATCH)
+            losses = [loss]
+        gpu.sync(losses)                     # loss scalars back to the host, as train-gpu.ts:221
+        opt.record_step()
+        gpu.sync([])
+        return float(np.mean(np.concatenate([l.data for l in losses])))
+
+    gpu.install()
+    try:
+        losses = [step(i) for i in range(a.warmup)]
+        gpu.sync([])
+        torch.cuda.synchronize()
+        gpu.start_profile("gemm.")           # HIP events on the library's stream around every GEMM launch
+        t0 = time.perf_counter()
+        for i in range(a.warmup, total):
+            losses.append(step(i))
+        gpu.sync([])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        prof = gpu.stop_profile()
+    finally:
+        gpu.uninstall()
+
+    tokens = a.steps * BATCH * SEQ
+    # dominant kernel: the backward GEMMs (NN = dX, TN = dW); the one tile shape with the most time stands for it
+    bwd = {k: v for k, v in prof.items() if k.startswith("gemm.nn") or k.startswith("gemm.tn")}
+    dom = max(bwd, key=lambda k: bwd[k][0]) if bwd else None
+    roof = None
+    if dom:
+        ms, cnt, work = bwd[dom]
+        ach = work / (ms * 1e-3)
+        all_ms = sum(v[0] for v in bwd.values())
+        all_work = sum(v[2] for v in bwd.values())
+        roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach / 1e12, 3), "peak": PEAK_FP32_MFMA / 1e12,
+                "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA, 4), "traffic": None,
+                "launches": int(cnt), "avg_launch_ms": round(ms / cnt, 4),
+                "all_bwd_gemms": {"achieved": round(all_work / (all_ms * 1e-3) / 1e12, 3), "ms_per_step": round(all_ms / a.steps, 2),
+                                  "frac": round(all_work / (all_ms * 1e-3) / PEAK_FP32_MFMA, 4)},
+                "per_kernel": {k: {"TFLOP/s": round(v[2] / (v[0] * 1e-3) / 1e12, 2), "ms_per_step": round(v[0] / a.steps, 2),
+                                   "launches_per_step": v[1] // a.steps} for k, v in sorted(prof.items())}}
+    out = {
+        "metric": "train tokens/s (SmolLM2-135M shape, 2048x8); bwd GEMM % FP32 MFMA peak",
+        "value": round(tokens / wall, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(1e3 * wall / a.steps, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic (weights N(0,0.02) random init, tokens Zipf(1.1) over the vocab)",
+        "config": {"workload": "configs[3]: SmolLM2-135M llama shape, fwd+bwd+AdamW, seq 2048 x batch 8, fp32",
+                   "params": n_params, "global_batch": BATCH, "seq_len": SEQ,
+                   "graph": "sequential micro-batches" if a.sequential else "8 sequences stacked into one 16384-row graph",
+                   "device": gpu.adapter_name},
+        "loss_first": round(losses[0], 4), "loss_last": round(losses[-1], 4),
+        "roofline": roof,
+        "cpu_baseline": None if a.no_cpu else cpu_baseline(),
+    }
+    gpu.destroy()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -224,7 +224,12 @@ static int check(gt_ctx *ctx, const char *who, int B, int T, int Hq, int Hkv, in
   return 0;
 }
 
-static bool g_no_mfma = false;
+// (query, key) pairs a causal / windowed sequence of T scores
+static double attn_pairs(int T, int window) {
+  double p = 0;
+  for (int t = 0; t < T; t++) p += (window > 0 && t + 1 > window) ? window : t + 1;
+  return p;
+}
 
 extern "C" {
 int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
@@ -233,10 +238,8 @@ int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   if (check(ctx, "gt_attn_fwd", B, T, Hq, Hkv, hd, window)) return 1;
   GT_REQUIRE(ctx, q && k && v && out && lse, "gt_attn_fwd: null operand");
   AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd)};
-  ProfScope ps(ctx, "attention");
-  static bool env = (g_no_mfma = getenv("GGUFHIP_ATTN_GENERIC") != nullptr, true);
-  (void)env;
-  if (!g_no_mfma && attn_mfma_supported(hd)) return attn_fwd_mfma(ctx, p, q, k, v, out, lse);
+  ProfScope ps(ctx, "attention", 2.0 * 2 * hd * attn_pairs(T, window) * Hq * B);   // QK^T and PV
+  if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) return attn_fwd_mfma(ctx, p, q, k, v, out, lse);
   int64_t rows = (int64_t)B * Hq * T;
   size_t smem = 4 * (size_t)(hd + WAVE) * sizeof(float);
   hipLaunchKernelGGL(attn_fwd_gen, dim3((unsigned)cdiv(rows, 4)), dim3(256), smem, ctx->stream, p, P<const float>(q),
@@ -252,25 +255,26 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   GT_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, "gt_attn_bwd: null operand");
   AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd)};
   int64_t rows = (int64_t)B * Hq * T, krows = (int64_t)B * Hkv * T;
+  ProfScope whole(ctx, "attention.bwd", 5.0 * 2 * hd * attn_pairs(T, window) * Hq * B);   // S, dP, dV, dK, dQ
   void *ws;
   if (gt_ws_reserve(ctx, (size_t)rows * sizeof(float), &ws)) return 1;
   float *Dr = static_cast<float *>(ws);
   {
-    ProfScope ps(ctx, "attention.bwdD");
+    ProfScope ps(ctx, "attention.bwd.D");
     hipLaunchKernelGGL(attn_bwd_d, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, p, P<const float>(out),
                        P<const float>(dout), Dr);
     GT_LAUNCHED(ctx);
   }
-  if (!g_no_mfma && attn_mfma_supported(hd)) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, dq, acc_q, dk, acc_k, dv, acc_v);
+  if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, dq, acc_q, dk, acc_k, dv, acc_v);
   {
-    ProfScope ps(ctx, "attention.bwdDq");
+    ProfScope ps(ctx, "attention.bwd.dq");
     size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);
     hipLaunchKernelGGL(attn_bwd_dq_gen, dim3((unsigned)cdiv(rows, 4)), dim3(256), smem, ctx->stream, p, P<const float>(q),
                        P<const float>(k), P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q);
     GT_LAUNCHED(ctx);
   }
   {
-    ProfScope ps(ctx, "attention.bwdDkv");
+    ProfScope ps(ctx, "attention.bwd.dkv");
     size_t smem = 4 * (size_t)(2 * hd + 2 * WAVE) * sizeof(float);
     hipLaunchKernelGGL(attn_bwd_dkv_gen, dim3((unsigned)cdiv(krows, 4)), dim3(256), smem, ctx->stream, p, P<const float>(q),
                        P<const float>(k), P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k,

@@ -218,7 +218,7 @@ int gt_ce_fwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 1 && V >= 1 && T >= 1 && rows % T == 0, "gt_ce_fwd: rows %d must be a positive multiple of T %d", rows, T);
   GT_REQUIRE(ctx, logits && targets && inv_denom && loss && lse, "gt_ce_fwd: null operand");
-  ProfScope ps(ctx, "ce");
+  ProfScope ps(ctx, "ce", 4.0 * rows * V);
   void *ws;
   if (gt_ws_reserve(ctx, (size_t)rows * sizeof(float), &ws)) return 1;
   hipLaunchKernelGGL(ce_fwd_rows, dim3(rows), dim3(256), 0, ctx->stream, V, P<const float>(logits), P<const int>(targets),
@@ -234,7 +234,7 @@ int gt_ce_bwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 1 && V >= 1 && T >= 1 && rows % T == 0, "gt_ce_bwd: rows %d must be a positive multiple of T %d", rows, T);
   GT_REQUIRE(ctx, logits && targets && inv_denom && lse && dlogits, "gt_ce_bwd: null operand");
-  ProfScope ps(ctx, "ce.bwd");
+  ProfScope ps(ctx, "ce.bwd", 8.0 * rows * V);          // read z, write dz
   hipLaunchKernelGGL(ce_bwd_k, dim3(rows, row_chunks(V)), dim3(256), 0, ctx->stream, V, T, P<const float>(logits),
                      P<const int>(targets), P<const float>(inv_denom), P<const float>(lse), seed, P<float>(dlogits), acc);
   GT_LAUNCHED(ctx);

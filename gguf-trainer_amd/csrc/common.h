@@ -13,7 +13,7 @@
 
 #define WAVE 64
 
-struct ProfEvent { std::string label; hipEvent_t a, b; };
+struct ProfEvent { std::string label; hipEvent_t a, b; double work; };
 
 struct gt_ctx {
   int device = 0;
@@ -30,7 +30,9 @@ struct gt_ctx {
   struct RopeKey { int T, hd, pos; double base; bool operator<(const RopeKey &o) const {
     if (T != o.T) return T < o.T; if (hd != o.hd) return hd < o.hd; if (pos != o.pos) return pos < o.pos; return base < o.base; } };
   std::map<RopeKey, float *> rope_tables;
+  int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1;
   bool prof_on = false;
+  std::string prof_prefix;
   std::vector<ProfEvent> prof;
 };
 
@@ -49,15 +51,17 @@ int gt_ws_reserve(gt_ctx *ctx, size_t bytes, void **out);
 
 // Brackets the launches made during its lifetime with a pair of events when profiling is on.
 struct ProfScope {
-  gt_ctx *c; bool on;
-  ProfScope(gt_ctx *ctx, const char *label) : c(ctx), on(ctx->prof_on) {
+  gt_ctx *c; bool on; size_t idx = 0;
+  ProfScope(gt_ctx *ctx, const char *label, double work = 0) : c(ctx), on(ctx->prof_on) {
+    if (on && !ctx->prof_prefix.empty() && strncmp(label, ctx->prof_prefix.c_str(), ctx->prof_prefix.size()) != 0) on = false;
     if (!on) return;
-    ProfEvent e; e.label = label;
+    ProfEvent e; e.label = label; e.work = work;
     (void)hipEventCreate(&e.a); (void)hipEventCreate(&e.b);
     (void)hipEventRecord(e.a, c->stream);
     c->prof.push_back(e);
+    idx = c->prof.size() - 1;
   }
-  ~ProfScope() { if (on) (void)hipEventRecord(c->prof.back().b, c->stream); }
+  ~ProfScope() { if (on) (void)hipEventRecord(c->prof[idx].b, c->stream); }
 };
 
 template <typename T> static inline T *P(gt_buf b) { return reinterpret_cast<T *>(b); }

@@ -119,8 +119,18 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes) {
   return 0;
 }
 
-int gt_prof_begin(gt_ctx *ctx) {
+int gt_set_option(gt_ctx *ctx, const char *key, int value) {
+  if (!ctx || !key) return 1;
+  if (!strcmp(key, "attn.generic")) ctx->opt_attn_generic = value;
+  else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
+  else if (!strcmp(key, "gemm.splitk")) ctx->opt_gemm_splitk = value;
+  else GT_FAIL(ctx, "gt_set_option: unknown key '%s'", key);
+  return 0;
+}
+
+int gt_prof_begin(gt_ctx *ctx, const char *prefix) {
   GT_ENTER(ctx);
+  ctx->prof_prefix = prefix ? prefix : "";
   for (auto &e : ctx->prof) { hipEventDestroy(e.a); hipEventDestroy(e.b); }
   ctx->prof.clear();
   ctx->prof_on = true;
@@ -131,14 +141,16 @@ int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n) {
   GT_ENTER(ctx);
   ctx->prof_on = false;
   GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  std::map<std::string, std::pair<double, int64_t>> sum;
+  struct Acc { double ms = 0, work = 0; int64_t n = 0; };
+  std::map<std::string, Acc> sum;
   std::vector<std::string> order;
   for (auto &e : ctx->prof) {
     float ms = 0;
     GT_HIP(ctx, hipEventElapsedTime(&ms, e.a, e.b));
     if (!sum.count(e.label)) order.push_back(e.label);
-    sum[e.label].first += ms;
-    sum[e.label].second += 1;
+    sum[e.label].ms += ms;
+    sum[e.label].n += 1;
+    sum[e.label].work += e.work;
     hipEventDestroy(e.a); hipEventDestroy(e.b);
   }
   ctx->prof.clear();
@@ -146,8 +158,9 @@ int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n) {
   for (auto &l : order) {
     if (k >= cap) break;
     snprintf(out[k].label, sizeof out[k].label, "%s", l.c_str());
-    out[k].ms = sum[l].first;
-    out[k].count = sum[l].second;
+    out[k].ms = sum[l].ms;
+    out[k].count = sum[l].n;
+    out[k].work = sum[l].work;
     k++;
   }
   if (n) *n = k;

@@ -105,11 +105,12 @@ static inline unsigned ew_grid(gt_ctx *ctx, int64_t n) {
 
 template <int OP, bool HASB>
 static int run_fwd(gt_ctx *ctx, const char *label, int64_t n, gt_buf a, gt_buf b, float c, gt_buf out) {
+  const double bytes = 4.0 * n * (HASB ? 3 : 2);
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, n >= 0 && a && out && (!HASB || b), "%s: null operand", label);
   GT_REQUIRE(ctx, (a | b | out) % 16 == 0, "%s: buffers must be 16-byte aligned", label);
   if (n == 0) return 0;
-  ProfScope ps(ctx, label);
+  ProfScope ps(ctx, label, bytes);
   hipLaunchKernelGGL((ew_fwd<OP, HASB>), dim3(ew_grid(ctx, n)), dim3(256), 0, ctx->stream, n, P<const float>(a),
                      P<const float>(b), c, P<float>(out));
   GT_LAUNCHED(ctx);
@@ -123,7 +124,9 @@ static int run_bwd(gt_ctx *ctx, const char *label, int64_t n, gt_buf g, gt_buf a
   GT_REQUIRE(ctx, (g | a | b | da | db) % 16 == 0, "%s: buffers must be 16-byte aligned", label);
   if (n == 0 || (!da && !db)) return 0;
   int same = (da && da == db) ? 1 : 0;
-  ProfScope ps(ctx, label);
+  // algorithmic bytes: g and the saved inputs read once, each destination written once
+  const double bytes = 4.0 * n * (1 + (NEEDA ? 1 : 0) + (NEEDB ? 1 : 0) + (da ? 1 : 0) + ((db && !same) ? 1 : 0));
+  ProfScope ps(ctx, label, bytes);
   hipLaunchKernelGGL((ew_bwd<OP, NEEDA, NEEDB>), dim3(ew_grid(ctx, n)), dim3(256), 0, ctx->stream, n, P<const float>(g),
                      P<const float>(a), P<const float>(b), c, P<float>(da), acc_a, P<float>(db), acc_b, same);
   GT_LAUNCHED(ctx);

@@ -118,7 +118,7 @@ int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, gt_buf ids, gt_buf W, gt_buf 
 int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, gt_buf dW, int acc) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 0 && d >= 1 && V >= 1 && ids && g && dW, "gt_embedding_bwd: bad arguments");
-  ProfScope ps(ctx, "embedding.bwd");
+  ProfScope ps(ctx, "embedding.bwd", 8.0 * rows * d);
   if (!acc) GT_HIP(ctx, hipMemsetAsync(P<void>(dW), 0, (size_t)V * d * sizeof(float), ctx->stream));
   if (rows == 0) return 0;
   void *ws;
@@ -137,7 +137,7 @@ int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, i
   GT_REQUIRE(ctx, rows >= 0 && T >= 1 && H >= 1 && hd >= 2 && hd % 2 == 0 && in && out, "gt_rope: bad arguments (hd %d)", hd);
   GT_REQUIRE(ctx, rows % T == 0, "gt_rope: rows %d is not a whole number of sequences of %d", rows, T);
   if (rows == 0) return 0;
-  ProfScope ps(ctx, backward ? "rope.bwd" : "rope");
+  ProfScope ps(ctx, backward ? "rope.bwd" : "rope", 8.0 * rows * H * hd);
   gt_ctx::RopeKey key{T, hd, pos, base};
   auto it = ctx->rope_tables.find(key);
   float *tab;

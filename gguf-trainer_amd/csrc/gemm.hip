@@ -216,15 +216,12 @@ static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
   return 0;
 }
 
-static int g_force_cfg = -1;     // tuning hook: GGUFHIP_GEMM_CFG=0..3 pins the tile shape
-
 static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
                      gt_buf C, int64_t sC, int count) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, kind >= 0 && kind <= 2, "gt_gemm: kind %d is not NT(0)/NN(1)/TN(2)", kind);
   GT_REQUIRE(ctx, M >= 1 && N >= 1 && K >= 1 && count >= 1, "gt_gemm: M,N,K,count must be >= 1 (got %d,%d,%d,%d)", M, N, K, count);
   GT_REQUIRE(ctx, A && B && C, "gt_gemm: null operand");
-  ProfScope ps(ctx, kind == GT_NT ? "gemm.nt" : kind == GT_NN ? "gemm.nn" : "gemm.tn");
   GemmArgs a;
   a.A = P<const float>(A); a.B = P<const float>(B); a.C = P<float>(C);
   a.M = M; a.N = N; a.K = K;
@@ -236,9 +233,6 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
              (sA % 4 == 0) && (sB % 4 == 0);
 
-  static bool env_read = false;
-  if (!env_read) { env_read = true; const char *e = getenv("GGUFHIP_GEMM_CFG"); if (e) g_force_cfg = atoi(e); }
-
   // Tile choice: the largest tile that still gives every CU a few workgroups; narrow N (heads,
   // LoRA rank) takes the 64-wide tile so columns are not wasted.
   int cfg;
@@ -247,7 +241,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   else if (N % 192 == 0 && N % 128 != 0 && blocks(128, 192) >= ctx->num_cu) cfg = 3;
   else if (blocks(128, 128) >= 2 * ctx->num_cu) cfg = 2;
   else cfg = 1;
-  if (g_force_cfg >= 0) cfg = g_force_cfg;
+  if (ctx->opt_gemm_tile >= 0 && ctx->opt_gemm_tile <= 3) cfg = ctx->opt_gemm_tile;
   int bm = cfg == 0 ? 64 : 128, bn = cfg == 0 ? 64 : cfg == 1 ? 64 : cfg == 2 ? 128 : 192;
 
   // split K when the output alone cannot fill the chip (dW: K = rows of the batch)
@@ -261,6 +255,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
       if (splits > 64) splits = 64;
     }
   }
+  if (count == 1 && ctx->opt_gemm_splitk >= 1) splits = ctx->opt_gemm_splitk;
   if (splits > 1) {
     int64_t kc = cdiv(cdiv(K, splits), BK) * BK;
     splits = (int)cdiv(K, kc);
@@ -272,6 +267,9 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
     a.splits = splits; a.Pp = static_cast<float *>(ws);
   }
   int zdim = splits > 1 ? splits : count;
+  char label[32];
+  snprintf(label, sizeof label, "gemm.%s.%dx%d%s", kind == GT_NT ? "nt" : kind == GT_NN ? "nn" : "tn", bm, bn, splits > 1 ? ".splitk" : "");
+  ProfScope ps(ctx, label, 2.0 * M * N * K * count);
   int rc;
   switch (cfg) {
     case 0: rc = launch_cfg<64, 64, 2, 2>(ctx, kind, vec, a, zdim); break;

@@ -121,12 +121,31 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const floa
   }
 }
 
+// dw[c] (+)= sum over the nparts partial rows, in a fixed order: 64 columns per workgroup, four
+// lane groups each summing every fourth partial row (eight independent loads in flight), then
+// the four group sums added in group order.
 __global__ __launch_bounds__(256) void colsum_reduce(const float *__restrict__ part, int nparts, int d, float *dw, int acc) {
-  int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= d) return;
+  __shared__ float sm[4][64];
+  const int cl = threadIdx.x % 64, grp = threadIdx.x / 64;
+  const int c = blockIdx.x * 64 + cl;
   float s = 0;
-  for (int p = 0; p < nparts; p++) s += part[(size_t)p * d + c];
-  dw[c] = acc ? dw[c] + s : s;
+  if (c < d) {
+    int p = grp;
+    for (; p + 28 < nparts; p += 32) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = part[(size_t)(p + 4 * u) * d + c];
+#pragma unroll
+      for (int u = 0; u < 8; u++) s += v[u];
+    }
+    for (; p < nparts; p += 4) s += part[(size_t)p * d + c];
+  }
+  sm[grp][cl] = s;
+  __syncthreads();
+  if (grp == 0 && c < d) {
+    float t = sm[0][cl] + sm[1][cl] + sm[2][cl] + sm[3][cl];
+    dw[c] = acc ? dw[c] + t : t;
+  }
 }
 
 // scalar fallback for d % 4 != 0 or very wide rows: one wavefront per row
@@ -176,7 +195,7 @@ template <int LPR, int NJ>
 static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
                        gt_buf dx, int acc_dx, gt_buf dw, int acc_dw) {
   constexpr int RPB = 4 * (WAVE / LPR);
-  int64_t nb = std::min<int64_t>(cdiv(rows, RPB), (int64_t)ctx->num_cu * 4);
+  int64_t nb = std::min<int64_t>(cdiv(rows, RPB), (int64_t)ctx->num_cu * 2);
   if (!bwd) {
     hipLaunchKernelGGL((rmsnorm_fwd_k<LPR, NJ>), dim3((unsigned)nb), dim3(256), 0, ctx->stream, rows, d, eps,
                        P<const float>(x), P<const float>(w), P<float>(y_or_g), P<float>(rinv));
@@ -195,7 +214,7 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
                      acc_dx, part);
   GT_LAUNCHED(ctx);
   if (dw) {
-    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 256)), dim3(256), 0, ctx->stream, part, (int)nb, d,
+    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 64)), dim3(256), 0, ctx->stream, part, (int)nb, d,
                        P<float>(dw), acc_dw);
     GT_LAUNCHED(ctx);
   }
@@ -234,7 +253,7 @@ static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x,
     hipLaunchKernelGGL(rmsnorm_dw_gen, dim3((unsigned)cdiv(d, 256), ns), dim3(256), 0, ctx->stream, rows, d, slab,
                        P<const float>(x), P<const float>(y_or_g), P<const float>(rinv), static_cast<float *>(ws));
     GT_LAUNCHED(ctx);
-    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 256)), dim3(256), 0, ctx->stream, static_cast<float *>(ws), ns,
+    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 64)), dim3(256), 0, ctx->stream, static_cast<float *>(ws), ns,
                        d, P<float>(dw), acc_dw);
     GT_LAUNCHED(ctx);
   }
@@ -246,7 +265,7 @@ int gt_rmsnorm_fwd(gt_ctx *ctx, int rows, int d, float eps, gt_buf x, gt_buf w, 
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 0 && d >= 1 && x && w && y && rinv, "gt_rmsnorm_fwd: bad arguments (rows %d, d %d)", rows, d);
   if (rows == 0) return 0;
-  ProfScope ps(ctx, "rmsnorm");
+  ProfScope ps(ctx, "rmsnorm", 8.0 * rows * d);
   return dispatch(ctx, false, rows, d, eps, x, w, y, rinv, 0, 0, 0, 0);
 }
 int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx, int acc_dx,
@@ -257,7 +276,7 @@ int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, g
     if (dw && !acc_dw) GT_HIP(ctx, hipMemsetAsync(P<void>(dw), 0, (size_t)d * 4, ctx->stream));
     return 0;
   }
-  ProfScope ps(ctx, "rmsnorm.bwd");
+  ProfScope ps(ctx, "rmsnorm.bwd", 12.0 * rows * d);   // read x, g; write dx
   return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dw, acc_dw);
 }
 }

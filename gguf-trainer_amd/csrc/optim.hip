@@ -25,7 +25,8 @@ struct TensorPtrs { float *w, *g, *m, *v; };
 
 struct gt_adamw {
   int n = 0, nchunks = 0;
-  float beta1, beta2, eps, wd, clip;
+  double total_elems = 0;
+  double beta1, beta2, eps, wd, clip;
   Chunk *chunks = nullptr;
   TensorPtrs *ptrs = nullptr;
   float *partial = nullptr;     // [nchunks]
@@ -64,21 +65,20 @@ __global__ __launch_bounds__(256) void adamw_scale_k(int nchunks, const float *_
     scale[1] = norm;
   }
 }
-__device__ __forceinline__ void adam1(float g, float &m, float &v, float &w, float b1, float b2, float eps, float wd,
-                                      float lr, float ibc1, float ibc2) {
-  m = b1 * m + (1.f - b1) * g;
-  v = b2 * v + (1.f - b2) * g * g;
+struct AdamH { float b1, b2, omb1, omb2, eps, wd, lr, ibc1, ibc2; };
+__device__ __forceinline__ void adam1(float g, float &m, float &v, float &w, const AdamH &h) {
+  const float b1 = h.b1, b2 = h.b2, eps = h.eps, wd = h.wd, lr = h.lr, ibc1 = h.ibc1, ibc2 = h.ibc2;
+  m = b1 * m + h.omb1 * g;
+  v = b2 * v + h.omb2 * g * g;
   float upd = (m * ibc1) / (sqrtf(v * ibc2) + eps);
   if (wd > 0.f) upd += wd * w;
   w -= lr * upd;
 }
 __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ chunks, const TensorPtrs *__restrict__ ptrs,
-                                                      const float *__restrict__ scale, float b1, float b2, float eps,
-                                                      float wd, float lr, float bc1, float bc2) {
+                                                      const float *__restrict__ scale, AdamH h) {
   Chunk c = chunks[blockIdx.x];
   TensorPtrs p = ptrs[c.tensor];
   const float sc = scale[0];
-  const float ibc1 = 1.0f / bc1, ibc2 = 1.0f / bc2;
   float *w = p.w + c.off, *m = p.m + c.off, *v = p.v + c.off;
   const float *g = p.g + c.off;
   bool vec = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(m) | reinterpret_cast<uintptr_t>(v) |
@@ -90,14 +90,14 @@ __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ 
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       float tm = mm[j], tv = vv[j], tw = ww[j];
-      adam1(gg[j], tm, tv, tw, b1, b2, eps, wd, lr, ibc1, ibc2);
+      adam1(gg[j], tm, tv, tw, h);
       mm[j] = tm; vv[j] = tv; ww[j] = tw;
     }
     reinterpret_cast<v4f *>(m)[i] = mm;
     reinterpret_cast<v4f *>(v)[i] = vv;
     reinterpret_cast<v4f *>(w)[i] = ww;
   }
-  for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) adam1(g[i] * sc, m[i], v[i], w[i], b1, b2, eps, wd, lr, ibc1, ibc2);
+  for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) adam1(g[i] * sc, m[i], v[i], w[i], h);
 }
 
 // ---- Muon -------------------------------------------------------------------------------------------
@@ -209,7 +209,7 @@ static void muon_release(gt_ctx *ctx, gt_muon *o) {
 extern "C" {
 
 int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *m, const gt_buf *v,
-                    const int64_t *sizes, float beta1, float beta2, float eps, float weight_decay, float clip, gt_adamw **out) {
+                    const int64_t *sizes, double beta1, double beta2, double eps, double weight_decay, double clip, gt_adamw **out) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, n >= 0 && out && (n == 0 || (w && g && m && v && sizes)), "gt_adamw_create: bad arguments");
   gt_adamw *o = new gt_adamw();
@@ -219,6 +219,7 @@ int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const 
   for (int i = 0; i < n; i++) {
     if (!(w[i] && g[i] && m[i] && v[i] && sizes[i] >= 0)) { delete o; GT_FAIL(ctx, "gt_adamw_create: tensor %d has a null buffer", i); }
     tp[i] = {P<float>(w[i]), P<float>(g[i]), P<float>(m[i]), P<float>(v[i])};
+    o->total_elems += (double)sizes[i];
     for (int64_t off = 0; off < sizes[i]; off += CHUNK) ch.push_back({i, (int)std::min<int64_t>(CHUNK, sizes[i] - off), off});
   }
   o->nchunks = (int)ch.size();
@@ -235,20 +236,24 @@ int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const 
   return 0;
 }
 
-int gt_adamw_step(gt_ctx *ctx, gt_adamw *o, float lr, float bc1, float bc2) {
+int gt_adamw_step(gt_ctx *ctx, gt_adamw *o, double lr, double bc1, double bc2) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, o, "gt_adamw_step: null optimizer");
   GT_REQUIRE(ctx, bc1 > 0 && bc2 > 0, "gt_adamw_step: bias corrections must be positive");
   if (o->nchunks == 0) return 0;
-  ProfScope ps(ctx, "adamw");
+  int64_t total = 0;
+  ProfScope ps(ctx, "adamw", o->total_elems * (o->clip > 0 ? 32.0 : 28.0));   // g,m,v,w read; m,v,w written; +g for the norm
+  (void)total;
   if (o->clip > 0) {
     hipLaunchKernelGGL(adamw_ssq_k, dim3(o->nchunks), dim3(256), 0, ctx->stream, o->chunks, o->ptrs, o->partial);
     GT_LAUNCHED(ctx);
-    hipLaunchKernelGGL(adamw_scale_k, dim3(1), dim3(256), 0, ctx->stream, o->nchunks, o->partial, o->clip, o->scale);
+    hipLaunchKernelGGL(adamw_scale_k, dim3(1), dim3(256), 0, ctx->stream, o->nchunks, o->partial, (float)o->clip, o->scale);
     GT_LAUNCHED(ctx);
   }
-  hipLaunchKernelGGL(adamw_update_k, dim3(o->nchunks), dim3(256), 0, ctx->stream, o->chunks, o->ptrs, o->scale, o->beta1,
-                     o->beta2, o->eps, o->wd, lr, bc1, bc2);
+  // every constant is formed in f64 and rounded to f32 once
+  AdamH h{(float)o->beta1, (float)o->beta2, (float)(1.0 - o->beta1), (float)(1.0 - o->beta2), (float)o->eps, (float)o->wd,
+          (float)lr, (float)(1.0 / bc1), (float)(1.0 / bc2)};
+  hipLaunchKernelGGL(adamw_update_k, dim3(o->nchunks), dim3(256), 0, ctx->stream, o->chunks, o->ptrs, o->scale, h);
   GT_LAUNCHED(ctx);
   return 0;
 }
@@ -273,11 +278,11 @@ int gt_adamw_destroy(gt_ctx *ctx, gt_adamw *o) {
 }
 
 int gt_muon_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *buf, const int *rows, const int *cols,
-                   float momentum, int nesterov, int ns_steps, gt_muon **out) {
+                   double momentum, int nesterov, int ns_steps, gt_muon **out) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, n >= 0 && out && ns_steps >= 0 && (n == 0 || (w && g && buf && rows && cols)), "gt_muon_create: bad arguments");
   gt_muon *o = new gt_muon();
-  o->momentum = momentum; o->nesterov = nesterov; o->ns_steps = ns_steps;
+  o->momentum = (float)momentum; o->nesterov = nesterov; o->ns_steps = ns_steps;
   size_t me = 1, mr = 1;
   for (int i = 0; i < n; i++) {
     if (!(w[i] && g[i] && buf[i] && rows[i] >= 1 && cols[i] >= 1)) { delete o; GT_FAIL(ctx, "gt_muon_create: matrix %d is malformed", i); }
@@ -290,7 +295,7 @@ int gt_muon_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const g
   return 0;
 }
 
-int gt_muon_step(gt_ctx *ctx, gt_muon *o, float lr) {
+int gt_muon_step(gt_ctx *ctx, gt_muon *o, double lr) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, o, "gt_muon_step: null optimizer");
   ProfScope ps(ctx, "muon");
@@ -300,7 +305,7 @@ int gt_muon_step(gt_ctx *ctx, gt_muon *o, float lr) {
     hipLaunchKernelGGL(muon_momentum_k, dim3(nb), dim3(256), 0, ctx->stream, size, mt.g, mt.buf, o->U, o->momentum, o->nesterov, o->part);
     GT_LAUNCHED(ctx);
     if (newton_schulz_run(ctx, mt.rows, mt.cols, o->ns_steps, o->U, o->X, o->A, o->AA, o->BX, o->part, (int)nb)) return 1;
-    float f = lr * sqrtf(std::max(1.0f, (float)mt.rows / (float)mt.cols));
+    float f = (float)(lr * sqrt(std::max(1.0, (double)mt.rows / (double)mt.cols)));
     hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, size)), dim3(256), 0, ctx->stream, mt.rows, mt.cols, mt.rows > mt.cols ? 1 : 0,
                        mt.w, o->X, f);
     GT_LAUNCHED(ctx);

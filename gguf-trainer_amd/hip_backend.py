@@ -242,6 +242,10 @@ class HipBackend:
         check(self._ctx, lib.gt_d2h(self._ctx, out.ctypes.data_as(C.c_void_p), b, out.nbytes), "gt_d2h")
         return out
 
+    def set_option(self, key: str, value: int):
+        """Kernel-selection switches for tests and tuning: "attn.generic", "gemm.tile", "gemm.splitk"."""
+        check(self._ctx, lib.gt_set_option(self._ctx, key.encode(), int(value)), "gt_set_option")
+
     def resident_bytes(self) -> int:
         v = C.c_uint64()
         lib.gt_resident_bytes(self._ctx, C.byref(v))
@@ -313,14 +317,16 @@ class HipBackend:
             lib.gt_ctx_destroy(self._ctx)
 
     # ---- profiling (webgpu.ts:830-880) -----------------------------------------------------------------------
-    def start_profile(self):
-        check(self._ctx, lib.gt_prof_begin(self._ctx), "gt_prof_begin")
+    def start_profile(self, prefix: str = ""):
+        """Time every launch whose label starts with `prefix` ("" = all) with HIP events on the stream."""
+        check(self._ctx, lib.gt_prof_begin(self._ctx, prefix.encode()), "gt_prof_begin")
 
     def stop_profile(self) -> dict:
-        recs = (ProfRec * 64)()
+        """label -> (total ms, launches, algorithmic work: FLOP or bytes)."""
+        recs = (ProfRec * 128)()
         n = C.c_int()
-        check(self._ctx, lib.gt_prof_end(self._ctx, recs, 64, C.byref(n)), "gt_prof_end")
-        return {recs[i].label.decode(): (recs[i].ms, recs[i].count) for i in range(n.value)}
+        check(self._ctx, lib.gt_prof_end(self._ctx, recs, 128, C.byref(n)), "gt_prof_end")
+        return {recs[i].label.decode(): (recs[i].ms, recs[i].count, recs[i].work) for i in range(n.value)}
 
     # ---- RegionBackend (webgpu.ts:639-761) ------------------------------------------------------------------------
     def begin_region(self) -> int:

@@ -25,7 +25,7 @@ i32, i64, f32, f64, sz = C.c_int, C.c_int64, C.c_float, C.c_double, C.c_size_t
 
 
 class ProfRec(C.Structure):
-    _fields_ = [("label", C.c_char * 32), ("ms", C.c_double), ("count", C.c_int64)]
+    _fields_ = [("label", C.c_char * 32), ("ms", C.c_double), ("count", C.c_int64), ("work", C.c_double)]
 
 
 _SIG = {
@@ -39,6 +39,7 @@ _SIG = {
     "gt_d2d": [ctxp, buf, buf, sz],
     "gt_sync": [ctxp],
     "gt_resident_bytes": [ctxp, C.POINTER(C.c_uint64)],
+    "gt_set_option": [ctxp, C.c_char_p, i32],
     "gt_gemm": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf],
     "gt_gemm_batched": [ctxp, i32, i32, i32, i32, i32, buf, i64, buf, i64, buf, i64, i32],
     "gt_add_fwd": [ctxp, i64, buf, buf, buf],
@@ -68,16 +69,16 @@ _SIG = {
     "gt_soft_ce_fwd": [ctxp, i32, i32, i32, buf, buf, buf, f32, buf, buf, buf],
     "gt_soft_ce_bwd": [ctxp, i32, i32, i32, buf, buf, buf, f32, buf, buf, f32, buf, i32],
     "gt_adamw_create": [ctxp, i32, C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(i64),
-                        f32, f32, f32, f32, f32, C.POINTER(C.c_void_p)],
-    "gt_adamw_step": [ctxp, C.c_void_p, f32, f32, f32],
+                        f64, f64, f64, f64, f64, C.POINTER(C.c_void_p)],
+    "gt_adamw_step": [ctxp, C.c_void_p, f64, f64, f64],
     "gt_adamw_grad_norm": [ctxp, C.c_void_p, C.POINTER(f32)],
     "gt_adamw_destroy": [ctxp, C.c_void_p],
     "gt_muon_create": [ctxp, i32, C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(i32), C.POINTER(i32),
-                       f32, i32, i32, C.POINTER(C.c_void_p)],
-    "gt_muon_step": [ctxp, C.c_void_p, f32],
+                       f64, i32, i32, C.POINTER(C.c_void_p)],
+    "gt_muon_step": [ctxp, C.c_void_p, f64],
     "gt_muon_destroy": [ctxp, C.c_void_p],
     "gt_newton_schulz": [ctxp, i32, i32, i32, buf, buf],
-    "gt_prof_begin": [ctxp],
+    "gt_prof_begin": [ctxp, C.c_char_p],
     "gt_prof_end": [ctxp, C.POINTER(ProfRec), i32, C.POINTER(i32)],
 }
 

@@ -56,6 +56,12 @@ int gt_d2h(gt_ctx *ctx, void *dst, gt_buf src, size_t bytes);         /* waits f
 int gt_d2d(gt_ctx *ctx, gt_buf dst, gt_buf src, size_t bytes);
 int gt_sync(gt_ctx *ctx);
 int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt_alloc bytes + workspace */
+/* Kernel-selection switches for tests and tuning (no reference counterpart; WebGPUBackend exposes
+ * attnFlashMinT as a public field for the same purpose, webgpu.ts:305):
+ *   "attn.generic" 1 = always take the shape-generic attention kernels, 0 = MFMA kernels where they apply
+ *   "gemm.tile"    -1 = heuristic, 0..3 = pin the GEMM tile (64x64, 128x64, 128x128, 128x192)
+ *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor */
+int gt_set_option(gt_ctx *ctx, const char *key, int value);
 
 /* ---- GEMM: srcGemm (src/backend/wgsl.ts:87-196), WebGPUBackend.gemm (webgpu.ts:1654) ---------
  * kind 0 "NT": C[M,N] = A[M,K] . B[N,K]^T      forward y = x W^T           (webgpu.ts:892)
@@ -140,11 +146,13 @@ int gt_soft_ce_bwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf te
 /* ---- AdamW: AdamWGpu (adamw-gpu.ts:131-251), spec src/train/adam.ts:46-82 --------------------
  * One object per parameter group; step() = global grad-norm clip over the whole group (when
  * clip > 0) followed by the fused element update, two launches for any number of tensors.
- * bc1 = 1 - beta1^t and bc2 = 1 - beta2^t come from the host, as in adamw-gpu.ts:211-218. */
+ * bc1 = 1 - beta1^t and bc2 = 1 - beta2^t come from the host, as in adamw-gpu.ts:211-218.
+ * Hyperparameters are doubles (JS numbers): 1 - beta and 1/bc are formed in f64 and rounded once,
+ * since 1.0f - 0.999f is already 1.3e-5 off. */
 int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *m, const gt_buf *v,
-                    const int64_t *sizes, float beta1, float beta2, float eps, float weight_decay, float clip,
+                    const int64_t *sizes, double beta1, double beta2, double eps, double weight_decay, double clip,
                     gt_adamw **out);
-int gt_adamw_step(gt_ctx *ctx, gt_adamw *opt, float lr, float bc1, float bc2);
+int gt_adamw_step(gt_ctx *ctx, gt_adamw *opt, double lr, double bc1, double bc2);
 int gt_adamw_grad_norm(gt_ctx *ctx, gt_adamw *opt, float *norm);   /* last step's global norm; waits */
 int gt_adamw_destroy(gt_ctx *ctx, gt_adamw *opt);
 
@@ -152,17 +160,20 @@ int gt_adamw_destroy(gt_ctx *ctx, gt_adamw *opt);
  * Matrices w[i] are [rows[i], cols[i]]; buf[i] is the momentum. step(): buf = mu*buf + g;
  * U = nesterov ? g + mu*buf : buf; X = NS(U); w -= lr*sqrt(max(1, rows/cols))*X. */
 int gt_muon_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const gt_buf *buf,
-                   const int *rows, const int *cols, float momentum, int nesterov, int ns_steps, gt_muon **out);
-int gt_muon_step(gt_ctx *ctx, gt_muon *opt, float lr);
+                   const int *rows, const int *cols, double momentum, int nesterov, int ns_steps, gt_muon **out);
+int gt_muon_step(gt_ctx *ctx, gt_muon *opt, double lr);
 int gt_muon_destroy(gt_ctx *ctx, gt_muon *opt);
 /* newtonSchulzGpu (muon-gpu.ts:259-283): out[m,n] = NS(G[m,n]) */
 int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out);
 
 /* ---- profiling: startProfile / stopProfile (webgpu.ts:830-880) --------------------------------
- * Between begin and end every launch is bracketed by HIP events on the context's stream and
- * summed per label. gt_prof_end waits, then fills up to `cap` records. */
-typedef struct gt_prof_rec { char label[32]; double ms; int64_t count; } gt_prof_rec;
-int gt_prof_begin(gt_ctx *ctx);
+ * Between begin and end every launch whose label starts with `prefix` (NULL or "" = all) is
+ * bracketed by HIP events on the context's stream and summed per label, together with the
+ * algorithmic work the call states for itself (FLOP for the contractions, bytes for the streaming
+ * kernels). GEMM labels carry the kernel's tile shape ("gemm.nn.128x192"). gt_prof_end waits, then
+ * fills up to `cap` records. */
+typedef struct gt_prof_rec { char label[32]; double ms; int64_t count; double work; } gt_prof_rec;
+int gt_prof_begin(gt_ctx *ctx, const char *prefix);
 int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n);
 
 #ifdef __cplusplus

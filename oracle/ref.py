@@ -54,6 +54,11 @@ _lib.or_fused_ce_fwd.restype = C.c_double
 _lib.or_soft_ce_fwd.restype = C.c_double
 
 
+# Timed CPU baseline only: route linear / attention backward through the OpenMP-safe variants in oracle.c
+# (per-output f64 dot products, rounded once). Parity tests leave this False and use the literal loops.
+PARALLEL_BWD = False
+
+
 def set_threads(n: int) -> None:
     _lib.or_set_threads(int(n))
 
@@ -218,8 +223,8 @@ def linear_raw(x: Tensor, w: Tensor) -> Tensor:
     wants_dw = w.requires_grad
 
     def bw():
-        _lib.or_linear_bwd(_f(x.data), _f(w.data), _f(out.grad), _f(x.grad),
-                           _f(w.grad) if wants_dw else None, T, ind, outd)
+        fn = _lib.or_linear_bwd_dots if PARALLEL_BWD else _lib.or_linear_bwd
+        fn(_f(x.data), _f(w.data), _f(out.grad), _f(x.grad), _f(w.grad) if wants_dw else None, T, ind, outd)
 
     out._backward = bw
     return out
@@ -321,9 +326,12 @@ def attention(q: Tensor, k: Tensor, v: Tensor, T: int, Hq: int, Hkv: int, hd: in
     _lib.or_attention_fwd(_f(q.data), _f(k.data), _f(v.data), _f(out.data), _f(probs), T, Hq, Hkv, hd, window)
     out._prev = [q, k, v]
     out.probs = probs
-    fn = _lib.or_attention_bwd_par if parallel_bwd else _lib.or_attention_bwd
-    out._backward = lambda: fn(_f(q.data), _f(k.data), _f(v.data), _f(probs), _f(out.grad),
-                               _f(q.grad), _f(k.grad), _f(v.grad), T, Hq, Hkv, hd, window)
+    def bw():
+        fn = _lib.or_attention_bwd_par if (parallel_bwd or PARALLEL_BWD) else _lib.or_attention_bwd
+        fn(_f(q.data), _f(k.data), _f(v.data), _f(probs), _f(out.grad), _f(q.grad), _f(k.grad), _f(v.grad),
+           T, Hq, Hkv, hd, window)
+
+    out._backward = bw
     return out
 
 

@@ -24,20 +24,22 @@ def mod(name):
     return importlib.import_module(f"{PKG}.{name}")
 
 
-def errs(got, want):
+def errs(got, want, floor=0.0):
     got = np.asarray(got, dtype=np.float64).ravel()
     want = np.asarray(want, dtype=np.float64).ravel()
     assert got.shape == want.shape, (got.shape, want.shape)
     assert np.all(np.isfinite(got)), "non-finite values from the device"
     nrm = np.linalg.norm(want)
     mx = np.abs(want).max() if want.size else 0.0
+    if floor > 0:                    # an exactly-zero gradient (attention window 1) compares absolutely
+        nrm, mx = max(nrm, floor), max(mx, floor)
     l2 = np.linalg.norm(got - want) / nrm if nrm > 0 else np.linalg.norm(got - want)
     mr = np.abs(got - want).max() / mx if mx > 0 else (np.abs(got - want).max() if want.size else 0.0)
     return l2, mr
 
 
-def assert_close(got, want, what="", rel_l2=REL_L2, max_rel=MAX_REL):
-    l2, mr = errs(got, want)
+def assert_close(got, want, what="", rel_l2=REL_L2, max_rel=MAX_REL, floor=0.0):
+    l2, mr = errs(got, want, floor)
     assert l2 <= rel_l2 and mr <= max_rel, f"{what}: rel L2 {l2:.3e} (<= {rel_l2:g}), max-rel {mr:.3e} (<= {max_rel:g})"
     return l2, mr
 
@@ -51,7 +53,7 @@ def backward_from(gpu, ag, out, grad_out):
         t._backward()
 
 
-def op_case(gpu, ref, arrays, fwd_hip, fwd_ref, what, frozen=(), rel_l2=REL_L2, max_rel=MAX_REL, seed=0xBEEF):
+def op_case(gpu, ref, arrays, fwd_hip, fwd_ref, what, frozen=(), rel_l2=REL_L2, max_rel=MAX_REL, seed=0xBEEF, floor=0.0):
     """tests/gpu-parity.ts:90-126: the same forward on both sides from the same arrays, the same seeded
     upstream gradient, compare the output and every input gradient."""
     ag = mod("autograd")
@@ -71,5 +73,5 @@ def op_case(gpu, ref, arrays, fwd_hip, fwd_ref, what, frozen=(), rel_l2=REL_L2, 
     for i, (h, r) in enumerate(zip(hts, rts)):
         if i in frozen:
             continue
-        assert_close(h.grad, r.grad, f"{what} grad[{i}]", rel_l2, max_rel)
+        assert_close(h.grad, r.grad, f"{what} grad[{i}]", rel_l2, max_rel, floor)
     return out_h, out_r

@@ -1,0 +1,138 @@
+"""BASELINE config 2 at full size (X [16384x576], W [576x1536], dY [16384x1536]; logits [16384x49152]; RMSNorm
+[16384x576]): too large for the scalar oracle end to end, so parity is through sampled entries computed in
+float64 on the host, the oracle on sampled rows, and size-independent properties."""
+import numpy as np
+import pytest
+
+from gpu_common import assert_close, mod
+
+pytestmark = pytest.mark.gpu
+
+ROWS, H, F, V = 16384, 576, 1536, 49152
+
+
+def dev(gpu, arr):
+    b = gpu.create_state_buffer(arr.nbytes)
+    gpu.write_state_buffer(b, arr)
+    return b
+
+
+def test_mlp_backward_gemms_full_size(gpu):
+    """dX = dY.W (NN) and dW = dY^T.X (TN), the up-projection of the SmolLM2 MLP: sampled outputs against float64 dot
+    products; accumulate mode adds exactly once; linearity in dY."""
+    lib = mod("lib")
+    rs = np.random.RandomState(0)
+    X = rs.standard_normal((ROWS, H)).astype(np.float32)
+    W = rs.standard_normal((F, H)).astype(np.float32)
+    dY = rs.standard_normal((ROWS, F)).astype(np.float32)
+    bX, bW, bdY = dev(gpu, X), dev(gpu, W), dev(gpu, dY)
+    bdX, bdW = gpu.create_state_buffer(X.nbytes), gpu.create_state_buffer(W.nbytes)
+    gpu.gemm(lib.NN, 0, ROWS, H, F, bdY, bW, bdX)
+    gpu.gemm(lib.TN, 0, F, H, ROWS, bdY, bX, bdW)
+    dX = gpu.read_state_buffer(bdX, X.size).reshape(ROWS, H)
+    dW = gpu.read_state_buffer(bdW, W.size).reshape(F, H)
+    W64, X64, dY64 = W.astype(np.float64), X.astype(np.float64), dY.astype(np.float64)
+    rr = rs.randint(0, ROWS, 64)
+    assert_close(dX[rr], dY64[rr] @ W64, "dX sampled rows")
+    rw = rs.randint(0, F, 48)
+    assert_close(dW[rw], dY64[:, rw].T @ X64, "dW sampled rows")
+    # accumulate: a second product on top doubles the value exactly (x + x is exact in f32)
+    gpu.gemm(lib.NN, 1, ROWS, H, F, bdY, bW, bdX)
+    gpu.gemm(lib.TN, 1, F, H, ROWS, bdY, bX, bdW)
+    assert np.array_equal(gpu.read_state_buffer(bdX, X.size).reshape(ROWS, H), 2 * dX)
+    assert np.array_equal(gpu.read_state_buffer(bdW, W.size).reshape(F, H), 2 * dW)
+    # forward NT on the same operands
+    bY = gpu.create_state_buffer(dY.nbytes)
+    gpu.gemm(lib.NT, 0, ROWS, F, H, bX, bW, bY)
+    Y = gpu.read_state_buffer(bY, dY.size).reshape(ROWS, F)
+    assert_close(Y[rr], X64[rr] @ W64.T, "Y sampled rows")
+
+
+def test_ce_backward_full_size(gpu, ref):
+    """logits [16384 x 49152] ~ N(0,2), uniform targets, 10% masked: every kept row of dz sums to zero and ignored
+    rows are zero (softmax - onehot), sampled rows equal the oracle's, the loss equals a float64 logsumexp."""
+    ag = mod("autograd")
+    rs = np.random.RandomState(1)
+    z = (2.0 * rs.standard_normal((ROWS, V))).astype(np.float32)
+    tg = rs.randint(0, V, ROWS)
+    tg[rs.rand(ROWS) < 0.1] = -1
+    hz = ag.Tensor(z, [ROWS, V], True)
+    gpu.install()
+    try:
+        loss = ag.cross_entropy(hz, tg)
+        ag.backward(loss, 1.0)
+        gpu.sync([loss])
+    finally:
+        gpu.uninstall()
+    dz = hz.grad.reshape(ROWS, V)
+    kept = tg >= 0
+    z64 = z[:512].astype(np.float64)
+    m = z64.max(axis=1)
+    lse = np.log(np.exp(z64 - m[:, None]).sum(axis=1)) + m
+    assert not np.any(dz[~kept])
+    rowsum = dz.astype(np.float64).sum(axis=1)
+    scale = 1.0 / kept.sum()
+    assert np.abs(rowsum[kept]).max() < 1e-4 * scale
+    sample = np.concatenate([np.arange(8), rs.randint(0, ROWS, 8)])
+    rz = ref.Tensor(z[sample], [len(sample), V], True)
+    rl = ref.cross_entropy(rz, [int(t) for t in tg[sample]])
+    ref.backward(rl, 1.0)
+    ks = max(int((tg[sample] >= 0).sum()), 1)
+    assert_close(dz[sample] * (kept.sum() / ks), rz.grad.reshape(len(sample), V), "CE dz sampled rows")
+    # loss over all kept rows, float64 on the host
+    zt = z[np.arange(ROWS), np.maximum(tg, 0)].astype(np.float64)
+    tot = 0.0
+    for r0 in range(0, ROWS, 1024):
+        blk = z[r0:r0 + 1024].astype(np.float64)
+        mm = blk.max(axis=1)
+        l = np.log(np.exp(blk - mm[:, None]).sum(axis=1)) + mm
+        k = kept[r0:r0 + 1024]
+        tot += (l[k] - zt[r0:r0 + 1024][k]).sum()
+    want = tot / kept.sum()
+    assert abs(loss.data[0] - want) <= 1e-5 * want
+
+
+def test_rmsnorm_backward_full_size(gpu, ref):
+    """RMSNorm backward on [16384 x 576] against the oracle directly (9.4 M elements)."""
+    ag = mod("autograd")
+    rs = np.random.RandomState(2)
+    x = rs.standard_normal((ROWS, H)).astype(np.float32)
+    w = (1 + 0.3 * rs.standard_normal(H)).astype(np.float32)
+    g = rs.standard_normal((ROWS, H)).astype(np.float32)
+    hx, hw = ag.Tensor(x, [ROWS, H], True), ag.Tensor(w, [H], True)
+    from gpu_common import backward_from
+    gpu.install()
+    try:
+        out = ag.rms_norm(hx, hw, 1e-5)
+        backward_from(gpu, ag, out, g)
+        gpu.sync([out])
+    finally:
+        gpu.uninstall()
+    rx, rw = ref.Tensor(x, [ROWS, H], True), ref.Tensor(w, [H], True)
+    ro = ref.rms_norm(rx, rw, 1e-5)
+    ref.backward_from(ro, g)
+    assert_close(out.data, ro.data, "rmsNorm full y")
+    assert_close(hx.grad, rx.grad, "rmsNorm full dx")
+    assert_close(hw.grad, rw.grad, "rmsNorm full dw")
+
+
+def test_glu_backward_full_size(gpu, ref):
+    """SwiGLU backward on [16384 x 1536] against the oracle (25 M elements)."""
+    ag = mod("autograd")
+    from gpu_common import backward_from
+    rs = np.random.RandomState(3)
+    a, b, g = (rs.standard_normal((ROWS, F)).astype(np.float32) for _ in range(3))
+    ha, hb2 = ag.Tensor(a, [ROWS, F], True), ag.Tensor(b, [ROWS, F], True)
+    gpu.install()
+    try:
+        out = ag.mul(ag.silu(ha), hb2)
+        backward_from(gpu, ag, out, g)
+        gpu.sync([out])
+    finally:
+        gpu.uninstall()
+    ra, rb = ref.Tensor(a, [ROWS, F], True), ref.Tensor(b, [ROWS, F], True)
+    ro = ref.mul(ref.silu(ra), rb)
+    ref.backward_from(ro, g)
+    assert_close(out.data, ro.data, "SwiGLU full out")
+    assert_close(ha.grad, ra.grad, "SwiGLU full dgate")
+    assert_close(hb2.grad, rb.grad, "SwiGLU full dup")

@@ -1,0 +1,209 @@
+"""Whole-graph parity: the three architectures, micro-batch accumulation, --recompute, LoRA, stacked
+sequences and BASELINE config 1, HIP backend (through the C ABI) against the CPU oracle."""
+import math
+
+import numpy as np
+import pytest
+
+from gpu_common import LOSS_REL, assert_close, mod
+
+pytestmark = pytest.mark.gpu
+
+SMALL = {
+    "llama": dict(arch="llama", vocab=61, hidden=48, layers=2, heads=6, kv_heads=2, head_dim=8, ffn=80, rope_base=1e5),
+    "qwen3": dict(arch="qwen3", vocab=61, hidden=48, layers=2, heads=4, kv_heads=2, head_dim=16, ffn=80, rope_base=1e6, rms_eps=1e-6),
+    "gemma3": dict(arch="gemma3", vocab=61, hidden=48, layers=3, heads=4, kv_heads=1, head_dim=16, ffn=80, rope_base=1e6,
+                   rope_base_local=1e4, sliding_window=7, swa_pattern=3, rms_eps=1e-6),
+}
+# BASELINE config 1
+TINY = dict(arch="llama", vocab=512, hidden=128, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=352, rope_base=1e4, rms_eps=1e-5)
+
+
+def build_pair(ref, kw, seed=0, std=0.02, jitter_gains=True):
+    arch = mod("arch")
+    rmodel = ref.Model(ref.ModelConfig(**kw), ref.Mulberry32(seed), std=std)
+    if jitter_gains:
+        rng = ref.Mulberry32(seed + 100)
+        for p in rmodel.params():
+            if len(p.shape) == 1:
+                p.data[:] = 1 + 0.2 * rng.fill_randn([p.size])
+    weights = {n: p.data.copy() for n, p in rmodel.named_params()}
+    return rmodel, arch.Model(arch.ModelConfig(**kw), weights)
+
+
+def batches(ref, vocab, T, n, seed, mask_every=0):
+    rng = ref.Mulberry32(seed)
+    out = []
+    for _ in range(n):
+        ids = [int(rng() * vocab) for _ in range(T + 1)]
+        tg = ids[1:]
+        if mask_every:
+            tg = [-1 if i % mask_every == 2 else g for i, g in enumerate(tg)]
+        out.append((ids[:-1], tg))
+    return out
+
+
+def hip_step(gpu, model, seqs, stacked, seq_len, loss_chunk=0, recompute=False):
+    ag, arch = mod("autograd"), mod("arch")
+    B = len(seqs)
+    gpu.install()
+    ag.set_checkpointing(recompute)
+    try:
+        losses = []
+        if stacked:
+            ids = np.concatenate([s[0] for s in seqs])
+            tg = np.concatenate([s[1] for s in seqs])
+            loss = arch.sequence_loss(model, ids, tg, loss_chunk, seq_len)
+            ag.backward(loss, 1.0 / B)
+            losses = [loss]
+        else:
+            for ids, tg in seqs:
+                loss = arch.sequence_loss(model, ids, tg, loss_chunk)
+                ag.backward(loss, 1.0 / B)
+                losses.append(loss)
+        gpu.sync(losses)
+    finally:
+        ag.set_checkpointing(False)
+        gpu.uninstall()
+    lv = np.concatenate([l.data for l in losses])
+    return lv, {n: p.grad.copy() for n, p in model.named_params()}
+
+
+def ref_step(ref, rmodel, seqs, loss_chunk=0):
+    B = len(seqs)
+    for p in rmodel.params():
+        p.zero_grad()
+    lv = []
+    for ids, tg in seqs:
+        l = ref.sequence_loss(rmodel, ids, tg, loss_chunk)
+        ref.backward(l, 1.0 / B)
+        lv.append(float(l.data[0]))
+    return np.array(lv), {n: p.grad.copy() for n, p in rmodel.named_params()}
+
+
+def compare(lh, gh, lr, gr, what):
+    assert np.all(np.abs(lh - lr) <= LOSS_REL * np.abs(lr)), f"{what}: loss {lh} vs {lr}"
+    for n in gr:
+        assert_close(gh[n], gr[n], f"{what} grad {n}")
+
+
+@pytest.mark.parametrize("arch_name", ["llama", "qwen3", "gemma3"])
+@pytest.mark.parametrize("stacked", [False, True])
+def test_whole_model_two_micro_batches(gpu, ref, arch_name, stacked):
+    """gpu-parity.ts:333-428: loss and every gradient tensor; two micro-batches accumulated with seed 1/2, masked
+    targets; the same step as one stacked graph over 2*T rows."""
+    kw = SMALL[arch_name]
+    rmodel, model = build_pair(ref, kw, seed=1, std=0.1)
+    seqs = batches(ref, kw["vocab"], 19, 2, seed=5, mask_every=5)
+    lh, gh = hip_step(gpu, model, seqs, stacked, 19)
+    lr, gr = ref_step(ref, rmodel, seqs)
+    compare(lh, gh, lr, gr, f"{arch_name} stacked={stacked}")
+
+
+@pytest.mark.parametrize("arch_name", ["llama", "qwen3", "gemma3"])
+def test_recompute_is_bit_identical_and_matches(gpu, ref, arch_name):
+    """gpu-parity.ts:536-564, 1299-1338: --recompute on/off gives bit-identical loss and gradients."""
+    kw = SMALL[arch_name]
+    seqs = batches(ref, kw["vocab"], 23, 2, seed=6, mask_every=4)
+    res = []
+    for rc in (False, True):
+        rmodel, model = build_pair(ref, kw, seed=2, std=0.1)
+        regions0 = gpu.region_count()
+        res.append(hip_step(gpu, model, seqs, False, 23, recompute=rc))
+        if rc:
+            assert gpu.region_count() > regions0
+    assert res[0][0].tobytes() == res[1][0].tobytes()
+    for n in res[0][1]:
+        assert res[0][1][n].tobytes() == res[1][1][n].tobytes(), n
+    lr, gr = ref_step(ref, rmodel, seqs)
+    compare(res[1][0], res[1][1], lr, gr, f"{arch_name} recompute")
+
+
+def test_run_to_run_determinism(gpu, ref):
+    kw = SMALL["llama"]
+    seqs = batches(ref, kw["vocab"], 40, 3, seed=9)
+    a = hip_step(gpu, build_pair(ref, kw, seed=3, std=0.1)[1], seqs, True, 40)
+    b = hip_step(gpu, build_pair(ref, kw, seed=3, std=0.1)[1], seqs, True, 40)
+    assert a[0].tobytes() == b[0].tobytes()
+    for n in a[1]:
+        assert a[1][n].tobytes() == b[1][n].tobytes(), n
+
+
+@pytest.mark.parametrize("chunk", [16, 61])
+def test_loss_chunk_path(gpu, ref, chunk):
+    """gpu-parity.ts:438-565: --loss-chunk gives the dense loss and gradients."""
+    kw = SMALL["qwen3"]
+    rmodel, model = build_pair(ref, kw, seed=4, std=0.1)
+    seqs = batches(ref, kw["vocab"], 17, 2, seed=7, mask_every=6)
+    lh, gh = hip_step(gpu, model, seqs, False, 17, loss_chunk=chunk)
+    lr, gr = ref_step(ref, rmodel, seqs)
+    compare(lh, gh, lr, gr, f"loss-chunk {chunk}")
+
+
+@pytest.mark.parametrize("recompute", [False, True])
+def test_lora(gpu, ref, recompute):
+    """gpu-parity.ts:2037-2138: base frozen (no gradient buffers), adapters trained; with --recompute too."""
+    ag, arch = mod("autograd"), mod("arch")
+    kw = SMALL["qwen3"]
+    rmodel, model = build_pair(ref, kw, seed=5, std=0.1)
+    rank, alpha = 4, 8.0
+    rmap, rparams = ref.attach_lora(rmodel, rank, alpha, ref.Mulberry32(11), a_std=0.1)
+    rng = ref.Mulberry32(12)
+    for a, b, _ in rmap.values():
+        b.data[:] = rng.fill_randn([b.size], 0.1)          # B != 0 so that dA is non-trivial
+    adapters = {}
+    for l, L in enumerate(rmodel.layers):
+        for k in ref.MATRIX_KEYS:
+            a, b, _ = rmap[id(L[k])]
+            adapters[f"L{l}.{k}"] = (a.data.copy(), b.data.copy())
+    aux = arch.apply_lora(model, rank, alpha, adapters)
+    ref.set_lora_adapters(rmap)
+    seqs = batches(ref, kw["vocab"], 15, 2, seed=8, mask_every=3)
+    try:
+        lh, _ = hip_step(gpu, model, seqs, False, 15, recompute=recompute)
+        lr, _ = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.set_lora_adapters({})
+        arch.clear_lora(model)
+    assert np.all(np.abs(lh - lr) <= LOSS_REL * np.abs(lr))
+    for i, (h, r) in enumerate(zip(aux, rparams)):
+        assert_close(h.grad, r.grad, f"lora adapter {i}")
+    for p in model.params():                                 # frozen base: no accumulator was ever created
+        assert gpu._entries[p].grad == 0
+
+
+def test_config1_tiny_llama_step(gpu, ref):
+    """BASELINE config 1: vocab 512, hidden 128, 2 layers, 4/2 heads x 32, SwiGLU 352, tied, weights N(0,0.02) seed 0,
+    4 sequences of 128 tokens, targets shifted by one; forward + backward + AdamW(lr 1e-3, betas 0.9/0.95, wd 0.1)."""
+    optim = mod("optim")
+    rmodel, model = build_pair(ref, TINY, seed=0, std=0.02, jitter_gains=False)
+    seqs = batches(ref, TINY["vocab"], 128, 4, seed=0)
+    ref.set_threads(min(8, ref.max_threads()))
+    try:
+        lr_, gr = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.set_threads(1)
+    opt = optim.AdamWHip(gpu, model.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
+    ag, arch = mod("autograd"), mod("arch")
+    gpu.install()
+    try:
+        ids = np.concatenate([s[0] for s in seqs])
+        tg = np.concatenate([s[1] for s in seqs])
+        loss = arch.sequence_loss(model, ids, tg, 0, 128)
+        ag.backward(loss, 0.25)
+        gpu.sync([loss])
+        gh = {n: gpu.read_state_buffer(gpu.buffers_for(p)["grad"], p.size) for n, p in model.named_params()}
+        opt.record_step()
+        gpu.sync([])
+        opt.sync_weights_to_host()
+    finally:
+        gpu.uninstall()
+    compare(loss.data.copy(), gh, lr_, gr, "config 1")
+    ropt = ref.AdamW(rmodel.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
+    ropt.step()
+    # The first Adam step is g/(|g|+eps): where |g| is near eps = 1e-8 the update turns rounding noise in g (1e-9
+    # absolute, far inside the gradient tolerance) into O(lr) differences in w. Gradients are held to 1e-5 above;
+    # the weights to 1e-4 relative L2 / 5e-3 max-rel. Identical gradients give 1e-5 (test_gpu_optim.py).
+    for n, p in rmodel.named_params():
+        assert_close(model.p[n].data, p.data, f"config 1 weight after AdamW {n}", rel_l2=1e-4, max_rel=5e-3)
+    assert gpu.grad_clears_issued < 400          # first-writer stores: no per-node gradient clears

@@ -123,7 +123,9 @@ def test_attention(gpu, ref, T, Hq, Hkv, hd, window):
     r = R(ref, T * 3 + hd + window)
     op_case(gpu, ref, [r(T, Hq * hd), r(T, Hkv * hd), r(T, Hkv * hd)],
             lambda ag, q, k, v: ag.attention(q, k, v, T, Hq, Hkv, hd, window),
-            lambda rf, q, k, v: rf.attention(q, k, v, T, Hq, Hkv, hd, window), f"attention {T},{Hq},{Hkv},{hd},w{window}")
+            lambda rf, q, k, v: rf.attention(q, k, v, T, Hq, Hkv, hd, window), f"attention {T},{Hq},{Hkv},{hd},w{window}",
+            # window 1: one key per query, dq and dk are exactly zero; both sides leave ~1e-8 of rounding there
+            floor=1.0 if window == 1 else 0.0)
 
 
 def test_attention_stacked_sequences(gpu, ref):
@@ -284,3 +286,58 @@ def test_late_backward_after_sync_is_refused(gpu, ref):
     finally:
         gpu.uninstall()
         gpu.sync([])
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 700, 4, 2, 64, 0), (2, 333, 6, 2, 64, 300), (1, 1024, 9, 3, 64, 0),
+                                                  (3, 129, 2, 1, 64, 33), (1, 512, 3, 3, 64, 512)])
+def test_attention_mfma_shapes(gpu, ref, B, T, Hq, Hkv, hd, window):
+    """The matrix-core kernels (hd = 64): tiles of 128 queries x 32 keys with ragged T, windows that cut tiles, GQA
+    group sums, stacked sequences; 1024 x 9/3 x 64 is one SmolLM2 layer at half the sequence length."""
+    ag = mod("autograd")
+    r = R(ref, T + Hq + window)
+    q, k, v = r(B * T, Hq * hd), r(B * T, Hkv * hd), r(B * T, Hkv * hd)
+    up = ref.Mulberry32(1).fill_uniform([B * T * Hq * hd])
+    hq, hk, hv = (ag.Tensor(a, list(a.shape), True) for a in (q, k, v))
+    gpu.install()
+    try:
+        out = ag.attention(hq, hk, hv, T, Hq, Hkv, hd, window)
+        backward_from(gpu, ag, out, up)
+        gpu.sync([out])
+    finally:
+        gpu.uninstall()
+    ref.set_threads(min(8, ref.max_threads()))
+    try:
+        for b in range(B):
+            s = slice(b * T, (b + 1) * T)
+            rq, rk, rv = (ref.Tensor(a[s], [T, a.shape[1]], True) for a in (q, k, v))
+            o = ref.attention(rq, rk, rv, T, Hq, Hkv, hd, window, parallel_bwd=True)
+            ref.backward_from(o, up.reshape(B, -1)[b])
+            assert_close(out.data.reshape(B, -1)[b], o.data, f"mfma attention out[{b}]")
+            for h, rr, nm in ((hq, rq, "q"), (hk, rk, "k"), (hv, rv, "v")):
+                assert_close(h.grad.reshape(B, -1)[b], rr.grad, f"mfma attention d{nm}[{b}]")
+    finally:
+        ref.set_threads(1)
+
+
+def test_attention_mfma_equals_generic_at_full_length(gpu, ref):
+    """T = 2048, 9/3 heads x 64 (the SmolLM2 layer), two stacked sequences: both kernel families against each other."""
+    ag = mod("autograd")
+    B, T, Hq, Hkv, hd = 2, 2048, 9, 3, 64
+    rs = np.random.RandomState(5)
+    q, k, v = (rs.standard_normal((B * T, n * hd)).astype(np.float32) for n in (Hq, Hkv, Hkv))
+    up = rs.standard_normal(B * T * Hq * hd).astype(np.float32)
+    res = []
+    for generic in (1, 0):
+        gpu.set_option("attn.generic", generic)
+        hq, hk, hv = (ag.Tensor(a, list(a.shape), True) for a in (q, k, v))
+        gpu.install()
+        try:
+            out = ag.attention(hq, hk, hv, T, Hq, Hkv, hd, 0)
+            backward_from(gpu, ag, out, up)
+            gpu.sync([out])
+        finally:
+            gpu.uninstall()
+            gpu.set_option("attn.generic", 0)
+        res.append((out.data.copy(), hq.grad.copy(), hk.grad.copy(), hv.grad.copy()))
+    for a, b, nm in zip(res[1], res[0], ("out", "dq", "dk", "dv")):
+        assert_close(a, b, f"mfma vs generic {nm}")
