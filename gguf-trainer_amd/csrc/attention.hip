@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
 
 int attn_mfma_supported(int hd);
 int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
-int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
+int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
                   gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 
 static int check(gt_ctx *ctx, const char *who, int B, int T, int Hq, int Hkv, int hd, int window) {
@@ -256,16 +256,22 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd)};
   int64_t rows = (int64_t)B * Hq * T, krows = (int64_t)B * Hkv * T;
   ProfScope whole(ctx, "attention.bwd", 5.0 * 2 * hd * attn_pairs(T, window) * Hq * B);   // S, dP, dV, dK, dQ
+  // workspace: D per (sequence, head, row), then (MFMA path, kv group > 1) one dK and one dV slice per query head
+  const bool mfma = !ctx->opt_attn_generic && attn_mfma_supported(hd);
+  const int group = Hq / Hkv;
+  const size_t d_floats = ((size_t)rows + 63) / 64 * 64;
+  const size_t part_floats = (mfma && group > 1) ? (size_t)2 * group * krows * hd : 0;
   void *ws;
-  if (gt_ws_reserve(ctx, (size_t)rows * sizeof(float), &ws)) return 1;
+  if (gt_ws_reserve(ctx, (d_floats + part_floats) * sizeof(float), &ws)) return 1;
   float *Dr = static_cast<float *>(ws);
+  float *part = part_floats ? Dr + d_floats : nullptr;
   {
     ProfScope ps(ctx, "attention.bwd.D");
     hipLaunchKernelGGL(attn_bwd_d, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, p, P<const float>(out),
                        P<const float>(dout), Dr);
     GT_LAUNCHED(ctx);
   }
-  if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, dq, acc_q, dk, acc_k, dv, acc_v);
+  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dq, acc_q, dk, acc_k, dv, acc_v);
   {
     ProfScope ps(ctx, "attention.bwd.dq");
     size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);

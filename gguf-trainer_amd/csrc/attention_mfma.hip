@@ -1,7 +1,6 @@
-// Attention forward / backward on the FP32 matrix cores (v_mfma_f32_32x32x2_f32) for head dims that
-// are multiples of 32 (64 and 128 are the shapes of every config). Same math and saved statistic as
-// the generic kernels in attention.hip: causal / sliding window, GQA, scores in the log2 domain,
-// softmax recomputed in backward from lse2.
+// Attention forward / backward on the FP32 matrix cores (v_mfma_f32_32x32x2_f32) for head dim 64.
+// Same math and saved statistic as the generic kernels in attention.hip: causal / sliding window,
+// GQA, scores in the log2 domain, softmax recomputed in backward from lse2.
 //
 // How the tiles map onto a 64-lane wavefront. A wavefront owns 32 queries (forward, dQ) or 32 keys
 // (dK/dV); a workgroup is four of them. Scores are computed TRANSPOSED, S^T[key][query] = K.Q^T
@@ -13,12 +12,19 @@
 // its half: the probability / dS tile feeds the second contraction (P.V, dS.K, P^T.dO, dS^T.Q)
 // straight from the accumulators, with no transpose through LDS.
 //
-// Operand staging. The 32-row tile that changes per iteration (K,V in forward and dQ; Q,dO in dK/dV)
-// is staged in LDS as [row][hd+4]. The first contraction reads it with ds_read_b128 (a lane's MFMA
-// inputs for four steps; row stride hd+4 words keeps every 8-lane group on distinct banks), the
-// second reads columns of the same tile with ds_read_b32 (consecutive lanes, consecutive banks).
+// Operand staging. The tile that changes per iteration (K,V in forward and dQ; Q,dO in dK/dV) is
+// staged in LDS in the layout its contraction reads with ds_read_b128, one read per four MFMAs:
+// row-major [row][hd+4] for the first contraction (a lane's four consecutive head dims of its row)
+// and transposed [hd][rows+4] for the second (a lane's four consecutive rows of its head dim).
+// Strides of 4 mod 32 words keep every 8-lane group of a b128 access on distinct banks, and the
+// global->LDS copy assigns consecutive lanes to consecutive rows so both stores are conflict-free.
 // The operand that stays fixed for the whole loop (this lane's query / key row) lives in registers.
-// Global loads of the next tile are issued into registers before the MFMAs of the current one.
+// Global loads of the next tile are issued into registers before the MFMAs of the current one, and
+// all LDS reads of a contraction are issued before its first MFMA.
+//
+// The running maximum of the online softmax is only raised, and the output accumulators rescaled,
+// when some lane of the wavefront actually sees a larger score (after the first few tiles it almost
+// never does), which keeps the accumulators out of the VALU in the steady state.
 //
 // dK/dV loops over the query heads of the kv group inside the workgroup and over query tiles in
 // increasing order, so the GQA sum has a fixed order and needs no atomics.
@@ -35,16 +41,20 @@ struct AttnP {
 };
 
 #define NEG_BIG (-1.0e30f)
+#define HD 64
+#define LD (HD + 4)          // row-major tile stride
 
 __device__ __forceinline__ int win_lo_m(int t, int window) { return (window > 0 && t + 1 > window) ? t + 1 - window : 0; }
-// row of accumulator register r (== K index of MFMA step r) for lane half g
 __device__ __forceinline__ int acc_row(int r, int g) { return 8 * (r / 4) + 4 * g + (r % 4); }
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int HD> struct TileIO {
-  static constexpr int LD = HD + 4;
-  static constexpr int PER = (32 * HD / 4) / 256;            // float4 units per thread
-  static_assert((32 * HD / 4) % 256 == 0, "head dim must be a multiple of 32");
-  // rows [row0, row0+32) of a row-major matrix with `stride` floats per row, columns [0,HD) at src
+// ROWS x HD tile. Global loads are coalesced (16 lanes cover one 256-byte row). Row-major copy:
+// [row][LD]. Transposed copy: [d][ROWS+4] with the 16-byte column chunks XOR-swizzled by (d/8)%8, which
+// makes the scalar transposing stores hit every bank exactly twice per 64 lanes (the minimum) while the
+// b128 reads of the second contraction stay conflict-free (an aligned group of 8 lanes shares d/8).
+template <int ROWS> struct TileIO {
+  static constexpr int LDT = ROWS + 4;
+  static constexpr int PER = (ROWS * HD / 4) / 256;
   __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ src, size_t stride, int row0, int rmax, int tid) {
 #pragma unroll
     for (int i = 0; i < PER; i++) {
@@ -54,17 +64,27 @@ template <int HD> struct TileIO {
       reg[i] = v;
     }
   }
-  __device__ static __forceinline__ void store(const v4f (&reg)[PER], float *lds, int tid) {
+  __device__ static __forceinline__ void store_rows(const v4f (&reg)[PER], float *lds, int tid) {
 #pragma unroll
     for (int i = 0; i < PER; i++) {
       int u = tid + i * 256, row = u / (HD / 4), c4 = u % (HD / 4);
       *reinterpret_cast<v4f *>(lds + row * LD + c4 * 4) = reg[i];
     }
   }
+  __device__ static __forceinline__ void store_t(const v4f (&reg)[PER], float *ldst, int tid) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      int u = tid + i * 256, row = u / (HD / 4), c4 = u % (HD / 4);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        int d = c4 * 4 + j;
+        ldst[d * LDT + 4 * ((row >> 2) ^ ((d >> 3) & 7)) + (row & 3)] = reg[i][j];
+      }
+    }
+  }
 };
 
 // this lane's row as MFMA B-operand registers: reg[4j+s] = x[8j + 4g + s] * mul
-template <int HD>
 __device__ __forceinline__ void load_row_regs(float (&reg)[HD / 2], const float *__restrict__ row, bool valid, int g, float mul) {
 #pragma unroll
   for (int j = 0; j < HD / 8; j++) {
@@ -75,36 +95,40 @@ __device__ __forceinline__ void load_row_regs(float (&reg)[HD / 2], const float 
   }
 }
 
-// acc = Tile(rows) . reg^T : A from LDS rows (b128), B from this lane's registers
-template <int HD>
-__device__ __forceinline__ v16f tile_dot_regs(const float *lds, const float (&reg)[HD / 2], int l32, int g) {
-  constexpr int LD = HD + 4;
+// acc = Tile(32 rows starting at `rows`) . reg^T : A = rows of the row-major tile, B = this lane's registers.
+__device__ __forceinline__ v16f rows_dot_regs(const float *rows, const float (&reg)[HD / 2], int l32, int g) {
+  v4f a[HD / 8];
+#pragma unroll
+  for (int j = 0; j < HD / 8; j++) a[j] = *reinterpret_cast<const v4f *>(rows + l32 * LD + 8 * j + 4 * g);
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
 #pragma unroll
-  for (int j = 0; j < HD / 8; j++) {
-    v4f a = *reinterpret_cast<const v4f *>(lds + l32 * LD + 8 * j + 4 * g);
+  for (int j = 0; j < HD / 8; j++)
 #pragma unroll
-    for (int s = 0; s < 4; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], reg[4 * j + s], acc, 0, 0, 0);
-  }
+    for (int s = 0; s < 4; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][s], reg[4 * j + s], acc, 0, 0, 0);
   return acc;
 }
 
-// out[dt] += Tile^T(cols of dt) . w : A = columns of the LDS tile (b32), B = the 16 accumulator-ordered weights
-template <int HD>
-__device__ __forceinline__ void tile_t_dot_acc(v16f (&out)[HD / 32], const float *lds, const float (&w)[16], int l32, int g) {
-  constexpr int LD = HD + 4;
+// out[dt] += TileT(cols [col0, col0+32)) . w : A = the transposed tile (stride LDT), B = 16 accumulator-ordered weights
+template <int LDT>
+__device__ __forceinline__ void t_dot_acc(v16f (&out)[HD / 32], const float *ldst, int col0, const float (&w)[16], int l32, int g) {
+  v4f a[HD / 32][4];
 #pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const float *rowp = lds + acc_row(i, g) * LD + l32;
+  for (int dt = 0; dt < HD / 32; dt++)
 #pragma unroll
-    for (int dt = 0; dt < HD / 32; dt++) out[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(rowp[dt * 32], w[i], out[dt], 0, 0, 0);
-  }
+    for (int q = 0; q < 4; q++) {
+      int d = dt * 32 + l32, chunk = (col0 >> 2) + 2 * q + g;
+      a[dt][q] = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * (chunk ^ ((d >> 3) & 7)));
+    }
+#pragma unroll
+  for (int q = 0; q < 4; q++)
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; dt++) out[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[dt][q][s], w[4 * q + s], out[dt], 0, 0, 0);
 }
 
-// write this lane's 32x(HD) transposed accumulator column (one row t of a [rows][stride] matrix)
-template <int HD>
 __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32], int g, float mul, int add) {
 #pragma unroll
   for (int dt = 0; dt < HD / 32; dt++)
@@ -117,18 +141,21 @@ __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32]
     }
 }
 
+#define KT 64      // keys per LDS stage in forward and dQ
+
 // ---- forward --------------------------------------------------------------------------------------
-template <int HD>
 __global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, float *__restrict__ out,
                                                        float *__restrict__ lse) {
-  using IO = TileIO<HD>;
-  constexpr int LD = HD + 4;
-  __shared__ __attribute__((aligned(16))) float sK[32 * LD];
-  __shared__ __attribute__((aligned(16))) float sV[32 * LD];
+  using IO = TileIO<KT>;
+  __shared__ __attribute__((aligned(16))) float sK[KT * LD];
+  __shared__ __attribute__((aligned(16))) float sVt[HD * IO::LDT];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
-  const int qtile = gridDim.x - 1 - blockIdx.x;          // longest rows first
-  const int h = blockIdx.y, b = blockIdx.z;
+  // 1-D grid ordered by work: every (head, sequence) pair's longest query tile is dispatched before any shorter
+  // one, so the causal triangle packs onto the CUs without a long tail
+  const int nhb = p.Hq * p.B;
+  const int qtile = (int)((p.T + 127) / 128) - 1 - (int)(blockIdx.x / nhb);
+  const int h = (blockIdx.x % nhb) % p.Hq, b = (blockIdx.x % nhb) / p.Hq;
   const int kvh = h / (p.Hq / p.Hkv);
   const size_t qstr = (size_t)p.Hq * HD, kstr = (size_t)p.Hkv * HD;
   const int tq0 = qtile * 128 + wave * 32, t = tq0 + l32;
@@ -137,11 +164,12 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__r
   const float *kb = k + (size_t)b * p.T * kstr + (size_t)kvh * HD;
   const float *vb = v + (size_t)b * p.T * kstr + (size_t)kvh * HD;
   float qreg[HD / 2];
-  load_row_regs<HD>(qreg, q + ((size_t)b * p.T + (tv ? t : 0)) * qstr + (size_t)h * HD, tv, g, p.c2);
+  load_row_regs(qreg, q + ((size_t)b * p.T + (tv ? t : 0)) * qstr + (size_t)h * HD, tv, g, p.c2);
   const int lo_t = win_lo_m(t, p.window);
-  const int kt_lo = win_lo_m(qtile * 128, p.window) / 32;
-  const int kt_hi = min(p.T - 1, qtile * 128 + 127) / 32;
-  const int wave_lo = win_lo_m(tq0, p.window);
+  const int kt_lo = win_lo_m(qtile * 128, p.window) / KT;
+  const int kt_hi = min(p.T - 1, qtile * 128 + 127) / KT;
+  const int wave_lo = win_lo_m(tq0, p.window), wave_lo_last = win_lo_m(tq1, p.window);
+  const bool ragged = tq0 + 31 >= p.T;
 
   v16f oacc[HD / 32];
 #pragma unroll
@@ -151,66 +179,88 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__r
   float m = NEG_BIG, l = 0.f;
 
   v4f pk[IO::PER], pv[IO::PER];
-  IO::load(pk, kb, kstr, kt_lo * 32, p.T, tid);
-  IO::load(pv, vb, kstr, kt_lo * 32, p.T, tid);
+  IO::load(pk, kb, kstr, kt_lo * KT, p.T, tid);
+  IO::load(pv, vb, kstr, kt_lo * KT, p.T, tid);
   for (int kt = kt_lo; kt <= kt_hi; kt++) {
     __syncthreads();
-    IO::store(pk, sK, tid);
-    IO::store(pv, sV, tid);
+    IO::store_rows(pk, sK, tid);
+    IO::store_t(pv, sVt, tid);
     __syncthreads();
     if (kt < kt_hi) {
-      IO::load(pk, kb, kstr, (kt + 1) * 32, p.T, tid);
-      IO::load(pv, vb, kstr, (kt + 1) * 32, p.T, tid);
+      IO::load(pk, kb, kstr, (kt + 1) * KT, p.T, tid);
+      IO::load(pv, vb, kstr, (kt + 1) * KT, p.T, tid);
     }
-    const int k0 = kt * 32;
-    if (k0 > tq1 || k0 + 31 < wave_lo || tq0 >= p.T) continue;      // wave-uniform: nothing of this tile is visible
-    v16f s = tile_dot_regs<HD>(sK, qreg, l32, g);
-    float pr[16];
+    if (tq0 >= p.T) continue;
+    float pr[2][16];
+    bool act[2];
     float mx = NEG_BIG;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      int key = k0 + acc_row(r, g);
-      bool ok = tv && key <= t && key >= lo_t;
-      pr[r] = ok ? s[r] : NEG_BIG;
-      mx = fmaxf(mx, pr[r]);
+    for (int sub = 0; sub < 2; sub++) {
+      const int k0 = kt * KT + sub * 32;
+      act[sub] = !(k0 > tq1 || k0 + 31 < wave_lo);           // wave-uniform: some (query, key) pair is visible
+      if (!act[sub]) continue;
+      v16f s = rows_dot_regs(sK + sub * 32 * LD, qreg, l32, g);
+      const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
+      if (need_mask) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          int key = k0 + acc_row(r, g);
+          pr[sub][r] = (tv && key <= t && key >= lo_t) ? s[r] : NEG_BIG;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) pr[sub][r] = s[r];
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) mx = fmaxf(mx, pr[sub][r]);
     }
+    if (!act[0] && !act[1]) continue;
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mn = fmaxf(m, mx);
-    const float alpha = exp2f(m - mn);
-    float ls = 0.f;
+    if (__any(mx > m)) {                                      // rare after the first tiles
+      const float mn = fmaxf(m, mx);
+      const float alpha = fast_exp2(m - mn);
+      l *= alpha;
+      m = mn;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      pr[r] = pr[r] > -1.0e29f ? exp2f(pr[r] - mn) : 0.f;
-      ls += pr[r];
+      for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
     }
-    l = l * alpha + ls;
-    m = mn;
 #pragma unroll
-    for (int dt = 0; dt < HD / 32; dt++)
+    for (int sub = 0; sub < 2; sub++) {
+      if (!act[sub]) continue;
+      float ls = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
-    tile_t_dot_acc<HD>(oacc, sV, pr, l32, g);
+      for (int r = 0; r < 16; r++) {
+        // a masked score is NEG_BIG; with m still NEG_BIG (no visible key yet) the difference would be 0
+        float e = pr[sub][r] > -1.0e29f ? fast_exp2(pr[sub][r] - m) : 0.f;
+        pr[sub][r] = e;
+        ls += e;
+      }
+      l += ls;
+      t_dot_acc<IO::LDT>(oacc, sVt, sub * 32, pr[sub], l32, g);
+    }
   }
   const float lt = l + __shfl_xor(l, 32, 64);
   if (tv) {
-    store_row<HD>(out + ((size_t)b * p.T + t) * qstr + (size_t)h * HD, oacc, g, 1.0f / lt, 0);
+    store_row(out + ((size_t)b * p.T + t) * qstr + (size_t)h * HD, oacc, g, 1.0f / lt, 0);
     if (g == 0) lse[((size_t)b * p.Hq + h) * p.T + t] = m + log2f(lt);
   }
 }
 
 // ---- dQ -----------------------------------------------------------------------------------------------
-template <int HD>
 __global__ __launch_bounds__(256) void attn_bwd_dq_mfma_k(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                           const float *__restrict__ v, const float *__restrict__ go,
                                                           const float *__restrict__ lse, const float *__restrict__ Dr,
                                                           float *dq, int acc_q) {
-  using IO = TileIO<HD>;
-  constexpr int LD = HD + 4;
-  __shared__ __attribute__((aligned(16))) float sK[32 * LD];
-  __shared__ __attribute__((aligned(16))) float sV[32 * LD];
+  using IO = TileIO<KT>;
+  __shared__ __attribute__((aligned(16))) float sK[KT * LD];
+  __shared__ __attribute__((aligned(16))) float sV[KT * LD];
+  __shared__ __attribute__((aligned(16))) float sKt[HD * IO::LDT];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
-  const int qtile = gridDim.x - 1 - blockIdx.x;
-  const int h = blockIdx.y, b = blockIdx.z;
+  const int nhb = p.Hq * p.B;
+  const int qtile = (int)((p.T + 127) / 128) - 1 - (int)(blockIdx.x / nhb);
+  const int h = (blockIdx.x % nhb) % p.Hq, b = (blockIdx.x % nhb) / p.Hq;
   const int kvh = h / (p.Hq / p.Hkv);
   const size_t qstr = (size_t)p.Hq * HD, kstr = (size_t)p.Hkv * HD;
   const int tq0 = qtile * 128 + wave * 32, t = tq0 + l32;
@@ -220,14 +270,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_mfma_k(AttnP p, const float *
   const float *vb = v + (size_t)b * p.T * kstr + (size_t)kvh * HD;
   const size_t qoff = ((size_t)b * p.T + (tv ? t : 0)) * qstr + (size_t)h * HD;
   float qreg[HD / 2], greg[HD / 2];
-  load_row_regs<HD>(qreg, q + qoff, tv, g, p.c2);
-  load_row_regs<HD>(greg, go + qoff, tv, g, 1.0f);
+  load_row_regs(qreg, q + qoff, tv, g, p.c2);
+  load_row_regs(greg, go + qoff, tv, g, 1.0f);
   const size_t sidx = ((size_t)b * p.Hq + h) * p.T + (tv ? t : 0);
   const float L2 = tv ? lse[sidx] : 0.f, Dt = tv ? Dr[sidx] : 0.f;
   const int lo_t = win_lo_m(t, p.window);
-  const int kt_lo = win_lo_m(qtile * 128, p.window) / 32;
-  const int kt_hi = min(p.T - 1, qtile * 128 + 127) / 32;
-  const int wave_lo = win_lo_m(tq0, p.window);
+  const int kt_lo = win_lo_m(qtile * 128, p.window) / KT;
+  const int kt_hi = min(p.T - 1, qtile * 128 + 127) / KT;
+  const int wave_lo = win_lo_m(tq0, p.window), wave_lo_last = win_lo_m(tq1, p.window);
+  const bool ragged = tq0 + 31 >= p.T;
 
   v16f dacc[HD / 32];
 #pragma unroll
@@ -236,61 +287,78 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_mfma_k(AttnP p, const float *
     for (int r = 0; r < 16; r++) dacc[dt][r] = 0.f;
 
   v4f pk[IO::PER], pv[IO::PER];
-  IO::load(pk, kb, kstr, kt_lo * 32, p.T, tid);
-  IO::load(pv, vb, kstr, kt_lo * 32, p.T, tid);
+  IO::load(pk, kb, kstr, kt_lo * KT, p.T, tid);
+  IO::load(pv, vb, kstr, kt_lo * KT, p.T, tid);
   for (int kt = kt_lo; kt <= kt_hi; kt++) {
     __syncthreads();
-    IO::store(pk, sK, tid);
-    IO::store(pv, sV, tid);
+    IO::store_rows(pk, sK, tid);
+    IO::store_t(pk, sKt, tid);
+    IO::store_rows(pv, sV, tid);
     __syncthreads();
     if (kt < kt_hi) {
-      IO::load(pk, kb, kstr, (kt + 1) * 32, p.T, tid);
-      IO::load(pv, vb, kstr, (kt + 1) * 32, p.T, tid);
+      IO::load(pk, kb, kstr, (kt + 1) * KT, p.T, tid);
+      IO::load(pv, vb, kstr, (kt + 1) * KT, p.T, tid);
     }
-    const int k0 = kt * 32;
-    if (k0 > tq1 || k0 + 31 < wave_lo || tq0 >= p.T) continue;
-    v16f s = tile_dot_regs<HD>(sK, qreg, l32, g);
-    v16f dp = tile_dot_regs<HD>(sV, greg, l32, g);
-    float ds[16];
+    if (tq0 >= p.T) continue;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      int key = k0 + acc_row(r, g);
-      bool ok = tv && key <= t && key >= lo_t;
-      float pr = ok ? exp2f(s[r] - L2) : 0.f;
-      ds[r] = pr * (dp[r] - Dt) * p.scale;
+    for (int sub = 0; sub < 2; sub++) {
+      const int k0 = kt * KT + sub * 32;
+      if (k0 > tq1 || k0 + 31 < wave_lo) continue;
+      v16f s = rows_dot_regs(sK + sub * 32 * LD, qreg, l32, g);
+      v16f dp = rows_dot_regs(sV + sub * 32 * LD, greg, l32, g);
+      const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
+      float ds[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        float pr = fast_exp2(s[r] - L2);
+        if (need_mask) {
+          int key = k0 + acc_row(r, g);
+          if (!(tv && key <= t && key >= lo_t)) pr = 0.f;
+        }
+        ds[r] = pr * (dp[r] - Dt) * p.scale;
+      }
+      t_dot_acc<IO::LDT>(dacc, sKt, sub * 32, ds, l32, g);
     }
-    tile_t_dot_acc<HD>(dacc, sK, ds, l32, g);
   }
-  if (tv) store_row<HD>(dq + qoff, dacc, g, 1.0f, acc_q);
+  if (tv) store_row(dq + qoff, dacc, g, 1.0f, acc_q);
 }
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------
-template <int HD>
+#define QT 32      // queries per LDS stage in dK/dV
 __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_k(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
-                                                           float *dk, int acc_k, float *dv, int acc_v) {
-  using IO = TileIO<HD>;
-  constexpr int LD = HD + 4;
-  __shared__ __attribute__((aligned(16))) float sQ[32 * LD];
-  __shared__ __attribute__((aligned(16))) float sG[32 * LD];
-  __shared__ float sL[32], sD[32];
+                                                           float *dk, int acc_k, float *dv, int acc_v, float *part) {
+  using IO = TileIO<QT>;
+  __shared__ __attribute__((aligned(16))) float sQ[QT * LD];
+  __shared__ __attribute__((aligned(16))) float sG[QT * LD];
+  __shared__ __attribute__((aligned(16))) float sQt[HD * IO::LDT];
+  __shared__ __attribute__((aligned(16))) float sGt[HD * IO::LDT];
+  __shared__ __attribute__((aligned(16))) float sL[QT], sD[QT];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
-  const int ktile = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  // 1-D grid, key tile slowest: the first key tiles are seen by the most queries and go first. One workgroup
+  // per QUERY head: with a kv group larger than one, each head's dK/dV goes to its own slice of the workspace
+  // and attn_group_sum adds the slices in head order (a fixed order, so still deterministic); splitting by
+  // head is what gives the dispatcher enough similar-sized pieces to fill 256 CUs.
+  const int nhb = p.Hq * p.B;
+  const int ktile = (int)(blockIdx.x / nhb);
+  const int h = (blockIdx.x % nhb) % p.Hq, b = (blockIdx.x % nhb) / p.Hq;
   const int group = p.Hq / p.Hkv;
+  const int kvh = h / group, hh = h % group;
   const size_t qstr = (size_t)p.Hq * HD, kstr = (size_t)p.Hkv * HD;
   const int sk0 = ktile * 128 + wave * 32, s = sk0 + l32;
   const bool sv = s < p.T;
   const size_t koff = ((size_t)b * p.T + (sv ? s : 0)) * kstr + (size_t)kvh * HD;
   float kreg[HD / 2], vreg[HD / 2];
-  load_row_regs<HD>(kreg, k + koff, sv, g, p.c2);
-  load_row_regs<HD>(vreg, v + koff, sv, g, 1.0f);
+  load_row_regs(kreg, k + koff, sv, g, p.c2);
+  load_row_regs(vreg, v + koff, sv, g, 1.0f);
   // queries that can see a key of this workgroup: t in [ktile*128, last key + window - 1]
-  const int qt_lo = ktile * 4;
+  const int qt_lo = ktile * (128 / QT);
   const int t_last = p.window > 0 ? min(p.T - 1, ktile * 128 + 127 + p.window - 1) : p.T - 1;
-  const int qt_hi = t_last / 32;
+  const int qt_hi = t_last / QT;
   const int nqt = qt_hi - qt_lo + 1;
   const int wave_t_hi = p.window > 0 ? sk0 + 31 + p.window - 1 : p.T - 1;   // last query that sees a key of this wave
+  const bool ragged_k = sk0 + 31 >= p.T;
 
   v16f kacc[HD / 32], vacc[HD / 32];
 #pragma unroll
@@ -298,79 +366,117 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_k(AttnP p, const float 
 #pragma unroll
     for (int r = 0; r < 16; r++) { kacc[dt][r] = 0.f; vacc[dt][r] = 0.f; }
 
-  const int niter = group * nqt;
+  const int niter = nqt;
   v4f pq[IO::PER], pg[IO::PER];
   float pstat = 0.f;
   auto prefetch = [&](int it) {
-    int hh = it / nqt, qt = qt_lo + it % nqt;
-    int h = kvh * group + hh;
+    int qt = qt_lo + it;
     const float *qb = q + (size_t)b * p.T * qstr + (size_t)h * HD;
     const float *gb = go + (size_t)b * p.T * qstr + (size_t)h * HD;
-    IO::load(pq, qb, qstr, qt * 32, p.T, tid);
-    IO::load(pg, gb, qstr, qt * 32, p.T, tid);
-    if (tid < 64) {
-      int tt = qt * 32 + (tid % 32);
+    IO::load(pq, qb, qstr, qt * QT, p.T, tid);
+    IO::load(pg, gb, qstr, qt * QT, p.T, tid);
+    if (tid < 2 * QT) {
+      int tt = qt * QT + (tid % QT);
       size_t si = ((size_t)b * p.Hq + h) * p.T + tt;
-      pstat = tt < p.T ? (tid < 32 ? lse[si] : Dr[si]) : 0.f;
+      pstat = tt < p.T ? (tid < QT ? lse[si] : Dr[si]) : 0.f;
     }
   };
   prefetch(0);
   for (int it = 0; it < niter; it++) {
     __syncthreads();
-    IO::store(pq, sQ, tid);
-    IO::store(pg, sG, tid);
-    if (tid < 32) sL[tid] = pstat;
-    else if (tid < 64) sD[tid - 32] = pstat;
+    IO::store_rows(pq, sQ, tid);
+    IO::store_t(pq, sQt, tid);
+    IO::store_rows(pg, sG, tid);
+    IO::store_t(pg, sGt, tid);
+    if (tid < QT) sL[tid] = pstat;
+    else if (tid < 2 * QT) sD[tid - QT] = pstat;
     __syncthreads();
     if (it + 1 < niter) prefetch(it + 1);
-    const int t0 = (qt_lo + it % nqt) * 32;
+    const int t0 = (qt_lo + it) * QT;
     if (t0 + 31 < sk0 || t0 > wave_t_hi || sk0 >= p.T) continue;      // wave-uniform: no (query, key) pair of this tile is live
-    v16f sc = tile_dot_regs<HD>(sQ, kreg, l32, g);
-    v16f dp = tile_dot_regs<HD>(sG, vreg, l32, g);
+    v16f sc = rows_dot_regs(sQ, kreg, l32, g);
+    v16f dp = rows_dot_regs(sG, vreg, l32, g);
+    // fully visible tile: every query is at or after every key of the wave, inside the window, and in range
+    const bool need_mask = ragged_k || t0 < sk0 + 31 || t0 + 31 >= p.T || (p.window > 0 && t0 + 31 > sk0 + p.window - 1);
     float pr[16], ds[16];
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      int ql = acc_row(r, g), tq = t0 + ql;
-      bool ok = sv && tq < p.T && s <= tq && (p.window == 0 || s + p.window > tq);
-      pr[r] = ok ? exp2f(sc[r] - sL[ql]) : 0.f;
-      ds[r] = pr[r] * (dp[r] - sD[ql]) * p.scale;
+    for (int a = 0; a < 4; a++) {
+      v4f lv = *reinterpret_cast<const v4f *>(sL + 8 * a + 4 * g), dv4 = *reinterpret_cast<const v4f *>(sD + 8 * a + 4 * g);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        int r = 4 * a + j;
+        float e = fast_exp2(sc[r] - lv[j]);
+        if (need_mask) {
+          int tq = t0 + 8 * a + 4 * g + j;
+          if (!(sv && tq < p.T && s <= tq && (p.window == 0 || s + p.window > tq))) e = 0.f;
+        }
+        pr[r] = e;
+        ds[r] = e * (dp[r] - dv4[j]) * p.scale;
+      }
     }
-    tile_t_dot_acc<HD>(vacc, sG, pr, l32, g);
-    tile_t_dot_acc<HD>(kacc, sQ, ds, l32, g);
+    t_dot_acc<IO::LDT>(vacc, sGt, 0, pr, l32, g);
+    t_dot_acc<IO::LDT>(kacc, sQt, 0, ds, l32, g);
   }
   if (sv) {
-    store_row<HD>(dk + koff, kacc, g, 1.0f, acc_k);
-    store_row<HD>(dv + koff, vacc, g, 1.0f, acc_v);
+    if (part) {            // slice hh of the workspace, same [row][Hkv*hd] layout as dk
+      const size_t slice = (size_t)p.B * p.T * kstr;
+      store_row(part + (size_t)hh * slice + koff, kacc, g, 1.0f, 0);
+      store_row(part + (size_t)(group + hh) * slice + koff, vacc, g, 1.0f, 0);
+    } else {
+      store_row(dk + koff, kacc, g, 1.0f, acc_k);
+      store_row(dv + koff, vacc, g, 1.0f, acc_v);
+    }
   }
 }
 
-int attn_mfma_supported(int hd) { return hd == 64; }
+// dk (+)= sum over the group's heads of their slices, in head order; same for dv
+__global__ __launch_bounds__(256) void attn_group_sum(const float *__restrict__ part, int group, size_t n4, float *dk, int acc_k,
+                                                      float *dv, int acc_v) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  const v4f *pp = reinterpret_cast<const v4f *>(part);
+  v4f sk = pp[i], sv = pp[(size_t)group * n4 + i];
+  for (int hh = 1; hh < group; hh++) { sk += pp[(size_t)hh * n4 + i]; sv += pp[(size_t)(group + hh) * n4 + i]; }
+  v4f *ok = reinterpret_cast<v4f *>(dk) + i, *ov = reinterpret_cast<v4f *>(dv) + i;
+  *ok = acc_k ? *ok + sk : sk;
+  *ov = acc_v ? *ov + sv : sv;
+}
+
+int attn_mfma_supported(int hd) { return hd == HD; }
 
 int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse) {
   GT_REQUIRE(ctx, (q | k | v | out) % 16 == 0, "attention: buffers must be 16-byte aligned");
-  dim3 grid((unsigned)cdiv(p.T, 128), p.Hq, p.B);
-  hipLaunchKernelGGL((attn_fwd_mfma_k<64>), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
+  dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
+  hipLaunchKernelGGL(attn_fwd_mfma_k, grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
                      P<const float>(v), P<float>(out), P<float>(lse));
   GT_LAUNCHED(ctx);
   return 0;
 }
 
-int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, gt_buf dq,
-                  int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+// Dr: the per-row sums D; part: workspace for the per-head dK/dV slices (2*group slices of B*T*Hkv*hd floats) or null
+int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
+                  gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
+  const int group = p.Hq / p.Hkv;
   {
     ProfScope ps(ctx, "attention.bwd.dq");
-    dim3 grid((unsigned)cdiv(p.T, 128), p.Hq, p.B);
-    hipLaunchKernelGGL((attn_bwd_dq_mfma_k<64>), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
+    dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
+    hipLaunchKernelGGL(attn_bwd_dq_mfma_k, grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
                        P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q);
     GT_LAUNCHED(ctx);
   }
   {
     ProfScope ps(ctx, "attention.bwd.dkv");
-    dim3 grid((unsigned)cdiv(p.T, 128), p.Hkv, p.B);
-    hipLaunchKernelGGL((attn_bwd_dkv_mfma_k<64>), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
-                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v);
+    dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
+    hipLaunchKernelGGL(attn_bwd_dkv_mfma_k, grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
+                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part);
     GT_LAUNCHED(ctx);
+    if (part) {
+      size_t n4 = (size_t)p.B * p.T * p.Hkv * HD / 4;
+      hipLaunchKernelGGL(attn_group_sum, dim3((unsigned)cdiv((int64_t)n4, 256)), dim3(256), 0, ctx->stream, part, group, n4,
+                         P<float>(dk), acc_k, P<float>(dv), acc_v);
+      GT_LAUNCHED(ctx);
+    }
   }
   return 0;
 }

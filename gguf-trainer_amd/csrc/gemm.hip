@@ -25,8 +25,8 @@
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-#define BK 16
-#define KS 20   // LDS row stride (words) of a k-contiguous operand tile
+// K depth of one LDS stage (BKT, 16 or 32) is a template parameter; a k-contiguous operand tile has
+// row stride BKT+4 words (20 or 36: both = 4 mod 32, see above).
 
 struct GemmArgs {
   const float *A, *B;
@@ -43,12 +43,14 @@ struct GemmArgs {
 
 // One operand tile of R rows x 16 k. KC: k contiguous in memory (element (r,k) at p[r*ld + k]);
 // otherwise row contiguous (element (r,k) at p[k*ld + r]).
-template <int R, bool KC, bool VEC, int NT>
+template <int R, bool KC, bool VEC, int NT, int BKT>
 struct Tile {
-  static constexpr int UNITS = R * 4;          // float4 units per tile
-  static constexpr int PER = UNITS / NT;       // per thread
-  static_assert(UNITS % NT == 0, "tile rows must be a multiple of threads/4");
-  static constexpr int LDS_WORDS = KC ? R * KS : BK * R;
+  static constexpr int KS = BKT + 4;
+  static constexpr int KQ = BKT / 4;           // float4 units along K
+  static constexpr int UNITS = R * KQ;         // float4 units per tile
+  static constexpr int PER = (UNITS + NT - 1) / NT;   // per thread (the last round may be partial)
+  static constexpr bool FULL = (UNITS % NT == 0);
+  static constexpr int LDS_WORDS = KC ? R * KS : BKT * R;
 
   // registers <- global, zero outside [0,Rtot) x [k0,kend)
   __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ p, int ld, int r0, int Rtot,
@@ -57,8 +59,9 @@ struct Tile {
     for (int i = 0; i < PER; i++) {
       int u = tid + i * NT;
       v4f v = {0.f, 0.f, 0.f, 0.f};
+      if (!FULL && u >= UNITS) { reg[i] = v; continue; }
       if (KC) {
-        int r = r0 + u / 4, k = k0 + (u % 4) * 4;
+        int r = r0 + u / KQ, k = k0 + (u % KQ) * 4;
         if (r < Rtot) {
           const float *q = p + (size_t)r * ld + k;
           if (VEC) { if (k < kend) v = *reinterpret_cast<const v4f *>(q); }
@@ -85,11 +88,12 @@ struct Tile {
 #pragma unroll
     for (int i = 0; i < PER; i++) {
       int u = tid + i * NT;
-      if (KC) *reinterpret_cast<v4f *>(lds + (u / 4) * KS + (u % 4) * 4) = reg[i];
+      if (!FULL && u >= UNITS) continue;
+      if (KC) *reinterpret_cast<v4f *>(lds + (u / KQ) * KS + (u % KQ) * 4) = reg[i];
       else *reinterpret_cast<v4f *>(lds + (u / (R / 4)) * R + (u % (R / 4)) * 4) = reg[i];
     }
   }
-  // MFMA inputs of this lane for the four steps of K-run c (0 or 1): row = tile row, g = lane/32
+  // MFMA inputs of this lane for the four steps of K-run c (0 .. BKT/8-1): row = tile row, g = lane/32
   __device__ static __forceinline__ v4f fetch(const float *lds, int row, int c, int g) {
     if (KC) return *reinterpret_cast<const v4f *>(lds + row * KS + c * 8 + g * 4);
     v4f v;
@@ -100,14 +104,15 @@ struct Tile {
   }
 };
 
-template <int BM, int BN, int WM, int WN, int KIND, bool VEC>
+template <int BM, int BN, int WM, int WN, int BKT, int KIND, bool VEC>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
+  constexpr int BK = BKT;
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be whole MFMA tiles");
   constexpr bool AKC = (KIND != GT_TN), BKC = (KIND == GT_NT);
-  using TA = Tile<BM, AKC, VEC, NT>;
-  using TB = Tile<BN, BKC, VEC, NT>;
+  using TA = Tile<BM, AKC, VEC, NT, BKT>;
+  using TB = Tile<BN, BKC, VEC, NT, BKT>;
   __shared__ __attribute__((aligned(16))) float sA[TA::LDS_WORDS];
   __shared__ __attribute__((aligned(16))) float sB[TB::LDS_WORDS];
 
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
       TB::load(rb, B, a.ldb, n0, a.N, k + BK, kend, tid);
     }
 #pragma unroll
-    for (int c = 0; c < 2; c++) {
+    for (int c = 0; c < BKT / 8; c++) {
       v4f fa[TM], fb[TN];
 #pragma unroll
       for (int i = 0; i < TM; i++) fa[i] = TA::fetch(sA, wm * (TM * 32) + i * 32 + l32, c, g);
@@ -202,12 +207,12 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ P
   C[i] = acc ? C[i] + s : s;
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int BKT>
 static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
   dim3 grid(a.nbm * a.nbn, 1, zdim), block(WM * WN * 64);
-#define GO(KIND, VEC) hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, KIND, VEC>), grid, block, 0, ctx->stream, a)
+#define GO(KIND, VEC) hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, BKT, KIND, VEC>), grid, block, 0, ctx->stream, a)
   if (kind == GT_NT) { if (vec) GO(GT_NT, true); else GO(GT_NT, false); }
   else if (kind == GT_NN) { if (vec) GO(GT_NN, true); else GO(GT_NN, false); }
   else { if (vec) GO(GT_TN, true); else GO(GT_TN, false); }
@@ -215,6 +220,11 @@ static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
   GT_LAUNCHED(ctx);
   return 0;
 }
+
+struct TileCfg { int bm, bn, bk; };
+static const TileCfg kTiles[] = {{64, 64, 16}, {128, 64, 16}, {128, 128, 16}, {128, 192, 16}, {128, 96, 16}, {256, 128, 16},
+                                 {128, 128, 32}, {128, 192, 32}, {128, 96, 32}, {256, 128, 32}, {64, 192, 16}, {128, 64, 32}};
+#define NCFG ((int)(sizeof(kTiles) / sizeof(kTiles[0])))
 
 static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
                      gt_buf C, int64_t sC, int count) {
@@ -233,31 +243,39 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
              (sA % 4 == 0) && (sB % 4 == 0);
 
-  // Tile choice: the largest tile that still gives every CU a few workgroups; narrow N (heads,
-  // LoRA rank) takes the 64-wide tile so columns are not wasted.
-  int cfg;
-  auto blocks = [&](int bm, int bn) { return cdiv(M, bm) * cdiv(N, bn) * count; };
-  if (N <= 64 || M <= 64) cfg = 0;
-  else if (N % 192 == 0 && N % 128 != 0 && blocks(128, 192) >= ctx->num_cu) cfg = 3;
-  else if (blocks(128, 128) >= 2 * ctx->num_cu) cfg = 2;
-  else cfg = 1;
-  if (ctx->opt_gemm_tile >= 0 && ctx->opt_gemm_tile <= 3) cfg = ctx->opt_gemm_tile;
-  int bm = cfg == 0 ? 64 : 128, bn = cfg == 0 ? 64 : cfg == 1 ? 64 : cfg == 2 ? 128 : 192;
-
-  // split K when the output alone cannot fill the chip (dW: K = rows of the batch)
-  int splits = 1;
-  if (count == 1) {
-    int64_t nb = blocks(bm, bn);
-    int64_t ksteps = cdiv(K, BK);
-    if (nb < 2 * ctx->num_cu && ksteps >= 16) {
-      splits = (int)std::min<int64_t>(cdiv(3 * ctx->num_cu, nb), ksteps / 8);
-      if (splits < 1) splits = 1;
-      if (splits > 64) splits = 64;
+  // Tile and split-K choice by a small cost model over the tile shapes that measured best on
+  // MI355X: time ~ flops / (tile efficiency x edge utilisation x wave quantisation) + the cost of
+  // the split-K reduction pass. N = 576 (SmolLM2) is 3x192 = 6x96; dW has a 1536x576 output and
+  // K = 16384 rows, which only fills 256 CUs when K is split.
+  static const struct { int cfg; double eff; } cand[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
+  int cfg = 0, splits = 1;
+  {
+    const double flops = 2.0 * M * N * K * count;
+    const double t0 = flops / 125e12;                     // seconds at the best tile's asymptotic rate
+    double best = 1e30;
+    for (auto &c : cand) {
+      const TileCfg &tc = kTiles[c.cfg];
+      const int64_t tiles = cdiv(M, tc.bm) * cdiv(N, tc.bn);
+      const double util = (double)M * N / ((double)tiles * tc.bm * tc.bn);
+      for (int sp = 1; sp <= 64; sp *= 2) {
+        // split only when the output tiles alone cannot give every CU a workgroup
+        if (sp > 1 && (count > 1 || tiles >= ctx->num_cu || K / sp < 8 * tc.bk)) break;
+        const double waves = (double)tiles * sp * count / ctx->num_cu;
+        const double quant = waves >= 4 ? 1.0 : waves / ceil(waves);
+        // short K per workgroup pays the prologue/epilogue more: ~2 K-steps of overhead
+        const double ksteps = (double)K / sp / tc.bk;
+        const double depth = ksteps / (ksteps + 2.0);
+        double t = t0 / (c.eff * util * quant * depth);
+        if (sp > 1) t += ((double)(sp + 2) * M * N * 4.0) / 3.5e12 + 4e-6;
+        if (t < best) { best = t; cfg = c.cfg; splits = sp; }
+      }
     }
   }
+  if (ctx->opt_gemm_tile >= 0 && ctx->opt_gemm_tile < NCFG) cfg = ctx->opt_gemm_tile;
+  const int bm = kTiles[cfg].bm, bn = kTiles[cfg].bn, bk = kTiles[cfg].bk;
   if (count == 1 && ctx->opt_gemm_splitk >= 1) splits = ctx->opt_gemm_splitk;
   if (splits > 1) {
-    int64_t kc = cdiv(cdiv(K, splits), BK) * BK;
+    int64_t kc = cdiv(cdiv(K, splits), bk) * bk;
     splits = (int)cdiv(K, kc);
     a.kchunk = (int)kc;
   }
@@ -268,14 +286,22 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   }
   int zdim = splits > 1 ? splits : count;
   char label[32];
-  snprintf(label, sizeof label, "gemm.%s.%dx%d%s", kind == GT_NT ? "nt" : kind == GT_NN ? "nn" : "tn", bm, bn, splits > 1 ? ".splitk" : "");
+  snprintf(label, sizeof label, "gemm.%s.%dx%dx%d%s", kind == GT_NT ? "nt" : kind == GT_NN ? "nn" : "tn", bm, bn, bk, splits > 1 ? ".splitk" : "");
   ProfScope ps(ctx, label, 2.0 * M * N * K * count);
   int rc;
   switch (cfg) {
-    case 0: rc = launch_cfg<64, 64, 2, 2>(ctx, kind, vec, a, zdim); break;
-    case 1: rc = launch_cfg<128, 64, 2, 2>(ctx, kind, vec, a, zdim); break;
-    case 2: rc = launch_cfg<128, 128, 2, 2>(ctx, kind, vec, a, zdim); break;
-    default: rc = launch_cfg<128, 192, 2, 2>(ctx, kind, vec, a, zdim); break;
+    case 0: rc = launch_cfg<64, 64, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
+    case 1: rc = launch_cfg<128, 64, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
+    case 2: rc = launch_cfg<128, 128, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
+    case 3: rc = launch_cfg<128, 192, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
+    case 4: rc = launch_cfg<128, 96, 4, 1, 16>(ctx, kind, vec, a, zdim); break;
+    case 5: rc = launch_cfg<256, 128, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
+    case 6: rc = launch_cfg<128, 128, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
+    case 7: rc = launch_cfg<128, 192, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
+    case 8: rc = launch_cfg<128, 96, 4, 1, 32>(ctx, kind, vec, a, zdim); break;
+    case 9: rc = launch_cfg<256, 128, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
+    case 10: rc = launch_cfg<64, 192, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
+    default: rc = launch_cfg<128, 64, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
   }
   if (rc) return rc;
   if (splits > 1) {
