@@ -51,13 +51,13 @@ def zipf_tokens(vocab, n, seed, s=1.1):
 
 def cpu_baseline(seconds_hint=20.0):
     """The CPU oracle (a C restatement of the reference's CPU ops) on a bounded sample of the same workload:
-    one 256-token sequence through 2 of the 30 layers (forward + backward), the full tied readout + cross-entropy,
+    one 512-token sequence through 3 of the 30 layers (forward + backward), the full tied readout + cross-entropy,
     and AdamW over those parameters; the per-token time is extrapolated to 30 layers. OpenMP over the host cores
     where the loops write disjoint outputs (dW/dX as per-output dot products). Reported, never a target."""
     from oracle import ref
     cores = max(1, min(ref.max_threads(), len(os.sched_getaffinity(0))))
     ref.set_threads(cores)
-    T, L = 256, 2
+    T, L = 512, 3
     kw = dict(SMOLLM2)
     kw["layers"] = L
     rs = np.random.RandomState(0)
