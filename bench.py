@@ -101,6 +101,79 @@ def cpu_baseline(seconds_hint=20.0):
                       f"per-token time extrapolated to 30 layers; attention is O(T) per token so T=2048 would be slower"}
 
 
+def micro_kernels(gpu, L, reps=10):
+    """BASELINE configs[1]: the isolated backward kernels at the SmolLM2 MLP shape, timed with HIP events on the
+    library's stream. fp32 dX = dY.W and dW = dY^T.X with X [16384x576], W [1536x576], dY [16384x1536]; softmax-CE
+    backward over logits [16384x49152] with 10% of the targets masked; RMSNorm backward on [16384x576]; SwiGLU
+    backward on [16384x1536]. Rates are algorithmic work (FLOP, or bytes each tensor is touched once) over time."""
+    import ctypes as C
+    rs = np.random.RandomState(7)
+    R, H, F, V = 16384, 576, 1536, 49152
+
+    def dev(shape, scale=1.0, dtype=np.float32, data=None):
+        a = data if data is not None else (scale * rs.standard_normal(shape)).astype(dtype)
+        b = gpu.create_state_buffer(a.nbytes)
+        gpu.write_state_buffer(b, a)
+        return b
+
+    def zeros(n):
+        return gpu.create_state_buffer(4 * n)
+
+    X, W, dY = dev((R, H)), dev((F, H)), dev((R, F))
+    dX, dW = zeros(R * H), zeros(F * H)
+    gate, up, dgate, dup = dev((R, F)), dev((R, F)), zeros(R * F), zeros(R * F)
+    g_n, w_n, rinv, y_n, dx_n, dw_n = dev((R, H)), dev((H,)), zeros(R), zeros(R * H), zeros(R * H), zeros(H)
+    blk = (2.0 * rs.standard_normal(1 << 24)).astype(np.float32)
+    z = gpu.create_state_buffer(4 * R * V)
+    for off in range(0, 4 * R * V, blk.nbytes):
+        n = min(blk.nbytes, 4 * R * V - off)
+        L.check(gpu.ctx, L.lib.gt_h2d(gpu.ctx, z + off, blk.ctypes.data_as(C.c_void_p), n), "h2d")
+    dz = zeros(R * V)
+    tg = rs.randint(0, V, R).astype(np.int32)
+    tg[rs.rand(R) < 0.1] = -1
+    tgb = dev(None, data=tg)
+    inv = dev(None, data=np.array([1.0 / max(int((tg >= 0).sum()), 1)], np.float32))
+    loss, lse = zeros(1), zeros(R)
+    c, lib = gpu.ctx, L.lib
+    L.check(c, lib.gt_rmsnorm_fwd(c, R, H, 1e-5, X, w_n, y_n, rinv), "rmsnorm")
+    L.check(c, lib.gt_ce_fwd(c, R, V, R, z, tgb, inv, loss, lse), "ce")
+
+    def run():
+        L.check(c, lib.gt_gemm(c, L.NN, 0, R, H, F, dY, W, dX), "dX")
+        L.check(c, lib.gt_gemm(c, L.TN, 0, F, H, R, dY, X, dW), "dW")
+        L.check(c, lib.gt_ce_fwd(c, R, V, R, z, tgb, inv, loss, lse), "ce")
+        L.check(c, lib.gt_ce_bwd(c, R, V, R, z, tgb, inv, lse, 1.0, dz, 0), "ce.bwd")
+        L.check(c, lib.gt_rmsnorm_bwd(c, R, H, X, w_n, g_n, rinv, dx_n, 0, dw_n, 0), "rmsnorm.bwd")
+        L.check(c, lib.gt_glu_bwd(c, 0, R * F, dY, gate, up, dgate, 0, dup, 0), "glu.bwd")
+        # a plain streaming kernel of known size (read 100.7 MB, write 100.7 MB): the yardstick the FETCH_SIZE /
+        # WRITE_SIZE counters are scaled by
+        L.check(c, lib.gt_scale_fwd(c, R * F, gate, 1.0, dgate), "scale")
+
+    run()
+    gpu.start_profile("")
+    for _ in range(reps):
+        run()
+    prof = gpu.stop_profile()
+    out = {}
+    names = {"gemm.nn": ("dX = dY.W  [16384x576x1536]", "mfma"), "gemm.tn": ("dW = dY^T.X [1536x576x16384]", "mfma"),
+             "ce.bwd": ("softmax-CE backward [16384x49152]", "hbm"), "ce": ("CE forward statistics [16384x49152]", "hbm"),
+             "rmsnorm.bwd": ("RMSNorm backward [16384x576]", "hbm"), "glu.bwd": ("SwiGLU backward [16384x1536]", "hbm"),
+             "scale": ("copy-like yardstick: out = 1.0*x [16384x1536]", "hbm")}
+    for label, (ms, cnt, work) in prof.items():
+        key = next((k for k in sorted(names, key=len, reverse=True) if label == k or label.startswith(k + ".")), None)
+        if key is None or cnt == 0:
+            continue
+        desc, bound = names[key]
+        rate = work / (ms * 1e-3)
+        peak = PEAK_FP32_MFMA if bound == "mfma" else PEAK_HBM
+        out[desc] = {"kernel": label, "bound": bound, "us_per_launch": round(1e3 * ms / cnt, 1),
+                     "achieved": round(rate / 1e12, 3), "unit": "TFLOP/s" if bound == "mfma" else "TB/s",
+                     "frac": round(rate / peak, 4)}
+    for b in (X, W, dY, dX, dW, gate, up, dgate, dup, g_n, w_n, rinv, y_n, dx_n, dw_n, z, dz, tgb, inv, loss, lse):
+        L.check(c, lib.gt_free(c, b), "gt_free")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -108,6 +181,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
+    ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (BASELINE configs[1] shapes)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -161,8 +235,19 @@ def main():
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
         prof = gpu.stop_profile()
+        opt_prof = None
+        gpu.start_profile("adamw")           # the optimizer kernel alone, outside the timed region
+        step(total - 1)
+        opt_prof = gpu.stop_profile().get("adamw")
     finally:
         gpu.uninstall()
+    Lmod = importlib.import_module(f"{PKG}.lib")
+    kernels = None if a.no_micro else micro_kernels(gpu, Lmod)
+    if kernels is not None and opt_prof:
+        ms, cnt, work = opt_prof
+        kernels[f"AdamW step, {n_params} params, clip on"] = {
+            "kernel": "adamw", "bound": "hbm", "us_per_launch": round(1e3 * ms / cnt, 1),
+            "achieved": round(work / (ms * 1e-3) / 1e12, 3), "unit": "TB/s", "frac": round(work / (ms * 1e-3) / PEAK_HBM, 4)}
 
     tokens = a.steps * BATCH * SEQ
     # dominant kernel: the backward GEMMs (NN = dX, TN = dW); the one tile shape with the most time stands for it
@@ -192,6 +277,7 @@ def main():
                    "device": gpu.adapter_name},
         "loss_first": round(losses[0], 4), "loss_last": round(losses[-1], 4),
         "roofline": roof,
+        "kernels": kernels,
         "cpu_baseline": None if a.no_cpu else cpu_baseline(),
     }
     gpu.destroy()

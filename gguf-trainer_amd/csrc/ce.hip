@@ -30,12 +30,22 @@ __device__ __forceinline__ void row_stats(const float *__restrict__ zr, int n, f
   const bool vec = ((reinterpret_cast<uintptr_t>(zr) & 15) == 0);
   if (vec) {
     int n4 = n / 4;
-    for (int i = threadIdx.x; i < n4; i += 256) {
-      v4f z = reinterpret_cast<const v4f *>(zr)[i];
-      float mx = fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3]));
-      float mn = fmaxf(m, mx);
-      l = l * __expf(m - mn) + __expf(z[0] - mn) + __expf(z[1] - mn) + __expf(z[2] - mn) + __expf(z[3] - mn);
-      m = mn;
+    const v4f *z4 = reinterpret_cast<const v4f *>(zr);
+    for (int i0 = threadIdx.x; i0 < n4; i0 += 1024) {
+      v4f zz[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        int i = i0 + u * 256;
+        zz[u] = i < n4 ? __builtin_nontemporal_load(z4 + i) : v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      }
+      float mx = m;
+#pragma unroll
+      for (int u = 0; u < 4; u++) mx = fmaxf(mx, fmaxf(fmaxf(zz[u][0], zz[u][1]), fmaxf(zz[u][2], zz[u][3])));
+      float acc = l * __expf(m - mx);
+#pragma unroll
+      for (int u = 0; u < 4; u++) acc += __expf(zz[u][0] - mx) + __expf(zz[u][1] - mx) + __expf(zz[u][2] - mx) + __expf(zz[u][3] - mx);
+      l = (mx == -INFINITY) ? 0.f : acc;
+      m = mx;
     }
     for (int i = n4 * 4 + threadIdx.x; i < n; i += 256) online(m, l, zr[i]);
   } else {
@@ -81,7 +91,8 @@ __global__ __launch_bounds__(256) void ce_seq_loss(int T, const float *__restric
   if (threadIdx.x == 0) loss[s] = a * inv_denom[s];
 }
 
-// dz[row, :] (+)= seed*inv_denom[seq] * (exp(z - lse) - onehot). grid = (chunks of the row, rows)
+// dz[row, :] (+)= seed*inv_denom[seq] * (exp(z - lse) - onehot). grid = (rows, chunks of the row). Each thread keeps
+// four float4 loads in flight; z and dz are touched exactly once, so both use streaming (non-temporal) accesses.
 __global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, const float *__restrict__ z, const int *__restrict__ tgt,
                                                 const float *__restrict__ inv_denom, const float *__restrict__ lse,
                                                 float seed, float *dz, int acc) {
@@ -94,16 +105,30 @@ __global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, const float *__res
   float *dr = dz + row * V;
   const bool vec = (V % 4 == 0) && (((reinterpret_cast<uintptr_t>(zr) | reinterpret_cast<uintptr_t>(dr)) & 15) == 0);
   if (vec) {
-    int n4 = V / 4;
-    for (int i = blockIdx.y * 256 + threadIdx.x; i < n4; i += gridDim.y * 256) {
-      v4f o = {0, 0, 0, 0};
-      if (g != IGN) {
-        v4f zz = reinterpret_cast<const v4f *>(zr)[i];
+    const int n4 = V / 4;
+    const v4f *z4 = reinterpret_cast<const v4f *>(zr);
+    v4f *d4 = reinterpret_cast<v4f *>(dr);
+    const int stride = gridDim.y * 256;
+    for (int i0 = blockIdx.y * 256 + threadIdx.x; i0 < n4; i0 += 4 * stride) {
+      v4f zz[4], dd[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) o[j] = sc * (__expf(zz[j] - ls) - ((i * 4 + j) == g ? 1.f : 0.f));
+      for (int u = 0; u < 4; u++) {
+        int i = i0 + u * stride;
+        if (g != IGN && i < n4) zz[u] = __builtin_nontemporal_load(z4 + i);
+        if (acc && i < n4) dd[u] = d4[i];
       }
-      if (acc) o += reinterpret_cast<v4f *>(dr)[i];
-      reinterpret_cast<v4f *>(dr)[i] = o;
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        int i = i0 + u * stride;
+        if (i >= n4) continue;
+        v4f o = {0, 0, 0, 0};
+        if (g != IGN) {
+#pragma unroll
+          for (int j = 0; j < 4; j++) o[j] = sc * (__expf(zz[u][j] - ls) - ((i * 4 + j) == g ? 1.f : 0.f));
+        }
+        if (acc) o += dd[u];
+        __builtin_nontemporal_store(o, d4 + i);
+      }
     }
   } else {
     for (int i = blockIdx.y * 256 + threadIdx.x; i < V; i += gridDim.y * 256) {

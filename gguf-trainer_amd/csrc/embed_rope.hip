@@ -31,28 +31,36 @@ __global__ __launch_bounds__(256) void embedding_fwd_k(int rows, int d, const in
   }
 }
 
-// pos[t] = #{t' : id[t'] < id[t]} + #{t' < t : id[t'] == id[t]}: the stable sorted position.
-__global__ __launch_bounds__(256) void rank_ids_k(int n, const int *__restrict__ ids, int *__restrict__ order,
-                                                  int *__restrict__ sorted) {
+// pos[t] = #{t' : id[t'] < id[t]} + #{t' < t : id[t'] == id[t]}: the stable sorted position. The T x T compare is
+// split over blockIdx.y segments of the t' range; the per-segment counts are integers, so adding them into pos[]
+// with atomicAdd is exact and order-independent (the float sums further down never use atomics).
+__global__ __launch_bounds__(256) void rank_ids_k(int n, int seg, const int *__restrict__ ids, int *__restrict__ pos) {
   __shared__ int tile[256];
   int t = blockIdx.x * 256 + threadIdx.x;
   int mine = t < n ? ids[t] : 0x7fffffff;
-  int pos = 0;
-  for (int base = 0; base < n; base += 256) {
+  int cnt = 0;
+  int b0 = blockIdx.y * seg, b1 = min(n, b0 + seg);
+  for (int base = b0; base < b1; base += 256) {
     int j = base + threadIdx.x;
     __syncthreads();
-    tile[threadIdx.x] = j < n ? ids[j] : 0x7fffffff;
+    tile[threadIdx.x] = j < b1 ? ids[j] : 0x7fffffff;
     __syncthreads();
-    int lim = min(256, n - base);
+    int lim = min(256, b1 - base);
     for (int q = 0; q < lim; q++) {
       int o = tile[q];
-      pos += (o < mine) || (o == mine && base + q < t);
+      cnt += (o < mine) || (o == mine && base + q < t);
     }
   }
-  if (t < n) { order[pos] = t; sorted[pos] = mine; }
+  if (t < n && cnt) atomicAdd(pos + t, cnt);
+}
+__global__ __launch_bounds__(256) void scatter_ids_k(int n, const int *__restrict__ ids, const int *__restrict__ pos,
+                                                     int *__restrict__ order, int *__restrict__ sorted) {
+  int t = blockIdx.x * 256 + threadIdx.x;
+  if (t < n) { order[pos[t]] = t; sorted[pos[t]] = ids[t]; }
 }
 
-// one workgroup per sorted slot; only the first slot of each id does work
+// one workgroup per sorted slot; only the first slot of each id does work: it sums that id's gradient rows in
+// position order (eight row loads in flight per thread) and adds the sum to the id's dW row
 __global__ __launch_bounds__(256) void embedding_bwd_k(int n, int d, const int *__restrict__ order,
                                                        const int *__restrict__ sorted, const float *__restrict__ g,
                                                        float *dW) {
@@ -62,10 +70,26 @@ __global__ __launch_bounds__(256) void embedding_bwd_k(int n, int d, const int *
   int e = p + 1;
   while (e < n && sorted[e] == id) e++;
   float *dst = dW + (size_t)id * d;
-  for (int c = threadIdx.x; c < d; c += 256) {
-    float s = 0;
-    for (int q = p; q < e; q++) s += g[(size_t)order[q] * d + c];
-    dst[c] += s;
+  if (d % 4 == 0) {
+    for (int c = threadIdx.x; c < d / 4; c += 256) {
+      v4f s = {0, 0, 0, 0};
+      int q = p;
+      for (; q + 8 <= e; q += 8) {
+        v4f r[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) r[u] = reinterpret_cast<const v4f *>(g + (size_t)order[q + u] * d)[c];
+#pragma unroll
+        for (int u = 0; u < 8; u++) s += r[u];
+      }
+      for (; q < e; q++) s += reinterpret_cast<const v4f *>(g + (size_t)order[q] * d)[c];
+      reinterpret_cast<v4f *>(dst)[c] += s;
+    }
+  } else {
+    for (int c = threadIdx.x; c < d; c += 256) {
+      float s = 0;
+      for (int q = p; q < e; q++) s += g[(size_t)order[q] * d + c];
+      dst[c] += s;
+    }
   }
 }
 
@@ -121,10 +145,17 @@ int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, 
   ProfScope ps(ctx, "embedding.bwd", 8.0 * rows * d);
   if (!acc) GT_HIP(ctx, hipMemsetAsync(P<void>(dW), 0, (size_t)V * d * sizeof(float), ctx->stream));
   if (rows == 0) return 0;
+  GT_REQUIRE(ctx, (g | dW) % 16 == 0, "gt_embedding_bwd: buffers must be 16-byte aligned");
   void *ws;
-  if (gt_ws_reserve(ctx, (size_t)rows * 2 * sizeof(int), &ws)) return 1;
-  int *order = static_cast<int *>(ws), *sorted = order + rows;
-  hipLaunchKernelGGL(rank_ids_k, dim3((unsigned)cdiv(rows, 256)), dim3(256), 0, ctx->stream, rows, P<const int>(ids), order, sorted);
+  if (gt_ws_reserve(ctx, (size_t)rows * 3 * sizeof(int), &ws)) return 1;
+  int *order = static_cast<int *>(ws), *sorted = order + rows, *pos = sorted + rows;
+  GT_HIP(ctx, hipMemsetAsync(pos, 0, (size_t)rows * sizeof(int), ctx->stream));
+  const int nseg = (int)std::max<int64_t>(1, std::min<int64_t>(32, cdiv(rows, 1024)));
+  const int seg = (int)(cdiv(cdiv(rows, nseg), 256) * 256);
+  hipLaunchKernelGGL(rank_ids_k, dim3((unsigned)cdiv(rows, 256), (unsigned)cdiv(rows, seg)), dim3(256), 0, ctx->stream, rows, seg,
+                     P<const int>(ids), pos);
+  GT_LAUNCHED(ctx);
+  hipLaunchKernelGGL(scatter_ids_k, dim3((unsigned)cdiv(rows, 256)), dim3(256), 0, ctx->stream, rows, P<const int>(ids), pos, order, sorted);
   GT_LAUNCHED(ctx);
   hipLaunchKernelGGL(embedding_bwd_k, dim3((unsigned)rows), dim3(256), 0, ctx->stream, rows, d, order, sorted,
                      P<const float>(g), P<float>(dW));

@@ -74,33 +74,51 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const floa
     wv[j] = c < d4 ? reinterpret_cast<const v4f *>(w)[c] : v4f{0, 0, 0, 0};
     dwv[j] = v4f{0, 0, 0, 0};
   }
-  for (int64_t row = ((int64_t)blockIdx.x * 4 + wave) * RPW + sub; row < rows; row += (int64_t)gridDim.x * 4 * RPW) {
-    const v4f *xr = reinterpret_cast<const v4f *>(x + row * d);
-    const v4f *gr = reinterpret_cast<const v4f *>(g + row * d);
-    v4f xv[NJ], gv[NJ];
-    float S = 0;
+  // two rows of this lane group in flight: the loads of the second are issued before the first is reduced
+  const int64_t rstep = (int64_t)gridDim.x * 4 * RPW;
+  for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW + sub; row0 < rows; row0 += 2 * rstep) {
+    v4f xv[2][NJ], gv[2][NJ];
+    float S[2] = {0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < NJ; j++) {
-      int c = li + j * LPR;
-      bool in = c < d4;
-      xv[j] = in ? xr[c] : v4f{0, 0, 0, 0};
-      gv[j] = in ? gr[c] : v4f{0, 0, 0, 0};
-      v4f t = gv[j] * wv[j] * xv[j];
-      S += t[0] + t[1] + t[2] + t[3];
-    }
-    S = group_sum<LPR>(S);
-    const float r = rinv[row];
-    const float k2 = r * r * r * S * invd;
-    v4f *dxr = reinterpret_cast<v4f *>(dx + row * d);
+    for (int u = 0; u < 2; u++) {
+      const int64_t row = row0 + u * rstep;
+      const bool live = row < rows;
+      const v4f *xr = reinterpret_cast<const v4f *>(x + (live ? row : 0) * d);
+      const v4f *gr = reinterpret_cast<const v4f *>(g + (live ? row : 0) * d);
 #pragma unroll
-    for (int j = 0; j < NJ; j++) {
-      int c = li + j * LPR;
-      if (c < d4) {
-        v4f o = wv[j] * gv[j] * r - xv[j] * k2;
-        if (acc_dx) o += dxr[c];
-        dxr[c] = o;
+      for (int j = 0; j < NJ; j++) {
+        int c = li + j * LPR;
+        bool in = live && c < d4;
+        xv[u][j] = in ? xr[c] : v4f{0, 0, 0, 0};
+        gv[u][j] = in ? gr[c] : v4f{0, 0, 0, 0};
       }
-      dwv[j] += gv[j] * xv[j] * r;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+#pragma unroll
+      for (int j = 0; j < NJ; j++) {
+        v4f t = gv[u][j] * wv[j] * xv[u][j];
+        S[u] += t[0] + t[1] + t[2] + t[3];
+      }
+      S[u] = group_sum<LPR>(S[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int64_t row = row0 + u * rstep;
+      if (row >= rows) continue;
+      const float r = rinv[row];
+      const float k2 = r * r * r * S[u] * invd;
+      v4f *dxr = reinterpret_cast<v4f *>(dx + row * d);
+#pragma unroll
+      for (int j = 0; j < NJ; j++) {
+        int c = li + j * LPR;
+        if (c < d4) {
+          v4f o = wv[j] * gv[u][j] * r - xv[u][j] * k2;
+          if (acc_dx) o += dxr[c];
+          dxr[c] = o;
+        }
+        dwv[j] += gv[u][j] * xv[u][j] * r;
+      }
     }
   }
   if (!dw_part) return;

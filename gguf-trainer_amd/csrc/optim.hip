@@ -84,18 +84,33 @@ __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ 
   bool vec = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(m) | reinterpret_cast<uintptr_t>(v) |
                reinterpret_cast<uintptr_t>(g)) & 15) == 0;
   int n4 = vec ? c.len / 4 : 0;
-  for (int i = threadIdx.x; i < n4; i += 256) {
-    v4f gg = reinterpret_cast<const v4f *>(g)[i] * sc;
-    v4f mm = reinterpret_cast<v4f *>(m)[i], vv = reinterpret_cast<v4f *>(v)[i], ww = reinterpret_cast<v4f *>(w)[i];
+  // every array is touched once per step: streaming accesses, two float4 per array in flight
+  for (int i0 = threadIdx.x; i0 < n4; i0 += 512) {
+    v4f gg[2], mm[2], vv[2], ww[2];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      float tm = mm[j], tv = vv[j], tw = ww[j];
-      adam1(gg[j], tm, tv, tw, h);
-      mm[j] = tm; vv[j] = tv; ww[j] = tw;
+    for (int u = 0; u < 2; u++) {
+      int i = i0 + u * 256;
+      if (i < n4) {
+        gg[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(g) + i) * sc;
+        mm[u] = __builtin_nontemporal_load(reinterpret_cast<v4f *>(m) + i);
+        vv[u] = __builtin_nontemporal_load(reinterpret_cast<v4f *>(v) + i);
+        ww[u] = __builtin_nontemporal_load(reinterpret_cast<v4f *>(w) + i);
+      }
     }
-    reinterpret_cast<v4f *>(m)[i] = mm;
-    reinterpret_cast<v4f *>(v)[i] = vv;
-    reinterpret_cast<v4f *>(w)[i] = ww;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      int i = i0 + u * 256;
+      if (i >= n4) continue;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float tm = mm[u][j], tv = vv[u][j], tw = ww[u][j];
+        adam1(gg[u][j], tm, tv, tw, h);
+        mm[u][j] = tm; vv[u][j] = tv; ww[u][j] = tw;
+      }
+      __builtin_nontemporal_store(mm[u], reinterpret_cast<v4f *>(m) + i);
+      __builtin_nontemporal_store(vv[u], reinterpret_cast<v4f *>(v) + i);
+      reinterpret_cast<v4f *>(w)[i] = ww[u];           // the next forward reads the weights: keep them cacheable
+    }
   }
   for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) adam1(g[i] * sc, m[i], v[i], w[i], h);
 }
