@@ -28,6 +28,18 @@ PEAK_HBM = 8.0e12              # B/s
 SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                rope_base=100000.0, rms_eps=1e-5, tie=True)
 SEQ, BATCH = 2048, 8
+# The other model-sized BASELINE configs, runnable with --config (the default line is configs[3]).
+GEMMA3_95M = dict(arch="gemma3", vocab=32768, hidden=640, layers=12, heads=10, kv_heads=2, head_dim=64, ffn=2048,
+                  rope_base=1e6, rope_base_local=1e4, sliding_window=512, swa_pattern=6, rms_eps=1e-6, tie=True)
+QWEN3_06B = dict(arch="qwen3", vocab=151936, hidden=1024, layers=28, heads=16, kv_heads=8, head_dim=128, ffn=3072,
+                 rope_base=1e6, rms_eps=1e-6, tie=True)
+WORKLOADS = {
+    3: dict(name="configs[3]: SmolLM2-135M llama shape, fwd+bwd+AdamW, seq 2048 x batch 8, fp32", model=SMOLLM2, batch=8),
+    2: dict(name="configs[2]: Gemma3-style 95M, --recompute, Muon (5 NS steps) + AdamW, seq 2048 x batch 8, fp32",
+            model=GEMMA3_95M, batch=8, muon=True, recompute=True),
+    4: dict(name="configs[4]: Qwen3-0.6B shape, base frozen, LoRA rank 16 on q/k/v/o/gate/up/down + AdamW, 60% loss mask, "
+                 "seq 2048 x batch 4, fp32", model=QWEN3_06B, batch=4, lora=16, mask=0.6),
+}
 
 
 def synth_weights(arch, cfg, seed=0):
@@ -182,6 +194,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
     ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (BASELINE configs[1] shapes)")
+    ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS),
+                    help="index into BASELINE.json configs (default 3, the headline SmolLM2 shape)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -197,24 +211,48 @@ def main():
     arch = importlib.import_module(f"{PKG}.arch")
     optim = importlib.import_module(f"{PKG}.optim")
 
-    cfg = arch.ModelConfig(**SMOLLM2)
+    wl = WORKLOADS[a.config]
+    BATCH = wl["batch"]
+    cfg = arch.ModelConfig(**wl["model"])
     model = arch.Model(cfg, synth_weights(arch, cfg))
     n_params = sum(p.size for p in model.params())
     gpu = hb.require_gpu("bench.py")
-    opt = optim.AdamWHip(gpu, model.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
+    if wl.get("lora"):
+        rs = np.random.RandomState(3)
+        rank = wl["lora"]
+        adapters = {}
+        for l in range(cfg.layers):
+            for k in arch.MATRIX_KEYS:
+                outd, ind = arch.layer_shapes(cfg)[k]
+                adapters[f"L{l}.{k}"] = ((0.02 * rs.standard_normal((rank, ind))).astype(np.float32), np.zeros((outd, rank), np.float32))
+        trainable = arch.apply_lora(model, rank, 16.0, adapters)
+        opt = optim.AdamWHip(gpu, trainable, lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.0, clip=1.0)
+    elif wl.get("muon"):
+        mu, aux = model.param_groups()
+        opt = optim.MuonHip(gpu, mu, aux, lr=0.01, momentum=0.95, nesterov=True, ns_steps=5, aux={"lr": 3e-3})
+    else:
+        opt = optim.AdamWHip(gpu, model.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
+    ag.set_checkpointing(bool(wl.get("recompute")))
     total = a.steps + a.warmup
-    toks = [zipf_tokens(cfg.vocab, BATCH * (SEQ + 1), 100 + i).reshape(BATCH, SEQ + 1) for i in range(total)]
+    if a.config == 3:
+        toks = [zipf_tokens(cfg.vocab, BATCH * (SEQ + 1), 100 + i).reshape(BATCH, SEQ + 1) for i in range(total)]
+    else:
+        toks = [np.random.RandomState(100 + i).randint(0, cfg.vocab, (BATCH, SEQ + 1)).astype(np.int64) for i in range(total)]
+    masks = [np.random.RandomState(500 + i).rand(BATCH, SEQ) < wl["mask"] for i in range(total)] if wl.get("mask") else None
 
     def step(i):
         t = toks[i]
+        tgt = t[:, 1:].copy()
+        if masks is not None:
+            tgt[~masks[i]] = -1                 # loss mask: only the kept positions carry a target
         if a.sequential:
             losses = []
             for b in range(BATCH):
-                loss = arch.sequence_loss(model, t[b, :-1], t[b, 1:], 0)
+                loss = arch.sequence_loss(model, t[b, :-1], tgt[b], 0)
                 ag.backward(loss, 1.0 / BATCH)
                 losses.append(loss)
         else:
-            loss = arch.sequence_loss(model, t[:, :-1].reshape(-1), t[:, 1:].reshape(-1), 0, SEQ)
+            loss = arch.sequence_loss(model, t[:, :-1].reshape(-1), tgt.reshape(-1), 0, SEQ)
             ag.backward(loss, 1.0 / BATCH)
             losses = [loss]
         gpu.sync(losses)                     # loss scalars back to the host, as train-gpu.ts:221
@@ -236,14 +274,17 @@ def main():
         wall = time.perf_counter() - t0
         prof = gpu.stop_profile()
         opt_prof = None
-        gpu.start_profile("adamw")           # the optimizer kernel alone, outside the timed region
+        gpu.start_profile("adamw")           # the AdamW kernels alone, outside the timed region
         step(total - 1)
         opt_prof = gpu.stop_profile().get("adamw")
     finally:
         gpu.uninstall()
+        ag.set_checkpointing(False)
+        if wl.get("lora"):
+            arch.clear_lora(model)
     Lmod = importlib.import_module(f"{PKG}.lib")
     kernels = None if a.no_micro else micro_kernels(gpu, Lmod)
-    if kernels is not None and opt_prof:
+    if kernels is not None and opt_prof and a.config == 3:
         ms, cnt, work = opt_prof
         kernels[f"AdamW step, {n_params} params, clip on"] = {
             "kernel": "adamw", "bound": "hbm", "us_per_launch": round(1e3 * ms / cnt, 1),
@@ -267,11 +308,12 @@ def main():
                 "per_kernel": {k: {"TFLOP/s": round(v[2] / (v[0] * 1e-3) / 1e12, 2), "ms_per_step": round(v[0] / a.steps, 2),
                                    "launches_per_step": v[1] // a.steps} for k, v in sorted(prof.items())}}
     out = {
-        "metric": "train tokens/s (SmolLM2-135M shape, 2048x8); bwd GEMM % FP32 MFMA peak",
+        "metric": "train tokens/s (SmolLM2-135M shape, 2048x8); bwd GEMM % FP32 MFMA peak" if a.config == 3 else
+                  "train tokens/s (" + wl["name"].split(":")[0] + ")",
         "value": round(tokens / wall, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(1e3 * wall / a.steps, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic (weights N(0,0.02) random init, tokens Zipf(1.1) over the vocab)",
-        "config": {"workload": "configs[3]: SmolLM2-135M llama shape, fwd+bwd+AdamW, seq 2048 x batch 8, fp32",
+        "config": {"workload": wl["name"],
                    "params": n_params, "global_batch": BATCH, "seq_len": SEQ,
                    "graph": "sequential micro-batches" if a.sequential else "8 sequences stacked into one 16384-row graph",
                    "device": gpu.adapter_name},

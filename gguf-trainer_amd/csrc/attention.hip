@@ -12,7 +12,7 @@
 // probabilities go through LDS, and the value/key accumulation runs with lanes across head dims,
 // so global reads of K/V/Q/dO rows in that phase are contiguous. dK/dV sums over the query heads
 // of the group and over queries in a fixed order; nothing is atomic.
-// The MFMA kernels for hd = 64 / 128 live in attention_mfma.hip and take over when they apply.
+// The MFMA kernels for hd = 64 and 128 live in attention_mfma.hip and take over when they apply.
 #include <algorithm>
 #include "common.h"
 
@@ -212,10 +212,22 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
   }
 }
 
-int attn_mfma_supported(int hd);
-int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
-int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                  gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+// attention_mfma.hip, compiled once per head dim
+int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
+int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
+int attn_bwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
+                    gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+int attn_bwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
+                     gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+static int attn_mfma_supported(int hd) { return hd == 64 || hd == 128; }
+static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse) {
+  return p.hd == 64 ? attn_fwd_mfma64(ctx, p, q, k, v, out, lse) : attn_fwd_mfma128(ctx, p, q, k, v, out, lse);
+}
+static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
+                         float *part, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+  return p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dq, acc_q, dk, acc_k, dv, acc_v)
+                    : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dq, acc_q, dk, acc_k, dv, acc_v);
+}
 
 static int check(gt_ctx *ctx, const char *who, int B, int T, int Hq, int Hkv, int hd, int window) {
   GT_REQUIRE(ctx, B >= 1 && T >= 1 && Hq >= 1 && Hkv >= 1 && hd >= 1 && window >= 0, "%s: bad shape", who);

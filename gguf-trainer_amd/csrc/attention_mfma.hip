@@ -1,4 +1,5 @@
-// Attention forward / backward on the FP32 matrix cores (v_mfma_f32_32x32x2_f32) for head dim 64.
+// Attention forward / backward on the FP32 matrix cores (v_mfma_f32_32x32x2_f32). This file is compiled once per
+// supported head dim (-DHD=64, -DHD=128); the entry points carry the head dim in their names.
 // Same math and saved statistic as the generic kernels in attention.hip: causal / sliding window,
 // GQA, scores in the log2 domain, softmax recomputed in backward from lse2.
 //
@@ -40,9 +41,16 @@ struct AttnP {
   float scale;
 };
 
+#ifndef HD
+#error "compile with -DHD=64 or -DHD=128"
+#endif
+#define CAT_(a, b) a##b
+#define CAT(a, b) CAT_(a, b)
+#define FN(name) CAT(name, HD)
 #define NEG_BIG (-1.0e30f)
-#define HD 64
 #define LD (HD + 4)          // row-major tile stride
+
+namespace {                  // per-head-dim helpers: each translation unit has its own
 
 __device__ __forceinline__ int win_lo_m(int t, int window) { return (window > 0 && t + 1 > window) ? t + 1 - window : 0; }
 __device__ __forceinline__ int acc_row(int r, int g) { return 8 * (r / 4) + 4 * g + (r % 4); }
@@ -96,37 +104,47 @@ __device__ __forceinline__ void load_row_regs(float (&reg)[HD / 2], const float 
 }
 
 // acc = Tile(32 rows starting at `rows`) . reg^T : A = rows of the row-major tile, B = this lane's registers.
+// The LDS reads are issued eight b128 at a time, ahead of the MFMAs that consume them.
 __device__ __forceinline__ v16f rows_dot_regs(const float *rows, const float (&reg)[HD / 2], int l32, int g) {
-  v4f a[HD / 8];
-#pragma unroll
-  for (int j = 0; j < HD / 8; j++) a[j] = *reinterpret_cast<const v4f *>(rows + l32 * LD + 8 * j + 4 * g);
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
 #pragma unroll
-  for (int j = 0; j < HD / 8; j++)
+  for (int j0 = 0; j0 < HD / 8; j0 += 8) {
+    v4f a[8];
 #pragma unroll
-    for (int s = 0; s < 4; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][s], reg[4 * j + s], acc, 0, 0, 0);
+    for (int j = 0; j < 8; j++) a[j] = *reinterpret_cast<const v4f *>(rows + l32 * LD + 8 * (j0 + j) + 4 * g);
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+      for (int s = 0; s < 4; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][s], reg[4 * (j0 + j) + s], acc, 0, 0, 0);
+  }
   return acc;
 }
 
 // out[dt] += TileT(cols [col0, col0+32)) . w : A = the transposed tile (stride LDT), B = 16 accumulator-ordered weights
 template <int LDT>
 __device__ __forceinline__ void t_dot_acc(v16f (&out)[HD / 32], const float *ldst, int col0, const float (&w)[16], int l32, int g) {
-  v4f a[HD / 32][4];
+  constexpr int DT = HD / 32;
+  constexpr int QB = DT <= 2 ? 4 : 2;          // column chunks fetched ahead: 8 b128 reads in flight either way
 #pragma unroll
-  for (int dt = 0; dt < HD / 32; dt++)
+  for (int q0 = 0; q0 < 4; q0 += QB) {
+    v4f a[DT][QB];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      int d = dt * 32 + l32, chunk = (col0 >> 2) + 2 * q + g;
-      a[dt][q] = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * (chunk ^ ((d >> 3) & 7)));
-    }
+    for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-  for (int q = 0; q < 4; q++)
+      for (int q = 0; q < QB; q++) {
+        int d = dt * 32 + l32, chunk = (col0 >> 2) + 2 * (q0 + q) + g;
+        a[dt][q] = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * (chunk ^ ((d >> 3) & 7)));
+      }
 #pragma unroll
-    for (int s = 0; s < 4; s++)
+    for (int q = 0; q < QB; q++)
 #pragma unroll
-      for (int dt = 0; dt < HD / 32; dt++) out[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[dt][q][s], w[4 * q + s], out[dt], 0, 0, 0);
+      for (int s = 0; s < 4; s++)
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+          out[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[dt][q][s], w[4 * (q0 + q) + s], out[dt], 0, 0, 0);
+  }
 }
 
 __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32], int g, float mul, int add) {
@@ -141,10 +159,13 @@ __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32]
     }
 }
 
-#define KT 64      // keys per LDS stage in forward and dQ
+}  // namespace
+
+#define KT (HD == 64 ? 64 : 32)      // keys per LDS stage in forward and dQ
+#define NSUB (KT / 32)
 
 // ---- forward --------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+__global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, float *__restrict__ out,
                                                        float *__restrict__ lse) {
   using IO = TileIO<KT>;
@@ -191,14 +212,16 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__r
       IO::load(pv, vb, kstr, (kt + 1) * KT, p.T, tid);
     }
     if (tq0 >= p.T) continue;
-    float pr[2][16];
-    bool act[2];
+    float pr[NSUB][16];
+    bool act[NSUB];
+    bool any_act = false;
     float mx = NEG_BIG;
 #pragma unroll
-    for (int sub = 0; sub < 2; sub++) {
+    for (int sub = 0; sub < NSUB; sub++) {
       const int k0 = kt * KT + sub * 32;
       act[sub] = !(k0 > tq1 || k0 + 31 < wave_lo);           // wave-uniform: some (query, key) pair is visible
       if (!act[sub]) continue;
+      any_act = true;
       v16f s = rows_dot_regs(sK + sub * 32 * LD, qreg, l32, g);
       const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
       if (need_mask) {
@@ -214,7 +237,7 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__r
 #pragma unroll
       for (int r = 0; r < 16; r++) mx = fmaxf(mx, pr[sub][r]);
     }
-    if (!act[0] && !act[1]) continue;
+    if (!any_act) continue;
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     if (__any(mx > m)) {                                      // rare after the first tiles
       const float mn = fmaxf(m, mx);
@@ -227,7 +250,7 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__r
         for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
     }
 #pragma unroll
-    for (int sub = 0; sub < 2; sub++) {
+    for (int sub = 0; sub < NSUB; sub++) {
       if (!act[sub]) continue;
       float ls = 0.f;
 #pragma unroll
@@ -249,7 +272,7 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_k(AttnP p, const float *__r
 }
 
 // ---- dQ -----------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void attn_bwd_dq_mfma_k(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+__global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                           const float *__restrict__ v, const float *__restrict__ go,
                                                           const float *__restrict__ lse, const float *__restrict__ Dr,
                                                           float *dq, int acc_q) {
@@ -301,7 +324,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_mfma_k(AttnP p, const float *
     }
     if (tq0 >= p.T) continue;
 #pragma unroll
-    for (int sub = 0; sub < 2; sub++) {
+    for (int sub = 0; sub < NSUB; sub++) {
       const int k0 = kt * KT + sub * 32;
       if (k0 > tq1 || k0 + 31 < wave_lo) continue;
       v16f s = rows_dot_regs(sK + sub * 32 * LD, qreg, l32, g);
@@ -325,16 +348,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_mfma_k(AttnP p, const float *
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------
 #define QT 32      // queries per LDS stage in dK/dV
-__global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_k(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+__global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
                                                            float *dk, int acc_k, float *dv, int acc_v, float *part) {
   using IO = TileIO<QT>;
-  __shared__ __attribute__((aligned(16))) float sQ[QT * LD];
-  __shared__ __attribute__((aligned(16))) float sG[QT * LD];
-  __shared__ __attribute__((aligned(16))) float sQt[HD * IO::LDT];
-  __shared__ __attribute__((aligned(16))) float sGt[HD * IO::LDT];
-  __shared__ __attribute__((aligned(16))) float sL[QT], sD[QT];
+  extern __shared__ __attribute__((aligned(16))) float dkv_smem[];      // 35 KB at hd 64, 69 KB at hd 128
+  float *sQ = dkv_smem, *sG = sQ + QT * LD, *sQt = sG + QT * LD, *sGt = sQt + HD * IO::LDT;
+  float *sL = sGt + HD * IO::LDT, *sD = sL + QT;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
   // 1-D grid, key tile slowest: the first key tiles are seen by the most queries and go first. One workgroup
   // per QUERY head: with a kv group larger than one, each head's dK/dV goes to its own slice of the workspace
@@ -430,7 +451,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_k(AttnP p, const float 
 }
 
 // dk (+)= sum over the group's heads of their slices, in head order; same for dv
-__global__ __launch_bounds__(256) void attn_group_sum(const float *__restrict__ part, int group, size_t n4, float *dk, int acc_k,
+__global__ __launch_bounds__(256) void FN(attn_group_sum)(const float *__restrict__ part, int group, size_t n4, float *dk, int acc_k,
                                                       float *dv, int acc_v) {
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n4) return;
@@ -442,38 +463,44 @@ __global__ __launch_bounds__(256) void attn_group_sum(const float *__restrict__ 
   *ov = acc_v ? *ov + sv : sv;
 }
 
-int attn_mfma_supported(int hd) { return hd == HD; }
+#define DKV_SMEM ((2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT) * sizeof(float))
 
-int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse) {
+int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse) {
   GT_REQUIRE(ctx, (q | k | v | out) % 16 == 0, "attention: buffers must be 16-byte aligned");
   dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
-  hipLaunchKernelGGL(attn_fwd_mfma_k, grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
+  hipLaunchKernelGGL(FN(attn_fwd_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
                      P<const float>(v), P<float>(out), P<float>(lse));
   GT_LAUNCHED(ctx);
   return 0;
 }
 
 // Dr: the per-row sums D; part: workspace for the per-head dK/dV slices (2*group slices of B*T*Hkv*hd floats) or null
-int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                  gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
+                      float *part, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
   const int group = p.Hq / p.Hkv;
+  static bool smem_set = false;
+  if (!smem_set) {            // more than the 64 KB a kernel gets by default at hd 128
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+    smem_set = true;
+  }
   {
     ProfScope ps(ctx, "attention.bwd.dq");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
-    hipLaunchKernelGGL(attn_bwd_dq_mfma_k, grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
+    hipLaunchKernelGGL(FN(attn_bwd_dq_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
                        P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q);
     GT_LAUNCHED(ctx);
   }
   {
     ProfScope ps(ctx, "attention.bwd.dkv");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
-    hipLaunchKernelGGL(attn_bwd_dkv_mfma_k, grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
+    hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k), grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
                        P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part);
     GT_LAUNCHED(ctx);
     if (part) {
       size_t n4 = (size_t)p.B * p.T * p.Hkv * HD / 4;
-      hipLaunchKernelGGL(attn_group_sum, dim3((unsigned)cdiv((int64_t)n4, 256)), dim3(256), 0, ctx->stream, part, group, n4,
+      hipLaunchKernelGGL(FN(attn_group_sum), dim3((unsigned)cdiv((int64_t)n4, 256)), dim3(256), 0, ctx->stream, part, group, n4,
                          P<float>(dk), acc_k, P<float>(dv), acc_v);
       GT_LAUNCHED(ctx);
     }

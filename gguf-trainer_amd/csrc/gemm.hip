@@ -223,7 +223,8 @@ static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
 
 struct TileCfg { int bm, bn, bk; };
 static const TileCfg kTiles[] = {{64, 64, 16}, {128, 64, 16}, {128, 128, 16}, {128, 192, 16}, {128, 96, 16}, {256, 128, 16},
-                                 {128, 128, 32}, {128, 192, 32}, {128, 96, 32}, {256, 128, 32}, {64, 192, 16}, {128, 64, 32}};
+                                 {128, 128, 32}, {128, 192, 32}, {128, 96, 32}, {256, 128, 32}, {64, 192, 16}, {128, 64, 32},
+                                 {64, 576, 16}, {128, 576, 16}};
 #define NCFG ((int)(sizeof(kTiles) / sizeof(kTiles[0])))
 
 static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
@@ -247,13 +248,19 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   // MI355X: time ~ flops / (tile efficiency x edge utilisation x wave quantisation) + the cost of
   // the split-K reduction pass. N = 576 (SmolLM2) is 3x192 = 6x96; dW has a 1536x576 output and
   // K = 16384 rows, which only fills 256 CUs when K is split.
-  static const struct { int cfg; double eff; } cand[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
+  // relative tile efficiencies as measured; the TN kernel (both operands fetched with ds_read_b32) does best
+  // with the 4x1-wave 128x96 tile, the others with 128x192
+  struct Cand { int cfg; double eff; };
+  static const Cand cand_nn[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
+  static const Cand cand_tn[] = {{8, 1.00}, {10, 0.97}, {6, 0.90}, {7, 0.78}, {11, 0.80}, {0, 0.72}};
+  const Cand *cand = kind == GT_TN ? cand_tn : cand_nn;
   int cfg = 0, splits = 1;
   {
     const double flops = 2.0 * M * N * K * count;
     const double t0 = flops / 125e12;                     // seconds at the best tile's asymptotic rate
     double best = 1e30;
-    for (auto &c : cand) {
+    for (int ci = 0; ci < 6; ci++) {
+      const Cand &c = cand[ci];
       const TileCfg &tc = kTiles[c.cfg];
       const int64_t tiles = cdiv(M, tc.bm) * cdiv(N, tc.bn);
       const double util = (double)M * N / ((double)tiles * tc.bm * tc.bn);
@@ -301,7 +308,9 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
     case 8: rc = launch_cfg<128, 96, 4, 1, 32>(ctx, kind, vec, a, zdim); break;
     case 9: rc = launch_cfg<256, 128, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
     case 10: rc = launch_cfg<64, 192, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
-    default: rc = launch_cfg<128, 64, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
+    case 11: rc = launch_cfg<128, 64, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
+    case 12: rc = launch_cfg<64, 576, 2, 6, 16>(ctx, kind, vec, a, zdim); break;     // a whole 576-wide row panel per workgroup, 12 waves
+    default: rc = launch_cfg<128, 576, 4, 3, 16>(ctx, kind, vec, a, zdim); break;
   }
   if (rc) return rc;
   if (splits > 1) {
