@@ -194,6 +194,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
     ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (BASELINE configs[1] shapes)")
+    ap.add_argument("--profile-all", action="store_true",
+                    help="time every kernel label (not only the GEMMs) over the timed region and print the table to stderr")
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS),
                     help="index into BASELINE.json configs (default 3, the headline SmolLM2 shape)")
     a = ap.parse_args()
@@ -265,7 +267,7 @@ def main():
         losses = [step(i) for i in range(a.warmup)]
         gpu.sync([])
         torch.cuda.synchronize()
-        gpu.start_profile("gemm.")           # HIP events on the library's stream around every GEMM launch
+        gpu.start_profile("" if a.profile_all else "gemm.")   # HIP events on the library's stream around every GEMM launch
         t0 = time.perf_counter()
         for i in range(a.warmup, total):
             losses.append(step(i))
@@ -290,6 +292,10 @@ def main():
             "kernel": "adamw", "bound": "hbm", "us_per_launch": round(1e3 * ms / cnt, 1),
             "achieved": round(work / (ms * 1e-3) / 1e12, 3), "unit": "TB/s", "frac": round(work / (ms * 1e-3) / PEAK_HBM, 4)}
 
+    if a.profile_all:
+        print(f"{'label':30s} {'ms/step':>9s} {'launches/step':>14s} {'T(FLOP|B)/s':>12s}", file=sys.stderr)
+        for k, v in sorted(prof.items(), key=lambda kv: -kv[1][0]):
+            print(f"{k:30s} {v[0] / a.steps:9.2f} {v[1] / a.steps:14.1f} {v[2] / (v[0] * 1e-3) / 1e12 if v[0] else 0:12.2f}", file=sys.stderr)
     tokens = a.steps * BATCH * SEQ
     # dominant kernel: the backward GEMMs (NN = dX, TN = dW); the one tile shape with the most time stands for it
     bwd = {k: v for k, v in prof.items() if k.startswith("gemm.nn") or k.startswith("gemm.tn")}

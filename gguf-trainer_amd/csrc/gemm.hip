@@ -7,14 +7,14 @@
 // 16 accumulator VGPRs each. Global loads for step i+1 are issued into registers before the
 // MFMAs of step i and stored to LDS after them, so HBM/L2 latency hides under 32+ MFMAs.
 //
-// LDS layouts. An operand whose K index is contiguous in memory (A of NT/NN, B of NT) is kept as
-// [row][16+4]: the float4 read from global is written as one ds_write_b128 and a lane fetches its
-// MFMA inputs for four consecutive steps with one ds_read_b128 (row stride 20 words makes every
-// 8-lane group of a b128 read touch all 32 banks). An operand whose row index is contiguous
-// (A of TN, B of NN/TN) is kept as [k][rows] and fetched with ds_read_b32, consecutive lanes on
-// consecutive banks. Because an MFMA step consumes K pairs (lane/32 selects which), the order in
-// which K is consumed is free as long as A and B agree: inside every run of 8, lane group g takes
-// k = 4g + i at step i, which is what lets the b128 fetch feed four steps.
+// LDS layout. Every operand tile is kept as [row][BK+4] so that a lane fetches its MFMA inputs for
+// four consecutive steps with one ds_read_b128 (row stride = 4 mod 32 words makes every 8-lane
+// group of a b128 read touch all 32 banks). An operand whose K index is contiguous in memory
+// (A of NT/NN, B of NT) is copied float4 for float4; one whose row index is contiguous (A of TN,
+// B of NN/TN) is transposed on the way in (see Tile). Because an MFMA step consumes K pairs
+// (lane/32 selects which), the order in which K is consumed is free as long as A and B agree:
+// inside every run of 8, lane group g takes k = 4g + i at step i, which is what lets the b128
+// fetch feed four steps.
 //
 // dW has a small output and a long K (rows of the batch), so it is split along K over blockIdx.z
 // into per-split partial tiles in the workspace, summed in split order by a second kernel: no
@@ -41,16 +41,26 @@ struct GemmArgs {
   int nbm, nbn;
 };
 
-// One operand tile of R rows x 16 k. KC: k contiguous in memory (element (r,k) at p[r*ld + k]);
-// otherwise row contiguous (element (r,k) at p[k*ld + r]).
+// One operand tile of R rows x BKT k, kept in LDS as [row][BKT+4] with the 16-byte K chunks of a row XOR-swizzled by
+// (row/8) mod (BKT/4). KC: k contiguous in memory (element (r,k) at p[r*ld + k]), copied with one ds_write_b128 per
+// float4. Otherwise row contiguous (element (r,k) at p[k*ld + r]): eight lanes read one 128-byte line of a k-row and
+// each float4 is transposed into LDS with four scalar stores; the swizzle makes those stores hit 32 distinct banks per
+// half-wavefront. Either way the MFMA inputs of four consecutive steps come from one conflict-free ds_read_b128.
 template <int R, bool KC, bool VEC, int NT, int BKT>
 struct Tile {
   static constexpr int KS = BKT + 4;
-  static constexpr int KQ = BKT / 4;           // float4 units along K
+  static constexpr int KQ = BKT / 4;           // float4 chunks along K
   static constexpr int UNITS = R * KQ;         // float4 units per tile
   static constexpr int PER = (UNITS + NT - 1) / NT;   // per thread (the last round may be partial)
   static constexpr bool FULL = (UNITS % NT == 0);
-  static constexpr int LDS_WORDS = KC ? R * KS : BKT * R;
+  static constexpr int LDS_WORDS = R * KS;
+  static_assert(R % 32 == 0, "tile rows must be a multiple of 32");
+
+  // unit u of a row-contiguous tile: float4 column c4 (rows 4*c4..4*c4+3) at k-row kk
+  __device__ static __forceinline__ void rc_unit(int u, int &c4, int &kk) {
+    c4 = (u / (8 * BKT)) * 8 + (u & 7);
+    kk = (u >> 3) % BKT;
+  }
 
   // registers <- global, zero outside [0,Rtot) x [k0,kend)
   __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ p, int ld, int r0, int Rtot,
@@ -71,7 +81,9 @@ struct Tile {
           }
         }
       } else {
-        int k = k0 + u / (R / 4), r = r0 + (u % (R / 4)) * 4;
+        int c4, kk;
+        rc_unit(u, c4, kk);
+        int k = k0 + kk, r = r0 + c4 * 4;
         if (k < kend) {
           const float *q = p + (size_t)k * ld + r;
           if (VEC) { if (r < Rtot) v = *reinterpret_cast<const v4f *>(q); }
@@ -89,18 +101,23 @@ struct Tile {
     for (int i = 0; i < PER; i++) {
       int u = tid + i * NT;
       if (!FULL && u >= UNITS) continue;
-      if (KC) *reinterpret_cast<v4f *>(lds + (u / KQ) * KS + (u % KQ) * 4) = reg[i];
-      else *reinterpret_cast<v4f *>(lds + (u / (R / 4)) * R + (u % (R / 4)) * 4) = reg[i];
+      if (KC) {
+        int row = u / KQ, chunk = u % KQ;
+        *reinterpret_cast<v4f *>(lds + row * KS + 4 * (chunk ^ ((row >> 3) & (KQ - 1)))) = reg[i];
+      } else {
+        int c4, kk;
+        rc_unit(u, c4, kk);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          int row = c4 * 4 + j;
+          lds[row * KS + 4 * ((kk >> 2) ^ ((row >> 3) & (KQ - 1))) + (kk & 3)] = reg[i][j];
+        }
+      }
     }
   }
   // MFMA inputs of this lane for the four steps of K-run c (0 .. BKT/8-1): row = tile row, g = lane/32
   __device__ static __forceinline__ v4f fetch(const float *lds, int row, int c, int g) {
-    if (KC) return *reinterpret_cast<const v4f *>(lds + row * KS + c * 8 + g * 4);
-    v4f v;
-    const float *q = lds + (c * 8 + g * 4) * R + row;
-#pragma unroll
-    for (int j = 0; j < 4; j++) v[j] = q[j * R];
-    return v;
+    return *reinterpret_cast<const v4f *>(lds + row * KS + 4 * ((2 * c + g) ^ ((row >> 3) & (KQ - 1))));
   }
 };
 

@@ -116,48 +116,64 @@ __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ 
 }
 
 // ---- Muon -------------------------------------------------------------------------------------------
+// Matrices of equal shape form a group that is stepped as one batch: every elementwise stage runs over the
+// group's concatenated work buffers (blockIdx.y = matrix), and each Newton-Schulz product is one batched GEMM
+// launch. A 12-layer model with four distinct projection shapes takes 4 x 29 launches per step instead of
+// 84 x 29.
 
-struct MuonMat { float *w, *g, *buf; int rows, cols; };
+struct MuonGroup {
+  int rows, cols, count;
+  float **w = nullptr, **g = nullptr, **buf = nullptr;          // device tables of per-matrix pointers
+  float *U = nullptr, *X = nullptr, *A = nullptr, *AA = nullptr, *BX = nullptr, *part = nullptr;
+  size_t bytes = 0;
+};
 struct gt_muon {
-  std::vector<MuonMat> mats;
+  std::vector<MuonGroup> groups;
   float momentum; int nesterov, ns_steps;
-  float *U = nullptr, *X = nullptr, *A = nullptr, *AA = nullptr, *BX = nullptr, *part = nullptr;   // sized for the largest matrix
-  size_t max_elems = 0, max_r = 0;
 };
 
 #define NS_A 3.4445f
 #define NS_B (-4.7750f)
 #define NS_C 2.0315f
-#define RED_BLOCKS 256
+#define RED_BLOCKS 64
 
-// buf = mu*buf + g; U = nesterov ? g + mu*buf : buf; per-workgroup sum of U^2 (muon-gpu.ts:51-92)
-__global__ __launch_bounds__(256) void muon_momentum_k(int64_t n, const float *__restrict__ g, float *buf, float *__restrict__ U,
-                                                       float mu, int nesterov, float *__restrict__ part) {
+// buf = mu*buf + g; U = nesterov ? g + mu*buf : buf; per-workgroup sum of U^2 (muon-gpu.ts:51-92).
+// With null tables (Newton-Schulz on a caller's matrix) U is only read.
+__global__ __launch_bounds__(256) void muon_momentum_k(int64_t n, float *const *__restrict__ gt, float *const *__restrict__ bt,
+                                                       float *__restrict__ Uall, float mu, int nesterov, float *__restrict__ part) {
   __shared__ float sm[4];
+  const int mi = blockIdx.y;
+  float *U = Uall + (size_t)mi * n;
+  const float *g = gt ? gt[mi] : nullptr;
+  float *buf = bt ? bt[mi] : nullptr;
   float s = 0;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    float gi = g ? g[i] : 0.f;
-    float b = buf ? mu * buf[i] + gi : gi;
-    if (buf) buf[i] = b;
-    float u = (buf && nesterov) ? gi + mu * b : b;
-    if (!buf) u = U[i];
-    else U[i] = u;
+    float u;
+    if (buf) {
+      float gi = g[i];
+      float b = mu * buf[i] + gi;
+      buf[i] = b;
+      u = nesterov ? gi + mu * b : b;
+      U[i] = u;
+    } else u = U[i];
     s += u * u;
   }
   s = block_sum<4>(s, sm);
-  if (threadIdx.x == 0) part[blockIdx.x] = s;
+  if (threadIdx.x == 0) part[(size_t)mi * gridDim.x + blockIdx.x] = s;
 }
 // X = (flip ? U^T : U) / (sqrt(sum part) + 1e-7); U is [m,n], X is [r,c] with r = min(m,n)
-__global__ __launch_bounds__(256) void muon_normalize_k(int m, int n, int flip, const float *__restrict__ U,
-                                                        const float *__restrict__ part, int nparts, float *__restrict__ X) {
+__global__ __launch_bounds__(256) void muon_normalize_k(int m, int n, int flip, const float *__restrict__ Uall,
+                                                        const float *__restrict__ part, int nparts, float *__restrict__ Xall) {
   __shared__ float sm[4];
+  const int mi = blockIdx.y;
+  const int64_t total = (int64_t)m * n;
+  const float *U = Uall + (size_t)mi * total;
+  float *X = Xall + (size_t)mi * total;
   float s = 0;
-  for (int i = threadIdx.x; i < nparts; i += 256) s += part[i];
+  for (int i = threadIdx.x; i < nparts; i += 256) s += part[(size_t)mi * nparts + i];
   s = block_sum<4>(s, sm);
   const float inv = 1.0f / (sqrtf(s) + 1e-7f);
-  int64_t total = (int64_t)m * n;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    // i indexes X row-major [r,c]
     float u;
     if (flip) { int64_t xr = i / m, xc = i % m; u = U[xc * n + xr]; }   // X[xr,xc] = U[xc,xr], X is [n,m]
     else u = U[i];
@@ -170,9 +186,13 @@ __global__ __launch_bounds__(256) void muon_combine_a_k(int64_t n, float *A, con
 __global__ __launch_bounds__(256) void muon_combine_x_k(int64_t n, float *X, const float *__restrict__ BX) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) X[i] = NS_A * X[i] + BX[i];
 }
-// W[m,n] -= f * (flip ? X^T : X)
-__global__ __launch_bounds__(256) void muon_apply_k(int m, int n, int flip, float *W, const float *__restrict__ X, float f) {
-  int64_t total = (int64_t)m * n;
+// W[m,n] -= f * (flip ? X^T : X), one matrix per blockIdx.y
+__global__ __launch_bounds__(256) void muon_apply_k(int m, int n, int flip, float *const *__restrict__ wt, float *Wone,
+                                                    const float *__restrict__ Xall, float f) {
+  const int mi = blockIdx.y;
+  const int64_t total = (int64_t)m * n;
+  float *W = wt ? wt[mi] : Wone;
+  const float *X = Xall + (size_t)mi * total;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     float x;
     if (flip) { int64_t wr = i / n, wc = i % n; x = X[wc * m + wr]; }    // X is [n,m]
@@ -183,42 +203,46 @@ __global__ __launch_bounds__(256) void muon_apply_k(int m, int n, int flip, floa
 
 static inline unsigned sgrid(gt_ctx *ctx, int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>(cdiv(n, 256), (int64_t)ctx->num_cu * 8)); }
 
-// Leaves NS(U) in X ([r,c]); U already holds the input, part its per-workgroup sums of squares.
-static int newton_schulz_run(gt_ctx *ctx, int m, int n, int steps, float *U, float *X, float *A, float *AA, float *BX,
-                             float *part, int nparts) {
-  int flip = m > n;
-  int r = flip ? n : m, c = flip ? m : n;
-  int64_t size = (int64_t)m * n;
-  hipLaunchKernelGGL(muon_normalize_k, dim3(sgrid(ctx, size)), dim3(256), 0, ctx->stream, m, n, flip, U, part, nparts, X);
+// Leaves NS(U) in X ([count][r,c]); U holds the inputs, part their per-workgroup sums of squares.
+static int newton_schulz_run(gt_ctx *ctx, const MuonGroup &G, int steps, int nparts) {
+  const int m = G.rows, n = G.cols, cnt = G.count;
+  const int flip = m > n;
+  const int r = flip ? n : m, c = flip ? m : n;
+  const int64_t size = (int64_t)m * n, rr = (int64_t)r * r;
+  hipLaunchKernelGGL(muon_normalize_k, dim3(sgrid(ctx, size), cnt), dim3(256), 0, ctx->stream, m, n, flip, G.U, G.part, nparts, G.X);
   GT_LAUNCHED(ctx);
-  gt_buf bX = reinterpret_cast<gt_buf>(X), bA = reinterpret_cast<gt_buf>(A), bAA = reinterpret_cast<gt_buf>(AA), bBX = reinterpret_cast<gt_buf>(BX);
+  gt_buf bX = reinterpret_cast<gt_buf>(G.X), bA = reinterpret_cast<gt_buf>(G.A), bAA = reinterpret_cast<gt_buf>(G.AA), bBX = reinterpret_cast<gt_buf>(G.BX);
   for (int s = 0; s < steps; s++) {
-    if (gt_gemm(ctx, GT_NT, 0, r, r, c, bX, bX, bA)) return 1;          // A = X X^T
-    if (gt_gemm(ctx, GT_NN, 0, r, r, r, bA, bA, bAA)) return 1;         // AA = A^2
-    hipLaunchKernelGGL(muon_combine_a_k, dim3(sgrid(ctx, (int64_t)r * r)), dim3(256), 0, ctx->stream, (int64_t)r * r, A, AA);
+    if (gt_gemm_batched(ctx, GT_NT, 0, r, r, c, bX, size, bX, size, bA, rr, cnt)) return 1;       // A = X X^T
+    if (gt_gemm_batched(ctx, GT_NN, 0, r, r, r, bA, rr, bA, rr, bAA, rr, cnt)) return 1;         // AA = A^2
+    hipLaunchKernelGGL(muon_combine_a_k, dim3(sgrid(ctx, rr * cnt)), dim3(256), 0, ctx->stream, rr * cnt, G.A, G.AA);
     GT_LAUNCHED(ctx);
-    if (gt_gemm(ctx, GT_NN, 0, r, c, r, bA, bX, bBX)) return 1;         // BX = (bA + cA^2) X
-    hipLaunchKernelGGL(muon_combine_x_k, dim3(sgrid(ctx, size)), dim3(256), 0, ctx->stream, size, X, BX);
+    if (gt_gemm_batched(ctx, GT_NN, 0, r, c, r, bA, rr, bX, size, bBX, size, cnt)) return 1;     // BX = (bA + cA^2) X
+    hipLaunchKernelGGL(muon_combine_x_k, dim3(sgrid(ctx, size * cnt)), dim3(256), 0, ctx->stream, size * cnt, G.X, G.BX);
     GT_LAUNCHED(ctx);
   }
   return 0;
 }
 
-static int muon_alloc(gt_ctx *ctx, gt_muon *o, size_t elems, size_t r) {
-  GT_HIP(ctx, hipMalloc((void **)&o->U, elems * 4));
-  GT_HIP(ctx, hipMalloc((void **)&o->X, elems * 4));
-  GT_HIP(ctx, hipMalloc((void **)&o->BX, elems * 4));
-  GT_HIP(ctx, hipMalloc((void **)&o->A, r * r * 4));
-  GT_HIP(ctx, hipMalloc((void **)&o->AA, r * r * 4));
-  GT_HIP(ctx, hipMalloc((void **)&o->part, RED_BLOCKS * 4));
-  ctx->live_bytes += elems * 12 + r * r * 8 + RED_BLOCKS * 4;
-  o->max_elems = elems; o->max_r = r;
+static int group_alloc(gt_ctx *ctx, MuonGroup &G) {
+  const size_t elems = (size_t)G.rows * G.cols * G.count, r = std::min(G.rows, G.cols);
+  GT_HIP(ctx, hipMalloc((void **)&G.U, elems * 4));
+  GT_HIP(ctx, hipMalloc((void **)&G.X, elems * 4));
+  GT_HIP(ctx, hipMalloc((void **)&G.BX, elems * 4));
+  GT_HIP(ctx, hipMalloc((void **)&G.A, r * r * G.count * 4));
+  GT_HIP(ctx, hipMalloc((void **)&G.AA, r * r * G.count * 4));
+  GT_HIP(ctx, hipMalloc((void **)&G.part, (size_t)RED_BLOCKS * G.count * 4));
+  G.bytes = elems * 12 + r * r * G.count * 8 + (size_t)RED_BLOCKS * G.count * 4;
+  ctx->live_bytes += G.bytes;
   return 0;
 }
-static void muon_release(gt_ctx *ctx, gt_muon *o) {
-  hipStreamSynchronize(ctx->stream);
-  hipFree(o->U); hipFree(o->X); hipFree(o->BX); hipFree(o->A); hipFree(o->AA); hipFree(o->part);
-  ctx->live_bytes -= o->max_elems * 12 + o->max_r * o->max_r * 8 + RED_BLOCKS * 4;
+static void group_release(gt_ctx *ctx, MuonGroup &G) {
+  (void)hipStreamSynchronize(ctx->stream);
+  (void)hipFree(G.U); (void)hipFree(G.X); (void)hipFree(G.BX); (void)hipFree(G.A); (void)hipFree(G.AA); (void)hipFree(G.part);
+  if (G.w) (void)hipFree(G.w);
+  if (G.g) (void)hipFree(G.g);
+  if (G.buf) (void)hipFree(G.buf);
+  ctx->live_bytes -= G.bytes;
 }
 
 extern "C" {
@@ -296,16 +320,34 @@ int gt_muon_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const g
                    double momentum, int nesterov, int ns_steps, gt_muon **out) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, n >= 0 && out && ns_steps >= 0 && (n == 0 || (w && g && buf && rows && cols)), "gt_muon_create: bad arguments");
+  for (int i = 0; i < n; i++)
+    GT_REQUIRE(ctx, w[i] && g[i] && buf[i] && rows[i] >= 1 && cols[i] >= 1, "gt_muon_create: matrix %d is malformed", i);
   gt_muon *o = new gt_muon();
   o->momentum = (float)momentum; o->nesterov = nesterov; o->ns_steps = ns_steps;
-  size_t me = 1, mr = 1;
+  std::vector<char> placed(n, 0);
   for (int i = 0; i < n; i++) {
-    if (!(w[i] && g[i] && buf[i] && rows[i] >= 1 && cols[i] >= 1)) { delete o; GT_FAIL(ctx, "gt_muon_create: matrix %d is malformed", i); }
-    o->mats.push_back({P<float>(w[i]), P<float>(g[i]), P<float>(buf[i]), rows[i], cols[i]});
-    me = std::max(me, (size_t)rows[i] * cols[i]);
-    mr = std::max(mr, (size_t)std::min(rows[i], cols[i]));
+    if (placed[i]) continue;
+    MuonGroup G;
+    G.rows = rows[i]; G.cols = cols[i];
+    std::vector<float *> pw, pg, pb;
+    for (int j = i; j < n; j++)
+      if (!placed[j] && rows[j] == G.rows && cols[j] == G.cols) {
+        placed[j] = 1;
+        pw.push_back(P<float>(w[j])); pg.push_back(P<float>(g[j])); pb.push_back(P<float>(buf[j]));
+      }
+    G.count = (int)pw.size();
+    size_t tb = pw.size() * sizeof(float *);
+    if (hipMalloc((void **)&G.w, tb) != hipSuccess || hipMalloc((void **)&G.g, tb) != hipSuccess ||
+        hipMalloc((void **)&G.buf, tb) != hipSuccess || group_alloc(ctx, G)) {
+      for (auto &gg : o->groups) group_release(ctx, gg);
+      delete o;
+      GT_FAIL(ctx, "gt_muon_create: out of device memory for the %dx%d group", G.rows, G.cols);
+    }
+    (void)hipMemcpy(G.w, pw.data(), tb, hipMemcpyHostToDevice);
+    (void)hipMemcpy(G.g, pg.data(), tb, hipMemcpyHostToDevice);
+    (void)hipMemcpy(G.buf, pb.data(), tb, hipMemcpyHostToDevice);
+    o->groups.push_back(G);
   }
-  if (muon_alloc(ctx, o, me, mr)) { delete o; return 1; }
   *out = o;
   return 0;
 }
@@ -314,15 +356,15 @@ int gt_muon_step(gt_ctx *ctx, gt_muon *o, double lr) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, o, "gt_muon_step: null optimizer");
   ProfScope ps(ctx, "muon");
-  for (auto &mt : o->mats) {
-    int64_t size = (int64_t)mt.rows * mt.cols;
-    unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv(size, 256));
-    hipLaunchKernelGGL(muon_momentum_k, dim3(nb), dim3(256), 0, ctx->stream, size, mt.g, mt.buf, o->U, o->momentum, o->nesterov, o->part);
+  for (auto &G : o->groups) {
+    const int64_t size = (int64_t)G.rows * G.cols;
+    const unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv(size, 256));
+    hipLaunchKernelGGL(muon_momentum_k, dim3(nb, G.count), dim3(256), 0, ctx->stream, size, G.g, G.buf, G.U, o->momentum, o->nesterov, G.part);
     GT_LAUNCHED(ctx);
-    if (newton_schulz_run(ctx, mt.rows, mt.cols, o->ns_steps, o->U, o->X, o->A, o->AA, o->BX, o->part, (int)nb)) return 1;
-    float f = (float)(lr * sqrt(std::max(1.0, (double)mt.rows / (double)mt.cols)));
-    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, size)), dim3(256), 0, ctx->stream, mt.rows, mt.cols, mt.rows > mt.cols ? 1 : 0,
-                       mt.w, o->X, f);
+    if (newton_schulz_run(ctx, G, o->ns_steps, (int)nb)) return 1;
+    const float f = (float)(lr * sqrt(std::max(1.0, (double)G.rows / (double)G.cols)));
+    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, size), G.count), dim3(256), 0, ctx->stream, G.rows, G.cols, G.rows > G.cols ? 1 : 0,
+                       G.w, (float *)nullptr, G.X, f);
     GT_LAUNCHED(ctx);
   }
   return 0;
@@ -331,7 +373,7 @@ int gt_muon_step(gt_ctx *ctx, gt_muon *o, double lr) {
 int gt_muon_destroy(gt_ctx *ctx, gt_muon *o) {
   GT_ENTER(ctx);
   if (!o) return 0;
-  muon_release(ctx, o);
+  for (auto &G : o->groups) group_release(ctx, G);
   delete o;
   return 0;
 }
@@ -340,23 +382,24 @@ int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out)
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, m >= 1 && n >= 1 && steps >= 0 && G && out, "gt_newton_schulz: bad arguments");
   ProfScope ps(ctx, "muon");
-  gt_muon tmp;
-  size_t size = (size_t)m * n;
-  if (muon_alloc(ctx, &tmp, size, (size_t)std::min(m, n))) return 1;
-  GT_HIP(ctx, hipMemcpyAsync(tmp.U, P<void>(G), size * 4, hipMemcpyDeviceToDevice, ctx->stream));
-  unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv((int64_t)size, 256));
+  MuonGroup T;
+  T.rows = m; T.cols = n; T.count = 1;
+  if (group_alloc(ctx, T)) return 1;
+  const size_t size = (size_t)m * n;
+  GT_HIP(ctx, hipMemcpyAsync(T.U, P<void>(G), size * 4, hipMemcpyDeviceToDevice, ctx->stream));
+  const unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv((int64_t)size, 256));
   // sums of squares of U only (no momentum buffer, no gradient)
-  hipLaunchKernelGGL(muon_momentum_k, dim3(nb), dim3(256), 0, ctx->stream, (int64_t)size, (const float *)nullptr, (float *)nullptr,
-                     tmp.U, 0.f, 0, tmp.part);
-  GT_LAUNCHED(ctx);
-  int rc = newton_schulz_run(ctx, m, n, steps, tmp.U, tmp.X, tmp.A, tmp.AA, tmp.BX, tmp.part, (int)nb);
+  hipLaunchKernelGGL(muon_momentum_k, dim3(nb, 1), dim3(256), 0, ctx->stream, (int64_t)size, (float *const *)nullptr,
+                     (float *const *)nullptr, T.U, 0.f, 0, T.part);
+  int rc = hipGetLastError() != hipSuccess;
+  if (!rc) rc = newton_schulz_run(ctx, T, steps, (int)nb);
   if (!rc) {
-    // out = 0 - (-1) * X(^T): reuse the apply kernel on a cleared destination
-    hipMemsetAsync(P<void>(out), 0, size * 4, ctx->stream);
-    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, (int64_t)size)), dim3(256), 0, ctx->stream, m, n, m > n ? 1 : 0, P<float>(out),
-                       tmp.X, -1.0f);
+    // out = 0 - (-1) * X(^T): the apply kernel on a cleared destination
+    (void)hipMemsetAsync(P<void>(out), 0, size * 4, ctx->stream);
+    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, (int64_t)size), 1), dim3(256), 0, ctx->stream, m, n, m > n ? 1 : 0,
+                       (float *const *)nullptr, P<float>(out), T.X, -1.0f);
   }
-  muon_release(ctx, &tmp);
+  group_release(ctx, T);
   return rc;
 }
 }
