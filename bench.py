@@ -24,6 +24,11 @@ PKG = "gguf-trainer_amd"
 
 PEAK_FP32_MFMA = 157.3e12      # MI355X dense FP32 matrix peak, FLOP/s
 PEAK_HBM = 8.0e12              # B/s
+# L2-miss traffic per launch (bytes) of the two backward GEMM kernels that lead the step, from two rocprofv3 --pmc
+# passes over this file (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the factors read off a plain streaming kernel of known
+# size; see profiles/bench_smollm2_135m_pmc_fetch_write.txt). Averages over the shapes each kernel serves in the step.
+MEASURED_TRAFFIC = {"gemm.tn.128x96x32.splitk": (2 * 232740.1 + 55296.0) * 1024,
+                    "gemm.nn.128x96x32": (2 * 195844.0 + 36864.0) * 1024}
 
 SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                rope_base=100000.0, rms_eps=1e-5, tie=True)
@@ -307,7 +312,8 @@ def main():
         all_ms = sum(v[0] for v in bwd.values())
         all_work = sum(v[2] for v in bwd.values())
         roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach / 1e12, 3), "peak": PEAK_FP32_MFMA / 1e12,
-                "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA, 4),
+                "traffic": MEASURED_TRAFFIC.get(dom) if a.config == 3 else None,
                 "launches": int(cnt), "avg_launch_ms": round(ms / cnt, 4),
                 "all_bwd_gemms": {"achieved": round(all_work / (all_ms * 1e-3) / 1e12, 3), "ms_per_step": round(all_ms / a.steps, 2),
                                   "frac": round(all_work / (all_ms * 1e-3) / PEAK_FP32_MFMA, 4)},

@@ -14,8 +14,10 @@
  *   - "acc" arguments: 0 = the kernel stores its result (the destination need not be cleared),
  *     1 = it adds to what the destination holds. The reference zeroes every gradient buffer and
  *     always adds (src/backend/webgpu.ts:21-26, 1397-1429); a host that knows a gradient's first
- *     writer can skip both the clear and the read. No kernel uses atomics: one thread owns one
- *     output element and every reduction has a fixed order, so results are run-to-run identical.
+ *     writer can skip both the clear and the read. No kernel uses floating-point atomics: one
+ *     thread owns one output element and every float reduction has a fixed order, so results
+ *     are run-to-run identical (the one integer atomicAdd, in the embedding id ranking, is exact
+ *     in any order).
  *   - rows-batched extension: where the reference runs one sequence of T rows per call, these take
  *     `rows` (= B*T, sequences stacked) plus what per-sequence structure the op needs (T for
  *     positions, B for attention, one denominator per sequence for the loss). B = 1 is the

@@ -207,3 +207,53 @@ def test_config1_tiny_llama_step(gpu, ref):
     for n, p in rmodel.named_params():
         assert_close(model.p[n].data, p.data, f"config 1 weight after AdamW {n}", rel_l2=1e-4, max_rel=5e-3)
     assert gpu.grad_clears_issued < 400          # first-writer stores: no per-node gradient clears
+
+
+def test_device_behaviour_gates(gpu, ref):
+    """gpu-parity.ts:1363-2028: after warm-up a device-resident step reads back the loss scalars only, issues no
+    gradient clears, stops allocating (the pool plateaus), and a stacked step uses B times fewer launches' worth of
+    regions than the sequential one when recomputing."""
+    optim, train = mod("optim"), mod("train")
+    kw = SMALL["llama"]
+    _, model = build_pair(ref, kw, seed=7, std=0.1)
+    seqs = batches(ref, kw["vocab"], 32, 12, seed=11)
+    opt = optim.AdamWHip(gpu, model.params(), lr=1e-3)
+    times = []
+    train.train_lm_hip_resident(model, gpu, opt, seqs[:4], 2, 2, 32, stacked=True,
+                                on_step_time=lambda a, b, rb: times.append(rb))
+    clears0, res0 = gpu.grad_clears_issued, gpu.resident_bytes()
+    pool0 = gpu._pool_bytes
+    train.train_lm_hip_resident(model, gpu, opt, seqs[4:], 4, 2, 32, stacked=True,
+                                on_step_time=lambda a, b, rb: times.append(rb))
+    assert gpu.grad_clears_issued == clears0            # first-writer stores: nothing to clear per step
+    assert gpu._pool_bytes == pool0 and gpu.resident_bytes() == res0   # no allocation after warm-up
+    assert all(rb == 0 for rb in times)                 # the optimizer-flush sync reads nothing back
+    # the loss sync itself: one f32 per sequence
+    ag, arch = mod("autograd"), mod("arch")
+    gpu.install()
+    try:
+        ids = np.concatenate([s[0] for s in seqs[:2]])
+        tg = np.concatenate([s[1] for s in seqs[:2]])
+        loss = arch.sequence_loss(model, ids, tg, 0, 32)
+        ag.backward(loss, 0.5)
+        gpu.sync([loss])
+        assert gpu.last_sync_readback_bytes == 8
+    finally:
+        gpu.uninstall()
+        gpu.sync([])
+
+
+def test_single_row_and_single_token_edges(gpu, ref):
+    """T = 1 (one query sees one key), one-row GEMMs, a one-token vocabulary span: the ragged-edge guards."""
+    from gpu_common import op_case
+    r = ref.Mulberry32(5)
+    R = lambda *s: r.fill_randn(list(s), 0.8)
+    op_case(gpu, ref, [R(1, 64), R(1, 64), R(1, 64)], lambda ag, q, k, v: ag.attention(q, k, v, 1, 1, 1, 64, 0),
+            lambda rf, q, k, v: rf.attention(q, k, v, 1, 1, 1, 64, 0), "attention T=1", floor=1.0)
+    op_case(gpu, ref, [R(1, 7), R(1, 7)], lambda ag, x, w: ag.linear(x, w), lambda rf, x, w: rf.linear(x, w), "linear 1x7x1")
+    op_case(gpu, ref, [R(1, 5)], lambda ag, z: ag.cross_entropy(z, [4]), lambda rf, z: rf.cross_entropy(z, [4]), "CE one row")
+    op_case(gpu, ref, [R(3, 1)], lambda ag, z: ag.cross_entropy(z, [0, -1, 0]), lambda rf, z: rf.cross_entropy(z, [0, -1, 0]),
+            "CE one-logit vocabulary", floor=1.0)
+    w = 1 + 0.3 * R(4)
+    op_case(gpu, ref, [R(1, 4), w], lambda ag, x, g: ag.rms_norm(x, g, 1e-6), lambda rf, x, g: rf.rms_norm(x, g, 1e-6), "rmsNorm one row")
+    op_case(gpu, ref, [R(5, 3)], lambda ag, e: ag.embedding(e, [4]), lambda rf, e: rf.embedding(e, [4]), "embedding one id")
