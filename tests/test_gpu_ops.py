@@ -32,6 +32,36 @@ def test_linear_frozen_weight_and_split_k(gpu, ref):
             "linear frozen", frozen=(1,))
 
 
+@pytest.mark.parametrize("M,N,K", [(200, 152, 200), (130, 100, 72), (70, 83, 75), (257, 193, 101)])
+def test_gemm_every_tile_shape_and_kind(gpu, M, N, K):
+    """Every tile configuration of the GEMM, NT / NN / TN, store and accumulate, split-K 1 and 3, on shapes that leave
+    partial tiles on both edges and a K tail (aligned leading dimensions take the vectorised loaders with the
+    steady-state loop, odd ones the tested loaders), against a float64 product."""
+    rs = np.random.RandomState(M + N + K)
+    a = rs.standard_normal((M, K)).astype(np.float32)
+    b = rs.standard_normal((N, K)).astype(np.float32)
+    c0 = rs.standard_normal((M, N)).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    da, db, dc = (gpu.create_state_buffer(x.nbytes) for x in (a, b, c0))
+    try:
+        for kind, (A, B) in enumerate([(a, b), (a, np.ascontiguousarray(b.T)), (np.ascontiguousarray(a.T), np.ascontiguousarray(b.T))]):
+            gpu.write_state_buffer(da, A)
+            gpu.write_state_buffer(db, B)
+            for tile in range(12):
+                for splitk in ((1, 3) if kind == 2 else (1,)):
+                    for acc in (0, 1):
+                        gpu.set_option("gemm.tile", tile)
+                        gpu.set_option("gemm.splitk", splitk)
+                        gpu.write_state_buffer(dc, c0)
+                        gpu.gemm(kind, acc, M, N, K, da, db, dc)
+                        got = gpu.read_state_buffer(dc, M * N).reshape(M, N)
+                        assert_close(got, (want + c0 if acc else want).astype(np.float32),
+                                     f"gemm kind {kind} tile {tile} splitk {splitk} acc {acc} {M}x{N}x{K}")
+    finally:
+        gpu.set_option("gemm.tile", -1)
+        gpu.set_option("gemm.splitk", -1)
+
+
 def test_elementwise(gpu, ref):
     r = R(ref, 11)
     for n in [(4, 6), (5, 7), (129, 33), (64, 1024)]:
