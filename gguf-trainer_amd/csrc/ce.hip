@@ -91,12 +91,16 @@ __global__ __launch_bounds__(256) void ce_seq_loss(int T, const float *__restric
   if (threadIdx.x == 0) loss[s] = a * inv_denom[s];
 }
 
-// dz[row, :] (+)= seed*inv_denom[seq] * (exp(z - lse) - onehot). grid = (rows, chunks of the row). Each thread keeps
-// four float4 loads in flight; z and dz are touched exactly once, so both use streaming (non-temporal) accesses.
-__global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, const float *__restrict__ z, const int *__restrict__ tgt,
-                                                const float *__restrict__ inv_denom, const float *__restrict__ lse,
-                                                float seed, float *dz, int acc) {
-  int64_t row = blockIdx.x;
+// dz[row, :] (+)= seed*inv_denom[seq] * (exp(z - lse) - onehot). One workgroup per contiguous span of CE_SPAN logits
+// of a row, spans of a row numbered fastest: workgroups that run at the same time then work on neighbouring memory,
+// which the DRAM pages like much better than 2048 rows streamed side by side. Each thread has four float4 loads in
+// flight; z and dz are touched exactly once, so both use streaming (non-temporal) accesses.
+#define CE_SPAN 4096
+__global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, int spans, const float *__restrict__ z,
+                                                const int *__restrict__ tgt, const float *__restrict__ inv_denom,
+                                                const float *__restrict__ lse, float seed, float *dz, int acc) {
+  const int64_t row = blockIdx.x / spans;
+  const int span = blockIdx.x % spans;
   int g = tgt[row];
   if (g == IGN && acc) return;                         // untouched, as the reference leaves it
   const float sc = seed * inv_denom[row / T];
@@ -108,30 +112,29 @@ __global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, const float *__res
     const int n4 = V / 4;
     const v4f *z4 = reinterpret_cast<const v4f *>(zr);
     v4f *d4 = reinterpret_cast<v4f *>(dr);
-    const int stride = gridDim.y * 256;
-    for (int i0 = blockIdx.y * 256 + threadIdx.x; i0 < n4; i0 += 4 * stride) {
-      v4f zz[4], dd[4];
+    const int i0 = span * (CE_SPAN / 4) + threadIdx.x;
+    v4f zz[4], dd[4];
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
-        int i = i0 + u * stride;
-        if (g != IGN && i < n4) zz[u] = __builtin_nontemporal_load(z4 + i);
-        if (acc && i < n4) dd[u] = d4[i];
+    for (int u = 0; u < 4; u++) {
+      int i = i0 + u * 256;
+      if (g != IGN && i < n4) zz[u] = __builtin_nontemporal_load(z4 + i);
+      if (acc && i < n4) dd[u] = d4[i];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      int i = i0 + u * 256;
+      if (i >= n4) continue;
+      v4f o = {0, 0, 0, 0};
+      if (g != IGN) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) o[j] = sc * (__expf(zz[u][j] - ls) - ((i * 4 + j) == g ? 1.f : 0.f));
       }
-#pragma unroll
-      for (int u = 0; u < 4; u++) {
-        int i = i0 + u * stride;
-        if (i >= n4) continue;
-        v4f o = {0, 0, 0, 0};
-        if (g != IGN) {
-#pragma unroll
-          for (int j = 0; j < 4; j++) o[j] = sc * (__expf(zz[u][j] - ls) - ((i * 4 + j) == g ? 1.f : 0.f));
-        }
-        if (acc) o += dd[u];
-        __builtin_nontemporal_store(o, d4 + i);
-      }
+      if (acc) o += dd[u];
+      __builtin_nontemporal_store(o, d4 + i);
     }
   } else {
-    for (int i = blockIdx.y * 256 + threadIdx.x; i < V; i += gridDim.y * 256) {
+    const int end = min(V, (span + 1) * CE_SPAN);
+    for (int i = span * CE_SPAN + threadIdx.x; i < end; i += 256) {
       float o = g == IGN ? 0.f : sc * (__expf(zr[i] - ls) - (i == g ? 1.f : 0.f));
       dr[i] = acc ? dr[i] + o : o;
     }
@@ -171,15 +174,18 @@ __global__ __launch_bounds__(256) void ce_loss_from_stats_k(int T, const int *__
   if (threadIdx.x == 0) loss[s] = a * inv_denom[s];
 }
 // in place: chunk logits -> chunk dlogits; ignored rows zeroed (wgsl.ts:1242)
-__global__ __launch_bounds__(256) void ce_chunk_grad_k(int vc, int v0, int T, float *chunk, const int *__restrict__ tgt,
-                                                       const float *__restrict__ inv_denom, const float *__restrict__ row_max,
-                                                       const float *__restrict__ row_sum, float seed) {
-  int64_t row = blockIdx.x;
+__global__ __launch_bounds__(256) void ce_chunk_grad_k(int vc, int v0, int T, int spans, float *chunk,
+                                                       const int *__restrict__ tgt, const float *__restrict__ inv_denom,
+                                                       const float *__restrict__ row_max, const float *__restrict__ row_sum,
+                                                       float seed) {
+  const int64_t row = blockIdx.x / spans;        // spans of a row are numbered fastest, as in ce_bwd_k
+  const int span = blockIdx.x % spans;
   int g = tgt[row];
   const float sc = seed * inv_denom[row / T];
   const float m = row_max[row], il = 1.0f / row_sum[row];
   float *zr = chunk + row * vc;
-  for (int i = blockIdx.y * 256 + threadIdx.x; i < vc; i += gridDim.y * 256)
+  const int end = min(vc, (span + 1) * CE_SPAN);
+  for (int i = span * CE_SPAN + threadIdx.x; i < end; i += 256)
     zr[i] = g == IGN ? 0.f : sc * (__expf(zr[i] - m) * il - ((i + v0) == g ? 1.f : 0.f));
 }
 
@@ -260,7 +266,9 @@ int gt_ce_bwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets
   GT_REQUIRE(ctx, rows >= 1 && V >= 1 && T >= 1 && rows % T == 0, "gt_ce_bwd: rows %d must be a positive multiple of T %d", rows, T);
   GT_REQUIRE(ctx, logits && targets && inv_denom && lse && dlogits, "gt_ce_bwd: null operand");
   ProfScope ps(ctx, "ce.bwd", 8.0 * rows * V);          // read z, write dz
-  hipLaunchKernelGGL(ce_bwd_k, dim3(rows, row_chunks(V)), dim3(256), 0, ctx->stream, V, T, P<const float>(logits),
+  const int spans = (int)cdiv(V, CE_SPAN);
+  GT_REQUIRE(ctx, (int64_t)rows * spans < (int64_t)1 << 31, "gt_ce_bwd: %d rows x %d logits is more than one launch covers", rows, V);
+  hipLaunchKernelGGL(ce_bwd_k, dim3((unsigned)((int64_t)rows * spans)), dim3(256), 0, ctx->stream, V, T, spans, P<const float>(logits),
                      P<const int>(targets), P<const float>(inv_denom), P<const float>(lse), seed, P<float>(dlogits), acc);
   GT_LAUNCHED(ctx);
   return 0;
@@ -293,8 +301,11 @@ int gt_ce_chunk_grad(gt_ctx *ctx, int rows, int vc, int v0, int T, gt_buf chunk,
   GT_REQUIRE(ctx, rows >= 1 && vc >= 1 && T >= 1 && rows % T == 0 && chunk && targets && inv_denom && row_max && row_sum,
              "gt_ce_chunk_grad: bad arguments");
   ProfScope ps(ctx, "ce.chunk.bwd");
-  hipLaunchKernelGGL(ce_chunk_grad_k, dim3(rows, row_chunks(vc)), dim3(256), 0, ctx->stream, vc, v0, T, P<float>(chunk),
-                     P<const int>(targets), P<const float>(inv_denom), P<const float>(row_max), P<const float>(row_sum), seed);
+  const int spans = (int)cdiv(vc, CE_SPAN);
+  GT_REQUIRE(ctx, (int64_t)rows * spans < (int64_t)1 << 31, "gt_ce_chunk_grad: %d rows x %d logits is more than one launch covers", rows, vc);
+  hipLaunchKernelGGL(ce_chunk_grad_k, dim3((unsigned)((int64_t)rows * spans)), dim3(256), 0, ctx->stream, vc, v0, T, spans,
+                     P<float>(chunk), P<const int>(targets), P<const float>(inv_denom), P<const float>(row_max),
+                     P<const float>(row_sum), seed);
   GT_LAUNCHED(ctx);
   return 0;
 }

@@ -3,22 +3,22 @@
 //
 // AdamW. The reference issues two reduction dispatches and one update dispatch per tensor (816
 // launches for a 272-tensor model). Here the group is described once by a chunk table on the
-// device (tensor index, offset, length per 64K-element chunk) and a step is three launches for any
+// device (tensor index, offset, length per 2048-element chunk) and a step is three launches for any
 // number of tensors: per-chunk sum of squares, a single-workgroup fold of the chunk sums into the
 // clip scale, and the fused element update. The fold runs in chunk order, so the norm and
 // everything downstream is identical from run to run.
 //
 // Muon. Per matrix: momentum + Nesterov + sum of squares, normalise (transposing tall matrices so
 // the Gram matrix is the small one), five quintic Newton-Schulz iterations as three MFMA GEMMs and
-// two fused elementwise combines each, then the scaled descent. Matrices are processed one after
-// another on the context's stream.
+// two fused elementwise combines each, then the scaled descent. Matrices of equal shape are stepped
+// together as one batch (see below).
 #include <algorithm>
 #include <vector>
 #include "common.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-#define CHUNK 65536
+#define CHUNK 2048
 
 struct Chunk { int tensor; int len; int64_t off; };
 struct TensorPtrs { float *w, *g, *m, *v; };
@@ -40,11 +40,20 @@ __global__ __launch_bounds__(256) void adamw_ssq_k(const Chunk *__restrict__ chu
   const float *g = ptrs[c.tensor].g + c.off;
   float s = 0;
   if ((reinterpret_cast<uintptr_t>(g) & 15) == 0) {
+    // read once: streaming loads, four float4 in flight per thread
     int n4 = c.len / 4;
-    for (int i = threadIdx.x; i < n4; i += 256) {
-      v4f x = reinterpret_cast<const v4f *>(g)[i];
-      s += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+    float s4[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int i0 = threadIdx.x; i0 < n4; i0 += 1024) {
+      v4f x[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        int i = i0 + u * 256;
+        x[u] = i < n4 ? __builtin_nontemporal_load(reinterpret_cast<const v4f *>(g) + i) : v4f{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) s4[u] += x[u][0] * x[u][0] + x[u][1] * x[u][1] + x[u][2] * x[u][2] + x[u][3] * x[u][3];
     }
+    s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
     for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) s += g[i] * g[i];
   } else {
     for (int i = threadIdx.x; i < c.len; i += 256) s += g[i] * g[i];
@@ -53,12 +62,21 @@ __global__ __launch_bounds__(256) void adamw_ssq_k(const Chunk *__restrict__ chu
   if (threadIdx.x == 0) partial[blockIdx.x] = s;
 }
 // scale = norm > clip ? clip/(norm + 1e-12) : 1   (adam.ts:56-62, adamw-gpu.ts:84-95)
-__global__ __launch_bounds__(256) void adamw_scale_k(int nchunks, const float *__restrict__ partial, float clip,
-                                                     float *__restrict__ scale) {
-  __shared__ float sm[4];
-  float s = 0;
-  for (int i = threadIdx.x; i < nchunks; i += 256) s += partial[i];
-  s = block_sum<4>(s, sm);
+__global__ __launch_bounds__(1024) void adamw_scale_k(int nchunks, const float *__restrict__ partial, float clip,
+                                                      float *__restrict__ scale) {
+  __shared__ float sm[16];
+  // eight independent loads per thread and round, so the fold is not a chain of dependent memory latencies; the
+  // order of the sum is fixed by the thread count, not by timing
+  float s8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int i0 = threadIdx.x; i0 < nchunks; i0 += 8 * 1024) {
+    float x[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) { int i = i0 + u * 1024; x[u] = i < nchunks ? partial[i] : 0.f; }
+#pragma unroll
+    for (int u = 0; u < 8; u++) s8[u] += x[u];
+  }
+  float s = ((s8[0] + s8[1]) + (s8[2] + s8[3])) + ((s8[4] + s8[5]) + (s8[6] + s8[7]));
+  s = block_sum<16>(s, sm);
   if (threadIdx.x == 0) {
     float norm = sqrtf(s);
     scale[0] = norm > clip ? clip / (norm + 1e-12f) : 1.0f;
@@ -84,11 +102,13 @@ __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ 
   bool vec = ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(m) | reinterpret_cast<uintptr_t>(v) |
                reinterpret_cast<uintptr_t>(g)) & 15) == 0;
   int n4 = vec ? c.len / 4 : 0;
-  // every array is touched once per step: streaming accesses, two float4 per array in flight
-  for (int i0 = threadIdx.x; i0 < n4; i0 += 512) {
-    v4f gg[2], mm[2], vv[2], ww[2];
+  // every array is touched once per step: streaming accesses (the weights too: 4 bytes per parameter of them do not
+  // stay cached until the next forward reads them), UF float4 per array in flight
+  constexpr int UF = 2;
+  for (int i0 = threadIdx.x; i0 < n4; i0 += 256 * UF) {
+    v4f gg[UF], mm[UF], vv[UF], ww[UF];
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
+    for (int u = 0; u < UF; u++) {
       int i = i0 + u * 256;
       if (i < n4) {
         gg[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(g) + i) * sc;
@@ -98,7 +118,7 @@ __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ 
       }
     }
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
+    for (int u = 0; u < UF; u++) {
       int i = i0 + u * 256;
       if (i >= n4) continue;
 #pragma unroll
@@ -109,7 +129,7 @@ __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ 
       }
       __builtin_nontemporal_store(mm[u], reinterpret_cast<v4f *>(m) + i);
       __builtin_nontemporal_store(vv[u], reinterpret_cast<v4f *>(v) + i);
-      reinterpret_cast<v4f *>(w)[i] = ww[u];           // the next forward reads the weights: keep them cacheable
+      __builtin_nontemporal_store(ww[u], reinterpret_cast<v4f *>(w) + i);
     }
   }
   for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) adam1(g[i] * sc, m[i], v[i], w[i], h);
@@ -286,7 +306,7 @@ int gt_adamw_step(gt_ctx *ctx, gt_adamw *o, double lr, double bc1, double bc2) {
   if (o->clip > 0) {
     hipLaunchKernelGGL(adamw_ssq_k, dim3(o->nchunks), dim3(256), 0, ctx->stream, o->chunks, o->ptrs, o->partial);
     GT_LAUNCHED(ctx);
-    hipLaunchKernelGGL(adamw_scale_k, dim3(1), dim3(256), 0, ctx->stream, o->nchunks, o->partial, (float)o->clip, o->scale);
+    hipLaunchKernelGGL(adamw_scale_k, dim3(1), dim3(1024), 0, ctx->stream, o->nchunks, o->partial, (float)o->clip, o->scale);
     GT_LAUNCHED(ctx);
   }
   // every constant is formed in f64 and rounded to f32 once
