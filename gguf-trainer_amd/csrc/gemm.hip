@@ -267,11 +267,10 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   // MI355X: time ~ flops / (tile efficiency x edge utilisation x wave quantisation) + the cost of
   // the split-K reduction pass. N = 576 (SmolLM2) is 3x192 = 6x96; dW has a 1536x576 output and
   // K = 16384 rows, which only fills 256 CUs when K is split.
-  // relative tile efficiencies as measured; the TN kernel (both operands fetched with ds_read_b32) does best
-  // with the 4x1-wave 128x96 tile, the others with 128x192
+  // relative tile efficiencies as measured (asymptotic rate of each tile over the best one's)
   struct Cand { int cfg; double eff; };
   static const Cand cand_nn[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
-  static const Cand cand_tn[] = {{8, 1.00}, {10, 0.97}, {6, 0.90}, {7, 0.78}, {11, 0.80}, {0, 0.72}};
+  static const Cand cand_tn[] = {{8, 1.00}, {11, 0.99}, {10, 0.92}, {6, 0.90}, {7, 0.78}, {0, 0.72}};
   const Cand *cand = kind == GT_TN ? cand_tn : cand_nn;
   int cfg = 0, splits = 1;
   {
@@ -283,15 +282,20 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
       const TileCfg &tc = kTiles[c.cfg];
       const int64_t tiles = cdiv(M, tc.bm) * cdiv(N, tc.bn);
       const double util = (double)M * N / ((double)tiles * tc.bm * tc.bn);
-      for (int sp = 1; sp <= 64; sp *= 2) {
+      // any split count, not only powers of two: 72 output tiles x 14 splits is 3.94 workgroups per CU, x 16 is 4.5,
+      // and with workgroups of equal length the CUs that get the fifth one set the time
+      for (int sp = 1; sp <= 64; sp++) {
         // split only when the output tiles alone cannot give every CU a workgroup
         if (sp > 1 && (count > 1 || tiles >= ctx->num_cu || K / sp < 8 * tc.bk)) break;
         const double waves = (double)tiles * sp * count / ctx->num_cu;
-        const double quant = waves >= 4 ? 1.0 : waves / ceil(waves);
+        const double quant = waves / ceil(waves);
+        // a CU with few workgroups over the whole launch overlaps their fills and write-backs less (fitted on the
+        // dW shapes: 1 workgroup per CU runs 15 % and 2 run 6 % below the rate reached from 4 per CU on)
+        const double conc = std::min(1.0, 1.0625 * waves / (waves + 0.25));
         // short K per workgroup pays the prologue/epilogue more: ~2 K-steps of overhead
         const double ksteps = (double)K / sp / tc.bk;
         const double depth = ksteps / (ksteps + 2.0);
-        double t = t0 / (c.eff * util * quant * depth);
+        double t = t0 / (c.eff * util * quant * depth * conc);
         if (sp > 1) t += ((double)(sp + 2) * M * N * 4.0) / 3.5e12 + 4e-6;
         if (t < best) { best = t; cfg = c.cfg; splits = sp; }
       }
