@@ -229,16 +229,32 @@ def linear(x: Tensor, w: Tensor) -> Tensor:
         ad = _lora.get(id(w))
         if ad is not None:
             a, b, sc = ad
+            be = _be()
+            if hasattr(be, "lora_linear"):
+                # the same composition as below, recorded as one op: the backend applies the scale to the rank-r
+                # activation instead of the [rows, out] product and accumulates into the base output in place
+                _check_linear_dims(x, w)
+                _check_linear_dims(x, a)
+                if b.shape[1] != a.shape[0]:
+                    raise ValueError(f"linear dim mismatch: x is [{x.shape[0]}, {a.shape[0]}] and w is "
+                                     f"[{', '.join(map(str, b.shape))}], so the contracted dimension is {a.shape[0]} on "
+                                     f"one side and {b.shape[1]} on the other. A projection wired to the wrong config "
+                                     "field is the usual cause.")
+                return be.lora_linear(x, w, a, b, sc)
             return add(_linear_raw(x, w), scale(_linear_raw(_linear_raw(x, a), b), sc))
     return _linear_raw(x, w)
 
 
-def _linear_raw(x, w):
+def _check_linear_dims(x, w):
     if x.shape[1] != w.shape[1]:
         raise ValueError(
             f"linear dim mismatch: x is [{', '.join(map(str, x.shape))}] and w is [{', '.join(map(str, w.shape))}], "
             f"so the contracted dimension is {x.shape[1]} on one side and {w.shape[1]} on the other. "
             "A projection wired to the wrong config field is the usual cause.")
+
+
+def _linear_raw(x, w):
+    _check_linear_dims(x, w)
     return _be().linear(x, w)
 
 

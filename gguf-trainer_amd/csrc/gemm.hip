@@ -38,6 +38,9 @@ struct GemmArgs {
   float *Pp;
   int64_t sA, sB, sC;      // batch strides (elements); batch index = blockIdx.z when splits == 1
   int nbm, nbn;
+  // optional second K segment: C = A.B (+) A2.B2 with the same M, N and operand orientation (K2 = 0: none)
+  const float *A2, *B2;
+  int K2, lda2, ldb2;
 };
 
 // One operand tile of R rows x BKT k, kept in LDS as [row][BKT+4] with the 16-byte K chunks of a row XOR-swizzled by
@@ -124,7 +127,7 @@ struct Tile {
   }
 };
 
-template <int BM, int BN, int WM, int WN, int BKT, int KIND, bool VEC>
+template <int BM, int BN, int WM, int WN, int BKT, int KIND, bool VEC, bool SEG2 = false>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
   constexpr int BK = BKT;
   constexpr int NT = WM * WN * 64;
@@ -168,31 +171,54 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
   TA::load(ra, A, a.lda, m0, a.M, k0, kend, tid);
   TB::load(rb, B, a.ldb, n0, a.N, k0, kend, tid);
 
-  for (int k = k0; k < kend; k += BK) {
-    __syncthreads();                       // previous step's LDS reads are done
-    TA::store(ra, sA, tid);
-    TB::store(rb, sB, tid);
-    __syncthreads();
-    if (k + BK < kend) {
-      TA::load(ra, A, a.lda, m0, a.M, k + BK, kend, tid);
-      TB::load(rb, B, a.ldb, n0, a.N, k + BK, kend, tid);
+  // MFMAs of one K step over the tiles in LDS
+#define GEMM_MFMA_STEP()                                                                                          \
+  _Pragma("unroll") for (int c = 0; c < BKT / 8; c++) {                                                           \
+    v4f fa[TM], fb[TN];                                                                                           \
+    _Pragma("unroll") for (int i = 0; i < TM; i++) fa[i] = TA::fetch(sA, wm * (TM * 32) + i * 32 + l32, c, g);     \
+    _Pragma("unroll") for (int j = 0; j < TN; j++) fb[j] = TB::fetch(sB, wn * (TN * 32) + j * 32 + l32, c, g);     \
+    _Pragma("unroll") for (int s = 0; s < 4; s++)                                                                 \
+      _Pragma("unroll") for (int i = 0; i < TM; i++)                                                              \
+        _Pragma("unroll") for (int j = 0; j < TN; j++)                                                            \
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);               \
+  }
+  if (!SEG2) {
+    for (int k = k0; k < kend; k += BK) {
+      __syncthreads();                     // previous step's LDS reads are done
+      TA::store(ra, sA, tid);
+      TB::store(rb, sB, tid);
+      __syncthreads();
+      if (k + BK < kend) {
+        TA::load(ra, A, a.lda, m0, a.M, k + BK, kend, tid);
+        TB::load(rb, B, a.ldb, n0, a.N, k + BK, kend, tid);
+      }
+      GEMM_MFMA_STEP()
     }
-#pragma unroll
-    for (int c = 0; c < BKT / 8; c++) {
-      v4f fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; i++) fa[i] = TA::fetch(sA, wm * (TM * 32) + i * 32 + l32, c, g);
-#pragma unroll
-      for (int j = 0; j < TN; j++) fb[j] = TB::fetch(sB, wn * (TN * 32) + j * 32 + l32, c, g);
-#pragma unroll
-      for (int s = 0; s < 4; s++)
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+  } else {
+    // The K loop runs over two segments (operand pointers, leading dimensions, K range); the step after the last one
+    // of the first segment is the first one of the second, so the pipeline of loads never drains in between.
+    int lda = a.lda, ldb = a.ldb, k = k0;
+    bool second = false;
+    for (;;) {
+      __syncthreads();
+      TA::store(ra, sA, tid);
+      TB::store(rb, sB, tid);
+      __syncthreads();
+      k += BK;
+      bool more = k < kend;
+      if (!more && !second) {
+        second = more = true;
+        A = a.A2; B = a.B2; lda = a.lda2; ldb = a.ldb2; k = 0; kend = a.K2;
+      }
+      if (more) {
+        TA::load(ra, A, lda, m0, a.M, k, kend, tid);
+        TB::load(rb, B, ldb, n0, a.N, k, kend, tid);
+      }
+      GEMM_MFMA_STEP()
+      if (!more) break;
     }
   }
+#undef GEMM_MFMA_STEP
 
   // accumulator register r of lane (g,l32) is C[8*(r/4) + 4*g + r%4][l32] of its 32x32 tile
   float *C;
@@ -233,9 +259,14 @@ static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
   a.nbn = (int)cdiv(a.N, BN);
   dim3 grid(a.nbm * a.nbn, 1, zdim), block(WM * WN * 64);
 #define GO(KIND, VEC) hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, BKT, KIND, VEC>), grid, block, 0, ctx->stream, a)
-  if (kind == GT_NT) { if (vec) GO(GT_NT, true); else GO(GT_NT, false); }
+#define GO2(KIND) hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, BKT, KIND, true, true>), grid, block, 0, ctx->stream, a)
+  if (a.K2 > 0) {                // two K segments: aligned NT / NN only (gemm_impl sends everything else as two launches)
+    if (kind == GT_NT) GO2(GT_NT); else GO2(GT_NN);
+  }
+  else if (kind == GT_NT) { if (vec) GO(GT_NT, true); else GO(GT_NT, false); }
   else if (kind == GT_NN) { if (vec) GO(GT_NN, true); else GO(GT_NN, false); }
   else { if (vec) GO(GT_TN, true); else GO(GT_TN, false); }
+#undef GO2
 #undef GO
   GT_LAUNCHED(ctx);
   return 0;
@@ -247,7 +278,7 @@ static const TileCfg kTiles[] = {{64, 64, 16}, {128, 64, 16}, {128, 128, 16}, {1
 #define NCFG ((int)(sizeof(kTiles) / sizeof(kTiles[0])))
 
 static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
-                     gt_buf C, int64_t sC, int count) {
+                     gt_buf C, int64_t sC, int count, int K2 = 0, gt_buf A2 = 0, gt_buf B2 = 0) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, kind >= 0 && kind <= 2, "gt_gemm: kind %d is not NT(0)/NN(1)/TN(2)", kind);
   GT_REQUIRE(ctx, M >= 1 && N >= 1 && K >= 1 && count >= 1, "gt_gemm: M,N,K,count must be >= 1 (got %d,%d,%d,%d)", M, N, K, count);
@@ -262,6 +293,10 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   a.sA = sA; a.sB = sB; a.sC = sC;
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
              (sA % 4 == 0) && (sB % 4 == 0);
+  a.K2 = K2; a.A2 = P<const float>(A2); a.B2 = P<const float>(B2);
+  a.lda2 = (kind == GT_TN) ? M : K2;
+  a.ldb2 = (kind == GT_NT) ? K2 : N;
+  if (K2 > 0) vec = vec && (a.lda2 % 4 == 0) && (a.ldb2 % 4 == 0) && (A2 % 16 == 0) && (B2 % 16 == 0);
 
   // Tile and split-K choice by a small cost model over the tile shapes that measured best on
   // MI355X: time ~ flops / (tile efficiency x edge utilisation x wave quantisation) + the cost of
@@ -286,7 +321,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
       // and with workgroups of equal length the CUs that get the fifth one set the time
       for (int sp = 1; sp <= 64; sp++) {
         // split only when the output tiles alone cannot give every CU a workgroup
-        if (sp > 1 && (count > 1 || tiles >= ctx->num_cu || K / sp < 8 * tc.bk)) break;
+        if (sp > 1 && (count > 1 || K2 > 0 || tiles >= ctx->num_cu || K / sp < 8 * tc.bk)) break;
         const double waves = (double)tiles * sp * count / ctx->num_cu;
         const double quant = waves / ceil(waves);
         // a CU with few workgroups over the whole launch overlaps their fills and write-backs less (fitted on the
@@ -303,7 +338,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   }
   if (ctx->opt_gemm_tile >= 0 && ctx->opt_gemm_tile < NCFG) cfg = ctx->opt_gemm_tile;
   const int bm = kTiles[cfg].bm, bn = kTiles[cfg].bn, bk = kTiles[cfg].bk;
-  if (count == 1 && ctx->opt_gemm_splitk >= 1) splits = ctx->opt_gemm_splitk;
+  if (count == 1 && K2 == 0 && ctx->opt_gemm_splitk >= 1) splits = ctx->opt_gemm_splitk;
   if (splits > 1) {
     int64_t kc = cdiv(cdiv(K, splits), bk) * bk;
     splits = (int)cdiv(K, kc);
@@ -317,7 +352,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   int zdim = splits > 1 ? splits : count;
   char label[32];
   snprintf(label, sizeof label, "gemm.%s.%dx%dx%d%s", kind == GT_NT ? "nt" : kind == GT_NN ? "nn" : "tn", bm, bn, bk, splits > 1 ? ".splitk" : "");
-  ProfScope ps(ctx, label, 2.0 * M * N * K * count);
+  ProfScope ps(ctx, label, 2.0 * M * N * ((double)K + K2) * count);
   int rc;
   switch (cfg) {
     case 0: rc = launch_cfg<64, 64, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
@@ -345,6 +380,17 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
 extern "C" {
 int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_buf B, gt_buf C) {
   return gemm_impl(ctx, kind, acc, M, N, K, A, 0, B, 0, C, 0, 1);
+}
+int gt_gemm_pair(gt_ctx *ctx, int kind, int acc, int M, int N, int K1, gt_buf A1, gt_buf B1, int K2, gt_buf A2, gt_buf B2,
+                 gt_buf C) {
+  if (ctx && (K2 < 1 || !A2 || !B2)) GT_FAIL(ctx, "gt_gemm_pair: the second product needs K2 >= 1 and both operands (got K2 = %d)", K2);
+  // one K loop over both products for 16-byte aligned NT / NN operands; otherwise two launches, the second adding
+  const int lda1 = kind == GT_TN ? M : K1, ldb1 = kind == GT_NT ? K1 : N, lda2 = kind == GT_TN ? M : K2, ldb2 = kind == GT_NT ? K2 : N;
+  const bool fused = kind != GT_TN && K1 >= 1 && (lda1 % 4 == 0) && (ldb1 % 4 == 0) && (lda2 % 4 == 0) && (ldb2 % 4 == 0) &&
+                     ((A1 | B1 | A2 | B2) % 16 == 0);
+  if (fused) return gemm_impl(ctx, kind, acc, M, N, K1, A1, 0, B1, 0, C, 0, 1, K2, A2, B2);
+  if (gemm_impl(ctx, kind, acc, M, N, K1, A1, 0, B1, 0, C, 0, 1)) return 1;
+  return gemm_impl(ctx, kind, 1, M, N, K2, A2, 0, B2, 0, C, 0, 1);
 }
 int gt_gemm_batched(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t strideA, gt_buf B,
                     int64_t strideB, gt_buf C, int64_t strideC, int count) {

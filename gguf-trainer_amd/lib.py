@@ -41,6 +41,7 @@ _SIG = {
     "gt_resident_bytes": [ctxp, C.POINTER(C.c_uint64)],
     "gt_set_option": [ctxp, C.c_char_p, i32],
     "gt_gemm": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf],
+    "gt_gemm_pair": [ctxp, i32, i32, i32, i32, i32, buf, buf, i32, buf, buf, buf],
     "gt_gemm_batched": [ctxp, i32, i32, i32, i32, i32, buf, i64, buf, i64, buf, i64, i32],
     "gt_add_fwd": [ctxp, i64, buf, buf, buf],
     "gt_mul_fwd": [ctxp, i64, buf, buf, buf],

@@ -72,6 +72,12 @@ int gt_set_option(gt_ctx *ctx, const char *key, int value);
  * FP32 MFMA, f32 accumulate. Any M, N, K >= 1. */
 enum { GT_NT = 0, GT_NN = 1, GT_TN = 2 };
 int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_buf B, gt_buf C);
+/* C (+)= A1.B1 + A2.B2: two products of the same kind, M and N summed in one K loop (K1 then K2). It is the LoRA
+ * linear of src/model/autograd.ts:760-781 without the [rows, out] add: y = x W^T + (s h) B^T with A2 = s h
+ * [rows, r], and in the backward dX = dY W + dH A. Bits differ from two gt_gemm calls with acc = 1 only by the order
+ * of the final additions. */
+int gt_gemm_pair(gt_ctx *ctx, int kind, int acc, int M, int N, int K1, gt_buf A1, gt_buf B1, int K2, gt_buf A2, gt_buf B2,
+                 gt_buf C);
 /* batch of `count` independent products with element strides between consecutive problems
  * (Newton-Schulz over same-shaped matrices; no counterpart call in the reference, which loops). */
 int gt_gemm_batched(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t strideA,

@@ -62,6 +62,37 @@ def test_gemm_every_tile_shape_and_kind(gpu, M, N, K):
         gpu.set_option("gemm.splitk", -1)
 
 
+@pytest.mark.parametrize("M,N,K1,K2", [(200, 152, 96, 16), (130, 100, 72, 5), (257, 193, 101, 33), (64, 64, 16, 16)])
+def test_gemm_pair(gpu, M, N, K1, K2):
+    """C (+)= A1.B1 + A2.B2 in one K loop (the LoRA linear and its dX): every kind, store and accumulate, a few tile
+    shapes, against a float64 sum of the two products."""
+    rs = np.random.RandomState(M + K2)
+    a1, b1 = rs.standard_normal((M, K1)).astype(np.float32), rs.standard_normal((N, K1)).astype(np.float32)
+    a2, b2 = rs.standard_normal((M, K2)).astype(np.float32), rs.standard_normal((N, K2)).astype(np.float32)
+    c0 = rs.standard_normal((M, N)).astype(np.float32)
+    want = a1.astype(np.float64) @ b1.astype(np.float64).T + a2.astype(np.float64) @ b2.astype(np.float64).T
+    bufs = [gpu.create_state_buffer(x.nbytes) for x in (a1, b1, a2, b2, c0)]
+    L = mod("lib")
+    T = lambda x: np.ascontiguousarray(x.T)
+    try:
+        for kind, ops in enumerate([(a1, b1, a2, b2), (a1, T(b1), a2, T(b2)), (T(a1), T(b1), T(a2), T(b2))]):
+            for buf, arr in zip(bufs, ops):
+                gpu.write_state_buffer(buf, arr)
+            for tile in (-1, 0, 7, 8, 10):
+                for acc in (0, 1):
+                    gpu.set_option("gemm.tile", tile)
+                    gpu.write_state_buffer(bufs[4], c0)
+                    L.check(gpu.ctx, L.lib.gt_gemm_pair(gpu.ctx, kind, acc, M, N, K1, bufs[0], bufs[1], K2, bufs[2], bufs[3],
+                                                        bufs[4]), "gt_gemm_pair")
+                    got = gpu.read_state_buffer(bufs[4], M * N).reshape(M, N)
+                    assert_close(got, (want + c0 if acc else want).astype(np.float32),
+                                 f"gemm pair kind {kind} tile {tile} acc {acc} {M}x{N}x({K1}+{K2})")
+        rc = L.lib.gt_gemm_pair(gpu.ctx, 0, 0, M, N, K1, bufs[0], bufs[1], 0, bufs[2], bufs[3], bufs[4])
+        assert rc != 0 and b"K2" in L.lib.gt_last_error(gpu.ctx)
+    finally:
+        gpu.set_option("gemm.tile", -1)
+
+
 def test_elementwise(gpu, ref):
     r = R(ref, 11)
     for n in [(4, 6), (5, 7), (129, 33), (64, 1024)]:
