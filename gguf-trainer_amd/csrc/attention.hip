@@ -22,6 +22,7 @@ struct AttnP {
   int B, T, Hq, Hkv, hd, window;
   float c2;              // log2(e)/sqrt(hd)
   float scale;           // 1/sqrt(hd)
+  int splits;            // MFMA kernels: workgroups per tile (1 unless the launch is small)
 };
 
 __device__ __forceinline__ int win_lo(int t, int window) { return (window > 0 && t + 1 > window) ? t + 1 - window : 0; }
@@ -213,20 +214,93 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
 }
 
 // attention_mfma.hip, compiled once per head dim
-int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
-int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse);
+int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
+int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
 int attn_bwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                    gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                    float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 int attn_bwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                     gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                     float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 static int attn_mfma_supported(int hd) { return hd == 64 || hd == 128; }
+
+// A launch with fewer 128-row tiles than three per CU is cut further (measured at T = 2048, 9 heads: 1 sequence runs
+// 2.3x faster with 6 workgroups per tile, 2 sequences 1.5x with 3, 4 sequences 1.13x with 2, 8 gain nothing): every tile's loop range goes to `splits`
+// workgroups (at most 8, at most one per 64-key stage of the longest tile) whose partial results are folded afterwards.
+static int attn_splits(gt_ctx *ctx, int B, int T, int Hq) {
+  const int64_t tiles = cdiv(T, 128) * Hq * B;
+  int s = 1;
+  if (tiles < 3 * (int64_t)ctx->num_cu) s = (int)std::min<int64_t>(8, cdiv(3 * (int64_t)ctx->num_cu, tiles));
+  if (ctx->opt_attn_splits >= 1) s = std::min(ctx->opt_attn_splits, 8);
+  return (int)std::max<int64_t>(1, std::min<int64_t>(s, cdiv(T, 64)));
+}
+
+// out = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), lse2 = m + log2(that sum), m = max_s m_s: the online-softmax
+// merge of the splits' partial results, in split order. One thread per float4 of the output.
+__global__ __launch_bounds__(256) void attn_fwd_combine(AttnP p, const float *__restrict__ fpart, float *__restrict__ out,
+                                                        float *__restrict__ lse) {
+  const int hd4 = p.hd / 4;
+  const int64_t n = (int64_t)p.B * p.T * p.Hq * hd4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int d4 = (int)(i % hd4), h = (int)((i / hd4) % p.Hq);
+  const int64_t row = i / ((int64_t)hd4 * p.Hq);            // b*T + t
+  const int64_t b = row / p.T, t = row % p.T;
+  const size_t slice = (size_t)p.B * p.T * p.Hq * p.hd, rows = (size_t)p.B * p.Hq * p.T;
+  const size_t sidx = ((size_t)b * p.Hq + h) * p.T + t;
+  const float *mp = fpart + (size_t)p.splits * slice, *lp = mp + (size_t)p.splits * rows;
+  float m = -1.0e30f;
+  for (int s = 0; s < p.splits; s++) m = fmaxf(m, mp[s * rows + sidx]);
+  float L = 0.f;
+  float4 o = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < p.splits; s++) {
+    const float wgt = __builtin_amdgcn_exp2f(mp[s * rows + sidx] - m);
+    L += lp[s * rows + sidx] * wgt;
+    const float4 x = reinterpret_cast<const float4 *>(fpart + s * slice)[i];
+    o.x += x.x * wgt; o.y += x.y * wgt; o.z += x.z * wgt; o.w += x.w * wgt;
+  }
+  const float inv = 1.0f / L;
+  reinterpret_cast<float4 *>(out)[i] = float4{o.x * inv, o.y * inv, o.z * inv, o.w * inv};
+  if (d4 == 0) lse[sidx] = m + log2f(L);
+}
+// dst (+)= sum of `ns` slices of n4 float4 each, in slice order
+__global__ __launch_bounds__(256) void attn_slice_sum(const float *__restrict__ part, int ns, size_t n4, float *dst, int acc) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  const float4 *pp = reinterpret_cast<const float4 *>(part);
+  float4 a = pp[i];
+  for (int s = 1; s < ns; s++) { float4 x = pp[(size_t)s * n4 + i]; a.x += x.x; a.y += x.y; a.z += x.z; a.w += x.w; }
+  float4 *o = reinterpret_cast<float4 *>(dst) + i;
+  if (acc) { float4 y = *o; a.x += y.x; a.y += y.y; a.z += y.z; a.w += y.w; }
+  *o = a;
+}
+
 static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse) {
-  return p.hd == 64 ? attn_fwd_mfma64(ctx, p, q, k, v, out, lse) : attn_fwd_mfma128(ctx, p, q, k, v, out, lse);
+  float *fpart = nullptr;
+  if (p.splits > 1) {
+    const size_t slice = (size_t)p.B * p.T * p.Hq * p.hd, rows = (size_t)p.B * p.Hq * p.T;
+    void *ws;
+    if (gt_ws_reserve(ctx, (size_t)p.splits * (slice + 2 * rows) * sizeof(float), &ws)) return 1;
+    fpart = static_cast<float *>(ws);
+  }
+  if (p.hd == 64 ? attn_fwd_mfma64(ctx, p, q, k, v, out, lse, fpart) : attn_fwd_mfma128(ctx, p, q, k, v, out, lse, fpart)) return 1;
+  if (p.splits > 1) {
+    const int64_t n = (int64_t)p.B * p.T * p.Hq * (p.hd / 4);
+    hipLaunchKernelGGL(attn_fwd_combine, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, p, fpart, P<float>(out), P<float>(lse));
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
 }
 static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
-                         float *part, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
-  return p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dq, acc_q, dk, acc_k, dv, acc_v)
-                    : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dq, acc_q, dk, acc_k, dv, acc_v);
+                         float *part, float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+  if (p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v)
+                 : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v))
+    return 1;
+  if (p.splits > 1) {
+    const size_t n4 = (size_t)p.B * p.T * p.Hq * p.hd / 4;
+    hipLaunchKernelGGL(attn_slice_sum, dim3((unsigned)cdiv((int64_t)n4, 256)), dim3(256), 0, ctx->stream, dqpart, p.splits, n4,
+                       P<float>(dq), acc_q);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
 }
 
 static int check(gt_ctx *ctx, const char *who, int B, int T, int Hq, int Hkv, int hd, int window) {
@@ -249,7 +323,8 @@ int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   GT_ENTER(ctx);
   if (check(ctx, "gt_attn_fwd", B, T, Hq, Hkv, hd, window)) return 1;
   GT_REQUIRE(ctx, q && k && v && out && lse, "gt_attn_fwd: null operand");
-  AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd)};
+  AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd), 1};
+  if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) p.splits = attn_splits(ctx, B, T, Hq);
   ProfScope ps(ctx, "attention", 2.0 * 2 * hd * attn_pairs(T, window) * Hq * B);   // QK^T and PV
   if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) return attn_fwd_mfma(ctx, p, q, k, v, out, lse);
   int64_t rows = (int64_t)B * Hq * T;
@@ -265,25 +340,29 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   GT_ENTER(ctx);
   if (check(ctx, "gt_attn_bwd", B, T, Hq, Hkv, hd, window)) return 1;
   GT_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, "gt_attn_bwd: null operand");
-  AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd)};
+  AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd), 1};
   int64_t rows = (int64_t)B * Hq * T, krows = (int64_t)B * Hkv * T;
   ProfScope whole(ctx, "attention.bwd", 5.0 * 2 * hd * attn_pairs(T, window) * Hq * B);   // S, dP, dV, dK, dQ
-  // workspace: D per (sequence, head, row), then (MFMA path, kv group > 1) one dK and one dV slice per query head
+  // workspace: D per (sequence, head, row); then (MFMA path) one dK and one dV slice per (split, query head of the kv
+  // group) when there is more than one, and one dQ partial per split when the launch is split
   const bool mfma = !ctx->opt_attn_generic && attn_mfma_supported(hd);
   const int group = Hq / Hkv;
+  if (mfma) p.splits = attn_splits(ctx, B, T, Hq);
   const size_t d_floats = ((size_t)rows + 63) / 64 * 64;
-  const size_t part_floats = (mfma && group > 1) ? (size_t)2 * group * krows * hd : 0;
+  const size_t part_floats = (mfma && p.splits * group > 1) ? (size_t)2 * p.splits * group * krows * hd : 0;
+  const size_t dq_floats = (mfma && p.splits > 1) ? (size_t)p.splits * rows * hd : 0;
   void *ws;
-  if (gt_ws_reserve(ctx, (d_floats + part_floats) * sizeof(float), &ws)) return 1;
+  if (gt_ws_reserve(ctx, (d_floats + part_floats + dq_floats) * sizeof(float), &ws)) return 1;
   float *Dr = static_cast<float *>(ws);
   float *part = part_floats ? Dr + d_floats : nullptr;
+  float *dqpart = dq_floats ? Dr + d_floats + part_floats : nullptr;
   {
     ProfScope ps(ctx, "attention.bwd.D");
     hipLaunchKernelGGL(attn_bwd_d, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, p, P<const float>(out),
                        P<const float>(dout), Dr);
     GT_LAUNCHED(ctx);
   }
-  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dq, acc_q, dk, acc_k, dv, acc_v);
+  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v);
   {
     ProfScope ps(ctx, "attention.bwd.dq");
     size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);

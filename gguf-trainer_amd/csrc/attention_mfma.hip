@@ -29,6 +29,11 @@
 //
 // dK/dV loops over the query heads of the kv group inside the workgroup and over query tiles in
 // increasing order, so the GQA sum has a fixed order and needs no atomics.
+//
+// Small launches (one short sequence, few heads) have fewer tiles than the chip has CUs and their time is the
+// serial loop of the longest tile. For them p.splits > 1 cuts every tile's loop range (key stages in forward and
+// dQ, query stages in dK/dV) into that many workgroups, which write partial results (unnormalised output with
+// its running maximum and sum; partial dQ; dK/dV slices) that a second kernel folds in split order.
 #include <algorithm>
 #include "common.h"
 
@@ -39,6 +44,7 @@ struct AttnP {
   int B, T, Hq, Hkv, hd, window;
   float c2;
   float scale;
+  int splits;               // >= 1: the loop range of every tile is cut into this many workgroups (small launches)
 };
 
 #ifndef HD
@@ -167,7 +173,7 @@ __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32]
 // ---- forward --------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, float *__restrict__ out,
-                                                       float *__restrict__ lse) {
+                                                       float *__restrict__ lse, float *__restrict__ fpart) {
   using IO = TileIO<KT>;
   __shared__ __attribute__((aligned(16))) float sK[KT * LD];
   __shared__ __attribute__((aligned(16))) float sVt[HD * IO::LDT];
@@ -175,8 +181,10 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
   // 1-D grid ordered by work: every (head, sequence) pair's longest query tile is dispatched before any shorter
   // one, so the causal triangle packs onto the CUs without a long tail
   const int nhb = p.Hq * p.B;
-  const int qtile = (int)((p.T + 127) / 128) - 1 - (int)(blockIdx.x / nhb);
-  const int h = (blockIdx.x % nhb) % p.Hq, b = (blockIdx.x % nhb) / p.Hq;
+  const int sp = (int)(blockIdx.x % p.splits);
+  const unsigned bid = blockIdx.x / p.splits;
+  const int qtile = (int)((p.T + 127) / 128) - 1 - (int)(bid / nhb);
+  const int h = (bid % nhb) % p.Hq, b = (bid % nhb) / p.Hq;
   const int kvh = h / (p.Hq / p.Hkv);
   const size_t qstr = (size_t)p.Hq * HD, kstr = (size_t)p.Hkv * HD;
   const int tq0 = qtile * 128 + wave * 32, t = tq0 + l32;
@@ -187,8 +195,13 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
   float qreg[HD / 2];
   load_row_regs(qreg, q + ((size_t)b * p.T + (tv ? t : 0)) * qstr + (size_t)h * HD, tv, g, p.c2);
   const int lo_t = win_lo_m(t, p.window);
-  const int kt_lo = win_lo_m(qtile * 128, p.window) / KT;
-  const int kt_hi = min(p.T - 1, qtile * 128 + 127) / KT;
+  int kt_lo = win_lo_m(qtile * 128, p.window) / KT;
+  int kt_hi = min(p.T - 1, qtile * 128 + 127) / KT;
+  if (p.splits > 1) {                      // this workgroup's share of the key stages (possibly none)
+    const int n = kt_hi - kt_lo + 1, first = kt_lo;
+    kt_lo = first + sp * n / p.splits;
+    kt_hi = first + (sp + 1) * n / p.splits - 1;
+  }
   const int wave_lo = win_lo_m(tq0, p.window), wave_lo_last = win_lo_m(tq1, p.window);
   const bool ragged = tq0 + 31 >= p.T;
 
@@ -265,25 +278,37 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
     }
   }
   const float lt = l + __shfl_xor(l, 32, 64);
-  if (tv) {
-    store_row(out + ((size_t)b * p.T + t) * qstr + (size_t)h * HD, oacc, g, 1.0f / lt, 0);
-    if (g == 0) lse[((size_t)b * p.Hq + h) * p.T + t] = m + log2f(lt);
+  if (!tv) return;
+  const size_t sidx = ((size_t)b * p.Hq + h) * p.T + t;
+  if (p.splits > 1) {        // partial: unnormalised output, running maximum and sum of this key range
+    const size_t slice = (size_t)p.B * p.T * qstr, rows = (size_t)p.B * p.Hq * p.T;
+    store_row(fpart + sp * slice + ((size_t)b * p.T + t) * qstr + (size_t)h * HD, oacc, g, 1.0f, 0);
+    if (g == 0) {
+      float *mp = fpart + (size_t)p.splits * slice;
+      mp[sp * rows + sidx] = m;
+      mp[((size_t)p.splits + sp) * rows + sidx] = lt;
+    }
+    return;
   }
+  store_row(out + ((size_t)b * p.T + t) * qstr + (size_t)h * HD, oacc, g, 1.0f / lt, 0);
+  if (g == 0) lse[sidx] = m + log2f(lt);
 }
 
 // ---- dQ -----------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                           const float *__restrict__ v, const float *__restrict__ go,
                                                           const float *__restrict__ lse, const float *__restrict__ Dr,
-                                                          float *dq, int acc_q) {
+                                                          float *dq, int acc_q, float *__restrict__ dqpart) {
   using IO = TileIO<KT>;
   __shared__ __attribute__((aligned(16))) float sK[KT * LD];
   __shared__ __attribute__((aligned(16))) float sV[KT * LD];
   __shared__ __attribute__((aligned(16))) float sKt[HD * IO::LDT];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
   const int nhb = p.Hq * p.B;
-  const int qtile = (int)((p.T + 127) / 128) - 1 - (int)(blockIdx.x / nhb);
-  const int h = (blockIdx.x % nhb) % p.Hq, b = (blockIdx.x % nhb) / p.Hq;
+  const int sp = (int)(blockIdx.x % p.splits);
+  const unsigned bid = blockIdx.x / p.splits;
+  const int qtile = (int)((p.T + 127) / 128) - 1 - (int)(bid / nhb);
+  const int h = (bid % nhb) % p.Hq, b = (bid % nhb) / p.Hq;
   const int kvh = h / (p.Hq / p.Hkv);
   const size_t qstr = (size_t)p.Hq * HD, kstr = (size_t)p.Hkv * HD;
   const int tq0 = qtile * 128 + wave * 32, t = tq0 + l32;
@@ -298,8 +323,13 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
   const size_t sidx = ((size_t)b * p.Hq + h) * p.T + (tv ? t : 0);
   const float L2 = tv ? lse[sidx] : 0.f, Dt = tv ? Dr[sidx] : 0.f;
   const int lo_t = win_lo_m(t, p.window);
-  const int kt_lo = win_lo_m(qtile * 128, p.window) / KT;
-  const int kt_hi = min(p.T - 1, qtile * 128 + 127) / KT;
+  int kt_lo = win_lo_m(qtile * 128, p.window) / KT;
+  int kt_hi = min(p.T - 1, qtile * 128 + 127) / KT;
+  if (p.splits > 1) {                      // this workgroup's share of the key stages (possibly none)
+    const int n = kt_hi - kt_lo + 1, first = kt_lo;
+    kt_lo = first + sp * n / p.splits;
+    kt_hi = first + (sp + 1) * n / p.splits - 1;
+  }
   const int wave_lo = win_lo_m(tq0, p.window), wave_lo_last = win_lo_m(tq1, p.window);
   const bool ragged = tq0 + 31 >= p.T;
 
@@ -343,7 +373,9 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
       t_dot_acc<IO::LDT>(dacc, sKt, sub * 32, ds, l32, g);
     }
   }
-  if (tv) store_row(dq + qoff, dacc, g, 1.0f, acc_q);
+  if (!tv) return;
+  if (p.splits > 1) store_row(dqpart + sp * ((size_t)p.B * p.T * qstr) + qoff, dacc, g, 1.0f, 0);
+  else store_row(dq + qoff, dacc, g, 1.0f, acc_q);
 }
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------
@@ -362,8 +394,10 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   // and attn_group_sum adds the slices in head order (a fixed order, so still deterministic); splitting by
   // head is what gives the dispatcher enough similar-sized pieces to fill 256 CUs.
   const int nhb = p.Hq * p.B;
-  const int ktile = (int)(blockIdx.x / nhb);
-  const int h = (blockIdx.x % nhb) % p.Hq, b = (blockIdx.x % nhb) / p.Hq;
+  const int sp = (int)(blockIdx.x % p.splits);
+  const unsigned bid = blockIdx.x / p.splits;
+  const int ktile = (int)(bid / nhb);
+  const int h = (bid % nhb) % p.Hq, b = (bid % nhb) / p.Hq;
   const int group = p.Hq / p.Hkv;
   const int kvh = h / group, hh = h % group;
   const size_t qstr = (size_t)p.Hq * HD, kstr = (size_t)p.Hkv * HD;
@@ -387,7 +421,9 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
 #pragma unroll
     for (int r = 0; r < 16; r++) { kacc[dt][r] = 0.f; vacc[dt][r] = 0.f; }
 
-  const int niter = nqt;
+  // this workgroup's share of the query stages
+  const int it_lo = p.splits > 1 ? sp * nqt / p.splits : 0;
+  const int niter = p.splits > 1 ? (sp + 1) * nqt / p.splits : nqt;
   v4f pq[IO::PER], pg[IO::PER];
   float pstat = 0.f;
   auto prefetch = [&](int it) {
@@ -402,8 +438,8 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
       pstat = tt < p.T ? (tid < QT ? lse[si] : Dr[si]) : 0.f;
     }
   };
-  prefetch(0);
-  for (int it = 0; it < niter; it++) {
+  prefetch(it_lo);
+  for (int it = it_lo; it < niter; it++) {
     __syncthreads();
     IO::store_rows(pq, sQ, tid);
     IO::store_t(pq, sQt, tid);
@@ -439,10 +475,11 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
     t_dot_acc<IO::LDT>(kacc, sQt, 0, ds, l32, g);
   }
   if (sv) {
-    if (part) {            // slice hh of the workspace, same [row][Hkv*hd] layout as dk
+    if (part) {            // slice (split, head of the group) of the workspace, same [row][Hkv*hd] layout as dk
       const size_t slice = (size_t)p.B * p.T * kstr;
-      store_row(part + (size_t)hh * slice + koff, kacc, g, 1.0f, 0);
-      store_row(part + (size_t)(group + hh) * slice + koff, vacc, g, 1.0f, 0);
+      const int nslice = p.splits * group, mine = sp * group + hh;
+      store_row(part + (size_t)mine * slice + koff, kacc, g, 1.0f, 0);
+      store_row(part + (size_t)(nslice + mine) * slice + koff, vacc, g, 1.0f, 0);
     } else {
       store_row(dk + koff, kacc, g, 1.0f, acc_k);
       store_row(dv + koff, vacc, g, 1.0f, acc_v);
@@ -450,7 +487,7 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   }
 }
 
-// dk (+)= sum over the group's heads of their slices, in head order; same for dv
+// dk (+)= sum of its slices (splits x heads of the group), in slice order; same for dv
 __global__ __launch_bounds__(256) void FN(attn_group_sum)(const float *__restrict__ part, int group, size_t n4, float *dk, int acc_k,
                                                       float *dv, int acc_v) {
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -465,20 +502,25 @@ __global__ __launch_bounds__(256) void FN(attn_group_sum)(const float *__restric
 
 #define DKV_SMEM ((2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT) * sizeof(float))
 
-int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse) {
+// fpart: workspace for the split partials (splits x output, then splits x rows maxima, splits x rows sums), or null
+int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart) {
   GT_REQUIRE(ctx, (q | k | v | out) % 16 == 0, "attention: buffers must be 16-byte aligned");
-  dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
+  GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || fpart), "attention: split forward without a workspace");
+  dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
   hipLaunchKernelGGL(FN(attn_fwd_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
-                     P<const float>(v), P<float>(out), P<float>(lse));
+                     P<const float>(v), P<float>(out), P<float>(lse), fpart);
   GT_LAUNCHED(ctx);
   return 0;
 }
 
-// Dr: the per-row sums D; part: workspace for the per-head dK/dV slices (2*group slices of B*T*Hkv*hd floats) or null
+// Dr: the per-row sums D; part: workspace for the dK/dV slices (2 * splits * group slices of B*T*Hkv*hd floats) or
+// null when there is one slice; dqpart: workspace for the dQ partials (splits x dq) or null when splits == 1
 int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
-                      float *part, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+                      float *part, float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
   const int group = p.Hq / p.Hkv;
+  GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart) && (p.splits * group == 1 || part),
+             "attention: split backward without a workspace");
   static bool smem_set = false;
   if (!smem_set) {            // more than the 64 KB a kernel gets by default at hd 128
     GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)),
@@ -487,20 +529,20 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
   }
   {
     ProfScope ps(ctx, "attention.bwd.dq");
-    dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
+    dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
     hipLaunchKernelGGL(FN(attn_bwd_dq_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
-                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q);
+                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q, dqpart);
     GT_LAUNCHED(ctx);
   }
   {
     ProfScope ps(ctx, "attention.bwd.dkv");
-    dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B));
+    dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
     hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k), grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
                        P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part);
     GT_LAUNCHED(ctx);
     if (part) {
       size_t n4 = (size_t)p.B * p.T * p.Hkv * HD / 4;
-      hipLaunchKernelGGL(FN(attn_group_sum), dim3((unsigned)cdiv((int64_t)n4, 256)), dim3(256), 0, ctx->stream, part, group, n4,
+      hipLaunchKernelGGL(FN(attn_group_sum), dim3((unsigned)cdiv((int64_t)n4, 256)), dim3(256), 0, ctx->stream, part, p.splits * group, n4,
                          P<float>(dk), acc_k, P<float>(dv), acc_v);
       GT_LAUNCHED(ctx);
     }

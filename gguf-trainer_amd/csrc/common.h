@@ -30,7 +30,7 @@ struct gt_ctx {
   struct RopeKey { int T, hd, pos; double base; bool operator<(const RopeKey &o) const {
     if (T != o.T) return T < o.T; if (hd != o.hd) return hd < o.hd; if (pos != o.pos) return pos < o.pos; return base < o.base; } };
   std::map<RopeKey, float *> rope_tables;
-  int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1;
+  int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1;
   bool prof_on = false;
   std::string prof_prefix;
   std::vector<ProfEvent> prof;

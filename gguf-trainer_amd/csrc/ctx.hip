@@ -122,6 +122,7 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes) {
 int gt_set_option(gt_ctx *ctx, const char *key, int value) {
   if (!ctx || !key) return 1;
   if (!strcmp(key, "attn.generic")) ctx->opt_attn_generic = value;
+  else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
   else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
   else if (!strcmp(key, "gemm.splitk")) ctx->opt_gemm_splitk = value;
   else GT_FAIL(ctx, "gt_set_option: unknown key '%s'", key);

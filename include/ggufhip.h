@@ -62,7 +62,8 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
  * attnFlashMinT as a public field for the same purpose, webgpu.ts:305):
  *   "attn.generic" 1 = always take the shape-generic attention kernels, 0 = MFMA kernels where they apply
  *   "gemm.tile"    -1 = heuristic, 0..3 = pin the GEMM tile (64x64, 128x64, 128x128, 128x192)
- *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor */
+ *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor
+ *   "attn.splits"  -1 = heuristic, n >= 1 = pin the workgroups per attention tile (MFMA kernels, at most 8) */
 int gt_set_option(gt_ctx *ctx, const char *key, int value);
 
 /* ---- GEMM: srcGemm (src/backend/wgsl.ts:87-196), WebGPUBackend.gemm (webgpu.ts:1654) ---------
