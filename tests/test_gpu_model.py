@@ -100,6 +100,39 @@ def test_whole_model_two_micro_batches(gpu, ref, arch_name, stacked):
     compare(lh, gh, lr, gr, f"{arch_name} stacked={stacked}")
 
 
+REAL = {
+    # SmolLM2-135M layer geometry (9/3 heads x 64, hidden 576, SwiGLU 1536), two layers, reduced vocabulary
+    "smollm2": dict(arch="llama", vocab=4096, hidden=576, layers=2, heads=9, kv_heads=3, head_dim=64, ffn=1536,
+                    rope_base=1e5, rms_eps=1e-5),
+    # Qwen3 head layout: head dim 128 with QK-norm, GQA 4/2
+    "qwen3-hd128": dict(arch="qwen3", vocab=2048, hidden=256, layers=2, heads=4, kv_heads=2, head_dim=128, ffn=512,
+                        rope_base=1e6, rms_eps=1e-6),
+    # Gemma3: GeGLU, sliding window that cuts the 128-row attention tiles, one global layer in three
+    "gemma3-window": dict(arch="gemma3", vocab=2048, hidden=320, layers=3, heads=5, kv_heads=1, head_dim=64, ffn=768,
+                          rope_base=1e6, rope_base_local=1e4, sliding_window=96, swa_pattern=3, rms_eps=1e-6),
+}
+
+
+@pytest.mark.parametrize("name", sorted(REAL))
+@pytest.mark.parametrize("stacked", [False, True])
+def test_whole_model_real_head_geometry(gpu, ref, name, stacked):
+    """The shapes the tuned kernels are built for, inside whole graphs: matrix-core attention (head dims 64 and 128, GQA,
+    windows), the large GEMM tiles with split-K dW, row lengths of 576 / 1536 in the normalisation and gated-activation
+    kernels. Two sequences of 200 tokens (ragged against every tile size), masked targets, loss and every gradient."""
+    kw = REAL[name]
+    rmodel, model = build_pair(ref, kw, seed=11, std=0.05)
+    seqs = batches(ref, kw["vocab"], 200, 2, seed=12, mask_every=7)
+    lh, gh = hip_step(gpu, model, seqs, stacked, 200)
+    ref.PARALLEL_BWD = True
+    ref.set_threads(min(16, ref.max_threads()))
+    try:
+        lr, gr = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.PARALLEL_BWD = False
+        ref.set_threads(1)
+    compare(lh, gh, lr, gr, f"{name} stacked={stacked}")
+
+
 @pytest.mark.parametrize("arch_name", ["llama", "qwen3", "gemma3"])
 def test_recompute_is_bit_identical_and_matches(gpu, ref, arch_name):
     """gpu-parity.ts:536-564, 1299-1338: --recompute on/off gives bit-identical loss and gradients."""
