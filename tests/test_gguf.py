@@ -1,0 +1,274 @@
+"""GGUF checkpoint wire format (host side, no GPU): the container against bytes assembled by hand from the GGUF v3
+layout, the float16 conversion against IEEE half precision, the block formats against known blocks and error bounds,
+llama's Q/K row order against the Hugging Face -> GGUF permutation, and the reference's own round-trip test
+(tests/arch-roundtrip.ts) for the three architectures: config, weights bit for bit at f32, logits within 5 % at
+q8_0, resume-gate messages."""
+import importlib
+import struct
+
+import numpy as np
+import pytest
+
+G = importlib.import_module("gguf-trainer_amd.gguf")
+arch = importlib.import_module("gguf-trainer_amd.arch")
+
+
+def test_f16_to_f32_is_ieee_for_every_pattern():
+    bits = np.arange(65536, dtype=np.uint16)
+    got = G.f16_bits_to_f32(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.all(np.isnan(got[np.isnan(want)]))
+
+
+def test_f32_to_f16_rounding():
+    # every finite half value converts back to itself
+    bits = np.arange(65536, dtype=np.uint16)
+    finite = bits[(bits & 0x7C00) != 0x7C00]
+    assert np.array_equal(G.f32_to_f16_bits(finite.view(np.float16).astype(np.float32)), finite)
+    # random values: IEEE round-to-nearest-even wherever the result is a normal half or not an exact tie
+    rs = np.random.RandomState(0)
+    x = np.concatenate([(rs.standard_normal(200000) * 10.0 ** rs.randint(-6, 5, 200000)).astype(np.float32),
+                        np.float32([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e10, -1e10, np.inf, -np.inf, 2.0 ** -14, 2.0 ** -24,
+                                    2.0 ** -26, 1.0009765625, 1.00048828125, 1.001464843750])])
+    assert x.dtype == np.float32
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(G.f32_to_f16_bits(x), want)
+    assert G.f32_to_f16_bits(np.float32([np.nan]))[0] == 0x7E00
+    # subnormal halves round half UP in the reference (f16.ts:33-37): 2.5 x 2^-24 -> 3, where IEEE gives 2
+    assert G.f32_to_f16_bits(np.float32([2.5 * 2.0 ** -24, 1.5 * 2.0 ** -24, -2.5 * 2.0 ** -24])).tolist() == [3, 2, 0x8003]
+    # below 2^-25 is flushed to a signed zero, 2^-25 itself rounds up to the smallest subnormal
+    assert G.f32_to_f16_bits(np.float32([2.0 ** -26, -2.0 ** -26, 2.0 ** -25])).tolist() == [0, 0x8000, 1]
+
+
+def test_q4_0_known_block_and_layout():
+    x = np.concatenate([np.arange(-8, 8), np.arange(7, -9, -1)]).astype(np.float32)      # max |x| is -8: scale = -8 / -8 = 1
+    t, b = G.serialize(x, "q4_0")
+    assert t == G.Q4_0 and len(b) == 18
+    assert b[:2] == struct.pack("<H", 0x3C00)                                              # f16 1.0
+    nib = x.astype(int) + 8                                                                # floor(x + 8.5)
+    assert list(b[2:]) == [int(nib[j]) | (int(min(15, nib[j + 16])) << 4) for j in range(16)]
+    assert np.array_equal(G.dequantize(G.Q4_0, b, 32), x)
+    # +8 cannot be represented (nibble 16 clamps to 15 -> 7)
+    y = np.zeros(32, np.float32); y[0] = -8; y[1] = 8
+    assert G.dequantize(G.Q4_0, G.serialize(y, "q4_0")[1], 32)[1] == 7
+
+
+def test_q8_0_known_block_and_bounds():
+    x = (np.arange(32) - 16).astype(np.float32) * 127.0 / 16.0        # max |x| = 127 -> scale 1, q = round(x), halves up
+    t, b = G.serialize(x, "q8_0")
+    assert t == G.Q8_0 and len(b) == 34 and b[:2] == struct.pack("<H", 0x3C00)
+    q = np.frombuffer(b[2:], dtype=np.int8)
+    assert np.array_equal(q, np.floor(x.astype(np.float64) + 0.5).astype(np.int8))
+    assert q[15] == -8 and q[17] == 8                                  # -7.9375 -> -8, 7.9375 -> 8
+    rs = np.random.RandomState(1)
+    z = rs.standard_normal(32 * 50).astype(np.float32)
+    for quant, ttype, steps in (("q8_0", G.Q8_0, 127.0), ("q4_0", G.Q4_0, 8.0)):
+        back = G.dequantize(ttype, G.serialize(z, quant)[1], z.size)
+        amax = np.abs(z.reshape(-1, 32)).max(axis=1, keepdims=True)
+        # half a step of the block's scale (a whole step for q4_0's clamped top nibble), plus the f16 rounding of the scale
+        bound = amax / steps * (0.5 if quant == "q8_0" else 1.0) + amax * 2.0 ** -10
+        assert np.all(np.abs(back.reshape(-1, 32) - z.reshape(-1, 32)) <= bound), quant
+    assert np.all(G.dequantize(G.Q8_0, G.serialize(np.zeros(32, np.float32), "q8_0")[1], 32) == 0)
+    with pytest.raises(ValueError, match="multiple of 32"):
+        G.serialize(np.zeros(33, np.float32), "q8_0")
+
+
+def test_dequantize_refuses_short_and_unknown():
+    with pytest.raises(ValueError, match="need 34 bytes, got 20"):
+        G.dequantize(G.Q8_0, bytes(20), 32)
+    with pytest.raises(ValueError, match="Q4_K"):
+        G.dequantize(12, bytes(200), 32)
+    with pytest.raises(ValueError, match="count multiple of 32"):
+        G.dequantize(G.Q4_0, bytes(200), 33)
+    # padding after the payload is fine; bf16 widens by a 16-bit shift
+    assert np.array_equal(G.dequantize(G.F32, struct.pack("<2f", 1.5, -2.0) + bytes(24), 2), np.float32([1.5, -2.0]))
+    assert np.array_equal(G.dequantize(G.BF16, struct.pack("<2H", 0x3FC0, 0xC000), 2), np.float32([1.5, -2.0]))
+
+
+def test_container_bytes_against_the_gguf_v3_layout():
+    w = G.GGUFWriter()
+    w.meta_string("general.architecture", "llama").meta_u32("llama.block_count", 2).meta_f32("f", 0.5)
+    w.meta_bool("b", True).meta_arr_str("toks", ["a", "bc"]).meta_arr_i32("ty", [1, -3]).meta_i32("i", -7).meta_u64("u", 2 ** 40)
+    w.meta_arr_f32("af", [1.0])
+    w.add_tensor("t0", [3, 2], G.serialize(np.arange(6, dtype=np.float32), "f32"))
+    w.add_tensor("v", [5], G.serialize(np.float32([1, 2, 3, 4, 5]), "f16"))
+    got = w.build()
+
+    def s(x):
+        return struct.pack("<Q", len(x)) + x.encode()
+    exp = struct.pack("<IIQQ", 0x46554747, 3, 2, 10)
+    exp += s("general.architecture") + struct.pack("<I", 8) + s("llama")
+    exp += s("llama.block_count") + struct.pack("<II", 4, 2)
+    exp += s("f") + struct.pack("<If", 6, 0.5)
+    exp += s("b") + struct.pack("<IB", 7, 1)
+    exp += s("toks") + struct.pack("<IIQ", 9, 8, 2) + s("a") + s("bc")
+    exp += s("ty") + struct.pack("<IIQii", 9, 5, 2, 1, -3)
+    exp += s("i") + struct.pack("<Ii", 5, -7)
+    exp += s("u") + struct.pack("<IQ", 10, 2 ** 40)
+    exp += s("af") + struct.pack("<IIQf", 9, 6, 1, 1.0)
+    exp += s("general.alignment") + struct.pack("<II", 4, 32)                    # appended by build()
+    exp += s("t0") + struct.pack("<IQQIQ", 2, 3, 2, 0, 0)                        # n_dims, ne[0], ne[1], type F32, offset 0
+    exp += s("v") + struct.pack("<IQIQ", 1, 5, 1, 32)                            # 24 bytes of t0 padded to 32
+    exp += bytes(-len(exp) % 32)
+    exp += struct.pack("<6f", *range(6)) + bytes(8)
+    exp += struct.pack("<5H", 0x3C00, 0x4000, 0x4200, 0x4400, 0x4500) + bytes(22)
+    assert got == exp
+    g = G.read_gguf(got)
+    assert g.version == 3 and g.alignment == 32
+    assert list(g.metadata) == ["general.architecture", "llama.block_count", "f", "b", "toks", "ty", "i", "u", "af", "general.alignment"]
+    assert g.metadata["toks"] == ["a", "bc"] and g.metadata["ty"] == [1, -3] and g.metadata["u"] == 2 ** 40 and g.metadata["b"] is True
+    assert [(t["name"], t["dims"], t["type"], t["offset"], len(t["data"])) for t in g.tensors] == [("t0", [3, 2], 0, 0, 32), ("v", [5], 1, 32, 32)]
+    with pytest.raises(ValueError, match="bad magic"):
+        G.read_gguf(b"GGUX" + got[4:])
+
+
+def test_reorder_qk_is_the_hf_to_gguf_permutation():
+    heads, hd, ind = 3, 8, 5
+    w = np.arange(heads * hd * ind, dtype=np.float32).reshape(heads * hd, ind)
+    out = G.reorder_qk(w, heads, hd, True)
+    # llama.cpp's converter: weights.reshape(n_head, 2, hd/2, in).swapaxes(1, 2).reshape(weights.shape)
+    assert np.array_equal(out, w.reshape(heads, 2, hd // 2, ind).swapaxes(1, 2).reshape(w.shape))
+    assert np.array_equal(G.reorder_qk(out, heads, hd, False), w)
+    assert not np.array_equal(G.reorder_qk(out, heads, hd, True), w)               # not idempotent
+    with pytest.raises(ValueError, match="does not tile"):
+        G.reorder_qk(w, 5, hd, True)
+
+
+TOK = dict(tokens=["<|bos|>", "<|eos|>", "<think>", "a", "b", "ab"] + [f"t{i}" for i in range(26)], merges=["a b"], bosId=0, eosId=1,
+           specials=["<|bos|>", "<|eos|>", "<think>"])
+# rms_eps and rope bases are powers of two or small integers here: the file stores them as f32, and a value that f32
+# cannot hold comes back rounded, which moves a logit by an ulp now and then and would blur the bit-for-bit check
+CFGS = {
+    "llama": dict(arch="llama", vocab=32, hidden=32, layers=2, heads=2, kv_heads=1, head_dim=16, ffn=64, rope_base=1e5, rms_eps=2.0 ** -17),
+    "llama-untied": dict(arch="llama", vocab=32, hidden=32, layers=1, heads=4, kv_heads=2, head_dim=8, ffn=32, rope_base=1e5, rms_eps=2.0 ** -17, tie=False),
+    "qwen3": dict(arch="qwen3", vocab=32, hidden=32, layers=2, heads=2, kv_heads=1, head_dim=32, ffn=64, rope_base=1e6, rms_eps=2.0 ** -20),
+    "gemma3": dict(arch="gemma3", vocab=32, hidden=32, layers=2, heads=2, kv_heads=1, head_dim=16, ffn=64, rope_base=1e6,
+                   rope_base_local=1e4, sliding_window=4, swa_pattern=2, rms_eps=2.0 ** -20),
+    # hidden 8: the block formats cannot tile an inner dimension of 8 and every matrix falls back to f16
+    "llama-narrow": dict(arch="llama", vocab=32, hidden=8, layers=2, heads=2, kv_heads=1, head_dim=4, ffn=16, rope_base=1e5, rms_eps=2.0 ** -17),
+}
+
+
+def _model(kw, seed=7):
+    cfg = arch.ModelConfig(**kw)
+    rs = np.random.RandomState(seed)
+    weights = {}
+    for n in arch.param_names(cfg):
+        shp = arch.param_shape(cfg, n)
+        weights[n] = (1 + 0.1 * rs.standard_normal(shp) if len(shp) == 1 else 0.05 * rs.standard_normal(shp)).astype(np.float32)
+    return arch.Model(cfg, weights)
+
+
+def _logits(ref, model, ids):
+    rcfg = ref.ModelConfig(**{k: getattr(model.cfg, k) for k in model.cfg.__dataclass_fields__})
+    rm = ref.Model(rcfg, weights={n: p.data.reshape(p.shape) for n, p in model.named_params()})
+    return rm.forward(ids).data.copy()
+
+
+@pytest.mark.parametrize("name", sorted(CFGS))
+def test_architecture_round_trip(ref, name):
+    """tests/arch-roundtrip.ts:49-123."""
+    model = _model(CFGS[name])
+    ids = [1, 5, 2, 9, 5, 3, 8]
+    before = _logits(ref, model, ids)
+    for quant, tol in (("f32", 0.0), ("f16", 0.01), ("q8_0", 0.05)):
+        blob = G.export_gguf(model, TOK, quant, max_seq=16)
+        loaded, cfg, max_seq, tok = G.load_model_from_gguf(blob)
+        assert cfg.arch == model.cfg.arch and max_seq == 16
+        assert G.config_matches(model.cfg, cfg, 16, max_seq) is None, quant            # floats to f32 precision
+        assert cfg.tie == model.cfg.tie and cfg.vocab == 32
+        assert tok["tokens"] == TOK["tokens"] and tok["merges"] == TOK["merges"] and tok["specials"] == TOK["specials"]
+        after = _logits(ref, loaded, ids)
+        if quant == "f32":
+            for (n, a), (_, b) in zip(model.named_params(), loaded.named_params()):
+                assert a.data.tobytes() == b.data.tobytes(), n
+            assert before.tobytes() == after.tobytes()
+        else:
+            assert np.abs(before - after).max() / np.abs(before).max() <= tol, quant
+    g = G.read_gguf(G.export_gguf(model, TOK, "q8_0", max_seq=16))
+    types = {t["name"]: t["type"] for t in g.tensors}
+    assert types["output_norm.weight"] == G.F32 and types["blk.0.attn_norm.weight"] == G.F32
+    assert types["blk.0.ffn_up.weight"] == (G.F16 if name == "llama-narrow" else G.Q8_0)
+    assert g.metadata["general.file_type"] == 7 and g.metadata["tokenizer.ggml.token_type"][:4] == [3, 3, 4, 1]
+    by = {t["name"]: t for t in g.tensors}
+    assert by["token_embd.weight"]["dims"] == [model.cfg.hidden, 32]                    # ggml order: [in, out]
+    assert ("output.weight" in by) == (not model.cfg.tie)
+
+
+def test_llama_export_stores_q_and_k_in_llama_cpp_row_order():
+    model = _model(CFGS["llama"])
+    g = G.read_gguf(G.export_gguf(model, TOK, "f32"))
+    by = {t["name"]: t for t in g.tensors}
+    c = model.cfg
+    q = G.dequantize(0, by["blk.1.attn_q.weight"]["data"], c.heads * c.head_dim * c.hidden).reshape(c.heads * c.head_dim, c.hidden)
+    mine = model.layers[1]["qProj"].data.reshape(c.heads * c.head_dim, c.hidden)
+    assert np.array_equal(q[0], mine[0]) and np.array_equal(q[1], mine[c.head_dim // 2]) and np.array_equal(q[2], mine[1])
+    v = G.dequantize(0, by["blk.1.attn_v.weight"]["data"], c.kv_heads * c.head_dim * c.hidden)
+    assert np.array_equal(v, model.layers[1]["vProj"].data.reshape(-1))                 # V is not permuted
+    # qwen3 rotates half-split in llama.cpp too: no permutation
+    m3 = _model(CFGS["qwen3"])
+    g3 = {t["name"]: t for t in G.read_gguf(G.export_gguf(m3, TOK, "f32")).tensors}
+    assert np.array_equal(G.dequantize(0, g3["blk.0.attn_q.weight"]["data"], m3.layers[0]["qProj"].size), m3.layers[0]["qProj"].data.reshape(-1))
+
+
+def test_metadata_keys_and_order_per_architecture():
+    keys = list(G.read_gguf(G.export_gguf(_model(CFGS["gemma3"]), TOK, "f32", max_seq=64)).metadata)
+    assert keys[:3] == ["general.architecture", "general.name", "general.file_type"]
+    a = [k for k in keys if k.startswith("gemma3.")]
+    assert a == ["gemma3." + k for k in ("context_length", "embedding_length", "block_count", "feed_forward_length", "attention.head_count",
+                                         "attention.head_count_kv", "attention.key_length", "attention.value_length",
+                                         "attention.layer_norm_rms_epsilon", "attention.sliding_window", "attention.sliding_window_pattern",
+                                         "rope.freq_base", "rope.freq_base_swa", "vocab_size")]
+    assert keys[-1] == "general.alignment"
+    names = [t["name"] for t in G.read_gguf(G.export_gguf(_model(CFGS["gemma3"]), TOK, "f32")).tensors]
+    assert names[:2] == ["token_embd.weight", "output_norm.weight"]
+    assert names[2:15] == ["blk.0." + k + ".weight" for k in ("attn_norm", "attn_q", "attn_k", "attn_v", "attn_q_norm", "attn_k_norm", "attn_output",
+                                                              "post_attention_norm", "ffn_norm", "ffn_gate", "ffn_up", "ffn_down", "post_ffw_norm")]
+    lk = [k for k in G.read_gguf(G.export_gguf(_model(CFGS["llama"]), TOK, "f32")).metadata if k.startswith("llama.")]
+    assert lk[-3:] == ["llama.rope.dimension_count", "llama.rope.freq_base", "llama.vocab_size"]
+
+
+def test_resume_gate_messages_and_loader_errors():
+    """arch-roundtrip.ts:125-190 and common.ts:134-181."""
+    c = arch.ModelConfig(**CFGS["llama"])
+    R = lambda **kw: arch.ModelConfig(**{**CFGS["llama"], **kw})
+    assert "layers" in G.config_matches(c, R(layers=3))
+    assert G.config_matches(c, c) is None
+    assert "rope-base" in G.config_matches(R(rope_base=1e5), R(rope_base=1e6))
+    assert "rope-base" in G.config_matches(R(rope_base=1_000_000), R(rope_base=1_000_001))
+    assert "rope-base" in G.config_matches(R(rope_base=1e8), R(rope_base=1e8 + 8))       # one f32 ulp at 1e8
+    assert G.config_matches(R(rope_base=1e8), R(rope_base=1e8 + 1)) is None               # below what the file can hold
+    assert "rms-eps" in G.config_matches(R(rms_eps=1e-5), R(rms_eps=2e-5))
+    assert G.config_matches(c, R(tie=False)) == "untied-embeddings: built false vs checkpoint true"
+    assert "max-seq" in G.config_matches(c, c, 16, 32)
+    g3 = arch.ModelConfig(**CFGS["gemma3"])
+    assert G.config_matches(g3, arch.ModelConfig(**{**CFGS["gemma3"], "head_dim": 32, "heads": 1})).startswith("head-dim")
+    assert G.config_matches(g3, arch.ModelConfig(**{**CFGS["gemma3"], "sliding_window": 8})).startswith("window")
+    blob = G.export_gguf(_model(CFGS["llama"]), TOK, "f32")
+    g = G.read_gguf(blob)
+    load = G.tensor_loader(g)
+    with pytest.raises(ValueError, match='missing tensor "nope"'):
+        load("nope", [3])
+    with pytest.raises(ValueError, match="has dims"):
+        load("output_norm.weight", [16])                      # a prefix of the stored tensor must not load silently
+    with pytest.raises(ValueError, match="has dims"):
+        load("token_embd.weight", [32 * 32])                   # same element count, different rank
+    with pytest.raises(ValueError, match="has dims"):
+        load("blk.0.ffn_up.weight", [32, 64])                  # transposed
+    assert load("output_norm.weight", [1, 32]).shape == (1, 32)          # ggml dims [32, 1]: a trailing one is no difference
+    # a non-integer rope base comes back as its f32 rounding and still matches the flag value (arch-roundtrip.ts:131-144)
+    odd = _model({**CFGS["llama"], "rope_base": 12345.6789})
+    _, back, _, _ = G.load_model_from_gguf(G.export_gguf(odd, TOK, "f32"))
+    assert back.rope_base != 12345.6789 and back.rope_base == float(np.float32(12345.6789))
+    assert G.config_matches(odd.cfg, back) is None
+    g.metadata.pop("llama.block_count")
+    with pytest.raises(ValueError, match='missing numeric metadata "llama.block_count"'):
+        G.config_from_gguf(g)
+    # optional llama keys fall back: key_length to hidden / heads, rope base to 10000, vocab to the token list
+    g = G.read_gguf(blob)
+    for k in ("llama.attention.key_length", "llama.rope.freq_base", "llama.vocab_size"):
+        g.metadata.pop(k)
+    cfg, _ = G.config_from_gguf(g)
+    assert cfg.head_dim == 16 and cfg.rope_base == 10000 and cfg.vocab == len(TOK["tokens"])

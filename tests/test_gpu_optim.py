@@ -165,3 +165,53 @@ def test_fifty_step_loss_curve(gpu, ref):
     worst = max(abs(a - b) / abs(b) for a, b in zip(hh, rh))
     assert worst <= 1e-3, worst
     assert rh[-1] < rh[0]
+
+
+@pytest.mark.parametrize("which", ["llama_adamw", "gemma3_muon"])
+def test_resume_through_gguf_and_optstate_is_bit_identical(gpu, ref, which):
+    """A run checkpointed after two steps as an F32 GGUF (llama: Q/K rows permuted out and back) plus the .optstate
+    sidecar bytes, rebuilt from those bytes alone and continued for two more steps, ends on the same losses and the same
+    weights, bit for bit, as the uninterrupted four-step run. rms_eps is a power of two: the file stores it as f32."""
+    optim, train, arch, gguf = mod("optim"), mod("train"), mod("arch"), mod("gguf")
+    kw = dict(SMALL["gemma3" if which == "gemma3_muon" else "llama"], rms_eps=2.0 ** -20)
+    seqs = batches(ref, kw["vocab"], 21, 8, seed=21, mask_every=6)
+    sched = ref.wsd_schedule(1, 1, 2, 0.1)
+    tok = dict(tokens=[f"t{i}" for i in range(kw["vocab"])], merges=[], bosId=0, eosId=1)
+
+    def make_opt(model):
+        if which == "llama_adamw":
+            return optim.AdamWHip(gpu, model.params(), lr=1e-3, beta2=0.95, weight_decay=0.1)
+        hm, ha = model.param_groups()
+        return optim.MuonHip(gpu, hm, ha, lr=0.01, aux={"lr": 3e-3})
+
+    def state_bytes(opt):
+        st = opt.export_state()
+        if which == "llama_adamw":
+            st = {"muonMomentum": [], "adamM": st["m"], "adamV": st["v"], "adamT": st["t"]}
+        return optim.serialize_opt_state(st)
+
+    def restore(opt, raw):
+        st = optim.deserialize_opt_state(raw)
+        opt.import_state({"m": st["adamM"], "v": st["adamV"], "t": st["adamT"]} if which == "llama_adamw" else st)
+
+    _, full = build_pair(ref, kw, seed=8, std=0.1)
+    fopt = make_opt(full)
+    hist_full = train.train_lm_hip_resident(full, gpu, fopt, seqs, 4, 2, 21, schedule=sched, stacked=True)
+    fopt.sync_weights_to_host()
+
+    _, first = build_pair(ref, kw, seed=8, std=0.1)
+    opt1 = make_opt(first)
+    hist_a = train.train_lm_hip_resident(first, gpu, opt1, seqs[:4], 2, 2, 21, schedule=sched, stacked=True)
+    opt1.sync_weights_to_host()
+    blob, side = gguf.export_gguf(first, tok, "f32", max_seq=64), state_bytes(opt1)
+    del first, opt1
+
+    second, cfg, max_seq, _ = gguf.load_model_from_gguf(blob)
+    assert gguf.config_matches(arch.ModelConfig(**kw), cfg, 64, max_seq) is None
+    opt2 = make_opt(second)
+    restore(opt2, side)
+    hist_b = train.train_lm_hip_resident(second, gpu, opt2, seqs[4:], 2, 2, 21, schedule=lambda s: sched(s + 2), stacked=True)
+    opt2.sync_weights_to_host()
+    assert hist_a + hist_b == hist_full
+    for n, p in full.named_params():
+        assert second.p[n].data.tobytes() == p.data.tobytes(), n
