@@ -107,13 +107,35 @@ def cpu_baseline(seconds_hint=20.0):
     finally:
         ref.PARALLEL_BWD = False
         ref.set_threads(1)
+    # the reference's CPU path is single-threaded: the literal serial loops, one thread, one layer at T = 256
+    T1 = 256
+    h1 = ref.Tensor(0.02 * rs.standard_normal((T1, cfg.hidden)).astype(np.float32), [T1, cfg.hidden], True)
+    t0 = time.perf_counter()
+    o1 = model._block(h1, model.layers[0], 0, T1)()
+    ref.backward_from(o1, np.ones(o1.size, np.float32))
+    t_layer_1t = time.perf_counter() - t0
+    ref.set_threads(cores)
+    ref.PARALLEL_BWD = True
+    try:
+        h1 = ref.Tensor(h1.data.copy(), [T1, cfg.hidden], True)
+        t0 = time.perf_counter()
+        o1 = model._block(h1, model.layers[0], 0, T1)()
+        ref.backward_from(o1, np.ones(o1.size, np.float32))
+        t_layer_mt = time.perf_counter() - t0
+    finally:
+        ref.PARALLEL_BWD = False
+        ref.set_threads(1)
     t_head = max(t_all - t_layers, 0.0)
     n_layer_params = sum(p.size for Lw in model.layers for p in Lw.values())
     n_head_params = model.tokenEmbd.size + model.outputNorm.size
     t_opt_full = t_opt * (n_head_params + n_layer_params / L * 30) / (n_head_params + n_layer_params)
     # one optimizer step serves BATCH*SEQ tokens
     per_token = (t_layers / L * 30 + t_head) / T + t_opt_full / (BATCH * SEQ)
+    slowdown = t_layer_1t / max(t_layer_mt, 1e-9)
     return {"value": round(1.0 / per_token, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "single_thread": {"value": round(1.0 / per_token / slowdown, 2), "unit": "tokens/s", "cores": 1,
+                              "sample": f"one layer fwd+bwd at T={T1}: serial loops on 1 thread {t_layer_1t:.2f}s, the same layer "
+                                        f"on {cores} threads {t_layer_mt:.2f}s; the {cores}-thread figure divided by that ratio"},
             "sample": f"oracle (C restatement of the reference's CPU ops), 1 sequence x {T} tokens through {L} of 30 layers "
                       f"fwd+bwd ({t_layers:.1f}s) + full readout and cross-entropy ({t_head:.1f}s) + AdamW ({t_opt:.1f}s); "
                       f"per-token time extrapolated to 30 layers; attention is O(T) per token so T=2048 would be slower"}
