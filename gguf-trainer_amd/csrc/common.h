@@ -34,6 +34,9 @@ struct gt_ctx {
   bool prof_on = false;
   std::string prof_prefix;
   std::vector<ProfEvent> prof;
+  int opt_prof_sample = 1;                      // events around every n-th launch of a label
+  struct ProfSeen { int64_t n = 0; double work = 0; };
+  std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not
 };
 
 extern thread_local char g_create_err[512];
@@ -55,6 +58,14 @@ struct ProfScope {
   ProfScope(gt_ctx *ctx, const char *label, double work = 0) : c(ctx), on(ctx->prof_on) {
     if (on && !ctx->prof_prefix.empty() && strncmp(label, ctx->prof_prefix.c_str(), ctx->prof_prefix.size()) != 0) on = false;
     if (!on) return;
+    // an event pair costs the stream about as much as a small kernel: with sampling only about 1 in n launches of a
+    // label is timed and gt_prof_end scales the timed sum up to the work of all of them. Which launches: a fixed
+    // pseudo-random choice over the label's launch numbers, so that a label whose launches cycle through a few
+    // shapes is not sampled in step with the cycle.
+    auto &seen = ctx->prof_seen[label];
+    const uint32_t nth = (uint32_t)(seen.n++);
+    seen.work += work;
+    if (ctx->opt_prof_sample > 1 && ((nth * 2654435761u) >> 15) % (uint32_t)ctx->opt_prof_sample != 0) { on = false; return; }
     ProfEvent e; e.label = label; e.work = work;
     (void)hipEventCreate(&e.a); (void)hipEventCreate(&e.b);
     (void)hipEventRecord(e.a, c->stream);

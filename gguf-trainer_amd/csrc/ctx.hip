@@ -123,6 +123,7 @@ int gt_set_option(gt_ctx *ctx, const char *key, int value) {
   if (!ctx || !key) return 1;
   if (!strcmp(key, "attn.generic")) ctx->opt_attn_generic = value;
   else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
+  else if (!strcmp(key, "prof.sample")) ctx->opt_prof_sample = value >= 1 ? value : 1;
   else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
   else if (!strcmp(key, "gemm.splitk")) ctx->opt_gemm_splitk = value;
   else GT_FAIL(ctx, "gt_set_option: unknown key '%s'", key);
@@ -134,6 +135,7 @@ int gt_prof_begin(gt_ctx *ctx, const char *prefix) {
   ctx->prof_prefix = prefix ? prefix : "";
   for (auto &e : ctx->prof) { hipEventDestroy(e.a); hipEventDestroy(e.b); }
   ctx->prof.clear();
+  ctx->prof_seen.clear();
   ctx->prof_on = true;
   return 0;
 }
@@ -159,9 +161,13 @@ int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n) {
   for (auto &l : order) {
     if (k >= cap) break;
     snprintf(out[k].label, sizeof out[k].label, "%s", l.c_str());
-    out[k].ms = sum[l].ms;
-    out[k].count = sum[l].n;
-    out[k].work = sum[l].work;
+    // count and work = every launch of the label; time = the timed launches' time scaled by all work / timed work
+    // (by all launches / timed launches for a label that states no work)
+    const auto &seen = ctx->prof_seen[l];
+    const double scale = sum[l].work > 0 ? seen.work / sum[l].work : (double)seen.n / (double)sum[l].n;
+    out[k].ms = sum[l].ms * scale;
+    out[k].count = seen.n;
+    out[k].work = seen.work;
     k++;
   }
   if (n) *n = k;

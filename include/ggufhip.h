@@ -63,7 +63,8 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
  *   "attn.generic" 1 = always take the shape-generic attention kernels, 0 = MFMA kernels where they apply
  *   "gemm.tile"    -1 = heuristic, 0..3 = pin the GEMM tile (64x64, 128x64, 128x128, 128x192)
  *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor
- *   "attn.splits"  -1 = heuristic, n >= 1 = pin the workgroups per attention tile (MFMA kernels, at most 8) */
+ *   "attn.splits"  -1 = heuristic, n >= 1 = pin the workgroups per attention tile (MFMA kernels, at most 8)
+ *   "prof.sample"  n >= 1: gt_prof_begin/end time about 1 in n launches of a label (default 1 = all) */
 int gt_set_option(gt_ctx *ctx, const char *key, int value);
 
 /* ---- GEMM: srcGemm (src/backend/wgsl.ts:87-196), WebGPUBackend.gemm (webgpu.ts:1654) ---------
@@ -180,7 +181,10 @@ int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out)
  * bracketed by HIP events on the context's stream and summed per label, together with the
  * algorithmic work the call states for itself (FLOP for the contractions, bytes for the streaming
  * kernels). GEMM labels carry the kernel's tile shape ("gemm.nn.128x192"). gt_prof_end waits, then
- * fills up to `cap` records. */
+ * fills up to `cap` records. An event pair delays the stream by a few microseconds; with the option
+ * "prof.sample" = n about 1 in n launches of a label is bracketed (a fixed pseudo-random choice over
+ * the label's launch numbers); `count` and `work` still cover every launch and `ms` is the timed
+ * launches' time scaled by all work / timed work. */
 typedef struct gt_prof_rec { char label[32]; double ms; int64_t count; double work; } gt_prof_rec;
 int gt_prof_begin(gt_ctx *ctx, const char *prefix);
 int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n);
