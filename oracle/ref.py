@@ -672,7 +672,57 @@ def attach_lora(model: Model, rank: int, alpha: float, rng: Mulberry32, a_std: f
     return m, params
 
 
-def train_lm(model: Model, optimizer, windows, batch_per_step: int, steps: int, loss_chunk=0, schedule=None):
+def qk_logit_scale(q_norm, k_norm, head_dim: int) -> float:
+    """src/train/qk-clip.ts:32-39: sqrt(sum_d (qNorm[d]*kNorm[d])^2) / sqrt(headDim), doubles over f32 gains."""
+    s = 0.0
+    for d in range(head_dim):
+        p = float(q_norm[d]) * float(k_norm[d])
+        s += p * p
+    return math.sqrt(s) / math.sqrt(head_dim)
+
+
+def apply_qk_clip(model: Model, tau: float) -> int:
+    """src/train/qk-clip.ts:46-66: a layer whose proxy s exceeds tau has qNorm and kNorm multiplied by
+    sqrt(tau/s) element by element (f32 stores), so the proxy lands on tau; returns the layers clipped."""
+    if not tau > 0:
+        raise ValueError("qk-clip tau must be > 0")
+    pairs = model.qk_norms()
+    if not pairs:
+        return 0
+    hd = model.cfg.head_dim
+    clipped = 0
+    for qn, kn in pairs:
+        s = qk_logit_scale(qn.data, kn.data, hd)
+        if s > tau:
+            f = math.sqrt(tau / s)
+            for d in range(hd):
+                qn.data[d] = np.float32(float(qn.data[d]) * f)
+                kn.data[d] = np.float32(float(kn.data[d]) * f)
+            clipped += 1
+    return clipped
+
+
+def draw_windows(tokens, seq_len: int, rng, count: int, supervised=None):
+    """The windows src/train/trainer.ts:56-70 draws: start = floor(rng() * (len - seq_len - 1)), inputs
+    tokens[start:start+T], targets tokens[start+1:start+1+T] with unsupervised positions set to -1
+    (maskWindow, trainer.ts:45-49). `rng` is a callable returning the next uniform."""
+    max_start = len(tokens) - seq_len - 1
+    if max_start <= 0:
+        raise ValueError("Not enough tokens for one training window")
+    out = []
+    for _ in range(count):
+        start = int(math.floor(rng() * max_start))
+        ids = [int(t) for t in tokens[start:start + seq_len]]
+        tg = [int(t) for t in tokens[start + 1:start + 1 + seq_len]]
+        if supervised is not None:
+            m = supervised[start + 1:start + 1 + seq_len]
+            tg = [t if m[k] else -1 for k, t in enumerate(tg)]
+        out.append((ids, tg))
+    return out
+
+
+def train_lm(model: Model, optimizer, windows, batch_per_step: int, steps: int, loss_chunk=0, schedule=None,
+             qk_clip_tau: float = 0.0):
     """src/train/trainer.ts:51-87 with the window sampling hoisted: `windows` yields
     (input_ids, target_ids) in the order the reference's rng would have drawn them."""
     hist = []
@@ -688,5 +738,7 @@ def train_lm(model: Model, optimizer, windows, batch_per_step: int, steps: int, 
             backward(loss, 1 / batch_per_step)
             loss_sum += float(loss.data[0])
         optimizer.step()
+        if qk_clip_tau:
+            apply_qk_clip(model, qk_clip_tau)
         hist.append(loss_sum / batch_per_step)
     return hist

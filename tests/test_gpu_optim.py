@@ -215,3 +215,72 @@ def test_resume_through_gguf_and_optstate_is_bit_identical(gpu, ref, which):
     assert hist_a + hist_b == hist_full
     for n, p in full.named_params():
         assert second.p[n].data.tobytes() == p.data.tobytes(), n
+
+
+# microConfig() of gpu-parity.ts:307-325
+MICRO = dict(arch="gemma3", vocab=50, hidden=32, layers=2, heads=4, kv_heads=2, head_dim=8, ffn=64, rope_base=1e6,
+             rope_base_local=1e4, rms_eps=1e-6, sliding_window=32, swa_pattern=2)
+MUON_HYPER = dict(lr=0.02, momentum=0.95, aux={"lr": 3e-3, "weight_decay": 0.0, "clip": 1.0})
+
+
+def micro_tokens(ref, seed):
+    r = ref.Mulberry32(seed)
+    return [int(math.floor(r() * MICRO["vocab"])) for _ in range(160)]
+
+
+@pytest.mark.parametrize("stacked", [False, True])
+def test_qk_clip_trajectory(gpu, ref, stacked):
+    """gpu-parity.ts:1233-1289: the logit clip is host math on the QK-norm gains between optimizer steps; tau = 0.5
+    triggers from initialisation (gains of one give proxy 1), so every step clips on both paths, windows are drawn
+    from the same token array by the same generator, and the trained model's proxies end at or under tau."""
+    ag, optim, train = mod("autograd"), mod("optim"), mod("train")
+    tokens = micro_tokens(ref, 0x70CC)
+    rmodel, model = build_pair(ref, MICRO, seed=5, jitter_gains=False)
+    rm, ra = rmodel.param_groups()
+    hm, ha = model.param_groups()
+    ropt = ref.Muon(rm, ra, **MUON_HYPER)
+    hopt = optim.MuonHip(gpu, hm, ha, **MUON_HYPER)
+    rh = ref.train_lm(rmodel, ropt, ref.draw_windows(tokens, 8, ref.Mulberry32(7), 8), 2, 4, qk_clip_tau=0.5)
+    log = []
+    hh = train.train_lm_hip_resident(model, gpu, hopt, train.WindowSampler(tokens, 8, ag.mulberry32(7)), 4, 2, 8,
+                                     stacked=stacked, qk_clip_tau=0.5, history=log)
+    assert [r["step"] for r in log] == [0, 1, 2, 3] and [r["loss"] for r in log] == hh
+    for a, b in zip(hh, rh):
+        assert abs(a - b) <= 1e-3 + 1e-3 * abs(b), (hh, rh)
+    for n, p in rmodel.named_params():
+        assert_close(model.p[n].data, p.data, f"qk-clip trajectory weight {n}", rel_l2=1e-3, max_rel=2e-2)
+    for q, k in model.qk_norms():
+        assert train.qk_logit_scale(q.data, k.data, MICRO["head_dim"]) <= 0.5 + 1e-4
+    # and without the clip the gains would have stayed near one: the clip is what moved them
+    assert max(float(np.abs(q.data).max()) for q, _ in model.qk_norms()) < 0.9
+
+
+def test_checkpoint_cadence(gpu, ref):
+    """gpu-parity.ts:2512-2563: the step trigger and the wall-clock trigger are ORed, never fire at step 0, and
+    the weights are on the host when the callback runs."""
+    ag, optim, train = mod("autograd"), mod("optim"), mod("train")
+    tokens = micro_tokens(ref, 0x5EC2)
+
+    def fired_at(**cadence):
+        _, model = build_pair(ref, MICRO, seed=5, jitter_gains=False)
+        hm, ha = model.param_groups()
+        hit, moved = [], []
+        w0 = model.p["tokenEmbd"].data.copy() if "tokenEmbd" in model.p else None
+
+        def on_checkpoint(step):
+            hit.append(step)
+            if w0 is not None:
+                moved.append(not np.array_equal(model.p["tokenEmbd"].data, w0))
+        train.train_lm_hip_resident(model, gpu, optim.MuonHip(gpu, hm, ha, **MUON_HYPER),
+                                    train.WindowSampler(tokens, 8, ag.mulberry32(7)), 6, 1, 8, log_every=100,
+                                    on_checkpoint=on_checkpoint, **cadence)
+        assert all(moved)               # trained weights, not the initial host copy
+        return hit
+
+    # a step takes milliseconds, so 1e-3 ms is due at every step and 1e9 ms at none
+    assert fired_at(checkpoint_every=2) == [2, 4]
+    assert fired_at(checkpoint_every_ms=1e-3) == [1, 2, 3, 4, 5]
+    assert fired_at(checkpoint_every=2, checkpoint_every_ms=1e9) == [2, 4]
+    assert fired_at(checkpoint_every=10 ** 9, checkpoint_every_ms=1e-3) == [1, 2, 3, 4, 5]
+    assert fired_at() == []
+    assert fired_at(checkpoint_every_ms=1e9) == []
