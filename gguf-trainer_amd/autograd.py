@@ -219,9 +219,9 @@ _lora: dict = {}
 
 
 def set_lora_adapters(m: dict):
-    """m: id(weight) -> (a [rank,in], b [out,rank], scale)."""
+    """m: id(weight) -> (a [rank,in], b [out,rank], scale); None or {} removes every adapter."""
     global _lora
-    _lora = m
+    _lora = m or {}
 
 
 def linear(x: Tensor, w: Tensor) -> Tensor:

@@ -198,9 +198,9 @@ _lora: dict[int, tuple] = {}
 
 
 def set_lora_adapters(m: dict):
-    """m maps id(weight tensor) -> (a, b, scale)."""
+    """m maps id(weight tensor) -> (a, b, scale); None or {} removes every adapter."""
     global _lora
-    _lora = m
+    _lora = m or {}
 
 
 def linear(x: Tensor, w: Tensor) -> Tensor:

@@ -142,10 +142,11 @@ def test_rms_norm(gpu, ref, rows, d):
             f"rmsNorm frozen gain {rows}x{d}", frozen=(1,))
 
 
-@pytest.mark.parametrize("T,H,hd", [(3, 2, 4), (17, 9, 64), (20, 16, 128), (11, 3, 32), (5, 2, 6)])
+@pytest.mark.parametrize("T,H,hd", [(3, 2, 4), (17, 9, 64), (20, 16, 128), (11, 3, 32), (5, 2, 6), (8200, 8, 4)])
 def test_rms_norm_heads(gpu, ref, T, H, hd):
     r = R(ref, T + hd)
     w = 1 + 0.3 * r(hd)
+    # (8200, 8, 4): 65600 rows, the count past one grid dimension's 65535 that gpu-parity.ts:690-702 folds into two
     op_case(gpu, ref, [r(T, H * hd), w], lambda ag, x, g: ag.rms_norm_heads(x, g, T, H, hd, 1e-6),
             lambda rf, x, g: rf.rms_norm_heads(x, g, T, H, hd, 1e-6), f"rmsNormHeads {T},{H},{hd}")
 
@@ -408,3 +409,46 @@ def test_attention_mfma_equals_generic_at_full_length(gpu, ref):
         res.append((out.data.copy(), hq.grad.copy(), hk.grad.copy(), hv.grad.copy()))
     for a, b, nm in zip(res[1], res[0], ("out", "dq", "dk", "dv")):
         assert_close(a, b, f"mfma vs generic {nm}")
+
+
+def test_flat_elementwise_past_65535_workgroups(gpu, ref):
+    """gpu-parity.ts:217-239: add over n = 65535*256 + 777 elements, every element exact."""
+    ag = mod("autograd")
+    n = 65535 * 256 + 777
+    a = ag.Tensor(np.full(n, 1.0, np.float32), [n], False)
+    b = ag.Tensor(np.full(n, 2.0, np.float32), [n], False)
+    gpu.install()
+    try:
+        y = ag.add(a, b)
+        gpu.sync([y])
+        assert int(np.count_nonzero(y.data != 3.0)) == 0
+    finally:
+        gpu.uninstall()
+        gpu.sync([])
+
+
+@pytest.mark.parametrize("sample", [1, 3])
+def test_profiler_labels_times_and_sampling(gpu, ref, sample):
+    """gpu-parity.ts:134-156: profile silu(linear(x, w)) with the default prefix: both kernels are reported with
+    non-negative times and positive counts. With sampling, counts and stated work still cover every launch."""
+    ag = mod("autograd")
+    r = R(ref, 5)
+    x, w = ag.Tensor(r(40, 48), [40, 48], True), ag.Tensor(r(40, 48), [40, 48], True)
+    gpu.install()
+    try:
+        gpu.set_option("prof.sample", sample)
+        gpu.start_profile()
+        for _ in range(7):
+            y = ag.silu(ag.linear(x, w))
+            gpu.sync([y])
+        prof = gpu.stop_profile()
+    finally:
+        gpu.set_option("prof.sample", 1)
+        gpu.uninstall()
+        gpu.sync([])
+    gemm = [k for k in prof if k.startswith("gemm.nt.")]
+    assert len(gemm) == 1 and "silu" in prof, prof
+    for label in (gemm[0], "silu"):
+        ms, count, work = prof[label]
+        assert ms >= 0 and count == 7
+    assert prof[gemm[0]][2] == 7 * 2 * 40 * 40 * 48
