@@ -136,3 +136,87 @@ def test_glu_backward_full_size(gpu, ref):
     assert_close(out.data, ro.data, "SwiGLU full out")
     assert_close(ha.grad, ra.grad, "SwiGLU full dgate")
     assert_close(hb2.grad, rb.grad, "SwiGLU full dup")
+
+
+FULL = {
+    # BASELINE configs 4, 3 and 5 at their real shapes
+    "smollm2": dict(model=dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
+                               rope_base=1e5, rms_eps=1e-5), batch=8),
+    "gemma3": dict(model=dict(arch="gemma3", vocab=32768, hidden=640, layers=12, heads=10, kv_heads=2, head_dim=64, ffn=2048,
+                              rope_base=1e6, rope_base_local=1e4, sliding_window=512, swa_pattern=6, rms_eps=1e-6), batch=8),
+    "qwen3_lora": dict(model=dict(arch="qwen3", vocab=151936, hidden=1024, layers=28, heads=16, kv_heads=8, head_dim=128, ffn=3072,
+                                  rope_base=1e6, rms_eps=1e-6), batch=4, lora=16),
+}
+
+
+@pytest.mark.parametrize("which", ["smollm2", "gemma3", "qwen3_lora"])
+def test_full_size_step_properties(gpu, which):
+    """BASELINE configs 4 (SmolLM2-135M shape), 3 (gemma-style, sliding window 512 on 5 of 6 layers, QK-norm) and 5
+    (Qwen3-0.6B shape, head dim 128, vocabulary 151936, frozen base with rank-16 LoRA) at their real sizes, sequences
+    of 2048 tokens, forward + backward. Far beyond the scalar oracle, so: the loss of a near-zero random init is ln(V)
+    per sequence; the stacked graph (one launch set over B*2048 rows) and the reference's sequential accumulation (B
+    graphs of 2048 rows: other GEMM tiles, split-K counts and attention splits) give the same gradients; --recompute
+    changes no bit; two runs are bit-identical; half the seed gives exactly half of every gradient (a power-of-two
+    factor commutes with every f32 rounding on the way); a frozen base never gets a gradient buffer."""
+    from test_gpu_model import hip_step
+    arch, ag = mod("arch"), mod("autograd")
+    spec = FULL[which]
+    cfg = arch.ModelConfig(**spec["model"])
+    rs = np.random.RandomState(0)
+    weights = {}
+    for n in arch.param_names(cfg):
+        shp = arch.param_shape(cfg, n)
+        weights[n] = (1 + 0.1 * rs.standard_normal(shp)).astype(np.float32) if len(shp) == 1 else (0.02 * rs.standard_normal(shp)).astype(np.float32)
+    model = arch.Model(cfg, weights)
+    base = list(model.params())
+    if spec.get("lora"):
+        r = spec["lora"]
+        adapters = {}
+        for l in range(cfg.layers):
+            for k in arch.MATRIX_KEYS:
+                outd, ind = arch.layer_shapes(cfg)[k]
+                adapters[f"L{l}.{k}"] = ((0.02 * rs.standard_normal((r, ind))).astype(np.float32),
+                                         (0.02 * rs.standard_normal((outd, r))).astype(np.float32))
+        trainable = arch.apply_lora(model, r, 16.0, adapters)
+    else:
+        trainable = base
+    B, T = spec["batch"], 2048
+    toks = rs.randint(0, cfg.vocab, (B, T + 1))
+    seqs = []
+    for b in range(B):
+        tg = toks[b, 1:].copy()
+        tg[rs.rand(T) < 0.1] = -1
+        seqs.append((toks[b, :-1].copy(), tg))
+
+    def grads():
+        return [p.grad.copy() for p in trainable]
+
+    try:
+        l_st, _ = hip_step(gpu, model, seqs, True, T)
+        g_st = grads()
+        assert l_st.shape == (B,) and np.all(np.abs(l_st - np.log(cfg.vocab)) < 0.05 * np.log(cfg.vocab)), l_st
+        assert all(np.isfinite(g).all() and np.abs(g).max() > 0 for g in g_st)
+        l2, _ = hip_step(gpu, model, seqs, True, T)
+        assert l2.tobytes() == l_st.tobytes()
+        assert all(a.tobytes() == p.grad.tobytes() for a, p in zip(g_st, trainable)), "run-to-run"
+        l2, _ = hip_step(gpu, model, seqs, True, T, recompute=True)
+        assert l2.tobytes() == l_st.tobytes()
+        assert all(a.tobytes() == p.grad.tobytes() for a, p in zip(g_st, trainable)), "recompute"
+        l2, _ = hip_step(gpu, model, seqs, False, T)
+        assert np.all(np.abs(l2 - l_st) <= 1e-5 * np.abs(l_st)), (l2, l_st)
+        for i, (a, p) in enumerate(zip(g_st, trainable)):
+            # two f32 device results with different summation orders, each held to 1e-5 of the exact value
+            # elsewhere: 2e-5 between them
+            assert_close(p.grad, a, f"{which}: sequential vs stacked, trainable tensor {i} {p.shape}", rel_l2=2e-5)
+        gpu.install()
+        try:
+            loss = arch.sequence_loss(model, np.concatenate([s[0] for s in seqs]), np.concatenate([s[1] for s in seqs]), 0, T)
+            ag.backward(loss, 0.5 / B)
+            gpu.sync([loss])
+        finally:
+            gpu.uninstall()
+        assert all(np.array_equal(p.grad * 2, a) for a, p in zip(g_st, trainable)), "seed linearity"
+        if spec.get("lora"):
+            assert all(gpu._entries[p].grad == 0 for p in base), "a frozen base parameter got a gradient buffer"
+    finally:
+        ag.set_lora_adapters(None)
