@@ -107,6 +107,39 @@ __global__ __launch_bounds__(256) void attn_bwd_d(AttnP p, const float *__restri
   if (lane == 0) Dr[rid] = s;
 }
 
+// The same sums for head dims that are 4 x a power of two (16 .. 256): G = hd/4 lanes take one (row, head) with one
+// float4 each, so a wavefront streams 1 KB of O and of dO per load in memory order [row][head][hd]; the G partial sums
+// are folded by a fixed butterfly. Eight items per lane group per workgroup pass keep enough loads in flight.
+template <int G>
+__global__ __launch_bounds__(256) void attn_bwd_d_vec(AttnP p, const float *__restrict__ o, const float *__restrict__ go,
+                                                      float *__restrict__ Dr) {
+  constexpr int PER = 8;                                   // items per lane group
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const unsigned items = (unsigned)p.B * p.T * p.Hq;       // numbered in memory order: (b*T + t)*Hq + h
+  const int sub = threadIdx.x % G;
+  const unsigned grp = blockIdx.x * (256 / G) + threadIdx.x / G;
+  const unsigned stride = gridDim.x * (256 / G);
+  f4 a[PER], g[PER];
+  // every load is issued before the first use; a group past the end re-reads the last item and drops the result
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    const unsigned m = min(grp + i * stride, items - 1);
+    a[i] = *(reinterpret_cast<const f4 *>(o + (size_t)m * p.hd) + sub);
+    g[i] = *(reinterpret_cast<const f4 *>(go + (size_t)m * p.hd) + sub);
+  }
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    const unsigned m = grp + i * stride;
+    float s = (a[i].x * g[i].x + a[i].y * g[i].y) + (a[i].z * g[i].z + a[i].w * g[i].w);
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+    if (sub == 0 && m < items) {
+      const unsigned bt = m / (unsigned)p.Hq, h = m - bt * (unsigned)p.Hq, b = bt / (unsigned)p.T, t = bt - b * (unsigned)p.T;
+      Dr[((size_t)b * p.Hq + h) * p.T + t] = s;
+    }
+  }
+}
+
 // ---- dQ: one wavefront per query row (srcAttnBwdDq, wgsl.ts:741-784) -----------------------------
 __global__ __launch_bounds__(256) void attn_bwd_dq_gen(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, const float *__restrict__ go,
@@ -358,8 +391,23 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   float *dqpart = dq_floats ? Dr + d_floats + part_floats : nullptr;
   {
     ProfScope ps(ctx, "attention.bwd.D");
-    hipLaunchKernelGGL(attn_bwd_d, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, p, P<const float>(out),
-                       P<const float>(dout), Dr);
+    const int G = p.hd / 4;
+    const bool vec = p.hd % 4 == 0 && G >= 4 && G <= 64 && (G & (G - 1)) == 0 && (out | dout) % 16 == 0 && rows < ((int64_t)1 << 31);
+    if (vec) {
+      const unsigned nb = (unsigned)cdiv(rows, (int64_t)(256 / G) * 8);
+#define GO_D(GG) hipLaunchKernelGGL((attn_bwd_d_vec<GG>), dim3(nb), dim3(256), 0, ctx->stream, p, P<const float>(out), P<const float>(dout), Dr)
+      switch (G) {
+        case 4: GO_D(4); break;
+        case 8: GO_D(8); break;
+        case 16: GO_D(16); break;
+        case 32: GO_D(32); break;
+        default: GO_D(64); break;
+      }
+#undef GO_D
+    } else {
+      hipLaunchKernelGGL(attn_bwd_d, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, p, P<const float>(out),
+                         P<const float>(dout), Dr);
+    }
     GT_LAUNCHED(ctx);
   }
   if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v);

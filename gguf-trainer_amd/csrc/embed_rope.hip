@@ -127,6 +127,48 @@ __global__ __launch_bounds__(256) void rope_k(int64_t npairs, int T, int H, int 
   }
 }
 
+// The same rotation four pairs at a time for hd % 8 == 0: a thread takes four consecutive j of one (row, head), i.e.
+// one float4 of each half of the head and two float4 of the table, with 32-bit index arithmetic (the scalar kernel's
+// 64-bit divisions cost more than its memory traffic). Two units per thread and pass, all loads before the first use.
+template <bool BWD>
+__global__ __launch_bounds__(256) void rope_vec_k(unsigned nunits, int T, int H, int hd, const float *__restrict__ tab,
+                                                  const float *__restrict__ in, float *out, int acc) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const unsigned q = (unsigned)hd / 8;                    // float4 units per half head
+  const unsigned stride = gridDim.x * 256;
+  for (unsigned i0 = blockIdx.x * 256 + threadIdx.x; i0 < nunits; i0 += 2 * stride) {
+    f4 a0[2], a1[2], c0[2], c1[2], o0[2], o1[2];
+    size_t off[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const unsigned i = min(i0 + u * stride, nunits - 1);
+      const unsigned rh = i / q, j4 = i - rh * q;           // rh = row*H + h
+      const unsigned row = rh / (unsigned)H, t = row % (unsigned)T;
+      off[u] = (size_t)rh * hd + 4 * j4;
+      const f4 *tp = reinterpret_cast<const f4 *>(tab + ((size_t)t * (hd / 2) + 4 * j4) * 2);
+      a0[u] = *reinterpret_cast<const f4 *>(in + off[u]);
+      a1[u] = *reinterpret_cast<const f4 *>(in + off[u] + hd / 2);
+      c0[u] = tp[0];                                        // cos, sin of pairs j, j+1
+      c1[u] = tp[1];                                        // and of pairs j+2, j+3
+      if (acc) {
+        o0[u] = *reinterpret_cast<const f4 *>(out + off[u]);
+        o1[u] = *reinterpret_cast<const f4 *>(out + off[u] + hd / 2);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      if (i0 + u * stride >= nunits) continue;
+      const f4 cs = {c0[u][0], c0[u][2], c1[u][0], c1[u][2]}, sn = {c0[u][1], c0[u][3], c1[u][1], c1[u][3]};
+      f4 r0, r1;
+      if (!BWD) { r0 = a0[u] * cs - a1[u] * sn; r1 = a0[u] * sn + a1[u] * cs; }
+      else { r0 = cs * a0[u] + sn * a1[u]; r1 = -sn * a0[u] + cs * a1[u]; }
+      if (acc) { r0 += o0[u]; r1 += o1[u]; }
+      *reinterpret_cast<f4 *>(out + off[u]) = r0;
+      *reinterpret_cast<f4 *>(out + off[u] + hd / 2) = r1;
+    }
+  }
+}
+
 extern "C" {
 int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, gt_buf ids, gt_buf W, gt_buf out) {
   GT_ENTER(ctx);
@@ -180,6 +222,16 @@ int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, i
     ctx->rope_tables[key] = tab;
   } else tab = it->second;
   int64_t npairs = (int64_t)rows * H * (hd / 2);
+  if (hd % 8 == 0 && npairs / 4 < ((int64_t)1 << 31) && (in | out) % 16 == 0) {
+    const unsigned nunits = (unsigned)(npairs / 4);
+    const unsigned nbv = (unsigned)std::min<int64_t>(cdiv(nunits, 512), (int64_t)ctx->num_cu * 16);
+    if (backward)
+      hipLaunchKernelGGL((rope_vec_k<true>), dim3(nbv), dim3(256), 0, ctx->stream, nunits, T, H, hd, tab, P<const float>(in), P<float>(out), acc);
+    else
+      hipLaunchKernelGGL((rope_vec_k<false>), dim3(nbv), dim3(256), 0, ctx->stream, nunits, T, H, hd, tab, P<const float>(in), P<float>(out), acc);
+    GT_LAUNCHED(ctx);
+    return 0;
+  }
   unsigned nb = (unsigned)std::min<int64_t>(cdiv(npairs, 256), (int64_t)ctx->num_cu * 16);
   if (backward)
     hipLaunchKernelGGL((rope_k<true>), dim3(nb), dim3(256), 0, ctx->stream, npairs, T, H, hd, reinterpret_cast<const float2 *>(tab),

@@ -39,9 +39,10 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_k(int rows, int d, float eps,
     v4f xv[NJ];
     float ss = 0;
 #pragma unroll
+    for (int j = 0; j < NJ; j++) xv[j] = xr[min(li + j * LPR, d4 - 1)];      // all loads first, none conditional
+#pragma unroll
     for (int j = 0; j < NJ; j++) {
-      int c = li + j * LPR;
-      xv[j] = c < d4 ? xr[c] : v4f{0, 0, 0, 0};
+      if (li + j * LPR >= d4) xv[j] = v4f{0, 0, 0, 0};
       ss += xv[j][0] * xv[j][0] + xv[j][1] * xv[j][1] + xv[j][2] * xv[j][2] + xv[j][3] * xv[j][3];
     }
     ss = group_sum<LPR>(ss);
@@ -74,24 +75,31 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const floa
     wv[j] = c < d4 ? reinterpret_cast<const v4f *>(w)[c] : v4f{0, 0, 0, 0};
     dwv[j] = v4f{0, 0, 0, 0};
   }
-  // two rows of this lane group in flight: the loads of the second are issued before the first is reduced
+  // Two rows of this lane group in flight, and every load of an iteration (x, g and, when accumulating, the old
+  // dx) issued before the first use, unconditionally: a chunk past the row end re-reads the row's last chunk and a
+  // row past the end re-reads row 0. Their products vanish where it matters (w is zero there, nothing is stored).
   const int64_t rstep = (int64_t)gridDim.x * 4 * RPW;
+  int cc[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; j++) cc[j] = min(li + j * LPR, d4 - 1);
   for (int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW + sub; row0 < rows; row0 += 2 * rstep) {
-    v4f xv[2][NJ], gv[2][NJ];
+    v4f xv[2][NJ], gv[2][NJ], ov[2][NJ];
+    float rr[2];
     float S[2] = {0.f, 0.f};
 #pragma unroll
     for (int u = 0; u < 2; u++) {
       const int64_t row = row0 + u * rstep;
-      const bool live = row < rows;
-      const v4f *xr = reinterpret_cast<const v4f *>(x + (live ? row : 0) * d);
-      const v4f *gr = reinterpret_cast<const v4f *>(g + (live ? row : 0) * d);
+      const int64_t rl = row < rows ? row : 0;
+      const v4f *xr = reinterpret_cast<const v4f *>(x + rl * d);
+      const v4f *gr = reinterpret_cast<const v4f *>(g + rl * d);
+      const v4f *dr = reinterpret_cast<const v4f *>(dx + rl * d);
 #pragma unroll
       for (int j = 0; j < NJ; j++) {
-        int c = li + j * LPR;
-        bool in = live && c < d4;
-        xv[u][j] = in ? xr[c] : v4f{0, 0, 0, 0};
-        gv[u][j] = in ? gr[c] : v4f{0, 0, 0, 0};
+        xv[u][j] = xr[cc[j]];
+        gv[u][j] = gr[cc[j]];
+        if (acc_dx) ov[u][j] = dr[cc[j]];
       }
+      rr[u] = rinv[rl];
     }
 #pragma unroll
     for (int u = 0; u < 2; u++) {
@@ -106,17 +114,15 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const floa
     for (int u = 0; u < 2; u++) {
       const int64_t row = row0 + u * rstep;
       if (row >= rows) continue;
-      const float r = rinv[row];
+      const float r = rr[u];
       const float k2 = r * r * r * S[u] * invd;
       v4f *dxr = reinterpret_cast<v4f *>(dx + row * d);
 #pragma unroll
       for (int j = 0; j < NJ; j++) {
         int c = li + j * LPR;
-        if (c < d4) {
-          v4f o = wv[j] * gv[u][j] * r - xv[u][j] * k2;
-          if (acc_dx) o += dxr[c];
-          dxr[c] = o;
-        }
+        v4f o = wv[j] * gv[u][j] * r - xv[u][j] * k2;
+        if (acc_dx) o += ov[u][j];
+        if (c < d4) dxr[c] = o;
         dwv[j] += gv[u][j] * xv[u][j] * r;
       }
     }
@@ -139,29 +145,32 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const floa
   }
 }
 
-// dw[c] (+)= sum over the nparts partial rows, in a fixed order: 64 columns per workgroup, four
-// lane groups each summing every fourth partial row (eight independent loads in flight), then
-// the four group sums added in group order.
+// dw[c] (+)= sum over the nparts partial rows, in a fixed order: 16 columns per workgroup (one 64-byte line per
+// load), sixteen lane groups each summing every sixteenth partial row with eight independent loads in flight, then
+// the group sums added in group order. Narrow workgroups because the launch is latency-bound: d = 576 gives 36 of them.
+#define CS_COLS 16
+#define CS_GRPS 16
 __global__ __launch_bounds__(256) void colsum_reduce(const float *__restrict__ part, int nparts, int d, float *dw, int acc) {
-  __shared__ float sm[4][64];
-  const int cl = threadIdx.x % 64, grp = threadIdx.x / 64;
-  const int c = blockIdx.x * 64 + cl;
+  __shared__ float sm[CS_GRPS][CS_COLS];
+  const int cl = threadIdx.x % CS_COLS, grp = threadIdx.x / CS_COLS;
+  const int c = blockIdx.x * CS_COLS + cl;
+  const int cr = min(c, d - 1);
   float s = 0;
-  if (c < d) {
-    int p = grp;
-    for (; p + 28 < nparts; p += 32) {
-      float v[8];
+  int p = grp;
+  for (; p + 7 * CS_GRPS < nparts; p += 8 * CS_GRPS) {
+    float v[8];
 #pragma unroll
-      for (int u = 0; u < 8; u++) v[u] = part[(size_t)(p + 4 * u) * d + c];
+    for (int u = 0; u < 8; u++) v[u] = part[(size_t)(p + CS_GRPS * u) * d + cr];
 #pragma unroll
-      for (int u = 0; u < 8; u++) s += v[u];
-    }
-    for (; p < nparts; p += 4) s += part[(size_t)p * d + c];
+    for (int u = 0; u < 8; u++) s += v[u];
   }
+  for (; p < nparts; p += CS_GRPS) s += part[(size_t)p * d + cr];
   sm[grp][cl] = s;
   __syncthreads();
   if (grp == 0 && c < d) {
-    float t = sm[0][cl] + sm[1][cl] + sm[2][cl] + sm[3][cl];
+    float t = sm[0][cl];
+#pragma unroll
+    for (int q = 1; q < CS_GRPS; q++) t += sm[q][cl];
     dw[c] = acc ? dw[c] + t : t;
   }
 }
@@ -232,7 +241,7 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
                      acc_dx, part);
   GT_LAUNCHED(ctx);
   if (dw) {
-    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 64)), dim3(256), 0, ctx->stream, part, (int)nb, d,
+    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, CS_COLS)), dim3(256), 0, ctx->stream, part, (int)nb, d,
                        P<float>(dw), acc_dw);
     GT_LAUNCHED(ctx);
   }
@@ -271,7 +280,7 @@ static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x,
     hipLaunchKernelGGL(rmsnorm_dw_gen, dim3((unsigned)cdiv(d, 256), ns), dim3(256), 0, ctx->stream, rows, d, slab,
                        P<const float>(x), P<const float>(y_or_g), P<const float>(rinv), static_cast<float *>(ws));
     GT_LAUNCHED(ctx);
-    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, 64)), dim3(256), 0, ctx->stream, static_cast<float *>(ws), ns,
+    hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, CS_COLS)), dim3(256), 0, ctx->stream, static_cast<float *>(ws), ns,
                        d, P<float>(dw), acc_dw);
     GT_LAUNCHED(ctx);
   }

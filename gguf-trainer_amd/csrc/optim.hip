@@ -71,9 +71,9 @@ __global__ __launch_bounds__(1024) void adamw_scale_k(int nchunks, const float *
   for (int i0 = threadIdx.x; i0 < nchunks; i0 += 8 * 1024) {
     float x[8];
 #pragma unroll
-    for (int u = 0; u < 8; u++) { int i = i0 + u * 1024; x[u] = i < nchunks ? partial[i] : 0.f; }
+    for (int u = 0; u < 8; u++) x[u] = partial[min(i0 + u * 1024, nchunks - 1)];       // unconditional: all in flight together
 #pragma unroll
-    for (int u = 0; u < 8; u++) s8[u] += x[u];
+    for (int u = 0; u < 8; u++) s8[u] += i0 + u * 1024 < nchunks ? x[u] : 0.f;
   }
   float s = ((s8[0] + s8[1]) + (s8[2] + s8[3])) + ((s8[4] + s8[5]) + (s8[6] + s8[7]));
   s = block_sum<16>(s, sm);
