@@ -247,13 +247,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
 }
 
 // attention_mfma.hip, compiled once per head dim
+int attn_fwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
+int attn_bwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
+                    float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
 int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
 int attn_bwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
                     float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 int attn_bwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
                      float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
-static int attn_mfma_supported(int hd) { return hd == 64 || hd == 128; }
+static int attn_mfma_supported(int hd) { return hd == 32 || hd == 64 || hd == 128; }
 
 // A launch with fewer 128-row tiles than three per CU is cut further (measured at T = 2048, 9 heads: 1 sequence runs
 // 2.3x faster with 6 workgroups per tile, 2 sequences 1.5x with 3, 4 sequences 1.13x with 2, 8 gain nothing): every tile's loop range goes to `splits`
@@ -314,7 +317,8 @@ static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
     if (gt_ws_reserve(ctx, (size_t)p.splits * (slice + 2 * rows) * sizeof(float), &ws)) return 1;
     fpart = static_cast<float *>(ws);
   }
-  if (p.hd == 64 ? attn_fwd_mfma64(ctx, p, q, k, v, out, lse, fpart) : attn_fwd_mfma128(ctx, p, q, k, v, out, lse, fpart)) return 1;
+  if (p.hd == 32 ? attn_fwd_mfma32(ctx, p, q, k, v, out, lse, fpart)
+      : p.hd == 64 ? attn_fwd_mfma64(ctx, p, q, k, v, out, lse, fpart) : attn_fwd_mfma128(ctx, p, q, k, v, out, lse, fpart)) return 1;
   if (p.splits > 1) {
     const int64_t n = (int64_t)p.B * p.T * p.Hq * (p.hd / 4);
     hipLaunchKernelGGL(attn_fwd_combine, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, p, fpart, P<float>(out), P<float>(lse));
@@ -324,8 +328,9 @@ static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
 }
 static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
                          float *part, float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
-  if (p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v)
-                 : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v))
+  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v)
+      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v)
+                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v))
     return 1;
   if (p.splits > 1) {
     const size_t n4 = (size_t)p.B * p.T * p.Hq * p.hd / 4;

@@ -1,5 +1,5 @@
 // Attention forward / backward on the FP32 matrix cores (v_mfma_f32_32x32x2_f32). This file is compiled once per
-// supported head dim (-DHD=64, -DHD=128); the entry points carry the head dim in their names.
+// supported head dim (-DHD=32, -DHD=64, -DHD=128); the entry points carry the head dim in their names.
 // Same math and saved statistic as the generic kernels in attention.hip: causal / sliding window,
 // GQA, scores in the log2 domain, softmax recomputed in backward from lse2.
 //
@@ -48,7 +48,7 @@ struct AttnP {
 };
 
 #ifndef HD
-#error "compile with -DHD=64 or -DHD=128"
+#error "compile with -DHD=32, -DHD=64 or -DHD=128"
 #endif
 #define CAT_(a, b) a##b
 #define CAT(a, b) CAT_(a, b)
@@ -115,13 +115,14 @@ __device__ __forceinline__ v16f rows_dot_regs(const float *rows, const float (&r
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  constexpr int NB = HD / 8 < 8 ? HD / 8 : 8;       // b128 reads in flight per batch
 #pragma unroll
-  for (int j0 = 0; j0 < HD / 8; j0 += 8) {
-    v4f a[8];
+  for (int j0 = 0; j0 < HD / 8; j0 += NB) {
+    v4f a[NB];
 #pragma unroll
-    for (int j = 0; j < 8; j++) a[j] = *reinterpret_cast<const v4f *>(rows + l32 * LD + 8 * (j0 + j) + 4 * g);
+    for (int j = 0; j < NB; j++) a[j] = *reinterpret_cast<const v4f *>(rows + l32 * LD + 8 * (j0 + j) + 4 * g);
 #pragma unroll
-    for (int j = 0; j < 8; j++)
+    for (int j = 0; j < NB; j++)
 #pragma unroll
       for (int s = 0; s < 4; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][s], reg[4 * (j0 + j) + s], acc, 0, 0, 0);
   }
@@ -167,7 +168,7 @@ __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32]
 
 }  // namespace
 
-#define KT (HD == 64 ? 64 : 32)      // keys per LDS stage in forward and dQ
+#define KT (HD <= 64 ? 64 : 32)      // keys per LDS stage in forward and dQ
 #define NSUB (KT / 32)
 
 // ---- forward --------------------------------------------------------------------------------------

@@ -103,9 +103,9 @@ def test_fd_embedding_and_rope(gpu, ref):
 
 
 @pytest.mark.parametrize("T,Hq,Hkv,hd,window", [(19, 4, 2, 8, 0), (19, 4, 2, 8, 5), (70, 2, 1, 64, 0), (70, 2, 1, 64, 33),
-                                                  (40, 2, 2, 128, 0), (150, 3, 1, 64, 0)])
+                                                  (40, 2, 2, 128, 0), (150, 3, 1, 64, 0), (90, 4, 2, 32, 0), (90, 4, 2, 32, 40)])
 def test_fd_attention(gpu, ref, T, Hq, Hkv, hd, window):
-    """Generic kernels (hd 8) and the matrix-core kernels (hd 64 / 128), GQA, full causal and windowed."""
+    """Generic kernels (hd 8) and the matrix-core kernels (hd 32 / 64 / 128), GQA, full causal and windowed."""
     g = R(ref, 5 + T + hd)
     fd_case(gpu, ref, [g(T, Hq * hd, scale=0.6), g(T, Hkv * hd, scale=0.6), g(T, Hkv * hd)],
             lambda ag, q, k, v: ag.attention(q, k, v, T, Hq, Hkv, hd, window), f"attention T={T} {Hq}/{Hkv}x{hd} w={window}")

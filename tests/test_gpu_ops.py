@@ -352,12 +352,13 @@ def test_late_backward_after_sync_is_refused(gpu, ref):
 
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 700, 4, 2, 64, 0), (2, 333, 6, 2, 64, 300), (1, 1024, 9, 3, 64, 0),
                                                   (3, 129, 2, 1, 64, 33), (1, 512, 3, 3, 64, 512),
-                                                  (1, 300, 4, 2, 128, 0), (2, 200, 8, 8, 128, 77), (1, 640, 16, 8, 128, 0)])
+                                                  (1, 300, 4, 2, 128, 0), (2, 200, 8, 8, 128, 77), (1, 640, 16, 8, 128, 0),
+                                                  (4, 128, 4, 2, 32, 0), (1, 450, 6, 3, 32, 100), (2, 261, 2, 2, 32, 0)])
 @pytest.mark.parametrize("splits", [-1, 1, 5])
 def test_attention_mfma_shapes(gpu, ref, B, T, Hq, Hkv, hd, window, splits):
-    """The matrix-core kernels (hd = 64 and 128): tiles of 128 queries x 32 keys with ragged T, windows that cut tiles,
+    """The matrix-core kernels (hd = 32, 64 and 128): tiles of 128 queries x 32 keys with ragged T, windows that cut tiles,
     GQA group sums, stacked sequences; 1024 x 9/3 x 64 is one SmolLM2 layer at half the sequence length, 16/8 x 128
-    the Qwen3-0.6B head layout. Each shape with one workgroup per tile, with the launch-size heuristic, and with five
+    the Qwen3-0.6B head layout, 4 x 128 x 4/2 x 32 the attention of BASELINE config 1. Each shape with one workgroup per tile, with the launch-size heuristic, and with five
     workgroups per tile (partial softmax / dQ / dK,dV folded afterwards, some of them over empty ranges)."""
     ag = mod("autograd")
     gpu.set_option("attn.splits", splits)
