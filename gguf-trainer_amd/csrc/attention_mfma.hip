@@ -522,11 +522,10 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
   const int group = p.Hq / p.Hkv;
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart) && (p.splits * group == 1 || part),
              "attention: split backward without a workspace");
-  static bool smem_set = false;
-  if (!smem_set) {            // more than the 64 KB a kernel gets by default at hd 128
+  if (!(ctx->attn_smem_set & HD)) {   // once per context (device): more than the 64 KB a kernel gets by default at hd 128
     GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
-    smem_set = true;
+    ctx->attn_smem_set |= HD;
   }
   {
     ProfScope ps(ctx, "attention.bwd.dq");

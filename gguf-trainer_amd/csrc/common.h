@@ -34,6 +34,7 @@ struct gt_ctx {
   bool prof_on = false;
   std::string prof_prefix;
   std::vector<ProfEvent> prof;
+  unsigned attn_smem_set = 0;                   // head dims (bits 32 | 64 | 128) whose dK/dV kernel has its LDS size attribute set
   int opt_prof_sample = 1;                      // events around every n-th launch of a label
   struct ProfSeen { int64_t n = 0; double work = 0; };
   std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not

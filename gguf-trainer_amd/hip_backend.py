@@ -380,7 +380,7 @@ class HipBackend:
 
     def lora_linear(self, x: Tensor, w: Tensor, a: Tensor, b: Tensor, sc: float) -> Tensor:
         """linear(x, w) + sc * linear(linear(x, a), b) (autograd.ts:760-781) as one recorded op. The scale is applied to
-        the rank-r activation h = x.a^T (a [rows, r] pass) instead of the [rows, out] product, the adapter product is
+        the rank-r activation h = x.a^T (inside the streaming rank kernels) instead of the [rows, out] product, the adapter product is
         accumulated into the base output by the GEMM itself, and the backward reads the upstream gradient directly:
         no [rows, out] elementwise pass in either direction."""
         T, ind = x.shape
@@ -388,8 +388,7 @@ class HipBackend:
         xd, wd, ad, bd = self._data(x), self._data(w), self._data(a), self._data(b)
         out, e = self._make_out([T, outd], [x, w, a, b])
         hs = self._scratch_buf(T * r * 4)
-        check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, T, r, ind, xd, ad, hs), "lora.h")
-        check(self._ctx, lib.gt_scale_fwd(self._ctx, T * r, hs, sc, hs), "lora.scale")
+        check(self._ctx, lib.gt_rank_down(self._ctx, T, ind, r, xd, ad, 0, sc, hs), "lora.h")
         check(self._ctx, lib.gt_gemm_pair(self._ctx, NT, 0, T, outd, ind, xd, wd, r, hs, bd, e.data), "lora.y")
         wants_dw, wants_da, wants_db = w.requires_grad, a.requires_grad, b.requires_grad
 
@@ -403,15 +402,14 @@ class HipBackend:
             if wants_db:
                 db, accb = self._gdst(b)
                 if db:
-                    check(self._ctx, lib.gt_gemm(self._ctx, TN, accb, outd, r, T, g, hs, db), "lora.db")
+                    check(self._ctx, lib.gt_rank_grad(self._ctx, T, outd, r, hs, g, 1, accb, db), "lora.db")
             if dx or wants_da:
                 dh = self._scratch_buf(T * r * 4)
-                check(self._ctx, lib.gt_gemm(self._ctx, NN, 0, T, r, outd, g, bd, dh), "lora.dh")
-                check(self._ctx, lib.gt_scale_fwd(self._ctx, T * r, dh, sc, dh), "lora.scale")
+                check(self._ctx, lib.gt_rank_down(self._ctx, T, outd, r, g, bd, 1, sc, dh), "lora.dh")
                 if wants_da:
                     da, acca = self._gdst(a)
                     if da:
-                        check(self._ctx, lib.gt_gemm(self._ctx, TN, acca, r, ind, T, dh, xd, da), "lora.da")
+                        check(self._ctx, lib.gt_rank_grad(self._ctx, T, ind, r, dh, xd, 0, acca, da), "lora.da")
                 if dx:      # dX (+)= dY.W + dH.A in one K loop
                     check(self._ctx, lib.gt_gemm_pair(self._ctx, NN, acc, T, ind, outd, g, wd, r, dh, ad, dx), "lora.dx")
 

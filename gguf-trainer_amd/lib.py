@@ -43,6 +43,8 @@ _SIG = {
     "gt_gemm": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf],
     "gt_gemm_pair": [ctxp, i32, i32, i32, i32, i32, buf, buf, i32, buf, buf, buf],
     "gt_gemm_batched": [ctxp, i32, i32, i32, i32, i32, buf, i64, buf, i64, buf, i64, i32],
+    "gt_rank_down": [ctxp, i32, i32, i32, buf, buf, i32, f32, buf],
+    "gt_rank_grad": [ctxp, i32, i32, i32, buf, buf, i32, i32, buf],
     "gt_add_fwd": [ctxp, i64, buf, buf, buf],
     "gt_mul_fwd": [ctxp, i64, buf, buf, buf],
     "gt_silu_fwd": [ctxp, i64, buf, buf],

@@ -80,6 +80,16 @@ int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_bu
  * of the final additions. */
 int gt_gemm_pair(gt_ctx *ctx, int kind, int acc, int M, int N, int K1, gt_buf A1, gt_buf B1, int K2, gt_buf A2, gt_buf B2,
                  gt_buf C);
+/* The rank-r products of the LoRA linear (src/model/autograd.ts:311-319 makes them `linear` calls; src/train/lora.ts:69-82
+ * sizes them), each one streaming pass over the [rows, K] operand:
+ *   gt_rank_down: h[rows, r] = alpha * x[rows, K] . s^T, s = [r, K] (s_kmajor = 0: h = x A^T) or [K, r] (s_kmajor = 1:
+ *                 dh = g B). alpha is the adapter scale, applied here instead of on a [rows, out] product.
+ *   gt_rank_grad: p (+)= h^T . y as [r, K] (transpose_out = 0: dA = dh^T x) or y^T . h as [K, r] (transpose_out = 1:
+ *                 dB = g^T h); h [rows, r], y [rows, K].
+ * Any r, K >= 1: r <= 32 with K a multiple of 16 (down) / 64 (grad) and 16-byte aligned operands take the streaming
+ * kernels, everything else the general GEMM. */
+int gt_rank_down(gt_ctx *ctx, int rows, int K, int r, gt_buf x, gt_buf s, int s_kmajor, float alpha, gt_buf h);
+int gt_rank_grad(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int transpose_out, int acc, gt_buf p);
 /* batch of `count` independent products with element strides between consecutive problems
  * (Newton-Schulz over same-shaped matrices; no counterpart call in the reference, which loops). */
 int gt_gemm_batched(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t strideA,

@@ -62,6 +62,41 @@ def test_gemm_every_tile_shape_and_kind(gpu, M, N, K):
         gpu.set_option("gemm.splitk", -1)
 
 
+@pytest.mark.parametrize("rows,K,r", [(16, 64, 16), (100, 192, 16), (257, 1024, 16), (333, 128, 8), (64, 64, 3), (129, 256, 32),
+                                      (200, 320, 20), (70, 48, 16), (50, 64, 40), (90, 100, 16), (2100, 576, 16)])
+def test_rank_products(gpu, rows, K, r):
+    """The rank-r products of the LoRA linear against float64: h = alpha x s^T for both layouts of s, p (+)= h^T y in both
+    output orientations, store and accumulate; rows and ranks that leave partial 16-blocks, K that does and does not
+    take the streaming kernels (48, 100: the GEMM fallback; r = 40: too wide), several row slices (2100 rows)."""
+    L = mod("lib")
+    rs = np.random.RandomState(rows + K + r)
+    x = rs.standard_normal((rows, K)).astype(np.float32)
+    s = rs.standard_normal((r, K)).astype(np.float32)
+    hh = rs.standard_normal((rows, r)).astype(np.float32)
+    p0 = rs.standard_normal((r, K)).astype(np.float32)
+    bx, bs, bh, bp = (gpu.create_state_buffer(a.nbytes) for a in (x, s, hh, p0))
+    bo = gpu.create_state_buffer(rows * r * 4)
+    gpu.write_state_buffer(bx, x)
+    gpu.write_state_buffer(bh, hh)
+    want_h = 0.37 * (x.astype(np.float64) @ s.astype(np.float64).T)
+    for kmajor, arr in ((0, s), (1, np.ascontiguousarray(s.T))):
+        gpu.write_state_buffer(bs, arr)
+        gpu.write_state_buffer(bo, np.full((rows, r), 7.0, np.float32))
+        L.check(gpu.ctx, L.lib.gt_rank_down(gpu.ctx, rows, K, r, bx, bs, kmajor, 0.37, bo), "gt_rank_down")
+        assert_close(gpu.read_state_buffer(bo, rows * r).reshape(rows, r), want_h.astype(np.float32), f"rank_down kmajor {kmajor} {rows}x{K}x{r}")
+    want_p = hh.astype(np.float64).T @ x.astype(np.float64)
+    for tr in (0, 1):
+        for acc in (0, 1):
+            base = p0 if not tr else np.ascontiguousarray(p0.T)
+            gpu.write_state_buffer(bp, base)
+            L.check(gpu.ctx, L.lib.gt_rank_grad(gpu.ctx, rows, K, r, bh, bx, tr, acc, bp), "gt_rank_grad")
+            got = gpu.read_state_buffer(bp, r * K).reshape((K, r) if tr else (r, K))
+            want = (want_p.T if tr else want_p) + (base if acc else 0)
+            assert_close(got, want.astype(np.float32), f"rank_grad transpose {tr} acc {acc} {rows}x{K}x{r}")
+    rc = L.lib.gt_rank_down(gpu.ctx, 0, K, r, bx, bs, 0, 1.0, bo)
+    assert rc != 0 and b"gt_rank_down" in L.lib.gt_last_error(gpu.ctx)
+
+
 @pytest.mark.parametrize("M,N,K1,K2", [(200, 152, 96, 16), (130, 100, 72, 5), (257, 193, 101, 33), (64, 64, 16, 16)])
 def test_gemm_pair(gpu, M, N, K1, K2):
     """C (+)= A1.B1 + A2.B2 in one K loop (the LoRA linear and its dX): every kind, store and accumulate, a few tile
