@@ -155,14 +155,20 @@ __device__ __forceinline__ void t_dot_acc(v16f (&out)[HD / 32], const float *lds
 }
 
 __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32], int g, float mul, int add) {
+  v4f old[HD / 32][4];
+  if (add) {          // every old value first: a load behind a store to the same array would wait for it
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) old[dt][a] = *reinterpret_cast<const v4f *>(row + dt * 32 + 8 * a + 4 * g);
+  }
 #pragma unroll
   for (int dt = 0; dt < HD / 32; dt++)
 #pragma unroll
     for (int a = 0; a < 4; a++) {
       v4f o = {acc[dt][4 * a] * mul, acc[dt][4 * a + 1] * mul, acc[dt][4 * a + 2] * mul, acc[dt][4 * a + 3] * mul};
-      v4f *dst = reinterpret_cast<v4f *>(row + dt * 32 + 8 * a + 4 * g);
-      if (add) o += *dst;
-      *dst = o;
+      if (add) o += old[dt][a];
+      *reinterpret_cast<v4f *>(row + dt * 32 + 8 * a + 4 * g) = o;
     }
 }
 

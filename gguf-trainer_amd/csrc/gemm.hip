@@ -226,19 +226,26 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
   bool add;
   if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
   else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0; }
+  // When accumulating, the sixteen old values of a 32x32 tile are loaded together (from clamped, always valid
+  // addresses) before the first store: a load placed after a store to the same array waits for it, and one round trip
+  // per element is what an interleaved read-add-write loop would pay.
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      int col = n0 + wn * (TN * 32) + j * 32 + l32;
+      const int col = n0 + wn * (TN * 32) + j * 32 + l32;
+      const int rbase = m0 + wm * (TM * 32) + i * 32 + 4 * g;
+      float old[16];
+      if (add) {
+        const float *cc = C + min(col, a.N - 1);
+#pragma unroll
+        for (int r = 0; r < 16; r++) old[r] = cc[(size_t)min(rbase + 8 * (r / 4) + (r % 4), a.M - 1) * ldc];
+      }
       if (col >= a.N) continue;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        int row = m0 + wm * (TM * 32) + i * 32 + 8 * (r / 4) + 4 * g + (r % 4);
-        if (row < a.M) {
-          float *q = C + (size_t)row * ldc + col;
-          *q = add ? *q + acc[i][j][r] : acc[i][j][r];
-        }
+        const int row = rbase + 8 * (r / 4) + (r % 4);
+        if (row < a.M) C[(size_t)row * ldc + col] = add ? old[r] + acc[i][j][r] : acc[i][j][r];
       }
     }
 }
