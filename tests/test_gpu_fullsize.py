@@ -220,3 +220,103 @@ def test_full_size_step_properties(gpu, which):
             assert all(gpu._entries[p].grad == 0 for p in base), "a frozen base parameter got a gradient buffer"
     finally:
         ag.set_lora_adapters(None)
+
+
+def test_adamw_full_size_tensor_list(gpu):
+    """BASELINE config 4's optimizer step at its real size: the 272 tensors of the SmolLM2-135M shape (134.5 M
+    parameters), two steps with the global clip active in the first and inactive in the second. Every tensor against
+    the closed form of src/train/adam.ts:46-82 evaluated in float64 (vectorised; the scalar oracle covers the small
+    cases), and the clip scale against a float64 norm over all gradients."""
+    ag, arch, optim = mod("autograd"), mod("arch"), mod("optim")
+    cfg = arch.ModelConfig(**FULL["smollm2"]["model"])
+    rs = np.random.RandomState(3)
+    names = arch.param_names(cfg)
+    params = []
+    for n in names:
+        shp = arch.param_shape(cfg, n)
+        params.append(ag.Tensor((0.05 * rs.standard_normal(shp)).astype(np.float32), list(shp), True))
+    assert len(params) == 272 and sum(p.size for p in params) == 134515008
+    lr, b1, b2, eps, wd, clip = 1e-3, 0.9, 0.95, 1e-8, 0.1, 1.0
+    opt = optim.AdamWHip(gpu, params, lr=lr, beta1=b1, beta2=b2, eps=eps, weight_decay=wd, clip=clip)
+    w = [p.data.astype(np.float64) for p in params]
+    m = [np.zeros(p.size) for p in params]
+    v = [np.zeros(p.size) for p in params]
+    for t, gscale in ((1, 3e-4), (2, 2e-5)):
+        grads = [(gscale * rs.standard_normal(p.size)).astype(np.float32) for p in params]
+        for p, g in zip(params, grads):
+            gpu.write_state_buffer(gpu.buffers_for(p)["grad"], g)
+            gpu._entries[p].grad_init = True
+        opt.record_step()
+        norm = np.sqrt(sum(float(np.dot(g.astype(np.float64), g.astype(np.float64))) for g in grads))
+        assert (norm > clip) == (t == 1)                         # the clip triggers in step 1 only
+        assert abs(opt.grad_norm() - norm) <= 1e-5 * norm
+        sc = clip / (norm + 1e-12) if norm > clip else 1.0
+        bc1, bc2 = 1 - b1 ** t, 1 - b2 ** t
+        for i, g in enumerate(grads):
+            g64 = g.astype(np.float64) * sc
+            m[i] = b1 * m[i] + (1 - b1) * g64
+            v[i] = b2 * v[i] + (1 - b2) * g64 * g64
+            w[i] -= lr * ((m[i] / bc1) / (np.sqrt(v[i] / bc2) + eps) + wd * w[i])
+    opt.sync_weights_to_host()
+    st = opt.export_state()
+    for i, p in enumerate(params):
+        assert_close(p.data, w[i], f"AdamW weights of {names[i]}")
+        assert_close(st["m"][i], m[i], f"AdamW first moment of {names[i]}")
+        assert_close(st["v"][i], v[i], f"AdamW second moment of {names[i]}")
+
+
+def test_muon_full_size_matrices(gpu):
+    """BASELINE config 3's Muon step on its real matrix shapes (640x640, 128x640, 2048x640, 640x2048; one layer's
+    seven matrices twice over so the per-shape batches hold several matrices): momentum, Nesterov, five Newton-Schulz
+    iterations and the scaled apply against a float64 evaluation of src/train/muon.ts:69-158, and the property the
+    quintic is built for: the singular values of the orthogonalised update land in about [0.7, 1.2]."""
+    ag, optim, L = mod("autograd"), mod("optim"), mod("lib")
+    rs = np.random.RandomState(4)
+    shapes = [(640, 640), (128, 640), (128, 640), (640, 640), (2048, 640), (2048, 640), (640, 2048)] * 2
+    params = [ag.Tensor((0.02 * rs.standard_normal(s)).astype(np.float32), list(s), True) for s in shapes]
+    aux = ag.Tensor(np.ones(640, np.float32), [640], True)
+    lr, mu = 0.01, 0.95
+    opt = optim.MuonHip(gpu, params, [aux], lr=lr, momentum=mu, nesterov=True, ns_steps=5, aux={"lr": 3e-3})
+    w = [p.data.astype(np.float64).reshape(s) for p, s in zip(params, shapes)]
+    buf = [np.zeros(s) for s in shapes]
+
+    def ns64(G):
+        tr = G.shape[0] > G.shape[1]
+        X = (G.T if tr else G) / (np.linalg.norm(G) + 1e-7)
+        for _ in range(5):
+            A = X @ X.T
+            X = 3.4445 * X + (-4.7750 * A + 2.0315 * (A @ A)) @ X
+        return X.T if tr else X
+
+    for step in range(2):
+        grads = [(0.01 * rs.standard_normal(s)).astype(np.float32) for s in shapes]
+        for p, g in zip(params + [aux], grads + [np.zeros(640, np.float32)]):
+            gpu.write_state_buffer(gpu.buffers_for(p)["grad"], g)
+            gpu._entries[p].grad_init = True
+        opt.record_step()
+        for i, (g, s) in enumerate(zip(grads, shapes)):
+            g64 = g.astype(np.float64)
+            buf[i] = mu * buf[i] + g64
+            O = ns64(g64 + mu * buf[i])
+            if step == 0 and i in (0, 1, 4, 6):
+                # (a square Gaussian matrix has singular values down to zero, which five steps cannot lift: there the
+                # bound holds for the bulk; a rectangular one is well conditioned and every value lands in the band)
+                sv = np.linalg.svd(O, compute_uv=False)
+                assert sv.max() < 1.25, (s, sv.max())
+                if s[0] != s[1]:
+                    assert sv.min() > 0.65, (s, sv.min())
+                else:
+                    assert np.mean((sv > 0.65) & (sv < 1.25)) > 0.85, (s, np.mean(sv > 0.65))
+            w[i] -= lr * np.sqrt(max(1.0, s[0] / s[1])) * O
+    opt.sync_weights_to_host()
+    st = opt.export_state()
+    for i, (p, s) in enumerate(zip(params, shapes)):
+        # the update is lr * O(1) on weights of 0.02: 2e-5 of the Newton-Schulz output is far inside 1e-5 of the weight
+        assert_close(p.data, w[i], f"Muon weights {s} #{i}")
+        assert_close(st["muonMomentum"][i], buf[i], f"Muon momentum {s} #{i}")
+    # the device Newton-Schulz alone on the widest shape
+    G = (0.01 * rs.standard_normal((2048, 640))).astype(np.float32)
+    bi, bo = gpu.create_state_buffer(G.nbytes), gpu.create_state_buffer(G.nbytes)
+    gpu.write_state_buffer(bi, G)
+    L.check(gpu.ctx, L.lib.gt_newton_schulz(gpu.ctx, 2048, 640, 5, bi, bo), "gt_newton_schulz")
+    assert_close(gpu.read_state_buffer(bo, G.size), ns64(G.astype(np.float64)), "Newton-Schulz 2048x640", rel_l2=2e-5)
