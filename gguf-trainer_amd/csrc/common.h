@@ -30,11 +30,12 @@ struct gt_ctx {
   struct RopeKey { int T, hd, pos; double base; bool operator<(const RopeKey &o) const {
     if (T != o.T) return T < o.T; if (hd != o.hd) return hd < o.hd; if (pos != o.pos) return pos < o.pos; return base < o.base; } };
   std::map<RopeKey, float *> rope_tables;
-  int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1;
+  int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1, opt_gemm_staged = 0;
   bool prof_on = false;
   std::string prof_prefix;
   std::vector<ProfEvent> prof;
   unsigned attn_smem_set = 0;                   // head dims (bits 32 | 64 | 128) whose dK/dV kernel has its LDS size attribute set
+  unsigned gemm_direct_set = 0;                 // direct-to-LDS GEMM variants whose LDS size attribute is set
   int opt_prof_sample = 1;                      // events around every n-th launch of a label
   struct ProfSeen { int64_t n = 0; double work = 0; };
   std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not

@@ -126,6 +126,7 @@ int gt_set_option(gt_ctx *ctx, const char *key, int value) {
   else if (!strcmp(key, "prof.sample")) ctx->opt_prof_sample = value >= 1 ? value : 1;
   else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
   else if (!strcmp(key, "gemm.splitk")) ctx->opt_gemm_splitk = value;
+  else if (!strcmp(key, "gemm.staged")) ctx->opt_gemm_staged = value;
   else GT_FAIL(ctx, "gt_set_option: unknown key '%s'", key);
   return 0;
 }

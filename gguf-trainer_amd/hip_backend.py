@@ -243,7 +243,7 @@ class HipBackend:
         return out
 
     def set_option(self, key: str, value: int):
-        """Kernel-selection switches for tests and tuning: "attn.generic", "attn.splits", "gemm.tile", "gemm.splitk",
+        """Kernel-selection switches for tests and tuning: "attn.generic", "attn.splits", "gemm.tile", "gemm.splitk", "gemm.staged",
         and "prof.sample" (time every n-th launch of a label)."""
         check(self._ctx, lib.gt_set_option(self._ctx, key.encode(), int(value)), "gt_set_option")
 

@@ -61,8 +61,9 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
 /* Kernel-selection switches for tests and tuning (no reference counterpart; WebGPUBackend exposes
  * attnFlashMinT as a public field for the same purpose, webgpu.ts:305):
  *   "attn.generic" 1 = always take the shape-generic attention kernels, 0 = MFMA kernels where they apply
- *   "gemm.tile"    -1 = heuristic, 0..3 = pin the GEMM tile (64x64, 128x64, 128x128, 128x192)
+ *   "gemm.tile"    -1 = heuristic, 0..12 = pin the GEMM tile configuration (tests and tuning)
  *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor
+ *   "gemm.staged"  1 = always stage GEMM operands through registers (0: aligned shapes load straight into LDS)
  *   "attn.splits"  -1 = heuristic, n >= 1 = pin the workgroups per attention tile (MFMA kernels, at most 8)
  *   "prof.sample"  n >= 1: gt_prof_begin/end time about 1 in n launches of a label (default 1 = all) */
 int gt_set_option(gt_ctx *ctx, const char *key, int value);

@@ -32,7 +32,8 @@ def test_linear_frozen_weight_and_split_k(gpu, ref):
             "linear frozen", frozen=(1,))
 
 
-@pytest.mark.parametrize("M,N,K", [(200, 152, 200), (130, 100, 72), (70, 83, 75), (257, 193, 101)])
+@pytest.mark.parametrize("M,N,K", [(200, 152, 200), (130, 100, 72), (70, 83, 75), (257, 193, 101), (200, 152, 96), (132, 100, 64),
+                                   (260, 196, 128)])
 def test_gemm_every_tile_shape_and_kind(gpu, M, N, K):
     """Every tile configuration of the GEMM, NT / NN / TN, store and accumulate, split-K 1 and 3, on shapes that leave
     partial tiles on both edges and a K tail (aligned leading dimensions take the vectorised loaders with the
@@ -47,19 +48,24 @@ def test_gemm_every_tile_shape_and_kind(gpu, M, N, K):
         for kind, (A, B) in enumerate([(a, b), (a, np.ascontiguousarray(b.T)), (np.ascontiguousarray(a.T), np.ascontiguousarray(b.T))]):
             gpu.write_state_buffer(da, A)
             gpu.write_state_buffer(db, B)
-            for tile in range(12):
+            for tile in range(13):
                 for splitk in ((1, 3) if kind == 2 else (1,)):
                     for acc in (0, 1):
-                        gpu.set_option("gemm.tile", tile)
-                        gpu.set_option("gemm.splitk", splitk)
-                        gpu.write_state_buffer(dc, c0)
-                        gpu.gemm(kind, acc, M, N, K, da, db, dc)
-                        got = gpu.read_state_buffer(dc, M * N).reshape(M, N)
-                        assert_close(got, (want + c0 if acc else want).astype(np.float32),
-                                     f"gemm kind {kind} tile {tile} splitk {splitk} acc {acc} {M}x{N}x{K}")
+                        # staged = 1 pins the register-staged kernels; 0 lets the aligned shapes (K a multiple of 32, whole
+                        # 16-byte chunks) take the kernels that load operands straight into LDS where the tile has one
+                        for staged in ((0, 1) if K % 32 == 0 else (0,)):
+                            gpu.set_option("gemm.tile", tile)
+                            gpu.set_option("gemm.splitk", splitk)
+                            gpu.set_option("gemm.staged", staged)
+                            gpu.write_state_buffer(dc, c0)
+                            gpu.gemm(kind, acc, M, N, K, da, db, dc)
+                            got = gpu.read_state_buffer(dc, M * N).reshape(M, N)
+                            assert_close(got, (want + c0 if acc else want).astype(np.float32),
+                                         f"gemm kind {kind} tile {tile} splitk {splitk} acc {acc} staged {staged} {M}x{N}x{K}")
     finally:
         gpu.set_option("gemm.tile", -1)
         gpu.set_option("gemm.splitk", -1)
+        gpu.set_option("gemm.staged", 0)
 
 
 @pytest.mark.parametrize("rows,K,r", [(16, 64, 16), (100, 192, 16), (257, 1024, 16), (333, 128, 8), (64, 64, 3), (129, 256, 32),
