@@ -363,7 +363,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
         for (int i = 0; i < TM; i++)
 #pragma unroll
           for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s4], fb[j][s4], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][s4], fa[i][s4], acc[i][j], 0, 0, 0);   // C^T tile
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
@@ -376,23 +376,46 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   bool add;
   if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
   else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0; }
+  // The MFMAs above take the B tile as their first operand, so an accumulator holds a C^T tile: lane l32 is the row
+  // of C, and registers 4q..4q+3 are four consecutive columns 8q + 4g + (0..3): one 16-byte store (and, when
+  // accumulating, one 16-byte load issued before any store) instead of four scalar ones.
+  const bool vec_c = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const int col = n0 + wn * (TN * 32) + j * 32 + l32;
-      const int rbase = m0 + wm * (TM * 32) + i * 32 + 4 * g;
-      float old[16];
-      if (add) {
-        const float *cc = C + min(col, a.N - 1);
+      const int row = m0 + wm * (TM * 32) + i * 32 + l32;
+      const int cbase = n0 + wn * (TN * 32) + j * 32 + 4 * g;
+      if (vec_c) {
+        v4f old[4];
+        if (add) {
+          const float *cr = C + (size_t)min(row, a.M - 1) * ldc;
 #pragma unroll
-        for (int r = 0; r < 16; r++) old[r] = cc[(size_t)min(rbase + 8 * (r / 4) + (r % 4), a.M - 1) * ldc];
-      }
-      if (col >= a.N) continue;
+          for (int q = 0; q < 4; q++) old[q] = *reinterpret_cast<const v4f *>(cr + min(cbase + 8 * q, a.N - 4));
+        }
+        if (row >= a.M) continue;
+        float *cr = C + (size_t)row * ldc;
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int row = rbase + 8 * (r / 4) + (r % 4);
-        if (row < a.M) C[(size_t)row * ldc + col] = add ? old[r] + acc[i][j][r] : acc[i][j][r];
+        for (int q = 0; q < 4; q++) {
+          const int col = cbase + 8 * q;
+          if (col >= a.N) continue;                       // N is a multiple of 4 here: a chunk is all in or all out
+          v4f o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          if (add) o += old[q];
+          *reinterpret_cast<v4f *>(cr + col) = o;
+        }
+      } else {
+        if (row >= a.M) continue;
+        float *cr = C + (size_t)row * ldc;
+        float old[16];
+        if (add) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) old[r] = cr[min(cbase + 8 * (r / 4) + (r % 4), a.N - 1)];
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int col = cbase + 8 * (r / 4) + (r % 4);
+          if (col < a.N) cr[col] = add ? old[r] + acc[i][j][r] : acc[i][j][r];
+        }
       }
     }
 }
