@@ -35,7 +35,7 @@ struct gt_ctx {
   std::string prof_prefix;
   std::vector<ProfEvent> prof;
   unsigned attn_smem_set = 0;                   // head dims (bits 32 | 64 | 128) whose dK/dV kernel has its LDS size attribute set
-  unsigned gemm_direct_set = 0;                 // direct-to-LDS GEMM variants whose LDS size attribute is set
+  uint64_t gemm_direct_set = 0;                 // direct-to-LDS GEMM variants whose LDS size attribute is set
   int opt_prof_sample = 1;                      // events around every n-th launch of a label
   struct ProfSeen { int64_t n = 0; double work = 0; };
   std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not

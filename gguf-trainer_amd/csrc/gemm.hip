@@ -271,37 +271,43 @@ __device__ __forceinline__ void load_to_lds16(const float *src, float *wave_base
 #endif
 }
 
-template <int R, bool KC, int NT>
+template <int R, bool KC, int NT, int BKD>
 struct DirectTile {
-  static constexpr int CH = R * 8;                 // 16-byte chunks per stage (R rows x 32 k)
-  static constexpr int PER = CH / NT;              // wave-level loads per wavefront and stage
-  static_assert(CH % NT == 0, "tile must be a whole number of wave loads");
+  static constexpr int CPR = BKD / 4;              // 16-byte chunks per row of a k-contiguous tile (8 or 4)
+  static constexpr int CH = R * CPR;               // chunks per stage (R rows x BKD k)
+  static constexpr int WL = CH / 64;               // wave-level loads per stage, dealt round-robin to the wavefronts
+  static constexpr int NW = NT / 64;
+  static constexpr int PER = (WL + NW - 1) / NW;   // per wavefront; when WL is not a multiple of NW the spare slots
+  static_assert(CH % 64 == 0, "tile must be a whole number of wave loads");   // repeat an earlier load (same data, same place)
+  __device__ static __forceinline__ int load_index(int wave, int i) { return (wave + i * NW) % WL; }
+  // XOR swizzle of a row's chunks: any 16 consecutive rows put a given chunk on 16 different bank groups
+  __device__ static __forceinline__ int sw(int row) { return CPR == 8 ? (row & 7) : ((row & 3) ^ ((row >> 2) & 3)); }
   // source of this lane's chunk in load i of its wavefront, for the stage that starts at k = 0
   __device__ static __forceinline__ const float *src(const float *p, int ld, int r0, int Rtot, int wave, int i, int lane) {
-    const int slot = (wave * PER + i) * 64 + lane;
+    const int slot = load_index(wave, i) * 64 + lane;
     if (KC) {
-      const int row = slot / 8, c = (slot % 8) ^ (row & 7);
+      const int row = slot / CPR, c = (slot % CPR) ^ sw(row);
       return p + (size_t)min(r0 + row, Rtot - 1) * ld + 4 * c;
     }
     const int k = slot / (R / 4), c4 = slot % (R / 4);
     return p + (size_t)k * ld + min(r0 + 4 * c4, Rtot - 4);
   }
-  __device__ static __forceinline__ size_t stage_step(int ld) { return KC ? (size_t)32 : (size_t)32 * ld; }
+  __device__ static __forceinline__ size_t stage_step(int ld) { return KC ? (size_t)BKD : (size_t)BKD * ld; }
   // MFMA inputs of this lane for the four steps of K-run c: tile row `row`, g = lane/32 (k = 8c + 4g + s at step s)
   __device__ static __forceinline__ v4f fetch(const float *lds, int row, int c, int g) {
-    if (KC) return *reinterpret_cast<const v4f *>(lds + row * 32 + 4 * ((2 * c + g) ^ (row & 7)));
+    if (KC) return *reinterpret_cast<const v4f *>(lds + row * BKD + 4 * ((2 * c + g) ^ sw(row)));
     const float *q = lds + (8 * c + 4 * g) * R + row;
     return v4f{q[0], q[R], q[2 * R], q[3 * R]};
   }
 };
 
-template <int BM, int BN, int WM, int WN, int KIND>
+template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
-  constexpr int BK = 32, NT = WM * WN * 64;
+  constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  using TA = DirectTile<BM, KIND != GT_TN, NT>;
-  using TB = DirectTile<BN, KIND == GT_NT, NT>;
-  extern __shared__ __attribute__((aligned(16))) float smem[];   // [2][A tile | B tile]
+  using TA = DirectTile<BM, KIND != GT_TN, NT, BK>;
+  using TB = DirectTile<BN, KIND == GT_NT, NT, BK>;
+  extern __shared__ __attribute__((aligned(16))) float smem[];   // [NSTG][A tile | B tile]
   constexpr int STAGE = (TA::CH + TB::CH) * 4;                // floats per stage
   if (a.M < 0) smem[threadIdx.x] = 0.f;                       // never taken: keeps the LDS array "written" for the compiler
 
@@ -324,15 +330,15 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
 
   const float *pa[TA::PER], *pb[TB::PER];
 #pragma unroll
-  for (int i = 0; i < TA::PER; i++) pa[i] = TA::src(A, a.lda, m0, a.M, wave, i, lane) + (size_t)(k0 / 32) * TA::stage_step(a.lda);
+  for (int i = 0; i < TA::PER; i++) pa[i] = TA::src(A, a.lda, m0, a.M, wave, i, lane) + (size_t)(k0 / BK) * TA::stage_step(a.lda);
 #pragma unroll
-  for (int i = 0; i < TB::PER; i++) pb[i] = TB::src(B, a.ldb, n0, a.N, wave, i, lane) + (size_t)(k0 / 32) * TB::stage_step(a.ldb);
+  for (int i = 0; i < TB::PER; i++) pb[i] = TB::src(B, a.ldb, n0, a.N, wave, i, lane) + (size_t)(k0 / BK) * TB::stage_step(a.ldb);
   const size_t sta = TA::stage_step(a.lda), stb = TB::stage_step(a.ldb);
 #define ISSUE(buf_)                                                                                              \
   {                                                                                                              \
     float *sa_ = smem + (buf_) * STAGE, *sb_ = sa_ + TA::CH * 4;                                                 \
-    _Pragma("unroll") for (int i = 0; i < TA::PER; i++) { load_to_lds16(pa[i], sa_ + (wave * TA::PER + i) * 256); pa[i] += sta; } \
-    _Pragma("unroll") for (int i = 0; i < TB::PER; i++) { load_to_lds16(pb[i], sb_ + (wave * TB::PER + i) * 256); pb[i] += stb; } \
+    _Pragma("unroll") for (int i = 0; i < TA::PER; i++) { load_to_lds16(pa[i], sa_ + TA::load_index(wave, i) * 256); pa[i] += sta; } \
+    _Pragma("unroll") for (int i = 0; i < TB::PER; i++) { load_to_lds16(pb[i], sb_ + TB::load_index(wave, i) * 256); pb[i] += stb; } \
   }
 
   v16f acc[TM][TN];
@@ -343,12 +349,23 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  ISSUE(0)
-  __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the direct loads have landed
-  __syncthreads();
+  // Ring of NSTG stages. Step k: wait until this wavefront's loads of stage k have landed (the younger stages may
+  // still be in flight), barrier (every wavefront's part of stage k is there, and everybody is done reading the
+  // buffer of stage k-1), issue stage k+NSTG-1 into that buffer, compute stage k.
+  constexpr int LPS = TA::PER + TB::PER;                      // loads per wavefront and stage
+  constexpr int INFLIGHT = (NSTG - 2) * LPS;                  // loads that may be outstanding when stage k is needed
+  static_assert(INFLIGHT < 64, "vmcnt holds six bits");
+  const int nstage = (kend - k0) / BK;
+#pragma unroll
+  for (int st = 0; st < NSTG - 1; st++)
+    if (st < nstage) ISSUE(st)
   int buf = 0;
-  for (int k = k0; k < kend; k += BK) {
-    if (k + BK < kend) ISSUE(buf ^ 1)
+  for (int st = 0; st < nstage; st++) {
+    // vmcnt(n): bits 3:0 and 15:14 of the immediate; the other counters are left at "no wait"
+    if (st + NSTG - 2 < nstage) __builtin_amdgcn_s_waitcnt(0x0F70 | (INFLIGHT & 15) | ((INFLIGHT >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                  // the tail: fewer stages are in flight than INFLIGHT assumes
+    __syncthreads();
+    if (st + NSTG - 1 < nstage) { const int nb = (buf + NSTG - 1) % NSTG; ISSUE(nb) }
     const float *sa = smem + buf * STAGE, *sb = sa + TA::CH * 4;
 #pragma unroll
     for (int c = 0; c < BK / 8; c++) {
@@ -365,9 +382,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
           for (int j = 0; j < TN; j++)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][s4], fa[i][s4], acc[i][j], 0, 0, 0);   // C^T tile
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    buf ^= 1;
+    buf = (buf + 1) % NSTG;
   }
 #undef ISSUE
 
@@ -420,25 +435,25 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
     }
 }
 
-template <int BM, int BN, int WM, int WN, int KIND>
+template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG>
 static int launch_direct_kind(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
-  constexpr int smem = 2 * (BM + BN) * 32 * 4;
-  if (!(ctx->gemm_direct_set & (1u << slot))) {       // once per context (device): more LDS than a kernel gets by default
-    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, KIND>),
+  constexpr int smem = NSTG * (BM + BN) * BK * 4;
+  if (!(ctx->gemm_direct_set & (1ull << slot))) {       // once per context (device): more LDS than a kernel gets by default
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    ctx->gemm_direct_set |= 1u << slot;
+    ctx->gemm_direct_set |= 1ull << slot;
   }
-  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, KIND>), dim3(a.nbm * a.nbn, 1, zdim), dim3(WM * WN * 64), smem, ctx->stream, a);
+  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG>), dim3(a.nbm * a.nbn, 1, zdim), dim3(WM * WN * 64), smem, ctx->stream, a);
   GT_LAUNCHED(ctx);
   return 0;
 }
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int BK, int NSTG>
 static int launch_direct(gt_ctx *ctx, int kind, GemmArgs &a, int zdim, int slot) {
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
-  if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT>(ctx, a, zdim, 3 * slot);
-  if (kind == GT_NN) return launch_direct_kind<BM, BN, WM, WN, GT_NN>(ctx, a, zdim, 3 * slot + 1);
-  return launch_direct_kind<BM, BN, WM, WN, GT_TN>(ctx, a, zdim, 3 * slot + 2);
+  if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG>(ctx, a, zdim, 3 * slot);
+  if (kind == GT_NN) return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG>(ctx, a, zdim, 3 * slot + 1);
+  return launch_direct_kind<BM, BN, WM, WN, GT_TN, BK, NSTG>(ctx, a, zdim, 3 * slot + 2);
 }
 
 // C (+)= sum over splits, in split order
@@ -571,11 +586,11 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   int rc;
   if (direct_ok && !ctx->opt_gemm_staged) {
     switch (cfg) {
-      case 6: return launch_direct<128, 128, 2, 2>(ctx, kind, a, zdim, 0) || reduce_splits(ctx, a, M, N, splits, acc);
-      case 7: return launch_direct<128, 192, 2, 2>(ctx, kind, a, zdim, 1) || reduce_splits(ctx, a, M, N, splits, acc);
-      case 8: return launch_direct<128, 96, 4, 1>(ctx, kind, a, zdim, 2) || reduce_splits(ctx, a, M, N, splits, acc);
-      case 11: return launch_direct<128, 64, 2, 2>(ctx, kind, a, zdim, 3) || reduce_splits(ctx, a, M, N, splits, acc);
-      case 12: return launch_direct<64, 192, 2, 2>(ctx, kind, a, zdim, 4) || reduce_splits(ctx, a, M, N, splits, acc);
+      case 6: return launch_direct<128, 128, 2, 2, 32, 2>(ctx, kind, a, zdim, 0) || reduce_splits(ctx, a, M, N, splits, acc);
+      case 7: return launch_direct<128, 192, 2, 2, 32, 2>(ctx, kind, a, zdim, 1) || reduce_splits(ctx, a, M, N, splits, acc);
+      case 8: return launch_direct<128, 96, 4, 1, 32, 2>(ctx, kind, a, zdim, 2) || reduce_splits(ctx, a, M, N, splits, acc);
+      case 11: return launch_direct<128, 64, 2, 2, 32, 2>(ctx, kind, a, zdim, 3) || reduce_splits(ctx, a, M, N, splits, acc);
+      case 12: return launch_direct<64, 192, 2, 2, 32, 2>(ctx, kind, a, zdim, 4) || reduce_splits(ctx, a, M, N, splits, acc);
       default: break;
     }
   }
