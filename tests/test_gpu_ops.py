@@ -494,3 +494,15 @@ def test_profiler_labels_times_and_sampling(gpu, ref, sample):
         ms, count, work = prof[label]
         assert ms >= 0 and count == 7
     assert prof[gemm[0]][2] == 7 * 2 * 40 * 40 * 48
+
+
+def test_unknown_option_is_an_error(gpu):
+    """gt_set_option refuses a key it does not know and says which; known keys round-trip."""
+    L = mod("lib")
+    rc = L.lib.gt_set_option(gpu.ctx, b"gemm.no_such_switch", 1)
+    assert rc != 0 and b"gemm.no_such_switch" in L.lib.gt_last_error(gpu.ctx)
+    with pytest.raises(RuntimeError, match="no_such_switch"):
+        gpu.set_option("attn.no_such_switch", 0)
+    for key, default in (("gemm.tile", -1), ("gemm.splitk", -1), ("gemm.staged", 0), ("attn.generic", 0), ("attn.splits", -1),
+                         ("prof.sample", 1)):
+        gpu.set_option(key, default)
