@@ -48,6 +48,28 @@ struct GemmArgs {
   int K2, lda2, ldb2;
 };
 
+// Which output tile (pid, N fastest) and which K split or batch member (z) a workgroup works on. Workgroups are handed
+// to the 8 XCDs round-robin in dispatch order (x fastest, then z), each XCD with its own L2. Renumber so that one XCD
+// walks a contiguous range of tiles: neighbours then share their A row panel in that L2. With K splits the range is over
+// the split-major list of (split, tile) pairs, so the workgroups resident on an XCD at one time are (nearly) all the
+// tiles of ONE split, walking the same K range: every operand slab they load is shared through that L2. (With the tiles
+// renumbered per split only, every XCD held a few tiles of every split in flight and dW missed L2 for 6x its operands.)
+__device__ __forceinline__ void tile_of_workgroup(const GemmArgs &a, int &pid, int &z) {
+  const int nblk = a.nbm * a.nbn;
+  if (a.splits > 1) {
+    const int total = nblk * a.splits, lin = blockIdx.x + blockIdx.z * nblk;
+    const int xcd = lin % 8, idx = lin / 8, base = total / 8, rem = total % 8;
+    const int w = xcd * base + (xcd < rem ? xcd : rem) + idx;
+    z = w / nblk;
+    pid = w % nblk;
+  } else {
+    const int p = blockIdx.x;
+    const int xcd = p % 8, idx = p / 8, base = nblk / 8, rem = nblk % 8;
+    pid = xcd * base + (xcd < rem ? xcd : rem) + idx;
+    z = blockIdx.z;
+  }
+}
+
 // One operand tile of R rows x BKT k, kept in LDS as [row][BKT+4] with the 16-byte K chunks of a row XOR-swizzled by
 // (row/8) mod (BKT/4). KC: k contiguous in memory (element (r,k) at p[r*ld + k]), copied with one ds_write_b128 per
 // float4. Otherwise row contiguous (element (r,k) at p[k*ld + r]): eight lanes read one 128-byte line of a k-row and
@@ -144,17 +166,10 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
   __shared__ __attribute__((aligned(16))) float sA[TA::LDS_WORDS];
   __shared__ __attribute__((aligned(16))) float sB[TB::LDS_WORDS];
 
-  // Workgroup i runs on XCD i mod 8, each XCD with its own L2. Renumber so that one XCD walks a
-  // contiguous range of tiles (N fastest): neighbours then share their A row panel in that L2.
-  int nblk = a.nbm * a.nbn;
-  int pid = blockIdx.x;
-  {
-    int xcd = pid % 8, idx = pid / 8, base = nblk / 8, rem = nblk % 8;
-    pid = xcd * base + (xcd < rem ? xcd : rem) + idx;
-  }
+  int pid, z;
+  tile_of_workgroup(a, pid, z);
   const int pm = pid / a.nbn, pn = pid % a.nbn;
   const int m0 = pm * BM, n0 = pn * BN;
-  const int z = blockIdx.z;
   const float *A = a.A, *B = a.B;
   int k0 = 0, kend = a.K;
   if (a.splits > 1) { k0 = z * a.kchunk; kend = min(a.K, k0 + a.kchunk); }
@@ -311,15 +326,10 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   constexpr int STAGE = (TA::CH + TB::CH) * 4;                // floats per stage
   if (a.M < 0) smem[threadIdx.x] = 0.f;                       // never taken: keeps the LDS array "written" for the compiler
 
-  int nblk = a.nbm * a.nbn;
-  int pid = blockIdx.x;
-  {
-    int xcd = pid % 8, idx = pid / 8, base = nblk / 8, rem = nblk % 8;
-    pid = xcd * base + (xcd < rem ? xcd : rem) + idx;
-  }
+  int pid, z;
+  tile_of_workgroup(a, pid, z);
   const int pm = pid / a.nbn, pn = pid % a.nbn;
   const int m0 = pm * BM, n0 = pn * BN;
-  const int z = blockIdx.z;
   const float *A = a.A, *B = a.B;
   int k0 = 0, kend = a.K;
   if (a.splits > 1) { k0 = z * a.kchunk; kend = min(a.K, k0 + a.kchunk); }
