@@ -317,6 +317,17 @@ struct DirectTile {
     const int k = slot / (R / 4), c4 = slot % (R / 4);
     return p + (size_t)k * ld + min(r0 + 4 * c4, Rtot - 4);
   }
+  // The same for a second K segment of K2 <= BKD (a multiple of 8) that fills one stage partly: chunks past K2 repeat
+  // valid ones (they are loaded but never fed to an MFMA), so nothing is read outside the operand.
+  __device__ static __forceinline__ const float *src2(const float *p, int ld, int r0, int Rtot, int K2, int wave, int i, int lane) {
+    const int slot = load_index(wave, i) * 64 + lane;
+    if (KC) {
+      const int row = slot / CPR, c = ((slot % CPR) ^ sw(row)) % (K2 / 4);
+      return p + (size_t)min(r0 + row, Rtot - 1) * ld + 4 * c;
+    }
+    const int k = (slot / (R / 4)) % K2, c4 = slot % (R / 4);
+    return p + (size_t)k * ld + min(r0 + 4 * c4, Rtot - 4);
+  }
   __device__ static __forceinline__ size_t stage_step(int ld) { return KC ? (size_t)BKD : (size_t)BKD * ld; }
   // MFMA inputs of this lane for the four steps of K-run c: tile row `row`, g = lane/32 (k = 8c + 4g + s at step s)
   __device__ static __forceinline__ v4f fetch(const float *lds, int row, int c, int g) {
@@ -326,7 +337,7 @@ struct DirectTile {
   }
 };
 
-template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG>
+template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -359,6 +370,16 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
     _Pragma("unroll") for (int i = 0; i < TA::PER; i++) { load_to_lds16(pa[i], sa_ + TA::load_index(wave, i) * 256); pa[i] += sta; } \
     _Pragma("unroll") for (int i = 0; i < TB::PER; i++) { load_to_lds16(pb[i], sb_ + TB::load_index(wave, i) * 256); pb[i] += stb; } \
   }
+  // the stage of the second segment (SEG2): its sources are computed when it is issued, once per workgroup
+#define ISSUE2(buf_)                                                                                             \
+  {                                                                                                              \
+    float *sa_ = smem + (buf_) * STAGE, *sb_ = sa_ + TA::CH * 4;                                                 \
+    _Pragma("unroll") for (int i = 0; i < TA::PER; i++)                                                          \
+      load_to_lds16(TA::src2(a.A2, a.lda2, m0, a.M, a.K2, wave, i, lane), sa_ + TA::load_index(wave, i) * 256);  \
+    _Pragma("unroll") for (int i = 0; i < TB::PER; i++)                                                          \
+      load_to_lds16(TB::src2(a.B2, a.ldb2, n0, a.N, a.K2, wave, i, lane), sb_ + TB::load_index(wave, i) * 256);  \
+  }
+#define ISSUE_STAGE(buf_, st_) { if (SEG2 && (st_) == nstage - 1) ISSUE2(buf_) else ISSUE(buf_) }
 
   v16f acc[TM][TN];
 #pragma unroll
@@ -374,35 +395,40 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   constexpr int LPS = TA::PER + TB::PER;                      // loads per wavefront and stage
   constexpr int INFLIGHT = (NSTG - 2) * LPS;                  // loads that may be outstanding when stage k is needed
   static_assert(INFLIGHT < 64, "vmcnt holds six bits");
-  const int nstage = (kend - k0) / BK;
+  const int nstage = (kend - k0) / BK + (SEG2 ? 1 : 0);
 #pragma unroll
   for (int st = 0; st < NSTG - 1; st++)
-    if (st < nstage) ISSUE(st)
+    if (st < nstage) ISSUE_STAGE(st, st)
   int buf = 0;
   for (int st = 0; st < nstage; st++) {
     // vmcnt(n): bits 3:0 and 15:14 of the immediate; the other counters are left at "no wait"
     if (st + NSTG - 2 < nstage) __builtin_amdgcn_s_waitcnt(0x0F70 | (INFLIGHT & 15) | ((INFLIGHT >> 4) << 14));
     else __builtin_amdgcn_s_waitcnt(0x0F70);                  // the tail: fewer stages are in flight than INFLIGHT assumes
     __syncthreads();
-    if (st + NSTG - 1 < nstage) { const int nb = (buf + NSTG - 1) % NSTG; ISSUE(nb) }
+    if (st + NSTG - 1 < nstage) { const int nb = (buf + NSTG - 1) % NSTG; ISSUE_STAGE(nb, st + NSTG - 1) }
     const float *sa = smem + buf * STAGE, *sb = sa + TA::CH * 4;
+    const int nrun = (SEG2 && st == nstage - 1) ? a.K2 / 8 : BK / 8;      // the second segment fills its stage partly
 #pragma unroll
     for (int c = 0; c < BK / 8; c++) {
-      v4f fa[TM], fb[TN];
+      if (!SEG2 || c < nrun) {                                             // wave-uniform
+        v4f fa[TM], fb[TN];
 #pragma unroll
-      for (int i = 0; i < TM; i++) fa[i] = TA::fetch(sa, wm * (TM * 32) + i * 32 + l32, c, g);
+        for (int i = 0; i < TM; i++) fa[i] = TA::fetch(sa, wm * (TM * 32) + i * 32 + l32, c, g);
 #pragma unroll
-      for (int j = 0; j < TN; j++) fb[j] = TB::fetch(sb, wn * (TN * 32) + j * 32 + l32, c, g);
+        for (int j = 0; j < TN; j++) fb[j] = TB::fetch(sb, wn * (TN * 32) + j * 32 + l32, c, g);
 #pragma unroll
-      for (int s4 = 0; s4 < 4; s4++)
+        for (int s4 = 0; s4 < 4; s4++)
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+          for (int i = 0; i < TM; i++)
 #pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][s4], fa[i][s4], acc[i][j], 0, 0, 0);   // C^T tile
+            for (int j = 0; j < TN; j++)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][s4], fa[i][s4], acc[i][j], 0, 0, 0);   // C^T tile
+      }
     }
     buf = (buf + 1) % NSTG;
   }
+#undef ISSUE_STAGE
+#undef ISSUE2
 #undef ISSUE
 
   float *C;
@@ -454,25 +480,30 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
     }
 }
 
-template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG>
+template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2>
 static int launch_direct_kind(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   constexpr int smem = NSTG * (BM + BN) * BK * 4;
   if (!(ctx->gemm_direct_set & (1ull << slot))) {       // once per context (device): more LDS than a kernel gets by default
-    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG>),
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG, SEG2>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     ctx->gemm_direct_set |= 1ull << slot;
   }
-  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG>), dim3(a.nbm * a.nbn, 1, zdim), dim3(WM * WN * 64), smem, ctx->stream, a);
+  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG, SEG2>), dim3(a.nbm * a.nbn, 1, zdim), dim3(WM * WN * 64), smem, ctx->stream, a);
   GT_LAUNCHED(ctx);
   return 0;
 }
+// slot: index of the tile shape (0..4); the bit of (shape, kind, one or two segments) in gemm_direct_set follows from it
 template <int BM, int BN, int WM, int WN, int BK, int NSTG>
 static int launch_direct(gt_ctx *ctx, int kind, GemmArgs &a, int zdim, int slot) {
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
-  if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG>(ctx, a, zdim, 3 * slot);
-  if (kind == GT_NN) return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG>(ctx, a, zdim, 3 * slot + 1);
-  return launch_direct_kind<BM, BN, WM, WN, GT_TN, BK, NSTG>(ctx, a, zdim, 3 * slot + 2);
+  if (a.K2 > 0) {                // two K segments: NT / NN only
+    if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG, true>(ctx, a, zdim, 15 + 2 * slot);
+    return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG, true>(ctx, a, zdim, 15 + 2 * slot + 1);
+  }
+  if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG, false>(ctx, a, zdim, 3 * slot);
+  if (kind == GT_NN) return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG, false>(ctx, a, zdim, 3 * slot + 1);
+  return launch_direct_kind<BM, BN, WM, WN, GT_TN, BK, NSTG, false>(ctx, a, zdim, 3 * slot + 2);
 }
 
 // C (+)= sum over splits, in split order
@@ -547,8 +578,8 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   // Tiles with a K step of 32 have a variant that loads operands straight into LDS (gemm_direct); it wants whole K
   // steps and whole 16-byte chunks along the contiguous index of every operand. Where it applies it is 2-8 % faster
   // than the register-staged kernel of the same tile and changes which tile is best, hence two tables.
-  const bool direct_ok = vec && K2 == 0 && K % 32 == 0 && (kind != GT_TN || (M % 4 == 0 && M >= 4)) &&
-                         (kind == GT_NT || (N % 4 == 0 && N >= 4));
+  const bool direct_ok = vec && K % 32 == 0 && (kind != GT_TN || (M % 4 == 0 && M >= 4)) && (kind == GT_NT || (N % 4 == 0 && N >= 4)) &&
+                         (K2 == 0 || (kind != GT_TN && K2 % 8 == 0 && K2 <= 32));   // a short second segment rides in one more stage
   struct Cand { int cfg; double eff; };
   static const Cand cand_nn[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
   static const Cand cand_tn[] = {{8, 1.00}, {11, 0.99}, {10, 0.92}, {6, 0.90}, {7, 0.78}, {0, 0.72}};

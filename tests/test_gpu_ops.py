@@ -103,10 +103,12 @@ def test_rank_products(gpu, rows, K, r):
     assert rc != 0 and b"gt_rank_down" in L.lib.gt_last_error(gpu.ctx)
 
 
-@pytest.mark.parametrize("M,N,K1,K2", [(200, 152, 96, 16), (130, 100, 72, 5), (257, 193, 101, 33), (64, 64, 16, 16)])
+@pytest.mark.parametrize("M,N,K1,K2", [(200, 152, 96, 16), (130, 100, 72, 5), (257, 193, 101, 33), (64, 64, 16, 16), (260, 196, 128, 8),
+                                       (132, 100, 64, 32), (300, 576, 192, 24), (200, 152, 96, 40)])
 def test_gemm_pair(gpu, M, N, K1, K2):
-    """C (+)= A1.B1 + A2.B2 in one K loop (the LoRA linear and its dX): every kind, store and accumulate, a few tile
-    shapes, against a float64 sum of the two products."""
+    """C (+)= A1.B1 + A2.B2 in one K loop (the LoRA linear and its dX): every kind, store and accumulate, several tile
+    shapes, against a float64 sum of the two products. K1 a multiple of 32 with K2 = 8 ... 32 takes the kernels that
+    load operands straight into LDS (the second segment fills one more stage partly); the rest the staged ones."""
     rs = np.random.RandomState(M + K2)
     a1, b1 = rs.standard_normal((M, K1)).astype(np.float32), rs.standard_normal((N, K1)).astype(np.float32)
     a2, b2 = rs.standard_normal((M, K2)).astype(np.float32), rs.standard_normal((N, K2)).astype(np.float32)
@@ -119,7 +121,7 @@ def test_gemm_pair(gpu, M, N, K1, K2):
         for kind, ops in enumerate([(a1, b1, a2, b2), (a1, T(b1), a2, T(b2)), (T(a1), T(b1), T(a2), T(b2))]):
             for buf, arr in zip(bufs, ops):
                 gpu.write_state_buffer(buf, arr)
-            for tile in (-1, 0, 7, 8, 10):
+            for tile in (-1, 0, 6, 7, 8, 10, 11, 12):
                 for acc in (0, 1):
                     gpu.set_option("gemm.tile", tile)
                     gpu.write_state_buffer(bufs[4], c0)
