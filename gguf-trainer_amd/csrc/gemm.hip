@@ -5,7 +5,7 @@
 // Two kernels share the tile shapes and the epilogue. gemm_direct (aligned shapes: K a multiple of 32, whole 16-byte
 // chunks along every operand's contiguous index) brings operand tiles from global memory straight into LDS, double
 // buffered, one barrier per K step; it is described where it is defined. gemm_kernel, described here, stages them
-// through registers and takes every shape, and the two-segment products.
+// through registers and takes every shape (two-segment products with a long or odd second segment included).
 //
 // Shape of the kernel. A workgroup of WM x WN wavefronts owns a BM x BN tile of C and walks K in
 // steps of 16 or 32. Each wavefront owns a (BM/WM) x (BN/WN) sub-tile as TM x TN MFMA tiles of 32x32,
