@@ -230,7 +230,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-              "(no collectives are part of it, see DESIGN.md on sharding)", file=sys.stderr)
+              "(no collectives are part of it: the path would shard over sequences with one gradient sum per step)", file=sys.stderr)
         sys.exit(2)
 
     import torch  # device plumbing only: make sure a GPU is there before touching the library
