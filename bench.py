@@ -223,6 +223,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
     ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (BASELINE configs[1] shapes)")
+    ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
     ap.add_argument("--profile-all", action="store_true",
                     help="time every kernel label (not only the GEMMs) over the timed region and print the table to stderr")
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS),
@@ -248,6 +249,7 @@ def main():
     model = arch.Model(cfg, synth_weights(arch, cfg))
     n_params = sum(p.size for p in model.params())
     gpu = hb.require_gpu("bench.py")
+    gpu.batch_linears = not a.no_pair
     if wl.get("lora"):
         rs = np.random.RandomState(3)
         rank = wl["lora"]

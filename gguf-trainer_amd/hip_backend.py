@@ -72,10 +72,20 @@ class HipBackend:
         self._transients: list = []       # (tensor weakref-free strong ref, entry) in creation order
         self._scratch: list = []          # (buf, nbytes) raw transients: id uploads, saved statistics
         self._regions_opened = 0
+        self._pend = None                 # (x, T, out, in, x data, w data, out data) of a held-back linear launch
+        self.batch_linears = True
         self._profiling = False
         self._destroyed = False
 
     # ---- install (webgpu.ts:393-399) ---------------------------------------------------------------
+    # ---- a linear's forward launch is held back by one op: two consecutive linears over the same input with the same
+    # shape (k and v, gate and up) then go out as ONE batched launch, which fills the chip better than two small ones
+    def _flush(self):
+        p = self._pend
+        if p is not None:
+            self._pend = None
+            check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, p[1], p[2], p[3], p[4], p[5], p[6]), "linear")
+
     def install(self):
         ag.set_ops_backend(self)
 
@@ -137,8 +147,11 @@ class HipBackend:
         self._transients.append((out, e))
         return out, e
 
-    def _data(self, t: Tensor) -> int:
-        """Device address of t's values, as an op input."""
+    def _data(self, t: Tensor, launch_held: bool = True) -> int:
+        """Device address of t's values, as an op input. launch_held = False is for an op that only records the
+        address for later (a lazy activation): a held-back linear launch may then stay held."""
+        if launch_held:
+            self._flush()
         e = self._entry_for(t)
         e.consumers += 1
         if e.lazy_act is not None:
@@ -146,6 +159,7 @@ class HipBackend:
         return e.data
 
     def _materialise(self, t: Tensor, e: _Entry):
+        self._flush()
         x, act = e.lazy_act
         e.lazy_act = None
         e.data = self._acquire(e.nbytes)
@@ -156,6 +170,7 @@ class HipBackend:
     def _gdst(self, t: Tensor) -> tuple:
         """(gradient buffer, acc) for a backward kernel about to contribute to t's gradient;
         (0, 0) when t takes no gradient (a frozen parameter)."""
+        self._flush()
         e = self._entries.get(t)
         if e is None:
             e = self._entry_for(t)
@@ -169,6 +184,7 @@ class HipBackend:
 
     def _gsrc(self, t: Tensor) -> int:
         """Gradient buffer of an op output inside its backward closure."""
+        self._flush()
         e = self._entries.get(t)
         if e is None:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
@@ -184,11 +200,13 @@ class HipBackend:
 
     # ---- public buffer surface (webgpu.ts:1432-1537) ----------------------------------------------------
     def upload_params(self, tensors):
+        self._flush()
         for t in tensors:
             e = self._entry_for(t)
             check(self._ctx, lib.gt_h2d(self._ctx, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
 
     def buffers_for(self, t: Tensor) -> dict:
+        self._flush()
         e = self._entry_for(t)
         if t.requires_grad and e.grad == 0:
             e.grad = self._acquire(e.nbytes)
@@ -219,6 +237,7 @@ class HipBackend:
                 e.grad_init = True
 
     def seed_grad_from_host(self, t: Tensor):
+        self._flush()
         e = self._entries.get(t)
         if e is None:
             raise RuntimeError("seed_grad_from_host: tensor has no device buffers")
@@ -234,10 +253,12 @@ class HipBackend:
         return out.value
 
     def write_state_buffer(self, b: int, arr: np.ndarray):
+        self._flush()
         arr = np.ascontiguousarray(arr)
         check(self._ctx, lib.gt_h2d(self._ctx, b, arr.ctypes.data_as(C.c_void_p), arr.nbytes), "gt_h2d")
 
     def read_state_buffer(self, b: int, n: int, dtype=np.float32) -> np.ndarray:
+        self._flush()
         out = np.empty(n, dtype=dtype)
         check(self._ctx, lib.gt_d2h(self._ctx, out.ctypes.data_as(C.c_void_p), b, out.nbytes), "gt_d2h")
         return out
@@ -282,6 +303,7 @@ class HipBackend:
         """Wait for the stream; read back `reads` (values) and the accumulated gradients of every
         trainable external tensor touched since the last sync that is not kept on the device; recycle
         all intermediates. The graph is unusable for backward afterwards."""
+        self._flush()
         nbytes = 0
         for t in reads:
             e = self._entries.get(t)
@@ -309,10 +331,12 @@ class HipBackend:
 
     def reclaim_step_transients(self, keep=()):
         """Free a finished micro-batch's intermediates mid-step; parameter gradients keep accumulating."""
+        self._flush()
         check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")
         self._release_transients(keep)
 
     def destroy(self):
+        self._pend = None
         if not self._destroyed:
             self._destroyed = True
             lib.gt_ctx_destroy(self._ctx)
@@ -320,10 +344,12 @@ class HipBackend:
     # ---- profiling (webgpu.ts:830-880) -----------------------------------------------------------------------
     def start_profile(self, prefix: str = ""):
         """Time every launch whose label starts with `prefix` ("" = all) with HIP events on the stream."""
+        self._flush()
         check(self._ctx, lib.gt_prof_begin(self._ctx, prefix.encode()), "gt_prof_begin")
 
     def stop_profile(self) -> dict:
         """label -> (total ms, launches, algorithmic work: FLOP or bytes)."""
+        self._flush()
         recs = (ProfRec * 128)()
         n = C.c_int()
         check(self._ctx, lib.gt_prof_end(self._ctx, recs, 128, C.byref(n)), "gt_prof_end")
@@ -335,6 +361,7 @@ class HipBackend:
         return len(self._transients)
 
     def end_region(self, mark: int, keep):
+        self._flush()
         keep_ids = {id(t) for t in keep}
         tail = self._transients[mark:]
         del self._transients[mark:]
@@ -360,9 +387,23 @@ class HipBackend:
     def linear(self, x: Tensor, w: Tensor) -> Tensor:
         T, ind = x.shape
         outd = w.shape[0]
+        p = self._pend
+        pair = self.batch_linears and p is not None and p[0] is x and p[1:4] == (T, outd, ind)
+        if pair:
+            self._pend = None               # taken: _data below must not launch it on its own
         xd, wd = self._data(x), self._data(w)
         out, e = self._make_out([T, outd], [x, w])
-        check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, T, outd, ind, xd, wd, e.data), "linear")
+        if pair and (wd - p[5]) % 16 == 0 and (e.data - p[6]) % 16 == 0:
+            # the held-back linear and this one as one batch of two: same input, weights and outputs a stride apart
+            check(self._ctx, lib.gt_gemm_batched(self._ctx, NT, 0, T, outd, ind, xd, 0, p[5], (wd - p[5]) // 4,
+                                                 p[6], (e.data - p[6]) // 4, 2), "linear x2")
+        else:
+            if pair:
+                check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, p[1], p[2], p[3], p[4], p[5], p[6]), "linear")
+            if self.batch_linears:
+                self._pend = (x, T, outd, ind, xd, wd, e.data)      # launched by the next op, or paired with it
+            else:
+                check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, T, outd, ind, xd, wd, e.data), "linear")
         wants_dw = w.requires_grad
 
         def bw():
@@ -474,7 +515,7 @@ class HipBackend:
         return out
 
     def _activation(self, x: Tensor, act: int) -> Tensor:
-        xd = self._data(x)
+        xd = self._data(x, launch_held=not self.fuse_glu)
         out, e = self._make_out(x.shape, [x], alloc=not self.fuse_glu)
         if self.fuse_glu:
             e.lazy_act = (x, act)
@@ -684,6 +725,7 @@ class HipBackend:
 
     # ---- raw GEMM for tests and benches (webgpu.ts:1654) --------------------------------------------------------------
     def gemm(self, kind: int, acc: int, M: int, N: int, K: int, a: int, b: int, c: int):
+        self._flush()
         check(self._ctx, lib.gt_gemm(self._ctx, kind, acc, M, N, K, a, b, c), "gemm")
 
 

@@ -508,3 +508,55 @@ def test_unknown_option_is_an_error(gpu):
     for key, default in (("gemm.tile", -1), ("gemm.splitk", -1), ("gemm.staged", 0), ("attn.generic", 0), ("attn.splits", -1),
                          ("prof.sample", 1)):
         gpu.set_option(key, default)
+
+
+def test_paired_linear_launches(gpu, ref):
+    """Two consecutive linears over the same input with the same shape (k and v, gate and up) go out as one batched
+    launch; results and gradients are those of two launches, also when a lazy activation sits between them, when the
+    first output is consumed by something else first, and when the second linear has another shape."""
+    ag = mod("autograd")
+    r = R(ref, 21)
+    x, w1, w2, w3 = r(70, 48), r(40, 48), r(40, 48), r(24, 48)
+
+    def pair(m, x_, a_, b_):
+        return m.add(m.linear(x_, a_), m.linear(x_, b_))
+
+    def gated(m, x_, a_, b_):                    # silu(linear) recorded between the two linears, then the fused product
+        g = m.silu(m.linear(x_, a_))
+        return m.mul(g, m.linear(x_, b_))
+
+    def act_then_add(m, x_, a_, b_):             # the activation is consumed by add, not by a gate*up product
+        g = m.silu(m.linear(x_, a_))
+        return m.add(g, m.linear(x_, b_))
+
+    def used_between(m, x_, a_, b_):             # the first output feeds another op before the second linear
+        y1 = m.linear(x_, a_)
+        s = m.scale(y1, 0.5)
+        return m.add(s, m.linear(x_, b_))
+
+    for name, fn in (("pair", pair), ("gated", gated), ("activation then add", act_then_add), ("used between", used_between)):
+        op_case(gpu, ref, [x, w1, w2], lambda m, *t, fn=fn: fn(m, *t), lambda m, *t, fn=fn: fn(m, *t), f"paired linears: {name}")
+    # a differently shaped second linear does not pair: q [40] then k [24] over the same input, summed over columns
+    def mixed(m, x_, a_, b_):
+        y1, y2 = m.linear(x_, a_), m.linear(x_, b_)
+        return m.add(m.linear(y1, m_ones(m, 24, 40)), y2)
+    ones = np.ones((24, 40), np.float32)
+
+    def m_ones(m, o, i):
+        return m.Tensor(ones, [o, i], False)
+    op_case(gpu, ref, [x, w1, w3], mixed, mixed, "paired linears: other shape second")
+    # the pair is one GEMM launch, the unpaired form two
+    counts = {}
+    for batch in (True, False):
+        gpu.batch_linears = batch
+        try:
+            hx, ha, hb = (ag.Tensor(a, list(a.shape), False) for a in (x, w1, w2))
+            gpu.install()
+            gpu.start_profile("gemm.")
+            y = pair(ag, hx, ha, hb)
+            gpu.sync([y])
+            counts[batch] = sum(v[1] for v in gpu.stop_profile().values())
+        finally:
+            gpu.uninstall()
+            gpu.batch_linears = True
+    assert counts == {True: 1, False: 2}, counts
