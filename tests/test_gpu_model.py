@@ -295,3 +295,34 @@ def test_single_row_and_single_token_edges(gpu, ref):
     w = 1 + 0.3 * R(4)
     op_case(gpu, ref, [R(1, 4), w], lambda ag, x, g: ag.rms_norm(x, g, 1e-6), lambda rf, x, g: rf.rms_norm(x, g, 1e-6), "rmsNorm one row")
     op_case(gpu, ref, [R(5, 3)], lambda ag, e: ag.embedding(e, [4]), lambda rf, e: rf.embedding(e, [4]), "embedding one id")
+
+
+@pytest.mark.parametrize("loss_chunk", [0, 64])
+def test_forward_only_scoring_reads_back_the_loss_alone(gpu, ref, loss_chunk):
+    """gpu-parity.ts:1430-1495 (eval freeze gate), for this backend's protocol: a scoring pass (forward, sync, no
+    backward) stages back the loss scalar and nothing else whether or not the parameters are frozen, allocates no
+    gradient accumulator in either arm (they are created by the first backward write), and freezing moves no bit of
+    the score."""
+    ag, arch = mod("autograd"), mod("arch")
+    kw = dict(arch="gemma3", vocab=64, hidden=64, layers=4, heads=4, kv_heads=2, head_dim=16, ffn=256, rope_base=1e6,
+              rope_base_local=1e4, sliding_window=16, swa_pattern=2, rms_eps=1e-6)
+    ids = np.array([(i * 11 + 5) % 64 for i in range(65)])
+    out = {}
+    for freeze in (False, True):
+        _, model = build_pair(ref, kw, seed=5, std=0.05)
+        if freeze:
+            for p in model.params():
+                p.requires_grad = False
+        gpu.install()
+        try:
+            gpu.upload_params(model.params())
+            loss = arch.sequence_loss(model, ids[:-1], ids[1:], loss_chunk)
+            gpu.sync([loss])
+            out[freeze] = (gpu.last_sync_readback_bytes, float(loss.data[0]),
+                           sum(1 for p in model.params() if gpu._entries[p].grad != 0))
+        finally:
+            gpu.uninstall()
+            gpu.sync([])
+    assert out[False][0] == 4 and out[True][0] == 4, out
+    assert out[False][2] == 0 and out[True][2] == 0, out
+    assert out[False][1] == out[True][1] and np.isfinite(out[True][1])
