@@ -315,14 +315,18 @@ class HipBackend:
             nbytes += e.nbytes
         for t in self._touched:
             e = self._entries.get(t)
-            if e is None or e.keep_grad or not t.requires_grad:
+            if e is None or e.keep_grad:
                 continue
-            if e.grad and e.grad_init:
-                check(self._ctx, lib.gt_d2h(self._ctx, t.grad.ctypes.data_as(C.c_void_p), e.grad, e.nbytes), "gt_d2h")
-                nbytes += e.nbytes
-            else:
-                t.grad.fill(0)
-            e.grad_init = False            # read back: the next step starts from zero
+            if t.requires_grad:
+                if e.grad and e.grad_init:
+                    check(self._ctx, lib.gt_d2h(self._ctx, t.grad.ctypes.data_as(C.c_void_p), e.grad, e.nbytes), "gt_d2h")
+                    nbytes += e.nbytes
+                else:
+                    t.grad.fill(0)
+            # The window ends here: the next one starts this accumulator from zero. Keyed on the accumulator, not on
+            # the flag as it reads now: a parameter frozen after its backward and thawed later would otherwise have the
+            # next window add on top of this one's gradients (gpu-parity.ts:1980-2028).
+            e.grad_init = False
         self._touched = []
         self._touched_ids = set()
         check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")

@@ -326,3 +326,42 @@ def test_forward_only_scoring_reads_back_the_loss_alone(gpu, ref, loss_chunk):
     assert out[False][0] == 4 and out[True][0] == 4, out
     assert out[False][2] == 0 and out[True][2] == 0, out
     assert out[False][1] == out[True][1] and np.isfinite(out[True][1])
+
+
+def test_gradient_rearm_survives_a_mid_window_freeze(gpu, ref):
+    """gpu-parity.ts:1980-2028: parameters frozen between a window's backward and its sync, thawed afterwards. The
+    accumulators still hold that window's gradients, so the window after the thaw must start them afresh: same inputs
+    and weights give the first window's gradients, not twice them."""
+    ag, arch = mod("autograd"), mod("arch")
+    kw = dict(arch="gemma3", vocab=64, hidden=64, layers=4, heads=4, kv_heads=2, head_dim=16, ffn=256, rope_base=1e6,
+              rope_base_local=1e4, sliding_window=16, swa_pattern=2, rms_eps=1e-6)
+    ids = np.array([(i * 11 + 5) % 64 for i in range(33)])
+    _, model = build_pair(ref, kw, seed=5, std=0.05)
+    gpu.install()
+    try:
+        gpu.upload_params(model.params())
+
+        def window(freeze_before_sync=False):
+            loss = arch.sequence_loss(model, ids[:-1], ids[1:], 0)
+            ag.backward(loss, 1.0)
+            if freeze_before_sync:
+                for p in model.params():
+                    p.requires_grad = False
+            gpu.sync([loss])
+            return [p.grad.copy() for p in model.params()]
+
+        first = window()
+        window(freeze_before_sync=True)
+        for p in model.params():
+            p.requires_grad = True
+        third = window()
+    finally:
+        gpu.uninstall()
+        gpu.sync([])
+    worst, n = 0.0, 0
+    for a, b in zip(first, third):
+        keep = np.abs(a) >= 1e-6
+        if keep.any():
+            worst = max(worst, float(np.abs(b[keep] / a[keep] - 1).max()))
+            n += int(keep.sum())
+    assert n > 0 and worst < 1e-4, (worst, n)
