@@ -316,8 +316,10 @@ def test_forward_only_scoring_reads_back_the_loss_alone(gpu, ref, loss_chunk):
         gpu.install()
         try:
             gpu.upload_params(model.params())
+            clears = gpu.grad_clears_issued
             loss = arch.sequence_loss(model, ids[:-1], ids[1:], loss_chunk)
             gpu.sync([loss])
+            assert gpu.grad_clears_issued == clears        # a forward-only window zeroes nothing (gpu-parity.ts:1825-1950)
             out[freeze] = (gpu.last_sync_readback_bytes, float(loss.data[0]),
                            sum(1 for p in model.params() if gpu._entries[p].grad != 0))
         finally:
@@ -365,3 +367,34 @@ def test_gradient_rearm_survives_a_mid_window_freeze(gpu, ref):
             worst = max(worst, float(np.abs(b[keep] / a[keep] - 1).max()))
             n += int(keep.sum())
     assert n > 0 and worst < 1e-4, (worst, n)
+
+
+def test_empty_sync_recycles_without_corrupting_queued_work(gpu, ref):
+    """gpu-parity.ts:2338-2410: with gradients kept on the device a bare sync() stages nothing and hands every
+    intermediate back to the pool; a second chain then reuses exactly those buffers (the pool does not grow) while the
+    first chain's gradients, already queued, still come out right."""
+    ag = mod("autograd")
+    T, HID, OUT = 24, 64, 40
+    r = ref.Mulberry32(0xFEED)
+    xs, w1s, w2s = r.fill_randn([T, HID], 0.8), r.fill_randn([HID, HID], 0.8), r.fill_randn([OUT, HID], 0.8)
+    targets = [(i * 7 + 3) % OUT for i in range(T)]
+    rt = [ref.Tensor(a, list(a.shape), True) for a in (xs, w1s, w2s)]
+    ref.backward(ref.cross_entropy(ref.linear(ref.gelu(ref.linear(rt[0], rt[1])), rt[2]), targets), 1.0)
+    ht = [ag.Tensor(a, list(a.shape), True) for a in (xs, w1s, w2s)]
+    for t in ht:
+        gpu.keep_grad_on_device(t)
+    gpu.install()
+    try:
+        ag.backward(ag.cross_entropy(ag.linear(ag.gelu(ag.linear(ht[0], ht[1])), ht[2]), targets), 1.0)
+        gpu.sync([])                         # stages nothing, recycles everything
+        assert gpu.last_sync_readback_bytes == 0
+        pool_before = gpu._pool_bytes
+        ag.gelu(ag.linear(ht[0], ht[1]))     # reuses the buffers the first chain released
+        assert gpu._pool_bytes == pool_before
+        gpu.sync([])
+        for t, rr, nm in zip(ht, rt, ("x", "w1", "w2")):
+            got = gpu.read_state_buffer(gpu.buffers_for(t)["grad"], t.size)
+            assert_close(got, rr.grad, f"recycle reuse d{nm}")
+    finally:
+        gpu.uninstall()
+        gpu.sync([])
