@@ -284,3 +284,37 @@ def test_checkpoint_cadence(gpu, ref):
     assert fired_at(checkpoint_every=10 ** 9, checkpoint_every_ms=1e-3) == [1, 2, 3, 4, 5]
     assert fired_at() == []
     assert fired_at(checkpoint_every_ms=1e9) == []
+
+
+def test_reclaim_transients_changes_no_bit(gpu, ref):
+    """gpu-parity.ts:438-565: freeing each micro-batch's intermediates mid-step only recycles pool buffers earlier.
+    Three micro-batches per step (two reclaim boundaries), Muon + AdamW, four steps: the dense loss, the chunked loss
+    (chunk 16 over a vocabulary of 50: four spans with a ragged tail, tied readout accumulating into the embedding
+    gradient) and the recomputed graph each give the same losses and weights with reclaim on and off, to the bit; the
+    recomputed losses equal the dense ones to the bit, the chunked ones to 1e-3."""
+    ag, optim, train = mod("autograd"), mod("optim"), mod("train")
+    tokens = micro_tokens(ref, 0x5EC1)
+
+    def run(reclaim, loss_chunk=0, recompute=False):
+        _, model = build_pair(ref, MICRO, seed=5, jitter_gains=False)
+        hm, ha = model.param_groups()
+        ag.set_checkpointing(recompute)
+        try:
+            hist = train.train_lm_hip_resident(model, gpu, optim.MuonHip(gpu, hm, ha, **MUON_HYPER),
+                                               train.WindowSampler(tokens, 8, ag.mulberry32(7)), 4, 3, 8, loss_chunk=loss_chunk,
+                                               stacked=False, reclaim=reclaim)
+        finally:
+            ag.set_checkpointing(False)
+        return hist, [p.data.copy() for p in model.params()]
+
+    dense_off, dense_on = run(False), run(True)
+    assert dense_on[0] == dense_off[0]
+    assert all(np.array_equal(a, b) for a, b in zip(dense_on[1], dense_off[1]))
+    chunk_off, chunk_on = run(False, 16), run(True, 16)
+    assert chunk_on[0] == chunk_off[0]
+    assert all(np.array_equal(a, b) for a, b in zip(chunk_on[1], chunk_off[1]))
+    for a, b in zip(chunk_off[0], dense_off[0]):
+        assert abs(a - b) <= 1e-3 + 1e-3 * abs(b), (chunk_off[0], dense_off[0])
+    rc_off, rc_on = run(False, 0, True), run(True, 0, True)
+    assert rc_off[0] == dense_off[0] and rc_on[0] == dense_off[0]
+    assert all(np.array_equal(a, b) for a, b in zip(rc_on[1], dense_off[1]))
