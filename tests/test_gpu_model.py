@@ -398,3 +398,34 @@ def test_empty_sync_recycles_without_corrupting_queued_work(gpu, ref):
     finally:
         gpu.uninstall()
         gpu.sync([])
+
+
+def test_recompute_memory_gate(ref):
+    """gpu-parity.ts:1363-1420: the buffer pool (a high-water mark) is flat in the number of steps (sync drains the
+    regions' buffers), flat in the number of micro-batches when transients are reclaimed between them, and clearly
+    smaller with recompute than without. A fresh backend per arm, sequential micro-batches of 128 tokens."""
+    ag, optim, train, hb = mod("autograd"), mod("optim"), mod("train"), mod("hip_backend")
+    kw = dict(arch="gemma3", vocab=64, hidden=64, layers=4, heads=4, kv_heads=2, head_dim=16, ffn=256, rope_base=1e6,
+              rope_base_local=1e4, sliding_window=16, swa_pattern=2, rms_eps=1e-6)
+    tokens = [(i * 7 + 3) % 64 for i in range(8192)]
+
+    def pool_for(recompute, reclaim, steps, batch):
+        g = hb.HipBackend(0)
+        _, model = build_pair(ref, kw, seed=5, std=0.05)
+        hm, ha = model.param_groups()
+        ag.set_checkpointing(recompute)
+        try:
+            train.train_lm_hip_resident(model, g, optim.MuonHip(g, hm, ha, lr=0.01, momentum=0.95, aux={"lr": 3e-3, "weight_decay": 0.0, "clip": 1.0}),
+                                        train.WindowSampler(tokens, 128, ag.mulberry32(7)), steps, batch, 128, stacked=False,
+                                        reclaim=reclaim, log_every=100)
+            return g._pool_bytes
+        finally:
+            ag.set_checkpointing(False)
+            g.destroy()
+
+    s2, s6 = pool_for(True, False, 2, 2), pool_for(True, False, 6, 2)
+    assert s6 <= s2 * 1.01, (s2, s6)
+    b2, b4 = pool_for(True, True, 3, 2), pool_for(True, True, 3, 4)
+    assert b4 <= b2 * 1.05, (b2, b4)
+    dense = pool_for(False, True, 3, 2)
+    assert b2 < 0.9 * dense, (b2, dense)
