@@ -429,3 +429,29 @@ def test_recompute_memory_gate(ref):
     assert b4 <= b2 * 1.05, (b2, b4)
     dense = pool_for(False, True, 3, 2)
     assert b2 < 0.9 * dense, (b2, dense)
+
+
+def test_resident_step_then_sample_readback(gpu, ref):
+    """gpu-parity.ts:1671-1735: a device-resident step stages back its loss scalars only, and a forward pass after it
+    (sampling) stages back its logits only: the optimizer's parameters keep their gradients on the device."""
+    ag, arch, optim, train = mod("autograd"), mod("arch"), mod("optim"), mod("train")
+    kw = dict(arch="gemma3", vocab=64, hidden=64, layers=4, heads=4, kv_heads=2, head_dim=16, ffn=256, rope_base=1e6,
+              rope_base_local=1e4, sliding_window=16, swa_pattern=2, rms_eps=1e-6)
+    tokens = [(i * 7 + 3) % 64 for i in range(2048)]
+    _, model = build_pair(ref, kw, seed=5, std=0.05)
+    hm, ha = model.param_groups()
+    seen = []
+    train.train_lm_hip_resident(model, gpu, optim.MuonHip(gpu, hm, ha, lr=0.01, momentum=0.95, aux={"lr": 3e-3}),
+                                train.WindowSampler(tokens, 64, ag.mulberry32(7)), 1, 1, 64, stacked=False, reclaim=True,
+                                on_step_time=lambda a, b, rb: seen.append(rb))
+    assert seen == [4]                                   # one micro-batch: one f32 loss
+    prompt = np.array([3, 11, 29, 5, 17])
+    gpu.install()
+    try:
+        logits = model.forward(prompt)
+        gpu.sync([logits])
+        assert gpu.last_sync_readback_bytes == len(prompt) * kw["vocab"] * 4
+        assert np.isfinite(logits.data).all()
+    finally:
+        gpu.uninstall()
+        gpu.sync([])
