@@ -175,10 +175,31 @@ def set_checkpointing(on: bool):
     _checkpointing = on
 
 
+def _assert_self_contained(out, inputs, born):
+    """src/model/autograd.ts:198-215: the block may read its declared inputs and leaves (parameters); a computed tensor
+    built before the block began would have its backward run once per block."""
+    seen = {id(t) for t in inputs}
+    if id(out) in seen:
+        raise ValueError("checkpoint: fn returned one of its inputs; there is nothing to recompute")
+    stack = [out]
+    while stack:
+        t = stack.pop()
+        if id(t) in seen:
+            continue
+        seen.add(id(t))
+        if t._prev and t.seq < born:
+            raise ValueError("checkpoint: the block reads a computed tensor it did not create. "
+                             "Pass it in `inputs`, or move its computation inside the block.")
+        stack.extend(t._prev)
+
+
 def checkpoint(inputs, fn):
+    """src/model/autograd.ts:234-273."""
     if not _checkpointing:
         return fn()
+    born = _created
     out = fn()
+    _assert_self_contained(out, inputs, born)
     out._prev = list(inputs)
 
     def bw():

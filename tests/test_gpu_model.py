@@ -455,3 +455,29 @@ def test_resident_step_then_sample_readback(gpu, ref):
     finally:
         gpu.uninstall()
         gpu.sync([])
+
+
+def test_checkpoint_input_guard_on_device(gpu, ref):
+    """gradcheck.ts:808-829 through the device backend: the guard runs above the dispatch, and a refused block leaves
+    the backend usable (its region is closed by the next sync)."""
+    ag = mod("autograd")
+    r = ref.Mulberry32(12)
+    x = ag.Tensor(r.fill_randn([5, 6], 0.8), [5, 6], True)
+    w1 = ag.Tensor(r.fill_randn([6, 6], 0.8), [6, 6], True)
+    gpu.install()
+    ag.set_checkpointing(True)
+    try:
+        shared = ag.linear(x, w1)
+        with pytest.raises(ValueError, match="did not create"):
+            ag.checkpoint([x], lambda: ag.add(ag.silu(ag.linear(x, w1)), shared))
+        with pytest.raises(ValueError, match="one of its inputs"):
+            ag.checkpoint([x], lambda: x)
+        out = ag.checkpoint([x, shared], lambda: ag.add(ag.silu(ag.linear(x, w1)), shared))
+        gpu.sync([out])
+        want = ref.add(ref.silu(ref.linear(ref.Tensor(x.data, [5, 6]), ref.Tensor(w1.data, [6, 6]))),
+                       ref.linear(ref.Tensor(x.data, [5, 6]), ref.Tensor(w1.data, [6, 6])))
+        assert_close(out.data, want.data, "checkpointed block with a declared shared input")
+    finally:
+        ag.set_checkpointing(False)
+        gpu.uninstall()
+        gpu.sync([])

@@ -204,3 +204,22 @@ def test_checkpoint_bit_identical(ref, arch):
     for g0, g1 in zip(res[0][1], res[1][1]):
         assert g0.tobytes() == g1.tobytes()
     assert any(np.any(g) for g in res[0][1])
+
+
+def test_checkpoint_input_guard(ref):
+    """gradcheck.ts:808-829: a checkpointed block that reads a computed tensor built outside it, or that returns one
+    of its inputs, is refused; the same tensor declared as an input is allowed."""
+    r = ref.Mulberry32(12)
+    x = ref.Tensor(r.fill_randn([5, 6], 0.8), [5, 6], True)
+    w1 = ref.Tensor(r.fill_randn([6, 6], 0.8), [6, 6], True)
+    ref.set_checkpointing(True)
+    try:
+        shared = ref.linear(x, w1)
+        with pytest.raises(ValueError, match="did not create"):
+            ref.checkpoint([x], lambda: ref.add(ref.silu(ref.linear(x, w1)), shared))
+        with pytest.raises(ValueError, match="one of its inputs"):
+            ref.checkpoint([x], lambda: x)
+        out = ref.checkpoint([x, shared], lambda: ref.add(ref.silu(ref.linear(x, w1)), shared))
+        assert out.shape == [5, 6]
+    finally:
+        ref.set_checkpointing(False)
