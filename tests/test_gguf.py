@@ -148,6 +148,8 @@ CFGS = {
                    rope_base_local=1e4, sliding_window=4, swa_pattern=2, rms_eps=2.0 ** -20),
     # hidden 8: the block formats cannot tile an inner dimension of 8 and every matrix falls back to f16
     "llama-narrow": dict(arch="llama", vocab=32, hidden=8, layers=2, heads=2, kv_heads=1, head_dim=4, ffn=16, rope_base=1e5, rms_eps=2.0 ** -17),
+    # tests/qwen3-wide-heads.ts:76-87: an attention block wider than the model, 3 heads of 8 over a width of 12
+    "qwen3-wide": dict(arch="qwen3", vocab=32, hidden=12, layers=2, heads=3, kv_heads=1, head_dim=8, ffn=32, rope_base=1e6, rms_eps=2.0 ** -20),
 }
 
 
@@ -190,7 +192,7 @@ def test_architecture_round_trip(ref, name):
     g = G.read_gguf(G.export_gguf(model, TOK, "q8_0", max_seq=16))
     types = {t["name"]: t["type"] for t in g.tensors}
     assert types["output_norm.weight"] == G.F32 and types["blk.0.attn_norm.weight"] == G.F32
-    assert types["blk.0.ffn_up.weight"] == (G.F16 if name == "llama-narrow" else G.Q8_0)
+    assert types["blk.0.ffn_up.weight"] == (G.Q8_0 if model.cfg.hidden % 32 == 0 else G.F16)
     assert g.metadata["general.file_type"] == 7 and g.metadata["tokenizer.ggml.token_type"][:4] == [3, 3, 4, 1]
     by = {t["name"]: t for t in g.tensors}
     assert by["token_embd.weight"]["dims"] == [model.cfg.hidden, 32]                    # ggml order: [in, out]

@@ -107,6 +107,9 @@ REAL = {
     # Qwen3 head layout: head dim 128 with QK-norm, GQA 4/2
     "qwen3-hd128": dict(arch="qwen3", vocab=2048, hidden=256, layers=2, heads=4, kv_heads=2, head_dim=128, ffn=512,
                         rope_base=1e6, rms_eps=1e-6),
+    # tests/qwen3-wide-heads.ts:30-43: the attention block wider than the model (16 heads of 128 over a width of 544)
+    "qwen3-wide": dict(arch="qwen3", vocab=1024, hidden=544, layers=1, heads=16, kv_heads=8, head_dim=128, ffn=2560,
+                       rope_base=1e6, rms_eps=1e-6),
     # Gemma3: GeGLU, sliding window that cuts the 128-row attention tiles, one global layer in three
     "gemma3-window": dict(arch="gemma3", vocab=2048, hidden=320, layers=3, heads=5, kv_heads=1, head_dim=64, ffn=768,
                           rope_base=1e6, rope_base_local=1e4, sliding_window=96, swa_pattern=3, rms_eps=1e-6),
