@@ -35,7 +35,7 @@ MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (2 * 85594.1 + 36868.8) * 1024,
 SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                rope_base=100000.0, rms_eps=1e-5, tie=True)
 SEQ, BATCH = 2048, 8
-# The other model-sized BASELINE configs, runnable with --config (the default line is configs[3]).
+# The other model-sized benchmark configs, runnable with --config (the default line is configs[3]).
 GEMMA3_95M = dict(arch="gemma3", vocab=32768, hidden=640, layers=12, heads=10, kv_heads=2, head_dim=64, ffn=2048,
                   rope_base=1e6, rope_base_local=1e4, sliding_window=512, swa_pattern=6, rms_eps=1e-6, tie=True)
 QWEN3_06B = dict(arch="qwen3", vocab=151936, hidden=1024, layers=28, heads=16, kv_heads=8, head_dim=128, ffn=3072,
@@ -143,7 +143,7 @@ def cpu_baseline(seconds_hint=20.0):
 
 
 def micro_kernels(gpu, L, reps=10):
-    """BASELINE configs[1]: the isolated backward kernels at the SmolLM2 MLP shape, timed with HIP events on the
+    """benchmark configs[1]: the isolated backward kernels at the SmolLM2 MLP shape, timed with HIP events on the
     library's stream. fp32 dX = dY.W and dW = dY^T.X with X [16384x576], W [1536x576], dY [16384x1536]; softmax-CE
     backward over logits [16384x49152] with 10% of the targets masked; RMSNorm backward on [16384x576]; SwiGLU
     backward on [16384x1536]. Rates are algorithmic work (FLOP, or bytes each tensor is touched once) over time."""
@@ -222,7 +222,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
-    ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (BASELINE configs[1] shapes)")
+    ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (benchmark configs[1] shapes)")
     ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
     ap.add_argument("--profile-all", action="store_true",
                     help="time every kernel label (not only the GEMMs) over the timed region and print the table to stderr")

@@ -1,4 +1,4 @@
-"""BASELINE config 2 at full size (X [16384x576], W [576x1536], dY [16384x1536]; logits [16384x49152]; RMSNorm
+"""benchmark config 2 at full size (X [16384x576], W [576x1536], dY [16384x1536]; logits [16384x49152]; RMSNorm
 [16384x576]): too large for the scalar oracle end to end, so parity is through sampled entries computed in
 float64 on the host, the oracle on sampled rows, and size-independent properties."""
 import numpy as np
@@ -139,7 +139,7 @@ def test_glu_backward_full_size(gpu, ref):
 
 
 FULL = {
-    # BASELINE configs 4, 3 and 5 at their real shapes
+    # benchmark configs 4, 3 and 5 at their real shapes
     "smollm2": dict(model=dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                                rope_base=1e5, rms_eps=1e-5), batch=8),
     "gemma3": dict(model=dict(arch="gemma3", vocab=32768, hidden=640, layers=12, heads=10, kv_heads=2, head_dim=64, ffn=2048,
@@ -151,7 +151,7 @@ FULL = {
 
 @pytest.mark.parametrize("which", ["smollm2", "gemma3", "qwen3_lora"])
 def test_full_size_step_properties(gpu, which):
-    """BASELINE configs 4 (SmolLM2-135M shape), 3 (gemma-style, sliding window 512 on 5 of 6 layers, QK-norm) and 5
+    """benchmark configs 4 (SmolLM2-135M shape), 3 (gemma-style, sliding window 512 on 5 of 6 layers, QK-norm) and 5
     (Qwen3-0.6B shape, head dim 128, vocabulary 151936, frozen base with rank-16 LoRA) at their real sizes, sequences
     of 2048 tokens, forward + backward. Far beyond the scalar oracle, so: the loss of a near-zero random init is ln(V)
     per sequence; the stacked graph (one launch set over B*2048 rows) and the reference's sequential accumulation (B
@@ -223,7 +223,7 @@ def test_full_size_step_properties(gpu, which):
 
 
 def test_adamw_full_size_tensor_list(gpu):
-    """BASELINE config 4's optimizer step at its real size: the 272 tensors of the SmolLM2-135M shape (134.5 M
+    """benchmark config 4's optimizer step at its real size: the 272 tensors of the SmolLM2-135M shape (134.5 M
     parameters), two steps with the global clip active in the first and inactive in the second. Every tensor against
     the closed form of src/train/adam.ts:46-82 evaluated in float64 (vectorised; the scalar oracle covers the small
     cases), and the clip scale against a float64 norm over all gradients."""
@@ -266,7 +266,7 @@ def test_adamw_full_size_tensor_list(gpu):
 
 
 def test_muon_full_size_matrices(gpu):
-    """BASELINE config 3's Muon step on its real matrix shapes (640x640, 128x640, 2048x640, 640x2048; one layer's
+    """benchmark config 3's Muon step on its real matrix shapes (640x640, 128x640, 2048x640, 640x2048; one layer's
     seven matrices twice over so the per-shape batches hold several matrices): momentum, Nesterov, five Newton-Schulz
     iterations and the scaled apply against a float64 evaluation of src/train/muon.ts:69-158, and the property the
     quintic is built for: the singular values of the orthogonalised update land in about [0.7, 1.2]."""

@@ -1,5 +1,5 @@
 """Whole-graph parity: the three architectures, micro-batch accumulation, --recompute, LoRA, stacked
-sequences and BASELINE config 1, HIP backend (through the C ABI) against the CPU oracle."""
+sequences and benchmark config 1, HIP backend (through the C ABI) against the CPU oracle."""
 import math
 
 import numpy as np
@@ -15,7 +15,7 @@ SMALL = {
     "gemma3": dict(arch="gemma3", vocab=61, hidden=48, layers=3, heads=4, kv_heads=1, head_dim=16, ffn=80, rope_base=1e6,
                    rope_base_local=1e4, sliding_window=7, swa_pattern=3, rms_eps=1e-6),
 }
-# BASELINE config 1
+# benchmark config 1
 TINY = dict(arch="llama", vocab=512, hidden=128, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=352, rope_base=1e4, rms_eps=1e-5)
 
 
@@ -209,7 +209,7 @@ def test_lora(gpu, ref, recompute):
 
 
 def test_config1_tiny_llama_step(gpu, ref):
-    """BASELINE config 1: vocab 512, hidden 128, 2 layers, 4/2 heads x 32, SwiGLU 352, tied, weights N(0,0.02) seed 0,
+    """benchmark config 1: vocab 512, hidden 128, 2 layers, 4/2 heads x 32, SwiGLU 352, tied, weights N(0,0.02) seed 0,
     4 sequences of 128 tokens, targets shifted by one; forward + backward + AdamW(lr 1e-3, betas 0.9/0.95, wd 0.1)."""
     optim = mod("optim")
     clears0 = gpu.grad_clears_issued

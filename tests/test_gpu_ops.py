@@ -401,7 +401,7 @@ def test_late_backward_after_sync_is_refused(gpu, ref):
 def test_attention_mfma_shapes(gpu, ref, B, T, Hq, Hkv, hd, window, splits):
     """The matrix-core kernels (hd = 32, 64 and 128): tiles of 128 queries x 32 keys with ragged T, windows that cut tiles,
     GQA group sums, stacked sequences; 1024 x 9/3 x 64 is one SmolLM2 layer at half the sequence length, 16/8 x 128
-    the Qwen3-0.6B head layout, 4 x 128 x 4/2 x 32 the attention of BASELINE config 1. Each shape with one workgroup per tile, with the launch-size heuristic, and with five
+    the Qwen3-0.6B head layout, 4 x 128 x 4/2 x 32 the attention of benchmark config 1. Each shape with one workgroup per tile, with the launch-size heuristic, and with five
     workgroups per tile (partial softmax / dQ / dK,dV folded afterwards, some of them over empty ranges)."""
     ag = mod("autograd")
     gpu.set_option("attn.splits", splits)
