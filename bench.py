@@ -224,6 +224,8 @@ def main():
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
     ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (benchmark configs[1] shapes)")
     ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
+    ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
+                    help="library option for an A/B run, e.g. attn.keep_ds=0 (dQ recomputes the scores) or gemm.staged=1")
     ap.add_argument("--profile-all", action="store_true",
                     help="time every kernel label (not only the GEMMs) over the timed region and print the table to stderr")
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS),
@@ -250,6 +252,9 @@ def main():
     n_params = sum(p.size for p in model.params())
     gpu = hb.require_gpu("bench.py")
     gpu.batch_linears = not a.no_pair
+    for kv in a.set:
+        key, _, val = kv.partition("=")
+        gpu.set_option(key, int(val))
     if wl.get("lora"):
         rs = np.random.RandomState(3)
         rank = wl["lora"]

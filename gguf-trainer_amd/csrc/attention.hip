@@ -249,13 +249,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
 // attention_mfma.hip, compiled once per head dim
 int attn_fwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
 int attn_bwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                    float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                    float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
 int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
 int attn_bwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                    float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                    float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 int attn_bwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                     float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                     float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 static int attn_mfma_supported(int hd) { return hd == 32 || hd == 64 || hd == 128; }
 
 // A launch with fewer 128-row tiles than three per CU is cut further (measured at T = 2048, 9 heads: 1 sequence runs
@@ -327,10 +327,10 @@ static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
   return 0;
 }
 static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
-                         float *part, float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
-  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v)
-      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v)
-                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v))
+                         float *part, float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v)
+      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v)
+                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v))
     return 1;
   if (p.splits > 1) {
     const size_t n4 = (size_t)p.B * p.T * p.Hq * p.hd / 4;
@@ -389,11 +389,16 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   const size_t d_floats = ((size_t)rows + 63) / 64 * 64;
   const size_t part_floats = (mfma && p.splits * group > 1) ? (size_t)2 * p.splits * group * krows * hd : 0;
   const size_t dq_floats = (mfma && p.splits > 1) ? (size_t)p.splits * rows * hd : 0;
+  // dS kept for the dQ product (one [T][T] matrix per sequence and head) when the launch is unsplit, the tiles are whole
+  // and the matrices fit the limit; otherwise dQ recomputes the scores in its own kernel
+  size_t ds_floats = (mfma && ctx->opt_attn_keep_ds && p.splits == 1 && T % 128 == 0 && hd >= 64) ? (size_t)rows * T : 0;
+  if (ds_floats * sizeof(float) > ((size_t)ctx->opt_attn_ds_limit_mb << 20)) ds_floats = 0;
   void *ws;
-  if (gt_ws_reserve(ctx, (d_floats + part_floats + dq_floats) * sizeof(float), &ws)) return 1;
+  if (gt_ws_reserve(ctx, (d_floats + part_floats + dq_floats + ds_floats) * sizeof(float), &ws)) return 1;
   float *Dr = static_cast<float *>(ws);
   float *part = part_floats ? Dr + d_floats : nullptr;
   float *dqpart = dq_floats ? Dr + d_floats + part_floats : nullptr;
+  float *dsb = ds_floats ? Dr + d_floats + part_floats + dq_floats : nullptr;
   {
     ProfScope ps(ctx, "attention.bwd.D");
     const int G = p.hd / 4;
@@ -415,7 +420,7 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
     }
     GT_LAUNCHED(ctx);
   }
-  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dq, acc_q, dk, acc_k, dv, acc_v);
+  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v);
   {
     ProfScope ps(ctx, "attention.bwd.dq");
     size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);

@@ -390,7 +390,8 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
-                                                           float *dk, int acc_k, float *dv, int acc_v, float *part) {
+                                                           float *dk, int acc_k, float *dv, int acc_v, float *part,
+                                                           float *dsb) {
   using IO = TileIO<QT>;
   extern __shared__ __attribute__((aligned(16))) float dkv_smem[];      // 35 KB at hd 64, 69 KB at hd 128
   float *sQ = dkv_smem, *sG = sQ + QT * LD, *sQt = sG + QT * LD, *sGt = sQt + HD * IO::LDT;
@@ -416,7 +417,11 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   load_row_regs(vreg, v + koff, sv, g, 1.0f);
   // queries that can see a key of this workgroup: t in [ktile*128, last key + window - 1]
   const int qt_lo = ktile * (128 / QT);
-  const int t_last = p.window > 0 ? min(p.T - 1, ktile * 128 + 127 + p.window - 1) : p.T - 1;
+  // With a dS matrix to fill (dsb: T a multiple of 128), the loop runs on to the end of the last 128-row tile whose
+  // band of keys (starting at a multiple of 128) still holds this key tile, so that every 32 x 32 block the banded
+  // dQ product will read has been written: zeros where no pair is live.
+  const int t_last = p.window > 0 ? min(p.T - 1, dsb ? ((ktile * 128 + 126 + p.window) & ~127) + 127 : ktile * 128 + 127 + p.window - 1)
+                                  : p.T - 1;
   const int qt_hi = t_last / QT;
   const int nqt = qt_hi - qt_lo + 1;
   const int wave_t_hi = p.window > 0 ? sk0 + 31 + p.window - 1 : p.T - 1;   // last query that sees a key of this wave
@@ -457,7 +462,18 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
     __syncthreads();
     if (it + 1 < niter) prefetch(it + 1);
     const int t0 = (qt_lo + it) * QT;
-    if (t0 + 31 < sk0 || t0 > wave_t_hi || sk0 >= p.T) continue;      // wave-uniform: no (query, key) pair of this tile is live
+    // this lane's column of the dS block of (query stage, keys of this wavefront): rows t0 + 8a + 4g + j. The matrix of a
+    // (sequence, head) is kept as [row tile of 128][key step of 32][128 rows][32 keys]: a wavefront's block is 4 KB in one piece
+    float *dsc = dsb ? dsb + ((((size_t)b * p.Hq + h) * (p.T / 128) + t0 / 128) * (p.T / 32) + sk0 / 32) * 4096 +
+                           (t0 % 128 + 4 * g) * 32 + l32
+                     : nullptr;
+    if (t0 + 31 < sk0 || t0 > wave_t_hi || sk0 >= p.T) {             // wave-uniform: no (query, key) pair of this tile is live
+      if (dsb) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = 0.f;
+      }
+      continue;
+    }
     v16f sc = rows_dot_regs(sQ, kreg, l32, g);
     v16f dp = rows_dot_regs(sG, vreg, l32, g);
     // fully visible tile: every query is at or after every key of the wave, inside the window, and in range
@@ -477,6 +493,10 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
         pr[r] = e;
         ds[r] = e * (dp[r] - dv4[j]) * p.scale;
       }
+    }
+    if (dsb) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = ds[r];
     }
     t_dot_acc<IO::LDT>(vacc, sGt, 0, pr, l32, g);
     t_dot_acc<IO::LDT>(kacc, sQt, 0, ds, l32, g);
@@ -522,8 +542,10 @@ int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
 
 // Dr: the per-row sums D; part: workspace for the dK/dV slices (2 * splits * group slices of B*T*Hkv*hd floats) or
 // null when there is one slice; dqpart: workspace for the dQ partials (splits x dq) or null when splits == 1
+// dsb: workspace for the B*Hq [T][T] dS matrices, or null. With it dK/dV writes dS as it goes and dQ is one banded
+// product dS.K afterwards (5 contractions in all); without it dQ recomputes S and dP in its own kernel (7).
 int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
-                      float *part, float *dqpart, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+                      float *part, float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
   const int group = p.Hq / p.Hkv;
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart) && (p.splits * group == 1 || part),
@@ -533,7 +555,8 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
     ctx->attn_smem_set |= HD;
   }
-  {
+  GT_REQUIRE(ctx, !dsb || (p.splits == 1 && p.T % 128 == 0 && HD >= 64), "attention: dS workspace with an unsupported shape");
+  if (!dsb) {
     ProfScope ps(ctx, "attention.bwd.dq");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
     hipLaunchKernelGGL(FN(attn_bwd_dq_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
@@ -544,7 +567,7 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
     ProfScope ps(ctx, "attention.bwd.dkv");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
     hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k), grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
-                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part);
+                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb);
     GT_LAUNCHED(ctx);
     if (part) {
       size_t n4 = (size_t)p.B * p.T * p.Hkv * HD / 4;
@@ -552,6 +575,10 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
                          P<float>(dk), acc_k, P<float>(dv), acc_v);
       GT_LAUNCHED(ctx);
     }
+  }
+  if (dsb) {
+    ProfScope ps(ctx, "attention.bwd.dq");
+    if (gemm_band_dq(ctx, p.B, p.T, p.Hq, p.Hkv, HD, p.window, dsb, P<const float>(k), P<float>(dq), acc_q)) return 1;
   }
   return 0;
 }

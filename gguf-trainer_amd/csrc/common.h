@@ -31,6 +31,7 @@ struct gt_ctx {
     if (T != o.T) return T < o.T; if (hd != o.hd) return hd < o.hd; if (pos != o.pos) return pos < o.pos; return base < o.base; } };
   std::map<RopeKey, float *> rope_tables;
   int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1, opt_gemm_staged = 0;
+  int opt_attn_keep_ds = 1, opt_attn_ds_limit_mb = 8192;
   bool prof_on = false;
   std::string prof_prefix;
   std::vector<ProfEvent> prof;
@@ -53,6 +54,8 @@ extern thread_local char g_create_err[512];
 #define GT_REQUIRE(ctx, cond, ...) do { if (!(cond)) GT_FAIL(ctx, __VA_ARGS__); } while (0)
 
 int gt_ws_reserve(gt_ctx *ctx, size_t bytes, void **out);
+// gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
+int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc);
 
 // Brackets the launches made during its lifetime with a pair of events when profiling is on.
 struct ProfScope {

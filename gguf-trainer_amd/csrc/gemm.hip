@@ -46,6 +46,11 @@ struct GemmArgs {
   // optional second K segment: C = A.B (+) A2.B2 with the same M, N and operand orientation (K2 = 0: none)
   const float *A2, *B2;
   int K2, lda2, ldb2;
+  // banded batch (gemm_direct<..., BAND>): batch member z = zb * zdiv + zh takes A + z*sA, B + zb*sB + (zh/zgroup)*sB2 and
+  // C + zb*sC + zh*sC2, and the row tile at m0 contracts over k in [band start of m0, m0 + BM) only: the product of a
+  // causal (optionally windowed) score-gradient matrix with the key rows, one (sequence, head) per batch member
+  int zdiv, zgroup, window;
+  int64_t sB2, sC2;
 };
 
 // Which output tile (pm, pn) and which K split or batch member (z) a workgroup works on. Workgroups are handed
@@ -337,7 +342,7 @@ struct DirectTile {
   }
 };
 
-template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2>
+template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2, bool BAND = false>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -348,11 +353,27 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   if (a.M < 0) smem[threadIdx.x] = 0.f;                       // never taken: keeps the LDS array "written" for the compiler
 
   int pm, pn, z;
-  tile_of_workgroup(a, pm, pn, z);
+  if (BAND) {
+    // Row tiles differ in K range (128 ... T keys) and workgroups go to the 8 XCDs round-robin in dispatch order: with a
+    // fixed tile per blockIdx.x one XCD would get every long tile. Rotating the tiles by the batch index hands every
+    // XCD every length in turn.
+    z = blockIdx.z;
+    pn = blockIdx.x % a.nbn;
+    pm = a.nbm - 1 - (int)((blockIdx.x / a.nbn + z) % a.nbm);
+  } else {
+    tile_of_workgroup(a, pm, pn, z);
+  }
   const int m0 = pm * BM, n0 = pn * BN;
   const float *A = a.A, *B = a.B;
   int k0 = 0, kend = a.K;
-  if (a.splits > 1) { k0 = z * a.kchunk; kend = min(a.K, k0 + a.kchunk); }
+  if (BAND) {
+    // A is kept in blocks: [z][row tile of 128][k step of 32][128 rows][32 k], one contiguous 16 KB block per stage
+    static_assert(!BAND || (BM == 128 && BK == 32), "banded A blocks are 128 rows x 32 k");
+    A += z * a.sA + (size_t)pm * (a.K / 32) * 4096;
+    B += (z / a.zdiv) * a.sB + ((z % a.zdiv) / a.zgroup) * a.sB2;
+    k0 = a.window > 0 ? (max(0, m0 - a.window + 1) & ~127) : 0;
+    kend = min(a.K, m0 + BM);
+  } else if (a.splits > 1) { k0 = z * a.kchunk; kend = min(a.K, k0 + a.kchunk); }
   else { A += z * a.sA; B += z * a.sB; }
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / WN, wn = wave % WN;
@@ -360,10 +381,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
 
   const float *pa[TA::PER], *pb[TB::PER];
 #pragma unroll
-  for (int i = 0; i < TA::PER; i++) pa[i] = TA::src(A, a.lda, m0, a.M, wave, i, lane) + (size_t)(k0 / BK) * TA::stage_step(a.lda);
+  for (int i = 0; i < TA::PER; i++)
+    pa[i] = BAND ? TA::src(A, 32, 0, BM, wave, i, lane) + (size_t)(k0 / BK) * 4096
+                 : TA::src(A, a.lda, m0, a.M, wave, i, lane) + (size_t)(k0 / BK) * TA::stage_step(a.lda);
 #pragma unroll
   for (int i = 0; i < TB::PER; i++) pb[i] = TB::src(B, a.ldb, n0, a.N, wave, i, lane) + (size_t)(k0 / BK) * TB::stage_step(a.ldb);
-  const size_t sta = TA::stage_step(a.lda), stb = TB::stage_step(a.ldb);
+  const size_t sta = BAND ? (size_t)4096 : TA::stage_step(a.lda), stb = TB::stage_step(a.ldb);
 #define ISSUE(buf_)                                                                                              \
   {                                                                                                              \
     float *sa_ = smem + (buf_) * STAGE, *sb_ = sa_ + TA::CH * 4;                                                 \
@@ -434,7 +457,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   float *C;
   int ldc;
   bool add;
-  if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
+  if (BAND) { C = a.C + (z / a.zdiv) * a.sC + (z % a.zdiv) * a.sC2; ldc = a.ldc; add = a.acc != 0; }
+  else if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
   else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0; }
   // The MFMAs above take the B tile as their first operand, so an accumulator holds a C^T tile: lane l32 is the row
   // of C, and registers 4q..4q+3 are four consecutive columns 8q + 4g + (0..3): one 16-byte store (and, when
@@ -563,6 +587,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   a.ldc = N;
   a.acc = acc; a.kchunk = K; a.splits = 1; a.Pp = nullptr;
   a.sA = sA; a.sB = sB; a.sC = sC;
+  a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0;
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
              (sA % 4 == 0) && (sB % 4 == 0);
   a.K2 = K2; a.A2 = P<const float>(A2); a.B2 = P<const float>(B2);
@@ -661,6 +686,43 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   }
   if (rc) return rc;
   return reduce_splits(ctx, a, M, N, splits, acc);
+}
+
+// dQ[b][t][h*hd + :] (+)= sum over the keys s visible from t of dS[b*Hq + h][t][s] * K[b][s][(h/group)*hd + :] for every
+// (sequence, head): one banded NN product per pair, all in one launch. dS holds B*Hq [T][T] matrices in blocks
+// [row tile of 128][key step of 32][128 rows][32 keys] (what one pipeline stage loads is one contiguous 16 KB block)
+// whose blocks inside each row tile's band are all written (zeros where a pair is masked); T is a multiple of 128.
+template <int BN>
+static int launch_band(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
+  constexpr int BM = 128, BK = 32, NSTG = 3, WM = 2, WN = 2;
+  constexpr int smem = NSTG * (BM + BN) * BK * 4;
+  if (!(ctx->gemm_direct_set & (1ull << slot))) {
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    ctx->gemm_direct_set |= 1ull << slot;
+  }
+  a.nbm = (int)cdiv(a.M, BM);
+  a.nbn = (int)cdiv(a.N, BN);
+  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>), dim3(a.nbm * a.nbn, 1, zdim), dim3(WM * WN * 64), smem,
+                     ctx->stream, a);
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc) {
+  GT_REQUIRE(ctx, T % 128 == 0 && (hd == 64 || hd == 128), "banded dQ product: T %d must be a multiple of 128 and hd %d 64 or 128", T, hd);
+  GT_REQUIRE(ctx, ((reinterpret_cast<uintptr_t>(dS) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(dQ)) & 15) == 0,
+             "banded dQ product: operands must be 16-byte aligned");
+  GemmArgs a;
+  a.A = dS; a.B = K; a.C = dQ;
+  a.M = T; a.N = hd; a.K = T;
+  a.lda = T; a.ldb = Hkv * hd; a.ldc = Hq * hd;
+  a.acc = acc; a.kchunk = T; a.splits = 1; a.Pp = nullptr;
+  a.sA = (int64_t)T * T; a.sB = (int64_t)T * Hkv * hd; a.sC = (int64_t)T * Hq * hd;
+  a.zdiv = Hq; a.zgroup = Hq / Hkv; a.window = window; a.sB2 = hd; a.sC2 = hd;
+  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0;
+  GT_REQUIRE(ctx, (int64_t)B * Hq <= 65535, "banded dQ product: %lld (sequence, head) pairs exceed the grid", (long long)B * Hq);
+  return hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26);
 }
 
 extern "C" {

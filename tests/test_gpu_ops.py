@@ -431,6 +431,58 @@ def test_attention_mfma_shapes(gpu, ref, B, T, Hq, Hkv, hd, window, splits):
         ref.set_threads(1)
 
 
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 512, 2, 1, 64, 128),
+                                                  (1, 512, 2, 1, 64, 127), (1, 640, 2, 2, 64, 129), (1, 256, 3, 1, 64, 1),
+                                                  (3, 128, 2, 2, 64, 0), (1, 768, 2, 1, 64, 300), (2, 256, 4, 2, 128, 0),
+                                                  (1, 384, 2, 1, 128, 130), (1, 1024, 9, 3, 64, 0)])
+@pytest.mark.parametrize("acc", [0, 1])
+def test_attention_backward_kept_ds_equals_recomputed(gpu, ref, B, T, Hq, Hkv, hd, window, acc):
+    """Whole 128-row tiles, unsplit launch: dK/dV writes the score gradients and dQ is one banded product over them. Against
+    the kernel pair that recomputes the scores for dQ (itself held to the oracle above) and, for the first sequence,
+    against the oracle; windows that end on, before and after a tile edge, window 1, accumulation into a used dq
+    (acc = 1: the gradient buffers start from the same random contents on both paths)."""
+    lib = mod("lib")
+    floor = 1.0 if window == 1 and not acc else 0.0        # window 1: dq and dk are zero up to rounding, compared absolutely
+    r = R(ref, 3 * T + Hq + window)
+    q, k, v = r(B * T, Hq * hd), r(B * T, Hkv * hd), r(B * T, Hkv * hd)
+    up = r(B * T, Hq * hd)
+    init = [r(B * T, Hq * hd), r(B * T, Hkv * hd), r(B * T, Hkv * hd)]
+    bufs = {n: gpu.create_state_buffer(a.nbytes) for n, a in (("q", q), ("k", k), ("v", v), ("up", up), ("out", q), ("dq", q), ("dk", k), ("dv", k))}
+    lse = gpu.create_state_buffer(B * Hq * T * 4)
+    for n, a in (("q", q), ("k", k), ("v", v), ("up", up)):
+        gpu.write_state_buffer(bufs[n], a)
+    gpu.set_option("attn.splits", 1)
+    res = []
+    try:
+        lib.check(gpu.ctx, lib.lib.gt_attn_fwd(gpu.ctx, B, T, Hq, Hkv, hd, window, bufs["q"], bufs["k"], bufs["v"], bufs["out"], lse), "fwd")
+        for keep in (0, 1):
+            gpu.set_option("attn.keep_ds", keep)
+            for n, a in zip(("dq", "dk", "dv"), init):
+                gpu.write_state_buffer(bufs[n], a)
+            lib.check(gpu.ctx, lib.lib.gt_attn_bwd(gpu.ctx, B, T, Hq, Hkv, hd, window, bufs["q"], bufs["k"], bufs["v"], bufs["out"],
+                                                   bufs["up"], lse, bufs["dq"], acc, bufs["dk"], acc, bufs["dv"], acc), "bwd")
+            res.append([gpu.read_state_buffer(bufs[n], a.size).copy() for n, a in zip(("dq", "dk", "dv"), init)])
+    finally:
+        gpu.set_option("attn.keep_ds", 1)
+        gpu.set_option("attn.splits", -1)
+    for a, b, nm in zip(res[1], res[0], ("dq", "dk", "dv")):
+        assert_close(a, b, f"kept dS vs recomputed {nm}", floor=floor)
+    assert np.array_equal(res[1][1], res[0][1]) and np.array_equal(res[1][2], res[0][2])     # dK, dV: the same arithmetic
+    ref.set_threads(min(8, ref.max_threads()))
+    try:
+        s = slice(0, T)
+        rq, rk, rv = (ref.Tensor(a[s], [T, a.shape[1]], True) for a in (q, k, v))
+        o = ref.attention(rq, rk, rv, T, Hq, Hkv, hd, window, parallel_bwd=True)
+        ref.backward_from(o, up[s].reshape(-1))
+        want = rq.grad.reshape(T, -1) + (init[0][s] if acc else 0)
+        if floor:       # exact result zero; f32 rounding of dP - D (two 64-term dot products of O(1) values) leaves ~1e-6 per element
+            assert np.abs(res[1][0].reshape(B * T, -1)[s] - want).max() < 1e-5
+        else:
+            assert_close(res[1][0].reshape(B * T, -1)[s], want, "kept dS dq vs oracle")
+    finally:
+        ref.set_threads(1)
+
+
 def test_attention_mfma_equals_generic_at_full_length(gpu, ref):
     """T = 2048, 9/3 heads x 64 (the SmolLM2 layer), two stacked sequences: both kernel families against each other."""
     ag = mod("autograd")
