@@ -30,6 +30,11 @@
 // dK/dV loops over the query heads of the kv group inside the workgroup and over query tiles in
 // increasing order, so the GQA sum has a fixed order and needs no atomics.
 //
+// Backward in five contractions. With a dS workspace (unsplit launches, T a multiple of 128) dK/dV stores the score
+// gradients it computes, and dQ = dS.K is one banded batched product afterwards (gemm.hip) instead of a kernel that
+// recomputes S and dP: one [T][T] matrix per (sequence, head), kept in blocks [row tile of 128][key step of 32]
+// [128 rows][32 keys], in which every block inside a row tile's band of keys is written (zeros where no pair is live).
+//
 // Small launches (one short sequence, few heads) have fewer tiles than the chip has CUs and their time is the
 // serial loop of the longest tile. For them p.splits > 1 cuts every tile's loop range (key stages in forward and
 // dQ, query stages in dK/dV) into that many workgroups, which write partial results (unnormalised output with
