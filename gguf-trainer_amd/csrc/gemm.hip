@@ -354,12 +354,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
 
   int pm, pn, z;
   if (BAND) {
-    // Row tiles differ in K range (128 ... T keys) and workgroups go to the 8 XCDs round-robin in dispatch order: with a
-    // fixed tile per blockIdx.x one XCD would get every long tile. Rotating the tiles by the batch index hands every
-    // XCD every length in turn.
-    z = blockIdx.z;
-    pn = blockIdx.x % a.nbn;
-    pm = a.nbm - 1 - (int)((blockIdx.x / a.nbn + z) % a.nbm);
+    // Row tiles differ in K range (128 ... T keys). The grid is (batch members, 1, row tiles): dispatch order runs over
+    // the batch members of the longest row tile first, then the next shorter one, so the long workgroups start first and
+    // the short ones fill the gaps at the end, and the 8 XCDs (fed round-robin in dispatch order) get equal lengths.
+    z = blockIdx.x;
+    pn = blockIdx.z % a.nbn;
+    pm = a.nbm - 1 - (int)(blockIdx.z / a.nbn);
   } else {
     tile_of_workgroup(a, pm, pn, z);
   }
@@ -703,7 +703,7 @@ static int launch_band(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   }
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
-  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>), dim3(a.nbm * a.nbn, 1, zdim), dim3(WM * WN * 64), smem,
+  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>), dim3(zdim, 1, a.nbm * a.nbn), dim3(WM * WN * 64), smem,
                      ctx->stream, a);
   GT_LAUNCHED(ctx);
   return 0;
@@ -721,7 +721,7 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.sA = (int64_t)T * T; a.sB = (int64_t)T * Hkv * hd; a.sC = (int64_t)T * Hq * hd;
   a.zdiv = Hq; a.zgroup = Hq / Hkv; a.window = window; a.sB2 = hd; a.sC2 = hd;
   a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0;
-  GT_REQUIRE(ctx, (int64_t)B * Hq <= 65535, "banded dQ product: %lld (sequence, head) pairs exceed the grid", (long long)B * Hq);
+  GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
   return hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26);
 }
 
