@@ -332,7 +332,7 @@ static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
       : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v)
                    : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v))
     return 1;
-  if (p.splits > 1) {
+  if (p.splits > 1 && !dsb) {
     const size_t n4 = (size_t)p.B * p.T * p.Hq * p.hd / 4;
     hipLaunchKernelGGL(attn_slice_sum, dim3((unsigned)cdiv((int64_t)n4, 256)), dim3(256), 0, ctx->stream, dqpart, p.splits, n4,
                        P<float>(dq), acc_q);
@@ -388,11 +388,11 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   if (mfma) p.splits = attn_splits(ctx, B, T, Hq);
   const size_t d_floats = ((size_t)rows + 63) / 64 * 64;
   const size_t part_floats = (mfma && p.splits * group > 1) ? (size_t)2 * p.splits * group * krows * hd : 0;
-  const size_t dq_floats = (mfma && p.splits > 1) ? (size_t)p.splits * rows * hd : 0;
-  // dS kept for the dQ product (one [T][T] matrix per sequence and head) when the launch is unsplit, the tiles are whole
-  // and the matrices fit the limit; otherwise dQ recomputes the scores in its own kernel
-  size_t ds_floats = (mfma && ctx->opt_attn_keep_ds && p.splits == 1 && T % 128 == 0 && hd >= 64) ? (size_t)rows * T : 0;
+  // dS kept for the dQ product (one [T][T] matrix per sequence and head) when the tiles are whole and the matrices fit
+  // the limit; otherwise dQ recomputes the scores in its own kernel (with one partial per split when the launch is split)
+  size_t ds_floats = (mfma && ctx->opt_attn_keep_ds && T % 128 == 0 && hd >= 64) ? (size_t)rows * T : 0;
   if (ds_floats * sizeof(float) > ((size_t)ctx->opt_attn_ds_limit_mb << 20)) ds_floats = 0;
+  const size_t dq_floats = (mfma && p.splits > 1 && !ds_floats) ? (size_t)p.splits * rows * hd : 0;
   void *ws;
   if (gt_ws_reserve(ctx, (d_floats + part_floats + dq_floats + ds_floats) * sizeof(float), &ws)) return 1;
   float *Dr = static_cast<float *>(ws);

@@ -30,7 +30,7 @@
 // dK/dV loops over the query heads of the kv group inside the workgroup and over query tiles in
 // increasing order, so the GQA sum has a fixed order and needs no atomics.
 //
-// Backward in five contractions. With a dS workspace (unsplit launches, T a multiple of 128) dK/dV stores the score
+// Backward in five contractions. With a dS workspace (T a multiple of 128) dK/dV stores the score
 // gradients it computes, and dQ = dS.K is one banded batched product afterwards (gemm.hip) instead of a kernel that
 // recomputes S and dP: one [T][T] matrix per (sequence, head), kept in blocks [row tile of 128][key step of 32]
 // [128 rows][32 keys], in which every block inside a row tile's band of keys is written (zeros where no pair is live).
@@ -553,14 +553,14 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
                       float *part, float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
   const int group = p.Hq / p.Hkv;
-  GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart) && (p.splits * group == 1 || part),
+  GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart || dsb) && (p.splits * group == 1 || part),
              "attention: split backward without a workspace");
   if (!(ctx->attn_smem_set & HD)) {   // once per context (device): more than the 64 KB a kernel gets by default at hd 128
     GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
     ctx->attn_smem_set |= HD;
   }
-  GT_REQUIRE(ctx, !dsb || (p.splits == 1 && p.T % 128 == 0 && HD >= 64), "attention: dS workspace with an unsupported shape");
+  GT_REQUIRE(ctx, !dsb || (p.T % 128 == 0 && HD >= 64), "attention: dS workspace with an unsupported shape");
   if (!dsb) {
     ProfScope ps(ctx, "attention.bwd.dq");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));

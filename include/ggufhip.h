@@ -66,7 +66,7 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
  *   "gemm.staged"  1 = always stage GEMM operands through registers (0: aligned shapes load straight into LDS)
  *   "attn.splits"  -1 = heuristic, n >= 1 = pin the workgroups per attention tile (MFMA kernels, at most 8)
  *   "attn.keep_ds" 1 (default) = attention backward keeps the score gradients dS in the workspace and computes dQ as one
- *                  banded product over them (unsplit launches, T a multiple of 128, hd 64 or 128); 0 = dQ always
+ *                  banded product over them (T a multiple of 128, hd 64 or 128); 0 = dQ always
  *                  recomputes the scores in its own kernel
  *   "attn.ds_limit_mb" largest dS workspace taken for that, in MiB (default 8192; B*Hq*T*T*4 bytes are needed)
  *   "prof.sample"  n >= 1: gt_prof_begin/end time about 1 in n launches of a label (default 1 = all) */

@@ -435,9 +435,9 @@ def test_attention_mfma_shapes(gpu, ref, B, T, Hq, Hkv, hd, window, splits):
                                                   (1, 512, 2, 1, 64, 127), (1, 640, 2, 2, 64, 129), (1, 256, 3, 1, 64, 1),
                                                   (3, 128, 2, 2, 64, 0), (1, 768, 2, 1, 64, 300), (2, 256, 4, 2, 128, 0),
                                                   (1, 384, 2, 1, 128, 130), (1, 1024, 9, 3, 64, 0)])
-@pytest.mark.parametrize("acc", [0, 1])
-def test_attention_backward_kept_ds_equals_recomputed(gpu, ref, B, T, Hq, Hkv, hd, window, acc):
-    """Whole 128-row tiles, unsplit launch: dK/dV writes the score gradients and dQ is one banded product over them. Against
+@pytest.mark.parametrize("acc,splits", [(0, 1), (1, 1), (0, 5), (1, 3)])
+def test_attention_backward_kept_ds_equals_recomputed(gpu, ref, B, T, Hq, Hkv, hd, window, acc, splits):
+    """Whole 128-row tiles, one or several workgroups per tile: dK/dV writes the score gradients and dQ is one banded product over them. Against
     the kernel pair that recomputes the scores for dQ (itself held to the oracle above) and, for the first sequence,
     against the oracle; windows that end on, before and after a tile edge, window 1, accumulation into a used dq
     (acc = 1: the gradient buffers start from the same random contents on both paths)."""
@@ -451,7 +451,7 @@ def test_attention_backward_kept_ds_equals_recomputed(gpu, ref, B, T, Hq, Hkv, h
     lse = gpu.create_state_buffer(B * Hq * T * 4)
     for n, a in (("q", q), ("k", k), ("v", v), ("up", up)):
         gpu.write_state_buffer(bufs[n], a)
-    gpu.set_option("attn.splits", 1)
+    gpu.set_option("attn.splits", splits)
     res = []
     try:
         lib.check(gpu.ctx, lib.lib.gt_attn_fwd(gpu.ctx, B, T, Hq, Hkv, hd, window, bufs["q"], bufs["k"], bufs["v"], bufs["out"], lse), "fwd")
@@ -467,7 +467,8 @@ def test_attention_backward_kept_ds_equals_recomputed(gpu, ref, B, T, Hq, Hkv, h
         gpu.set_option("attn.splits", -1)
     for a, b, nm in zip(res[1], res[0], ("dq", "dk", "dv")):
         assert_close(a, b, f"kept dS vs recomputed {nm}", floor=floor)
-    assert np.array_equal(res[1][1], res[0][1]) and np.array_equal(res[1][2], res[0][2])     # dK, dV: the same arithmetic
+    if splits == 1 or window == 0:      # dK, dV: the same arithmetic (a split windowed launch cuts its longer loop elsewhere)
+        assert np.array_equal(res[1][1], res[0][1]) and np.array_equal(res[1][2], res[0][2])
     ref.set_threads(min(8, ref.max_threads()))
     try:
         s = slice(0, T)
