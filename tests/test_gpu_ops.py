@@ -484,6 +484,35 @@ def test_attention_backward_kept_ds_equals_recomputed(gpu, ref, B, T, Hq, Hkv, h
         ref.set_threads(1)
 
 
+def test_attention_ds_workspace_limit_falls_back_to_recompute(gpu, ref):
+    """A dS workspace above "attn.ds_limit_mb" is not taken: the backward is then the recomputing kernel pair, bit for bit."""
+    lib = mod("lib")
+    B, T, Hq, Hkv, hd = 2, 256, 4, 2, 64              # dS would be 2 MiB
+    r = R(ref, 77)
+    arrs = dict(q=r(B * T, Hq * hd), k=r(B * T, Hkv * hd), v=r(B * T, Hkv * hd), up=r(B * T, Hq * hd))
+    bufs = {n: gpu.create_state_buffer(a.nbytes) for n, a in arrs.items()}
+    for n, a in arrs.items():
+        gpu.write_state_buffer(bufs[n], a)
+    out, dq = (gpu.create_state_buffer(arrs["q"].nbytes) for _ in range(2))
+    dk, dv = (gpu.create_state_buffer(arrs["k"].nbytes) for _ in range(2))
+    lse = gpu.create_state_buffer(B * Hq * T * 4)
+    lib.check(gpu.ctx, lib.lib.gt_attn_fwd(gpu.ctx, B, T, Hq, Hkv, hd, 0, bufs["q"], bufs["k"], bufs["v"], out, lse), "fwd")
+    res = {}
+    try:
+        for name, opts in (("recompute", {"attn.keep_ds": 0}), ("limited", {"attn.ds_limit_mb": 1}), ("kept", {"attn.ds_limit_mb": 2})):
+            for k_, v_ in {"attn.keep_ds": 1, "attn.ds_limit_mb": 8192, **opts}.items():
+                gpu.set_option(k_, v_)
+            lib.check(gpu.ctx, lib.lib.gt_attn_bwd(gpu.ctx, B, T, Hq, Hkv, hd, 0, bufs["q"], bufs["k"], bufs["v"], out, bufs["up"], lse,
+                                                   dq, 0, dk, 0, dv, 0), "bwd")
+            res[name] = gpu.read_state_buffer(dq, arrs["q"].size).copy()
+    finally:
+        gpu.set_option("attn.keep_ds", 1)
+        gpu.set_option("attn.ds_limit_mb", 8192)
+    assert np.array_equal(res["limited"], res["recompute"])
+    assert not np.array_equal(res["kept"], res["recompute"])          # another summation order, so not the same bits
+    assert_close(res["kept"], res["recompute"], "kept vs recomputed dq")
+
+
 def test_attention_mfma_equals_generic_at_full_length(gpu, ref):
     """T = 2048, 9/3 heads x 64 (the SmolLM2 layer), two stacked sequences: both kernel families against each other."""
     ag = mod("autograd")
