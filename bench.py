@@ -224,6 +224,8 @@ def main():
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
     ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (benchmark configs[1] shapes)")
     ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
+    ap.add_argument("--no-keep-scores", action="store_true",
+                    help="attention recomputes Q.K^T in the backward instead of keeping the forward's scores (saves B*Hq*T*T*4 bytes per layer)")
     ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
                     help="library option for an A/B run, e.g. attn.keep_ds=0 (dQ recomputes the scores) or gemm.staged=1")
     ap.add_argument("--profile-all", action="store_true",
@@ -252,6 +254,7 @@ def main():
     n_params = sum(p.size for p in model.params())
     gpu = hb.require_gpu("bench.py")
     gpu.batch_linears = not a.no_pair
+    gpu.attn_keep_scores = not a.no_keep_scores
     for kv in a.set:
         key, _, val = kv.partition("=")
         gpu.set_option(key, int(val))

@@ -189,7 +189,14 @@ def checkpoint(inputs, fn):
     rb = _region_backend()
     born = _created
     mark = rb.begin_region() if rb else 0
-    out = fn()
+    if rb is not None and hasattr(rb, "forward_only_region"):
+        rb.forward_only_region = True          # this pass's interior is thrown away: nothing worth saving for a backward
+        try:
+            out = fn()
+        finally:
+            rb.forward_only_region = False
+    else:
+        out = fn()
     _assert_self_contained(out, inputs, born)
     if rb:
         rb.end_region(mark, [out])

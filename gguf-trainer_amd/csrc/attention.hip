@@ -247,15 +247,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
 }
 
 // attention_mfma.hip, compiled once per head dim
-int attn_fwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
+int attn_fwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_bwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                    float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
-int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
-int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart);
+                    float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
+int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_bwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                    float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                    float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 int attn_bwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                     float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                     float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 static int attn_mfma_supported(int hd) { return hd == 32 || hd == 64 || hd == 128; }
 
 // A launch with fewer 128-row tiles than three per CU is cut further (measured at T = 2048, 9 heads: 1 sequence runs
@@ -309,7 +309,8 @@ __global__ __launch_bounds__(256) void attn_slice_sum(const float *__restrict__ 
   *o = a;
 }
 
-static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse) {
+static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, gt_buf scores) {
+  float *sco = P<float>(scores);
   float *fpart = nullptr;
   if (p.splits > 1) {
     const size_t slice = (size_t)p.B * p.T * p.Hq * p.hd, rows = (size_t)p.B * p.Hq * p.T;
@@ -317,8 +318,8 @@ static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
     if (gt_ws_reserve(ctx, (size_t)p.splits * (slice + 2 * rows) * sizeof(float), &ws)) return 1;
     fpart = static_cast<float *>(ws);
   }
-  if (p.hd == 32 ? attn_fwd_mfma32(ctx, p, q, k, v, out, lse, fpart)
-      : p.hd == 64 ? attn_fwd_mfma64(ctx, p, q, k, v, out, lse, fpart) : attn_fwd_mfma128(ctx, p, q, k, v, out, lse, fpart)) return 1;
+  if (p.hd == 32 ? attn_fwd_mfma32(ctx, p, q, k, v, out, lse, fpart, sco)
+      : p.hd == 64 ? attn_fwd_mfma64(ctx, p, q, k, v, out, lse, fpart, sco) : attn_fwd_mfma128(ctx, p, q, k, v, out, lse, fpart, sco)) return 1;
   if (p.splits > 1) {
     const int64_t n = (int64_t)p.B * p.T * p.Hq * (p.hd / 4);
     hipLaunchKernelGGL(attn_fwd_combine, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, p, fpart, P<float>(out), P<float>(lse));
@@ -327,10 +328,11 @@ static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
   return 0;
 }
 static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
-                         float *part, float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
-  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v)
-      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v)
-                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v))
+                         float *part, float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv,
+                         int acc_v) {
+  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v)
+      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v)
+                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v))
     return 1;
   if (p.splits > 1 && !dsb) {
     const size_t n4 = (size_t)p.B * p.T * p.Hq * p.hd / 4;
@@ -355,16 +357,22 @@ static double attn_pairs(int T, int window) {
   return p;
 }
 
-extern "C" {
-int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
-                gt_buf lse) {
+// kept scores: the MFMA kernels on whole 128-row tiles only (the blocks are addressed per 32 x 32 sub-tile)
+static bool scores_supported(gt_ctx *ctx, int T, int hd) {
+  return !ctx->opt_attn_generic && attn_mfma_supported(hd) && hd >= 64 && T % 128 == 0;
+}
+
+static int attn_fwd_impl(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                         gt_buf lse, gt_buf scores) {
   GT_ENTER(ctx);
   if (check(ctx, "gt_attn_fwd", B, T, Hq, Hkv, hd, window)) return 1;
   GT_REQUIRE(ctx, q && k && v && out && lse, "gt_attn_fwd: null operand");
+  GT_REQUIRE(ctx, !scores || (scores_supported(ctx, T, hd) && scores % 16 == 0),
+             "gt_attn_fwd_scores: scores are kept for T a multiple of 128 and head dim 64 or 128 only (T %d, hd %d)", T, hd);
   AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd), 1};
   if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) p.splits = attn_splits(ctx, B, T, Hq);
   ProfScope ps(ctx, "attention", 2.0 * 2 * hd * attn_pairs(T, window) * Hq * B);   // QK^T and PV
-  if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) return attn_fwd_mfma(ctx, p, q, k, v, out, lse);
+  if (!ctx->opt_attn_generic && attn_mfma_supported(hd)) return attn_fwd_mfma(ctx, p, q, k, v, out, lse, scores);
   int64_t rows = (int64_t)B * Hq * T;
   size_t smem = 4 * (size_t)(hd + WAVE) * sizeof(float);
   hipLaunchKernelGGL(attn_fwd_gen, dim3((unsigned)cdiv(rows, 4)), dim3(256), smem, ctx->stream, p, P<const float>(q),
@@ -373,11 +381,13 @@ int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
   return 0;
 }
 
-int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
-                gt_buf dout, gt_buf lse, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+static int attn_bwd_impl(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                         gt_buf dout, gt_buf lse, gt_buf scores, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
   GT_ENTER(ctx);
   if (check(ctx, "gt_attn_bwd", B, T, Hq, Hkv, hd, window)) return 1;
   GT_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, "gt_attn_bwd: null operand");
+  GT_REQUIRE(ctx, !scores || (scores_supported(ctx, T, hd) && scores % 16 == 0),
+             "gt_attn_bwd_scores: scores are kept for T a multiple of 128 and head dim 64 or 128 only (T %d, hd %d)", T, hd);
   AttnP p{B, T, Hq, Hkv, hd, window, 1.4426950408889634f / sqrtf((float)hd), 1.0f / sqrtf((float)hd), 1};
   int64_t rows = (int64_t)B * Hq * T, krows = (int64_t)B * Hkv * T;
   ProfScope whole(ctx, "attention.bwd", 5.0 * 2 * hd * attn_pairs(T, window) * Hq * B);   // S, dP, dV, dK, dQ
@@ -420,7 +430,7 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
     }
     GT_LAUNCHED(ctx);
   }
-  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, dq, acc_q, dk, acc_k, dv, acc_v);
+  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, P<const float>(scores), dq, acc_q, dk, acc_k, dv, acc_v);
   {
     ProfScope ps(ctx, "attention.bwd.dq");
     size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);
@@ -437,5 +447,32 @@ int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, 
     GT_LAUNCHED(ctx);
   }
   return 0;
+}
+
+extern "C" {
+int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                gt_buf lse) {
+  return attn_fwd_impl(ctx, B, T, Hq, Hkv, hd, window, q, k, v, out, lse, 0);
+}
+int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                gt_buf dout, gt_buf lse, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+  return attn_bwd_impl(ctx, B, T, Hq, Hkv, hd, window, q, k, v, out, dout, lse, 0, dq, acc_q, dk, acc_k, dv, acc_v);
+}
+int gt_attn_scores_bytes(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, uint64_t *bytes) {
+  GT_ENTER(ctx);
+  if (check(ctx, "gt_attn_scores_bytes", B, T, Hq, Hkv, hd, window)) return 1;
+  GT_REQUIRE(ctx, bytes, "gt_attn_scores_bytes: null result");
+  *bytes = scores_supported(ctx, T, hd) ? (uint64_t)B * Hq * T * T * sizeof(float) : 0;
+  return 0;
+}
+int gt_attn_fwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                       gt_buf lse, gt_buf scores) {
+  if (ctx && !scores) GT_FAIL(ctx, "gt_attn_fwd_scores: null scores buffer");
+  return attn_fwd_impl(ctx, B, T, Hq, Hkv, hd, window, q, k, v, out, lse, scores);
+}
+int gt_attn_bwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                       gt_buf dout, gt_buf lse, gt_buf scores, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+  if (ctx && !scores) GT_FAIL(ctx, "gt_attn_bwd_scores: null scores buffer");
+  return attn_bwd_impl(ctx, B, T, Hq, Hkv, hd, window, q, k, v, out, dout, lse, scores, dq, acc_q, dk, acc_k, dv, acc_v);
 }
 }

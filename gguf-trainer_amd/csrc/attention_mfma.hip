@@ -185,7 +185,7 @@ __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32]
 // ---- forward --------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, float *__restrict__ out,
-                                                       float *__restrict__ lse, float *__restrict__ fpart) {
+                                                       float *__restrict__ lse, float *__restrict__ fpart, float *sco) {
   using IO = TileIO<KT>;
   __shared__ __attribute__((aligned(16))) float sK[KT * LD];
   __shared__ __attribute__((aligned(16))) float sVt[HD * IO::LDT];
@@ -248,6 +248,11 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
       if (!act[sub]) continue;
       any_act = true;
       v16f s = rows_dot_regs(sK + sub * 32 * LD, qreg, l32, g);
+      if (sco) {      // keep the raw scores (log2 domain, unmasked) of this 32 x 32 block for dK/dV: [key][query], 4 KB in one piece
+        float *sb = sco + ((((size_t)b * p.Hq + h) * (p.T / 32) + k0 / 32) * (p.T / 32) + tq0 / 32) * 1024 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sb[acc_row(r, g) * 32] = s[r];
+      }
       const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
       if (need_mask) {
 #pragma unroll
@@ -392,11 +397,15 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------
 #define QT 32      // queries per LDS stage in dK/dV
+// KS: the forward kept its scores (sco: one [key][query] 32 x 32 block per (key sub-tile, query stage) of every
+// (sequence, head), T a multiple of 128). S is then read back, four 16-byte loads per lane and stage issued a stage
+// ahead, instead of recomputed: no key row in registers, no row-major query tile in LDS, three contractions per stage.
+template <bool KS>
 __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
                                                            float *dk, int acc_k, float *dv, int acc_v, float *part,
-                                                           float *dsb) {
+                                                           float *dsb, const float *__restrict__ sco) {
   using IO = TileIO<QT>;
   extern __shared__ __attribute__((aligned(16))) float dkv_smem[];      // 35 KB at hd 64, 69 KB at hd 128
   float *sQ = dkv_smem, *sG = sQ + QT * LD, *sQt = sG + QT * LD, *sGt = sQt + HD * IO::LDT;
@@ -417,8 +426,8 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   const int sk0 = ktile * 128 + wave * 32, s = sk0 + l32;
   const bool sv = s < p.T;
   const size_t koff = ((size_t)b * p.T + (sv ? s : 0)) * kstr + (size_t)kvh * HD;
-  float kreg[HD / 2], vreg[HD / 2];
-  load_row_regs(kreg, k + koff, sv, g, p.c2);
+  float kreg[KS ? 1 : HD / 2], vreg[HD / 2];
+  if constexpr (!KS) load_row_regs(kreg, k + koff, sv, g, p.c2);
   load_row_regs(vreg, v + koff, sv, g, 1.0f);
   // queries that can see a key of this workgroup: t in [ktile*128, last key + window - 1]
   const int qt_lo = ktile * (128 / QT);
@@ -441,10 +450,19 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   // this workgroup's share of the query stages
   const int it_lo = p.splits > 1 ? sp * nqt / p.splits : 0;
   const int niter = p.splits > 1 ? (sp + 1) * nqt / p.splits : nqt;
-  v4f pq[IO::PER], pg[IO::PER];
+  v4f pq[IO::PER], pg[IO::PER], psc[KS ? 4 : 1];
   float pstat = 0.f;
+  // this wavefront's block of kept scores for a query stage: lane = key row of the block, queries 8a + 4g + (0..3)
+  const float *scw = KS ? sco + (((size_t)b * p.Hq + h) * (p.T / 32) + sk0 / 32) * (p.T / 32) * 1024 + l32 * 32 + 4 * g : nullptr;
   auto prefetch = [&](int it) {
     int qt = qt_lo + it;
+    if (KS) {
+      const int t0n = qt * QT;
+      if (!(t0n + 31 < sk0 || t0n > wave_t_hi || sk0 >= p.T)) {           // only blocks the forward has written
+#pragma unroll
+        for (int a = 0; a < 4; a++) psc[a] = *reinterpret_cast<const v4f *>(scw + (size_t)qt * 1024 + 8 * a);
+      }
+    }
     const float *qb = q + (size_t)b * p.T * qstr + (size_t)h * HD;
     const float *gb = go + (size_t)b * p.T * qstr + (size_t)h * HD;
     IO::load(pq, qb, qstr, qt * QT, p.T, tid);
@@ -458,13 +476,18 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   prefetch(it_lo);
   for (int it = it_lo; it < niter; it++) {
     __syncthreads();
-    IO::store_rows(pq, sQ, tid);
+    if (!KS) IO::store_rows(pq, sQ, tid);
     IO::store_t(pq, sQt, tid);
     IO::store_rows(pg, sG, tid);
     IO::store_t(pg, sGt, tid);
     if (tid < QT) sL[tid] = pstat;
     else if (tid < 2 * QT) sD[tid - QT] = pstat;
     __syncthreads();
+    v16f sc;
+    if (KS) {            // out of the prefetch registers before the next stage's loads overwrite them
+#pragma unroll
+      for (int r = 0; r < 16; r++) sc[r] = psc[r / 4][r % 4];
+    }
     if (it + 1 < niter) prefetch(it + 1);
     const int t0 = (qt_lo + it) * QT;
     // this lane's column of the dS block of (query stage, keys of this wavefront): rows t0 + 8a + 4g + j. The matrix of a
@@ -479,7 +502,7 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
       }
       continue;
     }
-    v16f sc = rows_dot_regs(sQ, kreg, l32, g);
+    if constexpr (!KS) sc = rows_dot_regs(sQ, kreg, l32, g);
     v16f dp = rows_dot_regs(sG, vreg, l32, g);
     // fully visible tile: every query is at or after every key of the wave, inside the window, and in range
     const bool need_mask = ragged_k || t0 < sk0 + 31 || t0 + 31 >= p.T || (p.window > 0 && t0 + 31 > sk0 + p.window - 1);
@@ -535,12 +558,13 @@ __global__ __launch_bounds__(256) void FN(attn_group_sum)(const float *__restric
 #define DKV_SMEM ((2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT) * sizeof(float))
 
 // fpart: workspace for the split partials (splits x output, then splits x rows maxima, splits x rows sums), or null
-int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart) {
+// sco: where to keep the raw scores for the backward (B*Hq*T*T floats, T a multiple of 128), or null
+int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco) {
   GT_REQUIRE(ctx, (q | k | v | out) % 16 == 0, "attention: buffers must be 16-byte aligned");
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || fpart), "attention: split forward without a workspace");
   dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
   hipLaunchKernelGGL(FN(attn_fwd_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
-                     P<const float>(v), P<float>(out), P<float>(lse), fpart);
+                     P<const float>(v), P<float>(out), P<float>(lse), fpart, sco);
   GT_LAUNCHED(ctx);
   return 0;
 }
@@ -550,13 +574,17 @@ int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
 // dsb: workspace for the B*Hq [T][T] dS matrices, or null. With it dK/dV writes dS as it goes and dQ is one banded
 // product dS.K afterwards (5 contractions in all); without it dQ recomputes S and dP in its own kernel (7).
 int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
-                      float *part, float *dqpart, float *dsb, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+                      float *part, float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv,
+                      int acc_v) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
   const int group = p.Hq / p.Hkv;
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart || dsb) && (p.splits * group == 1 || part),
              "attention: split backward without a workspace");
+  GT_REQUIRE(ctx, !sco || (p.T % 128 == 0 && HD >= 64), "attention: kept scores with an unsupported shape");
   if (!(ctx->attn_smem_set & HD)) {   // once per context (device): more than the 64 KB a kernel gets by default at hd 128
-    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)),
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
     ctx->attn_smem_set |= HD;
   }
@@ -571,8 +599,12 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
   {
     ProfScope ps(ctx, "attention.bwd.dkv");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
-    hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k), grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
-                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb);
+    if (sco)
+      hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k)<true>, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
+                         P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco);
+    else
+      hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k)<false>, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
+                         P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco);
     GT_LAUNCHED(ctx);
     if (part) {
       size_t n4 = (size_t)p.B * p.T * p.Hkv * HD / 4;

@@ -60,7 +60,11 @@ int gt_alloc(gt_ctx *ctx, size_t bytes, int zero, gt_buf *out) {
   GT_REQUIRE(ctx, out, "gt_alloc: out is NULL");
   void *p = nullptr;
   size_t sz = bytes ? bytes : 4;
-  GT_HIP(ctx, hipMalloc(&p, sz));
+  hipError_t e = hipMalloc(&p, sz);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();       // a caller may free memory and ask again: the next launch check must not report this failure
+    GT_FAIL(ctx, "gt_alloc: hipMalloc of %zu bytes failed: %s", sz, hipGetErrorString(e));
+  }
   if (zero) GT_HIP(ctx, hipMemsetAsync(p, 0, sz, ctx->stream));
   ctx->allocs[reinterpret_cast<uint64_t>(p)] = sz;
   ctx->live_bytes += sz;

@@ -36,7 +36,7 @@ _ALIGN = 256
 
 class _Entry:
     __slots__ = ("data", "grad", "nbytes", "external", "grad_init", "lazy_act", "consumers", "fused_uses",
-                 "region", "keep_grad")
+                 "region", "keep_grad", "extra", "needs_grad")
 
     def __init__(self, nbytes, external):
         self.data = 0
@@ -49,6 +49,8 @@ class _Entry:
         self.fused_uses = 0
         self.region = 0
         self.keep_grad = False
+        self.extra = None           # (buf, nbytes) of a saved buffer that lives and dies with this output (attention scores)
+        self.needs_grad = False     # an intermediate below a trainable tensor: a backward through it may be asked for
 
 
 class HipBackend:
@@ -74,6 +76,14 @@ class HipBackend:
         self._regions_opened = 0
         self._pend = None                 # (x, T, out, in, x data, w data, out data) of a held-back linear launch
         self.batch_linears = True
+        # attention keeps its raw scores from the forward to the backward (one [T, T] matrix per sequence and head) when a
+        # gradient will be asked for, one call's matrices fit attn_scores_max_bytes and the live ones together stay
+        # within attn_scores_budget_bytes: memory spent to take one of four contractions out of dK/dV
+        self.attn_keep_scores = True
+        self.attn_scores_max_bytes = 4 << 30
+        self.attn_scores_budget_bytes = 96 << 30
+        self._scores_taken = 0
+        self.forward_only_region = False  # set by checkpoint() around a block's first forward, whose interior is never differentiated
         self._profiling = False
         self._destroyed = False
 
@@ -99,9 +109,26 @@ class HipBackend:
         if free:
             return free.pop()
         out = c_buf()
-        check(self._ctx, lib.gt_alloc(self._ctx, size, 0, C.byref(out)), "gt_alloc")
+        if lib.gt_alloc(self._ctx, size, 0, C.byref(out)) != 0:
+            # device memory is full of free buffers of other size classes (another model shape ran before): give them
+            # back and ask again; only then is it an error
+            if not self.trim_pool():
+                check(self._ctx, 1, "gt_alloc")
+            check(self._ctx, lib.gt_alloc(self._ctx, size, 0, C.byref(out)), "gt_alloc")
         self._pool_bytes += size
         return out.value
+
+    def trim_pool(self) -> int:
+        """Return every free buffer of the pool to the device (buffers in use stay). Gives the bytes freed."""
+        freed = 0
+        check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")      # queued kernels may still use a buffer recycled at a region's end
+        for size, free in self._pool.items():
+            for b in free:
+                check(self._ctx, lib.gt_free(self._ctx, b), "gt_free")
+                freed += size
+            free.clear()
+        self._pool_bytes -= freed
+        return freed
 
     def _recycle(self, b: int, nbytes: int):
         size = max(_ALIGN, (nbytes + _ALIGN - 1) // _ALIGN * _ALIGN)
@@ -143,6 +170,11 @@ class HipBackend:
         if alloc:
             e.data = self._acquire(e.nbytes)
         e.region = self._regions_opened
+        for p in prev:
+            pe = self._entries.get(p)
+            if p.requires_grad or (pe is not None and pe.needs_grad):
+                e.needs_grad = True
+                break
         self._entries[out] = e
         self._transients.append((out, e))
         return out, e
@@ -292,6 +324,10 @@ class HipBackend:
                 self._recycle(e.data, e.nbytes)
             if e.grad:
                 self._recycle(e.grad, e.nbytes)
+            if e.extra:
+                self._recycle(*e.extra)
+                self._scores_taken -= e.extra[1]
+                e.extra = None
             e.data = e.grad = 0
             self._entries.pop(t, None)
         self._transients = kept
@@ -332,6 +368,7 @@ class HipBackend:
         check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")
         self.last_sync_readback_bytes = nbytes
         self._release_transients()
+        self._scores_taken = 0
 
     def reclaim_step_transients(self, keep=()):
         """Free a finished micro-batch's intermediates mid-step; parameter gradients keep accumulating."""
@@ -377,6 +414,10 @@ class HipBackend:
                 self._recycle(e.data, e.nbytes)
             if e.grad:
                 self._recycle(e.grad, e.nbytes)
+            if e.extra:
+                self._recycle(*e.extra)
+                self._scores_taken -= e.extra[1]
+                e.extra = None
             e.data = e.grad = 0
             self._entries.pop(t, None)
 
@@ -628,7 +669,18 @@ class HipBackend:
         qd, kd, vd = self._data(q), self._data(k), self._data(v)
         out, e = self._make_out([rows, Hq * hd], [q, k, v])
         lse = self._scratch_buf(B * Hq * T * 4)
-        check(self._ctx, lib.gt_attn_fwd(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, e.data, lse), "attention")
+        scores = 0
+        if self.attn_keep_scores and not self.forward_only_region and e.needs_grad:
+            need = C.c_uint64(0)
+            check(self._ctx, lib.gt_attn_scores_bytes(self._ctx, B, T, Hq, Hkv, hd, window, C.byref(need)), "attention")
+            if 0 < need.value <= self.attn_scores_max_bytes and self._scores_taken + need.value <= self.attn_scores_budget_bytes:
+                scores = self._acquire(need.value)
+                e.extra = (scores, need.value)
+                self._scores_taken += need.value
+        if scores:
+            check(self._ctx, lib.gt_attn_fwd_scores(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, e.data, lse, scores), "attention")
+        else:
+            check(self._ctx, lib.gt_attn_fwd(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, e.data, lse), "attention")
         od = e.data
 
         def bw():
@@ -636,8 +688,12 @@ class HipBackend:
             dq, aq = self._gdst(q)
             dk, ak = self._gdst(k)
             dv, av = self._gdst(v)
-            check(self._ctx, lib.gt_attn_bwd(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, od, g, lse,
-                                             dq, aq, dk, ak, dv, av), "attention.bwd")
+            if scores:
+                check(self._ctx, lib.gt_attn_bwd_scores(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, od, g, lse, scores,
+                                                        dq, aq, dk, ak, dv, av), "attention.bwd")
+            else:
+                check(self._ctx, lib.gt_attn_bwd(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, od, g, lse,
+                                                 dq, aq, dk, ak, dv, av), "attention.bwd")
 
         out._backward = bw
         return out

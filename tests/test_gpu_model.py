@@ -333,6 +333,72 @@ def test_forward_only_scoring_reads_back_the_loss_alone(gpu, ref, loss_chunk):
     assert out[False][1] == out[True][1] and np.isfinite(out[True][1])
 
 
+@pytest.mark.parametrize("recompute", [False, True])
+def test_kept_attention_scores_policy(gpu, ref, recompute):
+    """The host keeps attention's scores from the forward to the backward only where a backward can come: a trainable
+    model takes one scores buffer per layer (recomputed layers: one at a time, and none in the discarded first pass), a
+    model frozen for scoring takes none; with and without them the step gives the same loss bits and gradients to the
+    parity bound, and both agree with the oracle."""
+    kw = dict(arch="qwen3", vocab=97, hidden=128, layers=3, heads=2, kv_heads=1, head_dim=64, ffn=192, rope_base=1e6, rms_eps=1e-6)
+    T, B = 128, 2
+    per_call = B * kw["heads"] * T * T * 4
+    rmodel, model = build_pair(ref, kw, seed=21, std=0.05)
+    seqs = batches(ref, kw["vocab"], T, B, seed=22, mask_every=6)
+    taken = []
+    acquire = gpu._acquire
+
+    def spy(nbytes):
+        taken.append(nbytes)
+        return acquire(nbytes)
+
+    gpu._acquire = spy
+    res = {}
+    try:
+        for keep in (True, False):
+            gpu.attn_keep_scores = keep
+            taken.clear()
+            res[keep] = hip_step(gpu, model, seqs, True, T, recompute=recompute)
+            assert taken.count(per_call) == (kw["layers"] if keep else 0), (keep, taken.count(per_call))
+            assert gpu._scores_taken == 0
+        gpu.attn_keep_scores = True
+        for p in model.params():
+            p.requires_grad = False
+        taken.clear()
+        gpu.install()
+        try:
+            loss = mod("arch").sequence_loss(model, np.concatenate([s[0] for s in seqs]), np.concatenate([s[1] for s in seqs]), 0, T)
+            gpu.sync([loss])
+        finally:
+            gpu.uninstall()
+        assert taken.count(per_call) == 0
+        assert np.array_equal(loss.data, res[True][0])
+    finally:
+        gpu._acquire = acquire
+        gpu.attn_keep_scores = True
+        for p in model.params():
+            p.requires_grad = True
+    assert np.array_equal(res[True][0], res[False][0])
+    for n in res[True][1]:
+        assert_close(res[True][1][n], res[False][1][n], f"kept scores vs recomputed, grad {n}")
+    lr, gr = ref_step(ref, rmodel, seqs)
+    compare(res[True][0], res[True][1], lr, gr, f"kept scores recompute={recompute}")
+
+
+def test_trim_pool_returns_free_buffers_and_work_goes_on(gpu, ref):
+    """Free buffers of the size-class pool go back to the device on request (and on their own when an allocation fails);
+    buffers in use stay, and the next step allocates afresh and gives the same bits."""
+    kw = SMALL["llama"]
+    _, model = build_pair(ref, kw, seed=3, std=0.1)
+    seqs = batches(ref, kw["vocab"], 19, 2, seed=4)
+    l0, g0 = hip_step(gpu, model, seqs, True, 19)
+    before = gpu.resident_bytes()
+    freed = gpu.trim_pool()
+    assert freed > 0 and gpu.resident_bytes() == before - freed
+    assert all(not free for free in gpu._pool.values())
+    l1, g1 = hip_step(gpu, model, seqs, True, 19)
+    assert np.array_equal(l0, l1) and all(np.array_equal(g0[n], g1[n]) for n in g0)
+
+
 def test_gradient_rearm_survives_a_mid_window_freeze(gpu, ref):
     """gpu-parity.ts:1980-2028: parameters frozen between a window's backward and its sync, thawed afterwards. The
     accumulators still hold that window's gradients, so the window after the thaw must start them afresh: same inputs

@@ -1,5 +1,6 @@
 """Per-op parity, HIP backend (through the C ABI) against the CPU oracle on identical seeded inputs:
 the op cases of tests/gpu-parity.ts:654-930 and the edge cases it names."""
+import ctypes as C
 import math
 
 import numpy as np
@@ -482,6 +483,77 @@ def test_attention_backward_kept_ds_equals_recomputed(gpu, ref, B, T, Hq, Hkv, h
             assert_close(res[1][0].reshape(B * T, -1)[s], want, "kept dS dq vs oracle")
     finally:
         ref.set_threads(1)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 512, 2, 1, 64, 128),
+                                                  (1, 640, 2, 2, 64, 129), (1, 256, 3, 1, 64, 1), (3, 128, 2, 2, 64, 0),
+                                                  (2, 256, 4, 2, 128, 0), (1, 384, 2, 1, 128, 130), (1, 1024, 9, 3, 64, 0)])
+@pytest.mark.parametrize("splits,keep_ds", [(1, 1), (3, 1), (1, 0)])
+def test_attention_kept_scores_equals_recomputed(gpu, ref, B, T, Hq, Hkv, hd, window, splits, keep_ds):
+    """gt_attn_fwd_scores / gt_attn_bwd_scores (the forward keeps S, dK/dV reads it back) against gt_attn_fwd / gt_attn_bwd
+    (dK/dV recomputes S): the same output and statistic bit for bit, the three gradients to the parity bound, and dq of
+    the first sequence against the oracle. Split and unsplit launches, with and without the kept dS."""
+    lib = mod("lib")
+    floor = 1.0 if window == 1 else 0.0
+    r = R(ref, 5 * T + Hq + window)
+    arrs = dict(q=r(B * T, Hq * hd), k=r(B * T, Hkv * hd), v=r(B * T, Hkv * hd), up=r(B * T, Hq * hd))
+    bufs = {n: gpu.create_state_buffer(a.nbytes) for n, a in arrs.items()}
+    for n, a in arrs.items():
+        gpu.write_state_buffer(bufs[n], a)
+    out, dq = (gpu.create_state_buffer(arrs["q"].nbytes) for _ in range(2))
+    dk, dv = (gpu.create_state_buffer(arrs["k"].nbytes) for _ in range(2))
+    lse = gpu.create_state_buffer(B * Hq * T * 4)
+    need = C.c_uint64(0)
+    lib.check(gpu.ctx, lib.lib.gt_attn_scores_bytes(gpu.ctx, B, T, Hq, Hkv, hd, window, C.byref(need)), "bytes")
+    assert need.value == B * Hq * T * T * 4
+    sco = gpu.create_state_buffer(need.value)
+    gpu.set_option("attn.splits", splits)
+    gpu.set_option("attn.keep_ds", keep_ds)
+    res = []
+    try:
+        for kept in (0, 1):
+            if kept:
+                lib.check(gpu.ctx, lib.lib.gt_attn_fwd_scores(gpu.ctx, B, T, Hq, Hkv, hd, window, bufs["q"], bufs["k"], bufs["v"], out, lse, sco), "fwd")
+                lib.check(gpu.ctx, lib.lib.gt_attn_bwd_scores(gpu.ctx, B, T, Hq, Hkv, hd, window, bufs["q"], bufs["k"], bufs["v"], out,
+                                                              bufs["up"], lse, sco, dq, 0, dk, 0, dv, 0), "bwd")
+            else:
+                lib.check(gpu.ctx, lib.lib.gt_attn_fwd(gpu.ctx, B, T, Hq, Hkv, hd, window, bufs["q"], bufs["k"], bufs["v"], out, lse), "fwd")
+                lib.check(gpu.ctx, lib.lib.gt_attn_bwd(gpu.ctx, B, T, Hq, Hkv, hd, window, bufs["q"], bufs["k"], bufs["v"], out,
+                                                       bufs["up"], lse, dq, 0, dk, 0, dv, 0), "bwd")
+            res.append([gpu.read_state_buffer(b_, n_).copy() for b_, n_ in ((out, arrs["q"].size), (lse, B * Hq * T), (dq, arrs["q"].size),
+                                                                            (dk, arrs["k"].size), (dv, arrs["k"].size))])
+    finally:
+        gpu.set_option("attn.splits", -1)
+        gpu.set_option("attn.keep_ds", 1)
+    assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1])
+    for a, b, nm in zip(res[1][2:], res[0][2:], ("dq", "dk", "dv")):
+        assert_close(a, b, f"kept scores vs recomputed {nm}", floor=floor)
+    ref.set_threads(min(8, ref.max_threads()))
+    try:
+        rq, rk, rv = (ref.Tensor(arrs[n][:T], [T, arrs[n].shape[1]], True) for n in ("q", "k", "v"))
+        o = ref.attention(rq, rk, rv, T, Hq, Hkv, hd, window, parallel_bwd=True)
+        ref.backward_from(o, arrs["up"][:T].reshape(-1))
+        for got, want, nm in ((res[1][2], rq.grad, "dq"), (res[1][3], rk.grad, "dk"), (res[1][4], rv.grad, "dv")):
+            got = got.reshape(B, -1)[0]
+            if floor and nm != "dv":
+                assert np.abs(got - want).max() < 1e-5
+            else:
+                assert_close(got, want, f"kept scores {nm} vs oracle")
+    finally:
+        ref.set_threads(1)
+
+
+def test_attention_scores_are_refused_where_not_kept(gpu):
+    lib = mod("lib")
+    need = C.c_uint64(7)
+    for B, T, Hq, Hkv, hd in ((1, 200, 4, 2, 64), (1, 256, 4, 2, 32), (1, 256, 4, 2, 16)):
+        lib.check(gpu.ctx, lib.lib.gt_attn_scores_bytes(gpu.ctx, B, T, Hq, Hkv, hd, 0, C.byref(need)), "bytes")
+        assert need.value == 0
+    b = gpu.create_state_buffer(1 << 20)
+    with pytest.raises(lib.HipError, match="scores are kept for T a multiple of 128"):
+        lib.check(gpu.ctx, lib.lib.gt_attn_fwd_scores(gpu.ctx, 1, 200, 4, 2, 64, 0, b, b, b, b, b, b), "fwd")
+    with pytest.raises(lib.HipError, match="null scores buffer"):
+        lib.check(gpu.ctx, lib.lib.gt_attn_fwd_scores(gpu.ctx, 1, 256, 4, 2, 64, 0, b, b, b, b, b, 0), "fwd")
 
 
 def test_attention_ds_workspace_limit_falls_back_to_recompute(gpu, ref):
