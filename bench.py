@@ -28,9 +28,9 @@ PROF_SAMPLE = 4                # the timed region brackets about 1 in 4 launches
 # L2-miss traffic per launch (bytes) of the two backward GEMM kernels that lead the step, from two rocprofv3 --pmc
 # passes over this file (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the factors read off a plain streaming kernel of known
 # size; see profiles/bench_smollm2_135m_pmc_fetch_write.txt). Averages over the shapes each kernel serves in the step.
-MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (2 * 85477.9 + 36866.6) * 1024,
-                    "gemm.tn.128x96x32.splitk": (2 * 91411.9 + 48384.1) * 1024,
-                    "gemm.tn.64x192x32.splitk": (90 * 360.0 + 180 * 126.8 + 180 * 67.0) / 450 * 1048576}
+MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (2 * 84713.0 + 36866.5) * 1024,
+                    "gemm.tn.128x96x32.splitk": (2 * 91430.1 + 48384.1) * 1024,
+                    "gemm.tn.64x192x32.splitk": (90 * 360.1 + 180 * 126.8 + 180 * 67.0) / 450 * 1048576}
 
 SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                rope_base=100000.0, rms_eps=1e-5, tie=True)

@@ -30,7 +30,11 @@
 // dK/dV loops over the query heads of the kv group inside the workgroup and over query tiles in
 // increasing order, so the GQA sum has a fixed order and needs no atomics.
 //
-// Backward in five contractions. With a dS workspace (T a multiple of 128) dK/dV stores the score
+// Kept scores. With a scores buffer (T a multiple of 128) the forward stores its raw scores, one [key][query] 32 x 32
+// block per (key sub-tile, query stage) of every (sequence, head), and dK/dV reads them back instead of recomputing
+// Q.K^T: three contractions per stage there instead of four.
+//
+// Kept score gradients. With a dS workspace (T a multiple of 128) dK/dV stores the score
 // gradients it computes, and dQ = dS.K is one banded batched product afterwards (gemm.hip) instead of a kernel that
 // recomputes S and dP: one [T][T] matrix per (sequence, head), kept in blocks [row tile of 128][key step of 32]
 // [128 rows][32 keys], in which every block inside a row tile's band of keys is written (zeros where no pair is live).
