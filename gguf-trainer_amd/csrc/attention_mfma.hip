@@ -255,7 +255,7 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
       if (sco) {      // keep the raw scores (log2 domain, unmasked) of this 32 x 32 block for dK/dV: [key][query], 4 KB in one piece
         float *sb = sco + ((((size_t)b * p.Hq + h) * (p.T / 32) + k0 / 32) * (p.T / 32) + tq0 / 32) * 1024 + l32;
 #pragma unroll
-        for (int r = 0; r < 16; r++) sb[acc_row(r, g) * 32] = s[r];
+        for (int r = 0; r < 16; r++) __builtin_nontemporal_store(s[r], sb + acc_row(r, g) * 32);   // read again only in the backward
       }
       const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
       if (need_mask) {
