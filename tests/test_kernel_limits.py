@@ -73,6 +73,9 @@ def test_every_kernel_family_is_in_the_library(kernels):
                    "attn_fwd_mfma_k64", "attn_fwd_mfma_k128", "attn_bwd_dq_mfma", "attn_bwd_dkv_mfma", "attn_bwd_d_vec",
                    "rmsnorm", "rope_vec_k", "adamw", "colsum"):
         assert family in names, family
+    # the kept-scores variant of dK/dV (template argument true) and the banded dQ product (last template argument true)
+    assert any("attn_bwd_dkv_mfma_k64ILb1E" in k["name"] for k in kernels)
+    assert any("gemm_direct" in k["name"] and k["name"].endswith("Lb0ELb1EEv8GemmArgs") for k in kernels)
 
 
 def test_wavefronts_are_64_wide(kernels):
