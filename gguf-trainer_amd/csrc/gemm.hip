@@ -51,6 +51,10 @@ struct GemmArgs {
   // causal (optionally windowed) score-gradient matrix with the key rows, one (sequence, head) per batch member
   int zdiv, zgroup, window;
   int64_t sB2, sC2;
+  // further whole K segments (gemm_direct<..., MSEG>): C = A.B + xA[0].xB[0] (+ xA[1].xB[1]), every K a multiple of the
+  // K step, same M, N and operand orientation: the dX of sibling projections of one input as one product
+  const float *xA[2], *xB[2];
+  int xK[2], xlda[2], xldb[2], nx;
 };
 
 // Which output tile (pm, pn) and which K split or batch member (z) a workgroup works on. Workgroups are handed
@@ -342,7 +346,7 @@ struct DirectTile {
   }
 };
 
-template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2, bool BAND = false>
+template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2, bool BAND = false, bool MSEG = false>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -386,7 +390,9 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
                  : TA::src(A, a.lda, m0, a.M, wave, i, lane) + (size_t)(k0 / BK) * TA::stage_step(a.lda);
 #pragma unroll
   for (int i = 0; i < TB::PER; i++) pb[i] = TB::src(B, a.ldb, n0, a.N, wave, i, lane) + (size_t)(k0 / BK) * TB::stage_step(a.ldb);
-  const size_t sta = BAND ? (size_t)4096 : TA::stage_step(a.lda), stb = TB::stage_step(a.ldb);
+  size_t sta = BAND ? (size_t)4096 : TA::stage_step(a.lda), stb = TB::stage_step(a.ldb);
+  // MSEG: stages of the current segment still to be issued, and the segment after it (wave-uniform)
+  int seg_left = MSEG ? a.K / BK : 0, seg_next = 0;
 #define ISSUE(buf_)                                                                                              \
   {                                                                                                              \
     float *sa_ = smem + (buf_) * STAGE, *sb_ = sa_ + TA::CH * 4;                                                 \
@@ -402,7 +408,21 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
     _Pragma("unroll") for (int i = 0; i < TB::PER; i++)                                                          \
       load_to_lds16(TB::src2(a.B2, a.ldb2, n0, a.N, a.K2, wave, i, lane), sb_ + TB::load_index(wave, i) * 256);  \
   }
-#define ISSUE_STAGE(buf_, st_) { if (SEG2 && (st_) == nstage - 1) ISSUE2(buf_) else ISSUE(buf_) }
+  // a further segment starts: this lane's sources move to its operands (once per segment and workgroup)
+#define NEXT_SEGMENT()                                                                                           \
+  {                                                                                                              \
+    const float *A_ = a.xA[seg_next], *B_ = a.xB[seg_next];                                                      \
+    const int lda_ = a.xlda[seg_next], ldb_ = a.xldb[seg_next];                                                  \
+    _Pragma("unroll") for (int i = 0; i < TA::PER; i++) pa[i] = TA::src(A_, lda_, m0, a.M, wave, i, lane);       \
+    _Pragma("unroll") for (int i = 0; i < TB::PER; i++) pb[i] = TB::src(B_, ldb_, n0, a.N, wave, i, lane);       \
+    sta = TA::stage_step(lda_); stb = TB::stage_step(ldb_);                                                      \
+    seg_left = a.xK[seg_next] / BK; seg_next++;                                                                  \
+  }
+#define ISSUE_STAGE(buf_, st_)                                                                                   \
+  {                                                                                                              \
+    if (MSEG) { if (seg_left == 0) NEXT_SEGMENT() seg_left--; }                                                  \
+    if (SEG2 && (st_) == nstage - 1) ISSUE2(buf_) else ISSUE(buf_)                                               \
+  }
 
   v16f acc[TM][TN];
 #pragma unroll
@@ -418,7 +438,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   constexpr int LPS = TA::PER + TB::PER;                      // loads per wavefront and stage
   constexpr int INFLIGHT = (NSTG - 2) * LPS;                  // loads that may be outstanding when stage k is needed
   static_assert(INFLIGHT < 64, "vmcnt holds six bits");
-  const int nstage = (kend - k0) / BK + (SEG2 ? 1 : 0);
+  int nstage = (kend - k0) / BK + (SEG2 ? 1 : 0);
+  if (MSEG) for (int i = 0; i < a.nx; i++) nstage += a.xK[i] / BK;
 #pragma unroll
   for (int st = 0; st < NSTG - 1; st++)
     if (st < nstage) ISSUE_STAGE(st, st)
@@ -451,6 +472,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
     buf = (buf + 1) % NSTG;
   }
 #undef ISSUE_STAGE
+#undef NEXT_SEGMENT
 #undef ISSUE2
 #undef ISSUE
 
@@ -587,7 +609,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   a.ldc = N;
   a.acc = acc; a.kchunk = K; a.splits = 1; a.Pp = nullptr;
   a.sA = sA; a.sB = sB; a.sC = sC;
-  a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0;
+  a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0; a.nx = 0;
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
              (sA % 4 == 0) && (sB % 4 == 0);
   a.K2 = K2; a.A2 = P<const float>(A2); a.B2 = P<const float>(B2);
@@ -720,12 +742,65 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.acc = acc; a.kchunk = T; a.splits = 1; a.Pp = nullptr;
   a.sA = (int64_t)T * T; a.sB = (int64_t)T * Hkv * hd; a.sC = (int64_t)T * Hq * hd;
   a.zdiv = Hq; a.zgroup = Hq / Hkv; a.window = window; a.sB2 = hd; a.sC2 = hd;
-  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0;
+  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0; a.nx = 0;
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
   return hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26);
 }
 
+// C (+)= sum over i of A_i.B_i with the K segments chained in one loop (NT / NN, every K_i a multiple of 32)
+template <int BM, int BN, int WM, int WN, int KIND>
+static int launch_multi(gt_ctx *ctx, GemmArgs &a, int slot) {
+  constexpr int BK = 32, NSTG = 2, smem = NSTG * (BM + BN) * BK * 4;
+  if (!(ctx->gemm_direct_set & (1ull << slot))) {
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG, false, false, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    ctx->gemm_direct_set |= 1ull << slot;
+  }
+  a.nbm = (int)cdiv(a.M, BM);
+  a.nbn = (int)cdiv(a.N, BN);
+  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, KIND, BK, NSTG, false, false, true>), dim3(a.nbm * a.nbn, 1, 1), dim3(WM * WN * 64), smem,
+                     ctx->stream, a);
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
 extern "C" {
+int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const int *K, const gt_buf *A, const gt_buf *B, gt_buf C) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, count >= 1 && count <= 3 && K && A && B && C, "gt_gemm_sum: 1 to 3 products with their sizes and operands (got %d)", count);
+  GT_REQUIRE(ctx, kind >= 0 && kind <= 2 && M >= 1 && N >= 1, "gt_gemm_sum: kind %d, M %d, N %d", kind, M, N);
+  bool fused = count > 1 && kind != GT_TN && !ctx->opt_gemm_staged && C % 16 == 0 && N % 4 == 0 && (kind == GT_NT || N >= 4);
+  for (int i = 0; i < count; i++) {
+    GT_REQUIRE(ctx, K[i] >= 1 && A[i] && B[i], "gt_gemm_sum: product %d has K %d or a null operand", i, K[i]);
+    fused = fused && K[i] % 32 == 0 && A[i] % 16 == 0 && B[i] % 16 == 0;
+  }
+  if (!fused) {        // one launch per product, each adding to the one before
+    for (int i = 0; i < count; i++)
+      if (gemm_impl(ctx, kind, i ? 1 : acc, M, N, K[i], A[i], 0, B[i], 0, C, 0, 1)) return 1;
+    return 0;
+  }
+  GemmArgs a;
+  a.A = P<const float>(A[0]); a.B = P<const float>(B[0]); a.C = P<float>(C);
+  a.M = M; a.N = N; a.K = K[0];
+  a.lda = K[0]; a.ldb = kind == GT_NT ? K[0] : N; a.ldc = N;
+  a.acc = acc; a.kchunk = K[0]; a.splits = 1; a.Pp = nullptr;
+  a.sA = a.sB = a.sC = 0;
+  a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0;
+  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0;
+  a.nx = count - 1;
+  double ksum = K[0];
+  for (int i = 1; i < count; i++) {
+    a.xA[i - 1] = P<const float>(A[i]); a.xB[i - 1] = P<const float>(B[i]);
+    a.xK[i - 1] = K[i]; a.xlda[i - 1] = K[i]; a.xldb[i - 1] = kind == GT_NT ? K[i] : N;
+    ksum += K[i];
+  }
+  const bool t96 = N % 96 == 0;
+  char label[32];
+  snprintf(label, sizeof label, "gemm.%s.128x%dx32", kind == GT_NT ? "nt" : "nn", t96 ? 96 : 128);
+  ProfScope ps(ctx, label, 2.0 * M * N * ksum);
+  if (kind == GT_NN) return t96 ? launch_multi<128, 96, 4, 1, GT_NN>(ctx, a, 30) : launch_multi<128, 128, 2, 2, GT_NN>(ctx, a, 31);
+  return t96 ? launch_multi<128, 96, 4, 1, GT_NT>(ctx, a, 32) : launch_multi<128, 128, 2, 2, GT_NT>(ctx, a, 33);
+}
 int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_buf B, gt_buf C) {
   return gemm_impl(ctx, kind, acc, M, N, K, A, 0, B, 0, C, 0, 1);
 }

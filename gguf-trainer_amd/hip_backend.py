@@ -75,6 +75,11 @@ class HipBackend:
         self._scratch: list = []          # (buf, nbytes) raw transients: id uploads, saved statistics
         self._regions_opened = 0
         self._pend = None                 # (x, T, out, in, x data, w data, out data) of a held-back linear launch
+        # input gradients of linears held back in the backward, by input tensor: id(x) -> (x, rows, in, [(dY, W, out), ...]).
+        # Sibling projections of one activation (q/k/v, gate/up) then leave as ONE product dX = sum of dY_i.W_i; whoever
+        # touches x's gradient next, and every point where buffers can change hands, sends what is held first.
+        self._pend_dx: dict = {}
+        self.fuse_sibling_dx = True
         self.batch_linears = True
         # attention keeps its raw scores from the forward to the backward (one [T, T] matrix per sequence and head) when a
         # gradient will be asked for, one call's matrices fit attn_scores_max_bytes and the live ones together stay
@@ -95,6 +100,32 @@ class HipBackend:
         if p is not None:
             self._pend = None
             check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, p[1], p[2], p[3], p[4], p[5], p[6]), "linear")
+
+    def _flush_dx(self, t: Tensor = None):
+        """Launch the held-back input-gradient products: those into t's gradient, or all of them."""
+        if not self._pend_dx:
+            return
+        if t is None:
+            items = list(self._pend_dx.values())
+            self._pend_dx.clear()
+        else:
+            it = self._pend_dx.pop(id(t), None)
+            if it is None:
+                return
+            items = [it]
+        for x, rows, ind, parts in items:
+            dx, acc = self._gdst(x)
+            if not dx:
+                continue
+            if len(parts) == 1:
+                g, wd, outd = parts[0]
+                check(self._ctx, lib.gt_gemm(self._ctx, NN, acc, rows, ind, outd, g, wd, dx), "linear.dx")
+            else:
+                n = len(parts)
+                ks = (C.c_int * n)(*[p[2] for p in parts])
+                gs = (c_buf * n)(*[p[0] for p in parts])
+                ws = (c_buf * n)(*[p[1] for p in parts])
+                check(self._ctx, lib.gt_gemm_sum(self._ctx, NN, acc, rows, ind, n, ks, gs, ws, dx), "linear.dx")
 
     def install(self):
         ag.set_ops_backend(self)
@@ -203,6 +234,8 @@ class HipBackend:
         """(gradient buffer, acc) for a backward kernel about to contribute to t's gradient;
         (0, 0) when t takes no gradient (a frozen parameter)."""
         self._flush()
+        if self._pend_dx:
+            self._flush_dx(t)       # products held back for this gradient go first: the order of its writers is kept
         e = self._entries.get(t)
         if e is None:
             e = self._entry_for(t)
@@ -217,6 +250,8 @@ class HipBackend:
     def _gsrc(self, t: Tensor) -> int:
         """Gradient buffer of an op output inside its backward closure."""
         self._flush()
+        if self._pend_dx:
+            self._flush_dx(t)
         e = self._entries.get(t)
         if e is None:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
@@ -233,12 +268,14 @@ class HipBackend:
     # ---- public buffer surface (webgpu.ts:1432-1537) ----------------------------------------------------
     def upload_params(self, tensors):
         self._flush()
+        self._flush_dx()
         for t in tensors:
             e = self._entry_for(t)
             check(self._ctx, lib.gt_h2d(self._ctx, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
 
     def buffers_for(self, t: Tensor) -> dict:
         self._flush()
+        self._flush_dx()
         e = self._entry_for(t)
         if t.requires_grad and e.grad == 0:
             e.grad = self._acquire(e.nbytes)
@@ -270,6 +307,7 @@ class HipBackend:
 
     def seed_grad_from_host(self, t: Tensor):
         self._flush()
+        self._flush_dx()
         e = self._entries.get(t)
         if e is None:
             raise RuntimeError("seed_grad_from_host: tensor has no device buffers")
@@ -286,11 +324,13 @@ class HipBackend:
 
     def write_state_buffer(self, b: int, arr: np.ndarray):
         self._flush()
+        self._flush_dx()
         arr = np.ascontiguousarray(arr)
         check(self._ctx, lib.gt_h2d(self._ctx, b, arr.ctypes.data_as(C.c_void_p), arr.nbytes), "gt_h2d")
 
     def read_state_buffer(self, b: int, n: int, dtype=np.float32) -> np.ndarray:
         self._flush()
+        self._flush_dx()
         out = np.empty(n, dtype=dtype)
         check(self._ctx, lib.gt_d2h(self._ctx, out.ctypes.data_as(C.c_void_p), b, out.nbytes), "gt_d2h")
         return out
@@ -340,6 +380,7 @@ class HipBackend:
         trainable external tensor touched since the last sync that is not kept on the device; recycle
         all intermediates. The graph is unusable for backward afterwards."""
         self._flush()
+        self._flush_dx()
         nbytes = 0
         for t in reads:
             e = self._entries.get(t)
@@ -373,11 +414,13 @@ class HipBackend:
     def reclaim_step_transients(self, keep=()):
         """Free a finished micro-batch's intermediates mid-step; parameter gradients keep accumulating."""
         self._flush()
+        self._flush_dx()
         check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")
         self._release_transients(keep)
 
     def destroy(self):
         self._pend = None
+        self._pend_dx = {}
         if not self._destroyed:
             self._destroyed = True
             lib.gt_ctx_destroy(self._ctx)
@@ -386,11 +429,13 @@ class HipBackend:
     def start_profile(self, prefix: str = ""):
         """Time every launch whose label starts with `prefix` ("" = all) with HIP events on the stream."""
         self._flush()
+        self._flush_dx()
         check(self._ctx, lib.gt_prof_begin(self._ctx, prefix.encode()), "gt_prof_begin")
 
     def stop_profile(self) -> dict:
         """label -> (total ms, launches, algorithmic work: FLOP or bytes)."""
         self._flush()
+        self._flush_dx()
         recs = (ProfRec * 128)()
         n = C.c_int()
         check(self._ctx, lib.gt_prof_end(self._ctx, recs, 128, C.byref(n)), "gt_prof_end")
@@ -403,6 +448,7 @@ class HipBackend:
 
     def end_region(self, mark: int, keep):
         self._flush()
+        self._flush_dx()
         keep_ids = {id(t) for t in keep}
         tail = self._transients[mark:]
         del self._transients[mark:]
@@ -453,9 +499,18 @@ class HipBackend:
 
         def bw():
             g = self._gsrc(out)
-            dx, acc = self._gdst(x)
-            if dx:
-                check(self._ctx, lib.gt_gemm(self._ctx, NN, acc, T, ind, outd, g, wd, dx), "linear.dx")
+            if self.fuse_sibling_dx:
+                held = self._pend_dx.get(id(x))
+                if held is None:
+                    self._pend_dx[id(x)] = (x, T, ind, [(g, wd, outd)])
+                else:
+                    held[3].append((g, wd, outd))
+                    if len(held[3]) == 3:
+                        self._flush_dx(x)
+            else:
+                dx, acc = self._gdst(x)
+                if dx:
+                    check(self._ctx, lib.gt_gemm(self._ctx, NN, acc, T, ind, outd, g, wd, dx), "linear.dx")
             if wants_dw:
                 dw, accw = self._gdst(w)
                 if dw:
@@ -786,6 +841,7 @@ class HipBackend:
     # ---- raw GEMM for tests and benches (webgpu.ts:1654) --------------------------------------------------------------
     def gemm(self, kind: int, acc: int, M: int, N: int, K: int, a: int, b: int, c: int):
         self._flush()
+        self._flush_dx()
         check(self._ctx, lib.gt_gemm(self._ctx, kind, acc, M, N, K, a, b, c), "gemm")
 
 

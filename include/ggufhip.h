@@ -95,6 +95,13 @@ int gt_gemm_pair(gt_ctx *ctx, int kind, int acc, int M, int N, int K1, gt_buf A1
  * kernels, everything else the general GEMM. */
 int gt_rank_down(gt_ctx *ctx, int rows, int K, int r, gt_buf x, gt_buf s, int s_kmajor, float alpha, gt_buf h);
 int gt_rank_grad(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int transpose_out, int acc, gt_buf p);
+/* C (+)= A_0.B_0 + A_1.B_1 (+ A_2.B_2): up to three products with the same M, N and kind summed in one launch, e.g. the
+ * input gradient of sibling projections of one activation, dX = dQ.Wq + dK.Wk + dV.Wv (the reference issues one
+ * accumulating GEMM per projection, webgpu.ts:893-901). K, A, B are host arrays of `count` entries; operand i is laid out
+ * as for gt_gemm with K = K[i]. NT / NN with every K[i] a multiple of 32 and 16-byte aligned operands chain the K
+ * segments in one loop; anything else is one gt_gemm per product, each adding to the one before. */
+int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const int *K, const gt_buf *A, const gt_buf *B,
+                gt_buf C);
 /* batch of `count` independent products with element strides between consecutive problems
  * (Newton-Schulz over same-shaped matrices; no counterpart call in the reference, which loops). */
 int gt_gemm_batched(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t strideA,

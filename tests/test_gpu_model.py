@@ -384,6 +384,66 @@ def test_kept_attention_scores_policy(gpu, ref, recompute):
     compare(res[True][0], res[True][1], lr, gr, f"kept scores recompute={recompute}")
 
 
+def test_sibling_input_gradients_leave_as_one_product(gpu, ref):
+    """The dX of linears that share their input is held back and sent as one summed product (q/k/v, gate/up). Same
+    gradients as one accumulating product per linear to the parity bound, against the oracle too, and fewer NN launches:
+    per layer q+k+v -> 1 and gate+up -> 1."""
+    kw = dict(arch="llama", vocab=64, hidden=128, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=256, rope_base=1e4, rms_eps=1e-5)
+    rmodel, model = build_pair(ref, kw, seed=31, std=0.05)
+    seqs = batches(ref, kw["vocab"], 64, 2, seed=32, mask_every=5)
+    res, launches = {}, {}
+    try:
+        for fuse in (True, False):
+            gpu.fuse_sibling_dx = fuse
+            gpu.start_profile("gemm.nn")
+            res[fuse] = hip_step(gpu, model, seqs, True, 64)
+            launches[fuse] = sum(v[1] for v in gpu.stop_profile().values())
+    finally:
+        gpu.fuse_sibling_dx = True
+    assert launches[False] - launches[True] == kw["layers"] * 3, launches      # (3 - 1) + (2 - 1) per layer
+    assert np.array_equal(res[True][0], res[False][0])
+    for n in res[True][1]:
+        assert_close(res[True][1][n], res[False][1][n], f"fused vs separate dX, grad {n}")
+    lr, gr = ref_step(ref, rmodel, seqs)
+    compare(res[True][0], res[True][1], lr, gr, "fused sibling dX")
+
+
+def test_held_back_input_gradient_keeps_the_order_of_writers(gpu, ref):
+    """x feeds two linears, an elementwise op and a third linear further on: whoever writes or reads dx while products
+    into it are held back sends them first. Against the oracle, with the elementwise consumer before, between and after."""
+    ag = mod("autograd")
+    r = ref.Mulberry32(77)
+    T, d = 70, 64
+    xa = r.fill_randn([T, d], 0.8)
+    ws = [r.fill_randn([d, d], 0.3) for _ in range(3)]
+    up = r.fill_uniform([T * d])
+
+    def graph(m, x, w1, w2, w3, order):
+        parts = {"a": lambda: m.linear(x, w1), "b": lambda: m.linear(x, w2), "e": lambda: m.mul(x, x)}
+        t = [parts[k]() for k in order]
+        y = m.add(m.add(t[0], t[1]), t[2])
+        return m.add(m.linear(m.silu(y), w3), x)
+
+    for order in ("abe", "aeb", "eab"):
+        hx, rx = ag.Tensor(xa, [T, d], True), ref.Tensor(xa, [T, d], True)
+        hw = [ag.Tensor(w, [d, d], True) for w in ws]
+        rw = [ref.Tensor(w, [d, d], True) for w in ws]
+        gpu.install()
+        try:
+            out = graph(ag, hx, *hw, order)
+            from gpu_common import backward_from
+            backward_from(gpu, ag, out, up)
+            gpu.sync([out])
+        finally:
+            gpu.uninstall()
+        rout = graph(ref, rx, *rw, order)
+        ref.backward_from(rout, up)
+        assert_close(out.data, rout.data, f"{order} forward")
+        assert_close(hx.grad, rx.grad, f"{order} dx")
+        for i, (h, rr) in enumerate(zip(hw, rw)):
+            assert_close(h.grad, rr.grad, f"{order} dw{i}")
+
+
 def test_trim_pool_returns_free_buffers_and_work_goes_on(gpu, ref):
     """Free buffers of the size-class pool go back to the device on request (and on their own when an allocation fails);
     buffers in use stay, and the next step allocates afresh and gives the same bits."""

@@ -219,6 +219,44 @@ def test_rope_far_positions(gpu, ref):
     op_case(gpu, ref, [r(T, H * hd)], lambda ag, x: ag.rope(x, T, H, hd, 1e5, 0), lambda rf, x: rf.rope(x, T, H, hd, 1e5, 0), "rope T=2048")
 
 
+@pytest.mark.parametrize("kind,M,N,Ks", [(1, 300, 576, (576, 192, 192)), (1, 257, 576, (1536, 1536)), (1, 128, 640, (640, 128, 128)),
+                                         (0, 200, 192, (64, 96)), (0, 130, 96, (32, 32, 32)), (1, 64, 576, (576,)),
+                                         (1, 100, 576, (576, 190)), (1, 100, 574, (64, 64)), (2, 96, 64, (128, 160))])
+@pytest.mark.parametrize("acc", [0, 1])
+def test_gemm_sum_equals_the_products_one_by_one(gpu, ref, kind, M, N, Ks, acc):
+    """gt_gemm_sum: up to three products summed in one launch (the K segments chained in one loop for aligned NT / NN
+    operands) against one accumulating gt_gemm per product, and against float64. Cases: the q/k/v and gate/up input
+    gradients at the SmolLM2 widths with ragged row counts, gemma's 640 width, NT, one product only, and the shapes that
+    fall back to single launches (a K that is no multiple of 32, an N that is no multiple of 4, TN)."""
+    lib = mod("lib")
+    r = R(ref, M + N + sum(Ks))
+    As, Bs = [], []
+    for K in Ks:
+        As.append(r(K, M) if kind == 2 else r(M, K))
+        Bs.append(r(N, K) if kind == 0 else r(K, N))
+    c0 = r(M, N)
+    ab = [(gpu.create_state_buffer(a_.nbytes), gpu.create_state_buffer(b_.nbytes)) for a_, b_ in zip(As, Bs)]
+    for (da, db), a_, b_ in zip(ab, As, Bs):
+        gpu.write_state_buffer(da, a_)
+        gpu.write_state_buffer(db, b_)
+    c = gpu.create_state_buffer(c0.nbytes)
+    n = len(Ks)
+    karr, aarr, barr = (C.c_int * n)(*Ks), (C.c_uint64 * n)(*[x[0] for x in ab]), (C.c_uint64 * n)(*[x[1] for x in ab])
+    gpu.write_state_buffer(c, c0)
+    lib.check(gpu.ctx, lib.lib.gt_gemm_sum(gpu.ctx, kind, acc, M, N, n, karr, aarr, barr, c), "gt_gemm_sum")
+    got = gpu.read_state_buffer(c, M * N).copy()
+    gpu.write_state_buffer(c, c0)
+    for i, K in enumerate(Ks):
+        lib.check(gpu.ctx, lib.lib.gt_gemm(gpu.ctx, kind, acc if i == 0 else 1, M, N, K, ab[i][0], ab[i][1], c), "gt_gemm")
+    one_by_one = gpu.read_state_buffer(c, M * N).copy()
+    want = c0.astype(np.float64) * acc
+    for a_, b_ in zip(As, Bs):
+        a64, b64 = a_.astype(np.float64), b_.astype(np.float64)
+        want = want + (a64.T @ b64 if kind == 2 else a64 @ (b64.T if kind == 0 else b64))
+    assert_close(got, want, "gemm_sum vs float64")
+    assert_close(got, one_by_one, "gemm_sum vs one by one")
+
+
 ATTN = [(5, 4, 2, 6, 0), (67, 4, 2, 16, 0), (130, 6, 2, 32, 0), (193, 9, 3, 64, 0), (64, 2, 2, 64, 0), (256, 4, 1, 64, 0),
         (96, 16, 8, 128, 0), (6, 4, 2, 6, 3), (130, 4, 2, 16, 17), (200, 10, 2, 64, 64), (150, 2, 1, 64, 1)]
 
