@@ -133,6 +133,7 @@ int gt_set_option(gt_ctx *ctx, const char *key, int value) {
   else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
   else if (!strcmp(key, "gemm.splitk")) ctx->opt_gemm_splitk = value;
   else if (!strcmp(key, "gemm.staged")) ctx->opt_gemm_staged = value;
+  else if (!strcmp(key, "gemm.sum_min_tiles")) ctx->opt_gemm_sum_min_tiles = value;
   else GT_FAIL(ctx, "gt_set_option: unknown key '%s'", key);
   return 0;
 }

@@ -774,6 +774,10 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
     GT_REQUIRE(ctx, K[i] >= 1 && A[i] && B[i], "gt_gemm_sum: product %d has K %d or a null operand", i, K[i]);
     fused = fused && K[i] % 32 == 0 && A[i] % 16 == 0 && B[i] % 16 == 0;
   }
+  // the chained loop has one tile shape and no K split: below one workgroup per CU the single products, which pick
+  // smaller tiles and split K, fill the chip better
+  const bool t96 = N % 96 == 0;
+  if (fused && cdiv(M, 128) * cdiv(N, t96 ? 96 : 128) < (ctx->opt_gemm_sum_min_tiles >= 0 ? ctx->opt_gemm_sum_min_tiles : ctx->num_cu)) fused = false;
   if (!fused) {        // one launch per product, each adding to the one before
     for (int i = 0; i < count; i++)
       if (gemm_impl(ctx, kind, i ? 1 : acc, M, N, K[i], A[i], 0, B[i], 0, C, 0, 1)) return 1;
@@ -794,7 +798,6 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
     a.xK[i - 1] = K[i]; a.xlda[i - 1] = K[i]; a.xldb[i - 1] = kind == GT_NT ? K[i] : N;
     ksum += K[i];
   }
-  const bool t96 = N % 96 == 0;
   char label[32];
   snprintf(label, sizeof label, "gemm.%s.128x%dx32", kind == GT_NT ? "nt" : "nn", t96 ? 96 : 128);
   ProfScope ps(ctx, label, 2.0 * M * N * ksum);

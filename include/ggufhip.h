@@ -64,6 +64,8 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
  *   "gemm.tile"    -1 = heuristic, 0..12 = pin the GEMM tile configuration (tests and tuning)
  *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor
  *   "gemm.staged"  1 = always stage GEMM operands through registers (0: aligned shapes load straight into LDS)
+ *   "gemm.sum_min_tiles" gt_gemm_sum chains its products in one loop from this many 128-row output tiles on
+ *                  (-1 = one per CU, the default; 0 = always, for tests of the chained kernel on small shapes)
  *   "attn.splits"  -1 = heuristic, n >= 1 = pin the workgroups per attention tile (MFMA kernels, at most 8)
  *   "attn.keep_ds" 1 (default) = attention backward keeps the score gradients dS in the workspace and computes dQ as one
  *                  banded product over them (T a multiple of 128, hd 64 or 128); 0 = dQ always
@@ -98,8 +100,9 @@ int gt_rank_grad(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int tr
 /* C (+)= A_0.B_0 + A_1.B_1 (+ A_2.B_2): up to three products with the same M, N and kind summed in one launch, e.g. the
  * input gradient of sibling projections of one activation, dX = dQ.Wq + dK.Wk + dV.Wv (the reference issues one
  * accumulating GEMM per projection, webgpu.ts:893-901). K, A, B are host arrays of `count` entries; operand i is laid out
- * as for gt_gemm with K = K[i]. NT / NN with every K[i] a multiple of 32 and 16-byte aligned operands chain the K
- * segments in one loop; anything else is one gt_gemm per product, each adding to the one before. */
+ * as for gt_gemm with K = K[i]. NT / NN with every K[i] a multiple of 32, 16-byte aligned operands and at least one
+ * 128-row output tile per CU chain the K segments in one loop; anything else is one gt_gemm per product, each adding to
+ * the one before. */
 int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const int *K, const gt_buf *A, const gt_buf *B,
                 gt_buf C);
 /* batch of `count` independent products with element strides between consecutive problems

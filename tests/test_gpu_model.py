@@ -392,6 +392,7 @@ def test_sibling_input_gradients_leave_as_one_product(gpu, ref):
     rmodel, model = build_pair(ref, kw, seed=31, std=0.05)
     seqs = batches(ref, kw["vocab"], 64, 2, seed=32, mask_every=5)
     res, launches = {}, {}
+    gpu.set_option("gemm.sum_min_tiles", 0)        # 128 rows: below the size from which the library chains the products
     try:
         for fuse in (True, False):
             gpu.fuse_sibling_dx = fuse
@@ -400,6 +401,7 @@ def test_sibling_input_gradients_leave_as_one_product(gpu, ref):
             launches[fuse] = sum(v[1] for v in gpu.stop_profile().values())
     finally:
         gpu.fuse_sibling_dx = True
+        gpu.set_option("gemm.sum_min_tiles", -1)
     assert launches[False] - launches[True] == kw["layers"] * 3, launches      # (3 - 1) + (2 - 1) per layer
     assert np.array_equal(res[True][0], res[False][0])
     for n in res[True][1]:

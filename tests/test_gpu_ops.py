@@ -221,7 +221,8 @@ def test_rope_far_positions(gpu, ref):
 
 @pytest.mark.parametrize("kind,M,N,Ks", [(1, 300, 576, (576, 192, 192)), (1, 257, 576, (1536, 1536)), (1, 128, 640, (640, 128, 128)),
                                          (0, 200, 192, (64, 96)), (0, 130, 96, (32, 32, 32)), (1, 64, 576, (576,)),
-                                         (1, 100, 576, (576, 190)), (1, 100, 574, (64, 64)), (2, 96, 64, (128, 160))])
+                                         (1, 100, 576, (576, 190)), (1, 100, 574, (64, 64)), (2, 96, 64, (128, 160)),
+                                         (1, 5600, 576, (576, 192, 192))])
 @pytest.mark.parametrize("acc", [0, 1])
 def test_gemm_sum_equals_the_products_one_by_one(gpu, ref, kind, M, N, Ks, acc):
     """gt_gemm_sum: up to three products summed in one launch (the K segments chained in one loop for aligned NT / NN
@@ -243,8 +244,16 @@ def test_gemm_sum_equals_the_products_one_by_one(gpu, ref, kind, M, N, Ks, acc):
     n = len(Ks)
     karr, aarr, barr = (C.c_int * n)(*Ks), (C.c_uint64 * n)(*[x[0] for x in ab]), (C.c_uint64 * n)(*[x[1] for x in ab])
     gpu.write_state_buffer(c, c0)
-    lib.check(gpu.ctx, lib.lib.gt_gemm_sum(gpu.ctx, kind, acc, M, N, n, karr, aarr, barr, c), "gt_gemm_sum")
+    gpu.set_option("gemm.sum_min_tiles", 0)          # the chained loop also below one tile per CU
+    try:
+        lib.check(gpu.ctx, lib.lib.gt_gemm_sum(gpu.ctx, kind, acc, M, N, n, karr, aarr, barr, c), "gt_gemm_sum")
+    finally:
+        gpu.set_option("gemm.sum_min_tiles", -1)
     got = gpu.read_state_buffer(c, M * N).copy()
+    if M * N < 256 * 128 * 96:                        # default threshold: a small output goes product by product, bit for bit
+        gpu.write_state_buffer(c, c0)
+        lib.check(gpu.ctx, lib.lib.gt_gemm_sum(gpu.ctx, kind, acc, M, N, n, karr, aarr, barr, c), "gt_gemm_sum")
+        small = gpu.read_state_buffer(c, M * N).copy()
     gpu.write_state_buffer(c, c0)
     for i, K in enumerate(Ks):
         lib.check(gpu.ctx, lib.lib.gt_gemm(gpu.ctx, kind, acc if i == 0 else 1, M, N, K, ab[i][0], ab[i][1], c), "gt_gemm")
@@ -255,6 +264,8 @@ def test_gemm_sum_equals_the_products_one_by_one(gpu, ref, kind, M, N, Ks, acc):
         want = want + (a64.T @ b64 if kind == 2 else a64 @ (b64.T if kind == 0 else b64))
     assert_close(got, want, "gemm_sum vs float64")
     assert_close(got, one_by_one, "gemm_sum vs one by one")
+    if M * N < 256 * 128 * 96:
+        assert np.array_equal(small, one_by_one)
 
 
 ATTN = [(5, 4, 2, 6, 0), (67, 4, 2, 16, 0), (130, 6, 2, 32, 0), (193, 9, 3, 64, 0), (64, 2, 2, 64, 0), (256, 4, 1, 64, 0),
