@@ -55,6 +55,9 @@ struct GemmArgs {
   // K step, same M, N and operand orientation: the dX of sibling projections of one input as one product
   const float *xA[2], *xB[2];
   int xK[2], xlda[2], xldb[2], nx;
+  // C = D + A.B: the matrix the product is added to when it is not C's own old contents (layout of C; null: none).
+  // Single products only (no batch); with K splits the reduce kernel adds it.
+  const float *D;
 };
 
 // Which output tile (pm, pn) and which K split or batch member (z) a workgroup works on. Workgroups are handed
@@ -264,7 +267,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
   int ldc;
   bool add;
   if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
-  else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0; }
+  else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0 || a.D != nullptr; }
+  const float *Cold = (a.D && a.splits == 1) ? a.D : C;
   // When accumulating, the sixteen old values of a 32x32 tile are loaded together (from clamped, always valid
   // addresses) before the first store: a load placed after a store to the same array waits for it, and one round trip
   // per element is what an interleaved read-add-write loop would pay.
@@ -276,7 +280,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
       const int rbase = m0 + wm * (TM * 32) + i * 32 + 4 * g;
       float old[16];
       if (add) {
-        const float *cc = C + min(col, a.N - 1);
+        const float *cc = Cold + min(col, a.N - 1);
 #pragma unroll
         for (int r = 0; r < 16; r++) old[r] = cc[(size_t)min(rbase + 8 * (r / 4) + (r % 4), a.M - 1) * ldc];
       }
@@ -481,11 +485,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   bool add;
   if (BAND) { C = a.C + (z / a.zdiv) * a.sC + (z % a.zdiv) * a.sC2; ldc = a.ldc; add = a.acc != 0; }
   else if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
-  else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0; }
+  else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0 || a.D != nullptr; }
+  const float *Cold = (!BAND && a.D && a.splits == 1) ? a.D : C;
   // The MFMAs above take the B tile as their first operand, so an accumulator holds a C^T tile: lane l32 is the row
   // of C, and registers 4q..4q+3 are four consecutive columns 8q + 4g + (0..3): one 16-byte store (and, when
   // accumulating, one 16-byte load issued before any store) instead of four scalar ones.
-  const bool vec_c = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
+  const bool vec_c = (ldc % 4 == 0) && (((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(Cold)) & 15) == 0);
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -495,7 +500,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
       if (vec_c) {
         v4f old[4];
         if (add) {
-          const float *cr = C + (size_t)min(row, a.M - 1) * ldc;
+          const float *cr = Cold + (size_t)min(row, a.M - 1) * ldc;
 #pragma unroll
           for (int q = 0; q < 4; q++) old[q] = *reinterpret_cast<const v4f *>(cr + min(cbase + 8 * q, a.N - 4));
         }
@@ -514,8 +519,9 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
         float *cr = C + (size_t)row * ldc;
         float old[16];
         if (add) {
+          const float *co = Cold + (size_t)row * ldc;
 #pragma unroll
-          for (int r = 0; r < 16; r++) old[r] = cr[min(cbase + 8 * (r / 4) + (r % 4), a.N - 1)];
+          for (int r = 0; r < 16; r++) old[r] = co[min(cbase + 8 * (r / 4) + (r % 4), a.N - 1)];
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -554,12 +560,12 @@ static int launch_direct(gt_ctx *ctx, int kind, GemmArgs &a, int zdim, int slot)
 
 // C (+)= sum over splits, in split order
 __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ Pp, float *__restrict__ C, int64_t n,
-                                                     int splits, int acc) {
+                                                     int splits, int acc, const float *__restrict__ D) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = Pp[i];
   for (int z = 1; z < splits; z++) s += Pp[(size_t)z * n + i];
-  C[i] = acc ? C[i] + s : s;
+  C[i] = D ? D[i] + s : acc ? C[i] + s : s;
 }
 
 template <int BM, int BN, int WM, int WN, int BKT>
@@ -584,7 +590,7 @@ static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
 static int reduce_splits(gt_ctx *ctx, const GemmArgs &a, int M, int N, int splits, int acc) {
   if (splits > 1) {
     int64_t n = (int64_t)M * N;
-    hipLaunchKernelGGL(splitk_reduce, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, a.Pp, a.C, n, splits, acc);
+    hipLaunchKernelGGL(splitk_reduce, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, a.Pp, a.C, n, splits, acc, a.D);
     GT_LAUNCHED(ctx);
   }
   return 0;
@@ -596,7 +602,7 @@ static const TileCfg kTiles[] = {{64, 64, 16}, {128, 64, 16}, {128, 128, 16}, {1
 #define NCFG ((int)(sizeof(kTiles) / sizeof(kTiles[0])))
 
 static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
-                     gt_buf C, int64_t sC, int count, int K2 = 0, gt_buf A2 = 0, gt_buf B2 = 0) {
+                     gt_buf C, int64_t sC, int count, int K2 = 0, gt_buf A2 = 0, gt_buf B2 = 0, gt_buf D = 0) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, kind >= 0 && kind <= 2, "gt_gemm: kind %d is not NT(0)/NN(1)/TN(2)", kind);
   GT_REQUIRE(ctx, M >= 1 && N >= 1 && K >= 1 && count >= 1, "gt_gemm: M,N,K,count must be >= 1 (got %d,%d,%d,%d)", M, N, K, count);
@@ -609,7 +615,8 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   a.ldc = N;
   a.acc = acc; a.kchunk = K; a.splits = 1; a.Pp = nullptr;
   a.sA = sA; a.sB = sB; a.sC = sC;
-  a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0; a.nx = 0;
+  a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0; a.nx = 0; a.D = P<const float>(D);
+  GT_REQUIRE(ctx, !D || (count == 1 && K2 == 0), "gt_gemm_add: one single product only");
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
              (sA % 4 == 0) && (sB % 4 == 0);
   a.K2 = K2; a.A2 = P<const float>(A2); a.B2 = P<const float>(B2);
@@ -742,7 +749,7 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.acc = acc; a.kchunk = T; a.splits = 1; a.Pp = nullptr;
   a.sA = (int64_t)T * T; a.sB = (int64_t)T * Hkv * hd; a.sC = (int64_t)T * Hq * hd;
   a.zdiv = Hq; a.zgroup = Hq / Hkv; a.window = window; a.sB2 = hd; a.sC2 = hd;
-  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0; a.nx = 0;
+  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0; a.nx = 0; a.D = nullptr;
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
   return hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26);
 }
@@ -791,7 +798,7 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
   a.sA = a.sB = a.sC = 0;
   a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0;
   a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0;
-  a.nx = count - 1;
+  a.nx = count - 1; a.D = nullptr;
   double ksum = K[0];
   for (int i = 1; i < count; i++) {
     a.xA[i - 1] = P<const float>(A[i]); a.xB[i - 1] = P<const float>(B[i]);
@@ -806,6 +813,10 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
 }
 int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_buf B, gt_buf C) {
   return gemm_impl(ctx, kind, acc, M, N, K, A, 0, B, 0, C, 0, 1);
+}
+int gt_gemm_add(gt_ctx *ctx, int kind, int M, int N, int K, gt_buf A, gt_buf B, gt_buf D, gt_buf C) {
+  if (ctx && !D) GT_FAIL(ctx, "gt_gemm_add: null addend");
+  return gemm_impl(ctx, kind, 0, M, N, K, A, 0, B, 0, C, 0, 1, 0, 0, 0, D);
 }
 int gt_gemm_pair(gt_ctx *ctx, int kind, int acc, int M, int N, int K1, gt_buf A1, gt_buf B1, int K2, gt_buf A2, gt_buf B2,
                  gt_buf C) {

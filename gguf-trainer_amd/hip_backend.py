@@ -36,7 +36,7 @@ _ALIGN = 256
 
 class _Entry:
     __slots__ = ("data", "grad", "nbytes", "external", "grad_init", "lazy_act", "consumers", "fused_uses",
-                 "region", "keep_grad", "extra", "needs_grad")
+                 "region", "keep_grad", "extra", "needs_grad", "lazy_lin")
 
     def __init__(self, nbytes, external):
         self.data = 0
@@ -51,6 +51,7 @@ class _Entry:
         self.keep_grad = False
         self.extra = None           # (buf, nbytes) of a saved buffer that lives and dies with this output (attention scores)
         self.needs_grad = False     # an intermediate below a trainable tensor: a backward through it may be asked for
+        self.lazy_lin = None        # (rows, out, in, x data, w data) while a linear's output lives only inside a fused add
 
 
 class HipBackend:
@@ -80,6 +81,7 @@ class HipBackend:
         # touches x's gradient next, and every point where buffers can change hands, sends what is held first.
         self._pend_dx: dict = {}
         self.fuse_sibling_dx = True
+        self.fuse_residual_add = True
         self.batch_linears = True
         # attention keeps its raw scores from the forward to the backward (one [T, T] matrix per sequence and head) when a
         # gradient will be asked for, one call's matrices fit attn_scores_max_bytes and the live ones together stay
@@ -219,6 +221,8 @@ class HipBackend:
         e.consumers += 1
         if e.lazy_act is not None:
             self._materialise(t, e)
+        if e.lazy_lin is not None:
+            self._materialise_lin(e)
         return e.data
 
     def _materialise(self, t: Tensor, e: _Entry):
@@ -229,6 +233,13 @@ class HipBackend:
         xe = self._entry_for(x)
         fn = lib.gt_silu_fwd if act == 0 else lib.gt_gelu_fwd
         check(self._ctx, fn(self._ctx, t.size, xe.data, e.data), "act.fwd")
+
+    def _materialise_lin(self, e: _Entry):
+        """A linear output that went straight into a residual add is wanted on its own after all: compute it now."""
+        rows, outd, ind, xd, wd = e.lazy_lin
+        e.lazy_lin = None
+        e.data = self._acquire(e.nbytes)
+        check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, rows, outd, ind, xd, wd, e.data), "linear")
 
     def _gdst(self, t: Tensor) -> tuple:
         """(gradient buffer, acc) for a backward kernel about to contribute to t's gradient;
@@ -388,6 +399,8 @@ class HipBackend:
                 raise RuntimeError("sync: tensor has no device buffers")
             if e.lazy_act is not None:
                 self._materialise(t, e)
+            if e.lazy_lin is not None:
+                self._materialise_lin(e)
             check(self._ctx, lib.gt_d2h(self._ctx, t.data.ctypes.data_as(C.c_void_p), e.data, e.nbytes), "gt_d2h")
             nbytes += e.nbytes
         for t in self._touched:
@@ -558,9 +571,31 @@ class HipBackend:
         return out
 
     def add(self, a: Tensor, b: Tensor) -> Tensor:
-        ad, bd = self._data(a), self._data(b)
-        out, e = self._make_out(a.shape, [a, b])
-        check(self._ctx, lib.gt_add_fwd(self._ctx, out.size, ad, bd, e.data), "add")
+        p = self._pend
+        lin = None
+        if self.fuse_residual_add and p is not None and a is not b:
+            # the linear whose launch is still held back is one of the operands and nothing else has read it: the residual
+            # add of a layer, h + linear(x, W). One launch writes h + x.W^T; the product never exists on its own.
+            for cand in (b, a):
+                ce = self._entries.get(cand)
+                if ce is not None and ce.data == p[6] and ce.consumers == 0 and not ce.external:
+                    lin = cand
+                    break
+        if lin is not None:
+            other = a if lin is b else b
+            le = self._entries[lin]
+            self._pend = None
+            od = self._data(other)
+            out, e = self._make_out(a.shape, [a, b])
+            check(self._ctx, lib.gt_gemm_add(self._ctx, NT, p[1], p[2], p[3], p[4], p[5], od, e.data), "linear+add")
+            le.consumers += 1
+            le.lazy_lin = (p[1], p[2], p[3], p[4], p[5])
+            self._recycle(le.data, le.nbytes)
+            le.data = 0
+        else:
+            ad, bd = self._data(a), self._data(b)
+            out, e = self._make_out(a.shape, [a, b])
+            check(self._ctx, lib.gt_add_fwd(self._ctx, out.size, ad, bd, e.data), "add")
 
         def bw():
             g = self._gsrc(out)

@@ -64,6 +64,7 @@ _SIG = {
     "gt_rope": [ctxp, i32, i32, i32, i32, f64, i32, i32, buf, buf, i32],
     "gt_attn_fwd": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf],
     "gt_attn_bwd": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, buf, buf, i32, buf, i32, buf, i32],
+    "gt_gemm_add": [ctxp, i32, i32, i32, i32, buf, buf, buf, buf],
     "gt_gemm_sum": [ctxp, i32, i32, i32, i32, i32, C.POINTER(i32), C.POINTER(buf), C.POINTER(buf), buf],
     "gt_attn_scores_bytes": [ctxp, i32, i32, i32, i32, i32, i32, C.POINTER(C.c_uint64)],
     "gt_attn_fwd_scores": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, buf],

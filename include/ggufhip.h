@@ -97,6 +97,10 @@ int gt_gemm_pair(gt_ctx *ctx, int kind, int acc, int M, int N, int K1, gt_buf A1
  * kernels, everything else the general GEMM. */
 int gt_rank_down(gt_ctx *ctx, int rows, int K, int r, gt_buf x, gt_buf s, int s_kmajor, float alpha, gt_buf h);
 int gt_rank_grad(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int transpose_out, int acc, gt_buf p);
+/* C = D + A.B with D a matrix laid out as C (it may be C itself): a linear whose output is at once added to the residual
+ * stream, add(h, linear(x, W)) in the reference's layer bodies (src/arch/llama.ts:131-222), as one launch
+ * with no [rows, out] round trip for the product. */
+int gt_gemm_add(gt_ctx *ctx, int kind, int M, int N, int K, gt_buf A, gt_buf B, gt_buf D, gt_buf C);
 /* C (+)= A_0.B_0 + A_1.B_1 (+ A_2.B_2): up to three products with the same M, N and kind summed in one launch, e.g. the
  * input gradient of sibling projections of one activation, dX = dQ.Wq + dK.Wk + dV.Wv (the reference issues one
  * accumulating GEMM per projection, webgpu.ts:893-901). K, A, B are host arrays of `count` entries; operand i is laid out

@@ -446,6 +446,70 @@ def test_held_back_input_gradient_keeps_the_order_of_writers(gpu, ref):
             assert_close(h.grad, rr.grad, f"{order} dw{i}")
 
 
+def test_residual_add_rides_the_linear_launch(gpu, ref):
+    """h + linear(x, W) leaves as one launch (the product is added to h in the GEMM's write-back): every bit of the loss
+    and of every gradient is what the linear and the add as two launches give, with two add launches fewer per layer."""
+    kw = dict(arch="llama", vocab=64, hidden=128, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=256, rope_base=1e4, rms_eps=1e-5)
+    _, model = build_pair(ref, kw, seed=41, std=0.05)
+    seqs = batches(ref, kw["vocab"], 50, 2, seed=42, mask_every=5)
+    res, adds = {}, {}
+    try:
+        for fuse in (True, False):
+            gpu.fuse_residual_add = fuse
+            gpu.start_profile("add")
+            res[fuse] = hip_step(gpu, model, seqs, True, 50)
+            adds[fuse] = sum(v[1] for k, v in gpu.stop_profile().items() if k == "add")
+    finally:
+        gpu.fuse_residual_add = True
+    assert adds[False] - adds[True] == 2 * kw["layers"], adds
+    assert np.array_equal(res[True][0], res[False][0])
+    for n in res[True][1]:
+        assert np.array_equal(res[True][1][n], res[False][1][n]), n
+
+
+def test_linear_output_used_again_after_its_fused_add(gpu, ref):
+    """The product that went straight into an add is computed after all when something else wants it: a later op, a
+    readback. Against the oracle."""
+    ag = mod("autograd")
+    r = ref.Mulberry32(91)
+    T, d = 70, 64
+    ha, xa, wa = r.fill_randn([T, d], 0.8), r.fill_randn([T, d], 0.8), r.fill_randn([d, d], 0.3)
+    up = r.fill_uniform([T * d])
+
+    def graph(m, h, x, w):
+        y = m.linear(x, w)
+        z = m.add(h, y)
+        return m.mul(z, y), y
+
+    hs = [ag.Tensor(a, list(a.shape), True) for a in (ha, xa, wa)]
+    rs = [ref.Tensor(a, list(a.shape), True) for a in (ha, xa, wa)]
+    gpu.install()
+    try:
+        out, y = graph(ag, *hs)
+        from gpu_common import backward_from
+        backward_from(gpu, ag, out, up)
+        gpu.sync([out, y])
+    finally:
+        gpu.uninstall()
+    rout, ry = graph(ref, *rs)
+    ref.backward_from(rout, up)
+    assert_close(out.data, rout.data, "forward")
+    assert_close(y.data, ry.data, "the product read back")
+    for h, rr, nm in zip(hs, rs, ("dh", "dx", "dw")):
+        assert_close(h.grad, rr.grad, nm)
+    # read back only: the product has no other consumer than the fused add
+    hs = [ag.Tensor(a, list(a.shape), False) for a in (ha, xa, wa)]
+    gpu.install()
+    try:
+        y = ag.linear(hs[1], hs[2])
+        z = ag.add(hs[0], y)
+        gpu.sync([z, y])
+    finally:
+        gpu.uninstall()
+    assert_close(y.data, ry.data, "the product read back, no other consumer")
+    assert_close(z.data, (ha + ry.data.reshape(T, d)).reshape(-1), "sum")
+
+
 def test_trim_pool_returns_free_buffers_and_work_goes_on(gpu, ref):
     """Free buffers of the size-class pool go back to the device on request (and on their own when an allocation fails);
     buffers in use stay, and the next step allocates afresh and gives the same bits."""

@@ -219,6 +219,32 @@ def test_rope_far_positions(gpu, ref):
     op_case(gpu, ref, [r(T, H * hd)], lambda ag, x: ag.rope(x, T, H, hd, 1e5, 0), lambda rf, x: rf.rope(x, T, H, hd, 1e5, 0), "rope T=2048")
 
 
+@pytest.mark.parametrize("kind,M,N,K", [(0, 300, 576, 576), (0, 257, 576, 1536), (0, 70, 83, 75), (0, 64, 64, 4096), (1, 130, 96, 64),
+                                        (2, 96, 64, 2048), (0, 1, 5, 3)])
+@pytest.mark.parametrize("in_place", [False, True])
+def test_gemm_add_is_the_product_plus_the_addend(gpu, ref, kind, M, N, K, in_place):
+    """gt_gemm_add: C = D + A.B in one call, bit for bit what gt_gemm into a buffer and an elementwise add give (the same
+    f32 sum of the same two numbers), for aligned and ragged shapes, the register-staged fallback, K splits (the reduce
+    kernel adds D) and D = C."""
+    lib = mod("lib")
+    r = R(ref, M + N + K)
+    a_ = r(K, M) if kind == 2 else r(M, K)
+    b_ = r(N, K) if kind == 0 else r(K, N)
+    d_ = r(M, N)
+    da, db, dd, dc, dy = (gpu.create_state_buffer(x.nbytes) for x in (a_, b_, d_, d_, d_))
+    gpu.write_state_buffer(da, a_)
+    gpu.write_state_buffer(db, b_)
+    gpu.write_state_buffer(dd, d_)
+    gpu.write_state_buffer(dc, d_ if in_place else np.zeros_like(d_))
+    lib.check(gpu.ctx, lib.lib.gt_gemm_add(gpu.ctx, kind, M, N, K, da, db, dc if in_place else dd, dc), "gt_gemm_add")
+    got = gpu.read_state_buffer(dc, M * N).copy()
+    lib.check(gpu.ctx, lib.lib.gt_gemm(gpu.ctx, kind, 0, M, N, K, da, db, dy), "gt_gemm")
+    y = gpu.read_state_buffer(dy, M * N).copy()
+    assert np.array_equal(got, (d_.reshape(-1) + y).astype(np.float32))
+    with pytest.raises(lib.HipError, match="null addend"):
+        lib.check(gpu.ctx, lib.lib.gt_gemm_add(gpu.ctx, kind, M, N, K, da, db, 0, dc), "gt_gemm_add")
+
+
 @pytest.mark.parametrize("kind,M,N,Ks", [(1, 300, 576, (576, 192, 192)), (1, 257, 576, (1536, 1536)), (1, 128, 640, (640, 128, 128)),
                                          (0, 200, 192, (64, 96)), (0, 130, 96, (32, 32, 32)), (1, 64, 576, (576,)),
                                          (1, 100, 576, (576, 190)), (1, 100, 574, (64, 64)), (2, 96, 64, (128, 160)),
