@@ -227,6 +227,8 @@ def main():
     ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
     ap.add_argument("--no-keep-scores", action="store_true",
                     help="attention recomputes Q.K^T in the backward instead of keeping the forward's scores (saves B*Hq*T*T*4 bytes per layer)")
+    ap.add_argument("--no-fuse", action="append", default=[], choices=["sibling_dx", "residual_add", "add_grads"],
+                    help="switch one of the host-side launch fusions off for an A/B run (repeatable)")
     ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
                     help="library option for an A/B run, e.g. attn.keep_ds=0 (dQ recomputes the scores) or gemm.staged=1")
     ap.add_argument("--profile-all", action="store_true",
@@ -256,6 +258,9 @@ def main():
     gpu = hb.require_gpu("bench.py")
     gpu.batch_linears = not a.no_pair
     gpu.attn_keep_scores = not a.no_keep_scores
+    gpu.fuse_sibling_dx = "sibling_dx" not in a.no_fuse
+    gpu.fuse_residual_add = "residual_add" not in a.no_fuse
+    gpu.alias_add_grads = "add_grads" not in a.no_fuse
     for kv in a.set:
         key, _, val = kv.partition("=")
         gpu.set_option(key, int(val))

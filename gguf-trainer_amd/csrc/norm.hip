@@ -61,7 +61,7 @@ template <int LPR, int NJ>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const float *__restrict__ x,
                                                      const float *__restrict__ w, const float *__restrict__ g,
                                                      const float *__restrict__ rinv, float *dx, int acc_dx,
-                                                     float *__restrict__ dw_part) {
+                                                     const float *dx_old, float *__restrict__ dw_part) {
   constexpr int RPW = WAVE / LPR;
   constexpr int NG = 4 * RPW;                    // row groups per workgroup
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const floa
       const int64_t rl = row < rows ? row : 0;
       const v4f *xr = reinterpret_cast<const v4f *>(x + rl * d);
       const v4f *gr = reinterpret_cast<const v4f *>(g + rl * d);
-      const v4f *dr = reinterpret_cast<const v4f *>(dx + rl * d);
+      const v4f *dr = reinterpret_cast<const v4f *>(dx_old + rl * d);     // what dx is added to (dx itself, or another buffer)
 #pragma unroll
       for (int j = 0; j < NJ; j++) {
         xv[u][j] = xr[cc[j]];
@@ -192,7 +192,8 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_gen(int rows, int d, float ep
 }
 __global__ __launch_bounds__(256) void rmsnorm_bwd_gen(int rows, int d, const float *__restrict__ x,
                                                        const float *__restrict__ w, const float *__restrict__ g,
-                                                       const float *__restrict__ rinv, float *dx, int acc_dx) {
+                                                       const float *__restrict__ rinv, float *dx, int acc_dx,
+                                                       const float *dx_old) {
   const int lane = threadIdx.x % WAVE;
   int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
   if (row >= rows) return;
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_gen(int rows, int d, const fl
   float r = rinv[row], k2 = r * r * r * S / (float)d;
   for (int j = lane; j < d; j += WAVE) {
     float o = w[j] * r * gr[j] - xr[j] * k2;
-    dx[row * d + j] = acc_dx ? dx[row * d + j] + o : o;
+    dx[row * d + j] = acc_dx ? dx_old[row * d + j] + o : o;
   }
 }
 // dw for the fallback: one thread per column over a slab of rows, partials per slab
@@ -220,7 +221,7 @@ __global__ __launch_bounds__(256) void rmsnorm_dw_gen(int rows, int d, int slab,
 
 template <int LPR, int NJ>
 static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
-                       gt_buf dx, int acc_dx, gt_buf dw, int acc_dw) {
+                       gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw) {
   constexpr int RPB = 4 * (WAVE / LPR);
   int64_t nb = std::min<int64_t>(cdiv(rows, RPB), (int64_t)ctx->num_cu * 2);
   if (!bwd) {
@@ -238,7 +239,7 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
   size_t smem = dw ? (size_t)RPB * d * sizeof(float) : 0;
   hipLaunchKernelGGL((rmsnorm_bwd_k<LPR, NJ>), dim3((unsigned)nb), dim3(256), smem, ctx->stream, rows, d,
                      P<const float>(x), P<const float>(w), P<const float>(y_or_g), P<const float>(rinv), P<float>(dx),
-                     acc_dx, part);
+                     acc_dx, P<const float>(dx_old), part);
   GT_LAUNCHED(ctx);
   if (dw) {
     hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, CS_COLS)), dim3(256), 0, ctx->stream, part, (int)nb, d,
@@ -249,10 +250,10 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
 }
 
 static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
-                    gt_buf dx, int acc_dx, gt_buf dw, int acc_dw) {
-  bool aligned = (x | w | y_or_g | dx) % 16 == 0;
+                    gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw) {
+  bool aligned = (x | w | y_or_g | dx | dx_old) % 16 == 0;
   int d4 = d / 4;
-#define FAST(LPR, NJ) return launch_fast<LPR, NJ>(ctx, bwd, rows, d, eps, x, w, y_or_g, rinv, dx, acc_dx, dw, acc_dw)
+#define FAST(LPR, NJ) return launch_fast<LPR, NJ>(ctx, bwd, rows, d, eps, x, w, y_or_g, rinv, dx, acc_dx, dx_old, dw, acc_dw)
   if (d % 4 == 0 && aligned && d <= 2048) {
     if (d4 <= 16) FAST(16, 1);
     if (d4 <= 32) FAST(32, 1);
@@ -271,7 +272,7 @@ static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x,
     return 0;
   }
   hipLaunchKernelGGL(rmsnorm_bwd_gen, dim3(nb), dim3(256), 0, ctx->stream, rows, d, P<const float>(x), P<const float>(w),
-                     P<const float>(y_or_g), P<const float>(rinv), P<float>(dx), acc_dx);
+                     P<const float>(y_or_g), P<const float>(rinv), P<float>(dx), acc_dx, P<const float>(dx_old));
   GT_LAUNCHED(ctx);
   if (dw) {
     int slab = 256, ns = (int)cdiv(rows, slab);
@@ -293,7 +294,7 @@ int gt_rmsnorm_fwd(gt_ctx *ctx, int rows, int d, float eps, gt_buf x, gt_buf w, 
   GT_REQUIRE(ctx, rows >= 0 && d >= 1 && x && w && y && rinv, "gt_rmsnorm_fwd: bad arguments (rows %d, d %d)", rows, d);
   if (rows == 0) return 0;
   ProfScope ps(ctx, "rmsnorm", 8.0 * rows * d);
-  return dispatch(ctx, false, rows, d, eps, x, w, y, rinv, 0, 0, 0, 0);
+  return dispatch(ctx, false, rows, d, eps, x, w, y, rinv, 0, 0, 0, 0, 0);
 }
 int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx, int acc_dx,
                    gt_buf dw, int acc_dw) {
@@ -304,6 +305,17 @@ int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, g
     return 0;
   }
   ProfScope ps(ctx, "rmsnorm.bwd", 12.0 * rows * d);   // read x, g; write dx
-  return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dw, acc_dw);
+  return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dx, dw, acc_dw);
+}
+int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
+                        gt_buf dw, int acc_dw) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && x && w && g && rinv && dx && dx_old, "gt_rmsnorm_bwd_from: bad arguments (rows %d, d %d)", rows, d);
+  if (rows == 0) {
+    if (dw && !acc_dw) GT_HIP(ctx, hipMemsetAsync(P<void>(dw), 0, (size_t)d * 4, ctx->stream));
+    return 0;
+  }
+  ProfScope ps(ctx, "rmsnorm.bwd", 12.0 * rows * d);
+  return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, 1, dx_old, dw, acc_dw);
 }
 }

@@ -36,7 +36,7 @@ _ALIGN = 256
 
 class _Entry:
     __slots__ = ("data", "grad", "nbytes", "external", "grad_init", "lazy_act", "consumers", "fused_uses",
-                 "region", "keep_grad", "extra", "needs_grad", "lazy_lin")
+                 "region", "keep_grad", "extra", "needs_grad", "lazy_lin", "grad_src")
 
     def __init__(self, nbytes, external):
         self.data = 0
@@ -52,6 +52,7 @@ class _Entry:
         self.extra = None           # (buf, nbytes) of a saved buffer that lives and dies with this output (attention scores)
         self.needs_grad = False     # an intermediate below a trainable tensor: a backward through it may be asked for
         self.lazy_lin = None        # (rows, out, in, x data, w data) while a linear's output lives only inside a fused add
+        self.grad_src = 0           # another tensor's gradient buffer that holds this gradient's value so far (add's backward)
 
 
 class HipBackend:
@@ -82,6 +83,12 @@ class HipBackend:
         self._pend_dx: dict = {}
         self.fuse_sibling_dx = True
         self.fuse_residual_add = True
+        # add's backward hands its upstream gradient on instead of copying it: an operand whose gradient has no writer yet
+        # points at the upstream buffer (grad_src). A reader takes that buffer as it is; the first later writer adds to its
+        # contents (rmsNorm's backward reads them from there, any other op has them copied first); aliases are settled
+        # before any buffer they point at can be recycled.
+        self.alias_add_grads = True
+        self._aliased: list = []
         self.batch_linears = True
         # attention keeps its raw scores from the forward to the backward (one [T, T] matrix per sequence and head) when a
         # gradient will be asked for, one call's matrices fit attn_scores_max_bytes and the live ones together stay
@@ -254,9 +261,48 @@ class HipBackend:
             return 0, 0
         if e.grad == 0:
             e.grad = self._acquire(e.nbytes)
+        if e.grad_src:
+            check(self._ctx, lib.gt_d2d(self._ctx, e.grad, e.grad_src, e.nbytes), "gt_d2d")
+            e.grad_src = 0
         acc = 1 if e.grad_init else 0
         e.grad_init = True
         return e.grad, acc
+
+    def _gdst_from(self, t: Tensor) -> tuple:
+        """(gradient buffer, acc, buffer holding its contents so far) for a kernel that can read the old contents from
+        another buffer than the one it writes: a handed-on upstream gradient is then never copied."""
+        e = self._entries.get(t)
+        if e is not None and e.grad_src:
+            self._flush()
+            if self._pend_dx:
+                self._flush_dx(t)
+        if e is not None and e.grad_src:
+            src = e.grad_src
+            e.grad_src = 0
+            if e.grad == 0:
+                e.grad = self._acquire(e.nbytes)
+            return e.grad, 1, src
+        dst, acc = self._gdst(t)
+        return dst, acc, dst
+
+    def _settle_aliases(self, released_ids):
+        """Before buffers are recycled: a handed-on gradient of a tensor that lives on gets its own copy, one of a tensor
+        that is being released is dropped."""
+        if not self._aliased:
+            return
+        for t in self._aliased:
+            e = self._entries.get(t)
+            if e is None or not e.grad_src:
+                continue
+            if id(t) in released_ids:
+                e.grad_src = 0
+                e.grad_init = False
+            else:
+                if e.grad == 0:
+                    e.grad = self._acquire(e.nbytes)
+                check(self._ctx, lib.gt_d2d(self._ctx, e.grad, e.grad_src, e.nbytes), "gt_d2d")
+                e.grad_src = 0
+        self._aliased = []
 
     def _gsrc(self, t: Tensor) -> int:
         """Gradient buffer of an op output inside its backward closure."""
@@ -267,6 +313,8 @@ class HipBackend:
         if e is None:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
                                "gradient buffers, so this backward would read pool garbage")
+        if e.grad_src:
+            return e.grad_src       # handed on by an add's backward and not written since: read it where it is
         if e.grad == 0 or not e.grad_init:
             # nothing downstream wrote it (an output the loss does not depend on): its gradient is zero
             if e.grad == 0:
@@ -326,6 +374,7 @@ class HipBackend:
             e.grad = self._acquire(e.nbytes)
         check(self._ctx, lib.gt_h2d(self._ctx, e.grad, t.grad.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
         e.grad_init = True
+        e.grad_src = 0
 
     def create_state_buffer(self, nbytes: int) -> int:
         out = c_buf()
@@ -366,6 +415,7 @@ class HipBackend:
     # ---- sync / reclaim (webgpu.ts:419-636) -------------------------------------------------------------
     def _release_transients(self, keep=()):
         keep_ids = {id(t) for t in keep}
+        self._settle_aliases({id(t) for t, _ in self._transients if id(t) not in keep_ids})
         kept = []
         for t, e in self._transients:
             if id(t) in keep_ids:
@@ -464,6 +514,7 @@ class HipBackend:
         self._flush_dx()
         keep_ids = {id(t) for t in keep}
         tail = self._transients[mark:]
+        self._settle_aliases({id(t) for t, _ in tail if id(t) not in keep_ids})
         del self._transients[mark:]
         for t, e in tail:
             if id(t) in keep_ids:
@@ -603,9 +654,24 @@ class HipBackend:
                 da, acc = self._gdst(a)
                 check(self._ctx, lib.gt_add_bwd(self._ctx, out.size, g, da, acc, da, acc), "add.bwd")
                 return
-            da, acca = self._gdst(a)
-            db, accb = self._gdst(b)
-            check(self._ctx, lib.gt_add_bwd(self._ctx, out.size, g, da, acca, db, accb), "add.bwd")
+            todo = []
+            for t in (a, b):
+                te = self._entries.get(t)
+                if (self.alias_add_grads and te is not None and not te.external and not te.keep_grad and not te.grad_init
+                        and not te.grad_src and id(t) not in self._pend_dx):
+                    te.grad_src = g             # first writer: the gradient IS the upstream one so far, nothing to launch
+                    te.grad_init = True
+                    self._aliased.append(t)
+                else:
+                    todo.append(t)
+            if len(todo) == 2:
+                da, acca = self._gdst(a)
+                db, accb = self._gdst(b)
+                check(self._ctx, lib.gt_add_bwd(self._ctx, out.size, g, da, acca, db, accb), "add.bwd")
+            elif todo:
+                d1, acc1 = self._gdst(todo[0])
+                if d1:
+                    check(self._ctx, lib.gt_scale_bwd(self._ctx, out.size, g, 1.0, d1, acc1), "add.bwd")
 
         out._backward = bw
         return out
@@ -664,7 +730,7 @@ class HipBackend:
                 raise RuntimeError("backward over a graph built before a sync()")
             if oe.fused_uses and oe.fused_uses == oe.consumers:
                 return                       # every use was a fused gate*up, which already wrote x's gradient
-            if oe.grad == 0 and oe.fused_uses:
+            if oe.grad == 0 and not oe.grad_src and oe.fused_uses:
                 return                       # its other consumers contributed nothing
             g = self._gsrc(out)
             dx, acc = self._gdst(x)
@@ -703,9 +769,12 @@ class HipBackend:
 
         def bw():
             g = self._gsrc(out)
-            dx, acc = self._gdst(x)
+            dx, acc, old = self._gdst_from(x)
             dw, accw = self._gdst(weight) if wants_dw else (0, 0)
-            check(self._ctx, lib.gt_rmsnorm_bwd(self._ctx, rows, d, xd, wd, g, rinv, dx, acc, dw, accw), "rmsnorm.bwd")
+            if old != dx:
+                check(self._ctx, lib.gt_rmsnorm_bwd_from(self._ctx, rows, d, xd, wd, g, rinv, old, dx, dw, accw), "rmsnorm.bwd")
+            else:
+                check(self._ctx, lib.gt_rmsnorm_bwd(self._ctx, rows, d, xd, wd, g, rinv, dx, acc, dw, accw), "rmsnorm.bwd")
 
         out._backward = bw
         return out

@@ -139,6 +139,11 @@ int gt_glu_bwd(gt_ctx *ctx, int act, int64_t n, gt_buf g, gt_buf gate, gt_buf up
 int gt_rmsnorm_fwd(gt_ctx *ctx, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y, gt_buf rinv);
 int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv,
                    gt_buf dx, int acc_dx, gt_buf dw, int acc_dw);
+/* The same with the gradient's old contents in another buffer: dx = dx_old + (the normalisation's input gradient). For a
+ * gradient whose only contribution so far is a copy of an upstream gradient (the add of a residual stream,
+ * webgpu.ts:921-937): the copy is skipped and the upstream buffer is read here instead. */
+int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
+                        gt_buf dw, int acc_dw);
 
 /* ---- embedding: srcEmbeddingFwd / Bwd (wgsl.ts:305-344) ------------------------------------- */
 int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, gt_buf ids, gt_buf W, gt_buf out);

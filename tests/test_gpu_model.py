@@ -510,6 +510,66 @@ def test_linear_output_used_again_after_its_fused_add(gpu, ref):
     assert_close(z.data, (ha + ry.data.reshape(T, d)).reshape(-1), "sum")
 
 
+@pytest.mark.parametrize("arch_name", ["llama", "gemma3"])
+@pytest.mark.parametrize("recompute", [False, True])
+def test_add_backward_hands_its_gradient_on(gpu, ref, arch_name, recompute):
+    """add's backward launches nothing where it is the first writer of an intermediate's gradient: the operand points at
+    the upstream buffer, a reader takes it there, rmsNorm's backward adds to it from there, anything else gets a copy
+    first, and aliases are settled before a region's buffers are recycled. Every bit of the step is what the copying
+    backward gives, with fewer add.bwd launches; also against the oracle."""
+    kw = SMALL[arch_name]
+    rmodel, model = build_pair(ref, kw, seed=51, std=0.1)
+    seqs = batches(ref, kw["vocab"], 23, 2, seed=52, mask_every=5)
+    res, n = {}, {}
+    try:
+        for alias in (True, False):
+            gpu.alias_add_grads = alias
+            gpu.start_profile("")
+            res[alias] = hip_step(gpu, model, seqs, True, 23, recompute=recompute)
+            prof = gpu.stop_profile()
+            n[alias] = sum(v[1] for k, v in prof.items() if k == "add.bwd")
+    finally:
+        gpu.alias_add_grads = True
+    assert n[True] < n[False], n
+    assert np.array_equal(res[True][0], res[False][0])
+    for name in res[True][1]:
+        assert np.array_equal(res[True][1][name], res[False][1][name]), name
+    lr, gr = ref_step(ref, rmodel, seqs)
+    compare(res[True][0], res[True][1], lr, gr, f"{arch_name} handed-on add gradients recompute={recompute}")
+
+
+def test_handed_on_gradient_with_other_readers_and_writers(gpu, ref):
+    """An intermediate whose gradient was handed on by an add and is then written by a product, an elementwise op and
+    another add, or only read. Against the oracle."""
+    ag = mod("autograd")
+    r = ref.Mulberry32(61)
+    T, d = 40, 64
+    xa, wa, ga = r.fill_randn([T, d], 0.8), r.fill_randn([d, d], 0.3), 1 + 0.2 * r.fill_randn([d])
+    up = r.fill_uniform([T * d])
+
+    def graph(m, x, w, gain):
+        t = m.scale(x, 0.5)                                  # an intermediate with four consumers
+        u = m.add(t, m.silu(t))                              # handed on to t first (add runs its backward first)
+        v = m.add(u, m.linear(t, w))                         # a product into t's gradient
+        return m.add(m.mul(v, t), m.rms_norm(m.add(t, u), gain, 1e-5))
+
+    hs = [ag.Tensor(a, list(a.shape), True) for a in (xa, wa, ga)]
+    rs = [ref.Tensor(a, list(a.shape), True) for a in (xa, wa, ga)]
+    gpu.install()
+    try:
+        out = graph(ag, *hs)
+        from gpu_common import backward_from
+        backward_from(gpu, ag, out, up)
+        gpu.sync([out])
+    finally:
+        gpu.uninstall()
+    rout = graph(ref, *rs)
+    ref.backward_from(rout, up)
+    assert_close(out.data, rout.data, "forward")
+    for h, rr, nm in zip(hs, rs, ("dx", "dw", "dgain")):
+        assert_close(h.grad, rr.grad, nm)
+
+
 def test_trim_pool_returns_free_buffers_and_work_goes_on(gpu, ref):
     """Free buffers of the size-class pool go back to the device on request (and on their own when an allocation fails);
     buffers in use stay, and the next step allocates afresh and gives the same bits."""
