@@ -29,9 +29,9 @@ PROF_SAMPLE = 4                # the timed region brackets about 1 in 4 launches
 # passes over this file (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the factors read off a plain streaming kernel of known
 # size; see profiles/bench_smollm2_135m_pmc_fetch_write.txt). Averages over the shapes each label serves in the step (the NN label:
 # 60 summed sibling products, the 30 dX of the o projection and the readout's).
-MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (60 * (2 * 110791.6 + 36864.0) + 30 * (2 * 29745.5 + 36864.2) + (2 * 4516752.8 + 36864.2)) / 91 * 1024,
-                    "gemm.tn.128x96x32.splitk": (2 * 91859.9 + 48384.1) * 1024,
-                    "gemm.tn.64x192x32.splitk": (90 * 359.9 + 180 * 126.8 + 180 * 67.0) / 450 * 1048576}
+MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (60 * (2 * 110763.7 + 36864.0) + 30 * (2 * 29758.3 + 36864.3) + (2 * 4481555.6 + 36864.3)) / 91 * 1024,
+                    "gemm.tn.128x96x32.splitk": (2 * 91867.3 + 48384.1) * 1024,
+                    "gemm.tn.64x192x32.splitk": (90 * 360.1 + 180 * 126.8 + 180 * 67.0) / 450 * 1048576}
 
 SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                rope_base=100000.0, rms_eps=1e-5, tie=True)
