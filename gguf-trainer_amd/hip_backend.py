@@ -18,6 +18,15 @@ What differs from the reference, on purpose:
     the fused gated-activation kernels on the pre-activation and the activation tensor never
     exists in memory. Any other consumer materialises it and the unfused kernels run.
   * Host arrays of intermediates are never allocated unless sync() is asked to read them.
+  * Launches are held back where the next op can ride them. A linear's forward waits one op: a second linear of the
+    same shape over the same input joins it as a batch of two (k and v, gate and up), an add of its output is written
+    by the product's own write-back (the residual add). A linear's input gradient waits until that gradient is next
+    touched: sibling projections then leave as one summed product. add's backward launches nothing where it is the
+    first writer: the operand's gradient points at the upstream buffer until somebody adds to it.
+  * attention keeps its raw scores from the forward to the backward where a backward can come and a byte budget allows,
+    as the reference's small-T path keeps its probabilities (webgpu.ts:1176-1189).
+  Each of these has a switch (batch_linears, fuse_residual_add, fuse_sibling_dx, alias_add_grads, attn_keep_scores) and
+  gives the same gradients as the one-launch-per-op form: bit for bit, or to rounding where a sum changes its order.
 """
 from __future__ import annotations
 
