@@ -1,5 +1,5 @@
 /* A plain C host of libggufhip.so: no Python, no torch, only include/ggufhip.h. It runs y = x W^T, the two backward
- * products and one AdamW step on small matrices, checks them against straightforward loops, and prints "ok".
+ * products, the product-plus-matrix and sum-of-products calls and one AdamW step on small matrices, checks them against straightforward loops, and prints "ok".
  * Built and run by tests/test_gpu_abi_c.py:  gcc abi_host.c -I include -L <pkg> -lggufhip */
 #include <math.h>
 #include <stdio.h>
@@ -48,6 +48,19 @@ int main(void) {
       worst = fmax(worst, fabs(s - dw[o * IN + k]));
     }
   if (worst > 2e-5) { fprintf(stderr, "GEMM mismatch %g\n", worst); return 1; }
+
+  /* product plus matrix, and a sum of two products, each in one call: y + x W^T = 2y and dY W + dY W = 2 dX */
+  {
+    static float y2[T * OUT], dx2[T * IN];
+    const int ks[2] = {OUT, OUT};
+    const gt_buf as[2] = {bdy, bdy}, bs[2] = {bw, bw};
+    CHECK(gt_gemm_add(ctx, GT_NT, T, OUT, IN, bx, bw, by, by));
+    CHECK(gt_gemm_sum(ctx, GT_NN, 0, T, IN, 2, ks, as, bs, bdx));
+    CHECK(gt_d2h(ctx, y2, by, sizeof y2)); CHECK(gt_d2h(ctx, dx2, bdx, sizeof dx2));
+    for (int i = 0; i < T * OUT; i++) worst = fmax(worst, fabs(2.0 * y[i] - y2[i]));
+    for (int i = 0; i < T * IN; i++) worst = fmax(worst, fabs(2.0 * dx[i] - dx2[i]));
+    if (worst > 4e-5) { fprintf(stderr, "gemm_add / gemm_sum mismatch %g\n", worst); return 1; }
+  }
 
   /* one AdamW step on w with gradient dw, no clipping, against adam.ts:46-82 in double */
   gt_adamw *opt = NULL;
