@@ -23,7 +23,11 @@
  *   attention          central finite differences with the reference's recipe
  *                      (tests/gradcheck.ts:100-168) and torch float64 autograd
  *   or_fused_ce_*      equals dense CE of or_linear (tests/gradcheck.ts:854-877)
- *   or_soft_ce_*       finite differences; reduces to hard CE for one-hot q
+ *   or_soft_ce_*       finite differences; reduces to hard CE for one-hot q;
+ *                      k = 3 float64 closed form sum_j q_j (lse - z[id_j]) with a
+ *                      duplicated id, a zero-probability slot, mass < 1
+ *   or_linear_bwd_dots or_linear_bwd and a float64 product, ragged shapes,
+ *                      non-zero starting gradients, frozen weight
  *   or_adamw_step      torch.optim.AdamW in float64 (same closed form)
  *   or_newton_schulz   SVD closed form (the quintic acts on singular values),
  *                      flip invariance
@@ -122,8 +126,11 @@ void or_linear_bwd(const float *x, const float *w, const float *gout, float *gx,
 }
 
 /* Same gradients with the per-output f64 dot product the forward uses: one f32
- * rounding per element instead of one per term. Used only to time a CPU
- * baseline in parallel; or_linear_bwd stays the parity oracle. */
+ * rounding per element instead of one per term, every output element owned by
+ * one iteration (OpenMP-safe). It is the checker of the whole-model GPU
+ * comparisons at real head geometry, where the serial form would take minutes,
+ * and the linear backward of the timed CPU baseline. Pinned against
+ * or_linear_bwd and a float64 product (tests/test_oracle_torch64.py). */
 void or_linear_bwd_dots(const float *x, const float *w, const float *gout, float *gx, float *gw,
                         int T, int in, int outd) {
   OR_PAR

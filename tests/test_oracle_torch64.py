@@ -108,6 +108,77 @@ def test_attention_parallel_bwd_variant_matches(ref):
         assert relerr(a, b) < 1e-6
 
 
+@pytest.mark.parametrize("T,ind,outd,frozen", [(7, 12, 9, False), (33, 17, 5, False), (1, 3, 40, False), (19, 31, 23, True)])
+def test_linear_dots_bwd_variant_matches_serial_and_float64(ref, T, ind, outd, frozen):
+    """or_linear_bwd_dots (the OpenMP-safe backward the whole-model GPU comparisons at tuned shapes and the timed CPU
+    baseline run through) against the reference-ordered or_linear_bwd and against a float64 matrix product, from non-zero
+    starting gradients, on ragged shapes, with a frozen weight (no dW) as one case, and with zeros in the upstream
+    gradient (the serial form skips those terms)."""
+    rng = ref.Mulberry32(T * 1009 + ind * 31 + outd)
+    x, w = rng.fill_randn([T, ind], 0.8), rng.fill_randn([outd, ind], 0.8)
+    gx0, gw0 = rng.fill_randn([T, ind], 0.5), rng.fill_randn([outd, ind], 0.5)
+    up = rng.fill_uniform([T * outd]).reshape(T, outd)
+    up[::3, ::2] = 0.0
+    res = []
+    for par in (False, True):
+        ref.PARALLEL_BWD = par
+        try:
+            xt, wt = ref.Tensor(x, [T, ind], True), ref.Tensor(w, [outd, ind], not frozen)
+            xt.grad[:] = gx0.ravel()
+            wt.grad[:] = gw0.ravel()
+            out = ref.linear(xt, wt)
+            out.grad[:] = up.ravel()
+            out._backward()
+        finally:
+            ref.PARALLEL_BWD = False
+        res.append((xt.grad.copy(), wt.grad.copy()))
+    x64, w64, up64 = x.astype(np.float64).reshape(T, ind), w.astype(np.float64).reshape(outd, ind), up.astype(np.float64)
+    want_gx = gx0.astype(np.float64).reshape(T, ind) + up64 @ w64
+    want_gw = gw0.astype(np.float64).reshape(outd, ind) + (0 if frozen else up64.T @ x64)
+    for gx, gw in res:
+        assert relerr(gx, want_gx) < 2e-7
+        assert relerr(gw, want_gw) < 2e-7
+    assert relerr(res[1][0], res[0][0]) < 2e-7 and relerr(res[1][1], res[0][1]) < 2e-7
+    if frozen:
+        assert np.array_equal(res[0][1], gw0.ravel()) and np.array_equal(res[1][1], gw0.ravel())
+
+
+def test_soft_ce_k3_vs_float64_closed_form(ref):
+    """softCrossEntropy with k = 3 teachers per row (autograd.ts:1076-1138) against its closed form written with library
+    routines in float64: loss = (1/kept) sum_rows sum_j q_j (logsumexp(z) - z[id_j]), gradient by torch autograd. The rows
+    hold a duplicated id (its two probabilities both count), a zero-probability pad slot, a teacher mass below 1, and an
+    ignored row (first id -1); a forward that mis-weights teachers j >= 1 fails the loss, a backward that drops the
+    duplicate's second term fails the gradient."""
+    rng = ref.Mulberry32(77)
+    T, V, k = 6, 29, 3
+    z = rng.fill_randn([T, V], 2.0)
+    ids = [[4, 17, 9], [5, 5, 2], [28, 0, 3], [-1, 0, 0], [11, 12, 12], [7, 1, 20]]
+    q = [[0.5, 0.3, 0.2], [0.4, 0.35, 0.1], [0.7, 0.0, 0.25], [0.0, 0.0, 0.0], [0.2, 0.3, 0.1], [0.05, 0.9, 0.05]]
+    flat_ids = [i for r in ids for i in r]
+    flat_q = [p for r in q for p in r]
+    zt = ref.Tensor(z, [T, V], True)
+    loss = ref.soft_cross_entropy(zt, flat_ids, flat_q, k)
+    ref.backward(loss, 0.75)
+
+    z64 = t64(z, [T, V])
+    lse = torch.logsumexp(z64, dim=1)
+    total = torch.zeros((), dtype=torch.float64)
+    kept = 0
+    for t in range(T):
+        if ids[t][0] < 0:
+            continue
+        kept += 1
+        for j in range(k):
+            total = total + q[t][j] * (lse[t] - z64[t, ids[t][j]])
+    want = total / kept
+    want.backward(torch.tensor(0.75, dtype=torch.float64))
+    want = float(want.detach())
+    assert kept == 5
+    assert abs(float(loss.data[0]) - want) <= 2e-7 * abs(want)
+    assert relerr(zt.grad, z64.grad.numpy()) < 2e-7
+    assert np.all(zt.grad.reshape(T, V)[3] == 0)
+
+
 def test_ce_vs_torch64(ref):
     rng = ref.Mulberry32(31)
     T, V = 9, 37
