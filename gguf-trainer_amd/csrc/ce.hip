@@ -67,7 +67,7 @@ __device__ __forceinline__ void row_stats(const float *__restrict__ zr, int n, f
 
 // one workgroup per row: lse[row] = M + log(L); nll[row] = lse - z_target (0 when ignored)
 __global__ __launch_bounds__(256) void ce_fwd_rows(int V, const float *__restrict__ z, const int *__restrict__ tgt,
-                                                   float *__restrict__ lse, float *__restrict__ nll) {
+                                                   float *__restrict__ lse, float *__restrict__ nll, int *bad) {
   __shared__ float sm[8];
   int64_t row = blockIdx.x;
   const float *zr = z + row * V;
@@ -77,6 +77,10 @@ __global__ __launch_bounds__(256) void ce_fwd_rows(int V, const float *__restric
     float ls = M + logf(L);
     lse[row] = ls;
     int g = tgt[row];
+    if (g < IGN || g >= V) {                    // no such logit: the row counts as ignored here and the host hears of it
+      note_bad_id(bad, GT_BAD_TARGET, row, g, V);
+      g = IGN;
+    }
     nll[row] = g == IGN ? 0.f : (logf(L) + M - zr[g]);
   }
 }
@@ -192,7 +196,7 @@ __global__ __launch_bounds__(256) void ce_chunk_grad_k(int vc, int v0, int T, in
 // ---- sparse-teacher soft CE (autograd.ts:1076-1138) -------------------------------------------------
 __global__ __launch_bounds__(256) void soft_ce_fwd_rows(int V, int k, const float *__restrict__ z, const int *__restrict__ tid,
                                                         const float *__restrict__ tq, float *__restrict__ lse,
-                                                        float *__restrict__ mass, float *__restrict__ nll) {
+                                                        float *__restrict__ mass, float *__restrict__ nll, int *bad) {
   __shared__ float sm[8];
   int64_t row = blockIdx.x;
   const float *zr = z + row * V;
@@ -206,7 +210,9 @@ __global__ __launch_bounds__(256) void soft_ce_fwd_rows(int V, int k, const floa
       for (int j = 0; j < k; j++) {
         float qv = tq[row * k + j];
         if (qv == 0.f) continue;
-        tot += qv * (logf(L) + M - zr[tid[row * k + j]]);
+        const int id = tid[row * k + j];
+        if (id < 0 || id >= V) { note_bad_id(bad, GT_BAD_TEACHER_ID, row, id, V); continue; }
+        tot += qv * (logf(L) + M - zr[id]);
         ms += qv;
       }
     }
@@ -236,10 +242,14 @@ __global__ __launch_bounds__(256) void soft_ce_bwd_p(int V, int k, const float *
   }
 }
 __global__ __launch_bounds__(64) void soft_ce_bwd_q(int rows, int V, int k, const int *__restrict__ tid,
-                                                    const float *__restrict__ tq, float sc, float *dz) {
+                                                    const float *__restrict__ tq, float sc, float *dz, int *bad) {
   int64_t row = (int64_t)blockIdx.x * 64 + threadIdx.x;
   if (row >= rows || tid[row * k] == IGN) return;
-  for (int j = 0; j < k; j++) dz[row * V + tid[row * k + j]] -= sc * tq[row * k + j];
+  for (int j = 0; j < k; j++) {
+    const int id = tid[row * k + j];
+    if (id < 0 || id >= V) { note_bad_id(bad, GT_BAD_TEACHER_ID, row, id, V); continue; }
+    dz[row * V + id] -= sc * tq[row * k + j];
+  }
 }
 
 static inline unsigned row_chunks(int V) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>(cdiv(V, 4 * 256 * 4), 64)); }
@@ -253,7 +263,7 @@ int gt_ce_fwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets
   void *ws;
   if (gt_ws_reserve(ctx, (size_t)rows * sizeof(float), &ws)) return 1;
   hipLaunchKernelGGL(ce_fwd_rows, dim3(rows), dim3(256), 0, ctx->stream, V, P<const float>(logits), P<const int>(targets),
-                     P<float>(lse), static_cast<float *>(ws));
+                     P<float>(lse), static_cast<float *>(ws), ctx->bad_dev);
   GT_LAUNCHED(ctx);
   hipLaunchKernelGGL(ce_seq_loss, dim3(rows / T), dim3(256), 0, ctx->stream, T, static_cast<const float *>(ws),
                      P<const float>(inv_denom), P<float>(loss));
@@ -319,7 +329,7 @@ int gt_soft_ce_fwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf te
   if (gt_ws_reserve(ctx, (size_t)rows * sizeof(float), &ws)) return 1;
   hipLaunchKernelGGL(soft_ce_fwd_rows, dim3(rows), dim3(256), 0, ctx->stream, V, k, P<const float>(logits),
                      P<const int>(teacher_ids), P<const float>(teacher_probs), P<float>(lse), P<float>(row_mass),
-                     static_cast<float *>(ws));
+                     static_cast<float *>(ws), ctx->bad_dev);
   GT_LAUNCHED(ctx);
   hipLaunchKernelGGL(sum_scale_k, dim3(1), dim3(256), 0, ctx->stream, rows, static_cast<const float *>(ws), inv_denom, P<float>(loss));
   GT_LAUNCHED(ctx);
@@ -336,7 +346,7 @@ int gt_soft_ce_bwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf te
                      P<const int>(teacher_ids), P<const float>(lse), P<const float>(row_mass), sc, P<float>(dlogits), acc);
   GT_LAUNCHED(ctx);
   hipLaunchKernelGGL(soft_ce_bwd_q, dim3((unsigned)cdiv(rows, 64)), dim3(64), 0, ctx->stream, rows, V, k,
-                     P<const int>(teacher_ids), P<const float>(teacher_probs), sc, P<float>(dlogits));
+                     P<const int>(teacher_ids), P<const float>(teacher_probs), sc, P<float>(dlogits), ctx->bad_dev);
   GT_LAUNCHED(ctx);
   return 0;
 }

@@ -38,6 +38,9 @@ struct gt_ctx {
   unsigned attn_smem_set = 0;                   // head dims (bits 32 | 64 | 128) whose dK/dV kernel has its LDS size attribute set
   uint64_t gemm_direct_set = 0;                 // direct-to-LDS GEMM variants whose LDS size attribute is set
   int opt_prof_sample = 1;                      // events around every n-th launch of a label
+  // Pinned host words a kernel writes when it meets an id / target outside its range (it skips that row):
+  // [0] = which check (GT_BAD_*), [1] = row, [2] = the value, [3] = the bound. Read after the stream has drained.
+  int *bad_host = nullptr, *bad_dev = nullptr;
   struct ProfSeen { int64_t n = 0; double work = 0; };
   std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not
 };
@@ -54,6 +57,13 @@ extern thread_local char g_create_err[512];
 #define GT_REQUIRE(ctx, cond, ...) do { if (!(cond)) GT_FAIL(ctx, __VA_ARGS__); } while (0)
 
 int gt_ws_reserve(gt_ctx *ctx, size_t bytes, void **out);
+// ids, targets and teacher ids live on the device, so the host cannot look at them before a launch: a kernel that meets
+// one outside its range skips the row and notes it here; gt_sync / gt_d2h / gt_prof_end then fail once with that note.
+enum { GT_BAD_EMBED_ID = 1, GT_BAD_TARGET = 2, GT_BAD_TEACHER_ID = 3 };
+__device__ __forceinline__ void note_bad_id(int *bad, int what, int64_t row, int value, int bound) {
+  bad[1] = (int)row; bad[2] = value; bad[3] = bound; bad[0] = what;
+}
+int gt_report_bad_id(gt_ctx *ctx);
 // gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
 int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc);
 

@@ -35,6 +35,15 @@ int gt_ctx_create(int device, gt_ctx **out) {
     delete c;
     return 1;
   }
+  if ((e = hipHostMalloc(reinterpret_cast<void **>(&c->bad_host), 4 * sizeof(int), hipHostMallocMapped)) != hipSuccess ||
+      (e = hipHostGetDevicePointer(reinterpret_cast<void **>(&c->bad_dev), c->bad_host, 0)) != hipSuccess) {
+    snprintf(g_create_err, sizeof g_create_err, "context setup failed: %s", hipGetErrorString(e));
+    if (c->bad_host) hipHostFree(c->bad_host);
+    hipStreamDestroy(c->stream);
+    delete c;
+    return 1;
+  }
+  memset(c->bad_host, 0, 4 * sizeof(int));
   *out = c;
   return 0;
 }
@@ -46,6 +55,7 @@ int gt_ctx_destroy(gt_ctx *ctx) {
   for (auto &kv : ctx->allocs) hipFree(reinterpret_cast<void *>(kv.first));
   for (auto &kv : ctx->rope_tables) hipFree(kv.second);
   if (ctx->ws) hipFree(ctx->ws);
+  if (ctx->bad_host) hipHostFree(ctx->bad_host);
   for (auto &e : ctx->prof) { hipEventDestroy(e.a); hipEventDestroy(e.b); }
   hipStreamDestroy(ctx->stream);
   delete ctx;
@@ -101,7 +111,7 @@ int gt_d2h(gt_ctx *ctx, void *dst, gt_buf src, size_t bytes) {
   GT_ENTER(ctx);
   if (bytes) GT_HIP(ctx, hipMemcpyAsync(dst, P<void>(src), bytes, hipMemcpyDeviceToHost, ctx->stream));
   GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  return 0;
+  return gt_report_bad_id(ctx);
 }
 
 int gt_d2d(gt_ctx *ctx, gt_buf dst, gt_buf src, size_t bytes) {
@@ -114,7 +124,7 @@ int gt_d2d(gt_ctx *ctx, gt_buf dst, gt_buf src, size_t bytes) {
 int gt_sync(gt_ctx *ctx) {
   GT_ENTER(ctx);
   GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  return 0;
+  return gt_report_bad_id(ctx);
 }
 
 int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes) {
@@ -179,10 +189,21 @@ int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n) {
     k++;
   }
   if (n) *n = k;
-  return 0;
+  return gt_report_bad_id(ctx);
 }
 
 }  // extern "C"
+
+// Call with the stream drained. Reports an out-of-range id once and re-arms the note.
+int gt_report_bad_id(gt_ctx *ctx) {
+  volatile int *b = ctx->bad_host;
+  const int what = b[0];
+  if (!what) return 0;
+  const int row = b[1], value = b[2], bound = b[3];
+  b[0] = 0;
+  const char *name = what == GT_BAD_EMBED_ID ? "embedding id" : what == GT_BAD_TARGET ? "cross-entropy target" : "teacher id";
+  GT_FAIL(ctx, "%s %d at row %d is outside [%d, %d): that row was skipped", name, value, row, what == GT_BAD_TARGET ? -1 : 0, bound);
+}
 
 int gt_ws_reserve(gt_ctx *ctx, size_t bytes, void **out) {
   if (bytes > ctx->ws_bytes) {

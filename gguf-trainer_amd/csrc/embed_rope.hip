@@ -16,14 +16,20 @@
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(256) void embedding_fwd_k(int rows, int d, const int *__restrict__ ids,
-                                                       const float *__restrict__ W, float *__restrict__ out) {
+__global__ __launch_bounds__(256) void embedding_fwd_k(int rows, int d, int V, const int *__restrict__ ids,
+                                                       const float *__restrict__ W, float *__restrict__ out, int *bad) {
   // one wavefront per row, float4 when d % 4 == 0
   const int lane = threadIdx.x % WAVE;
   int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
   if (row >= rows) return;
-  const float *src = W + (size_t)ids[row] * d;
+  const int id = ids[row];
   float *dst = out + row * d;
+  if (id < 0 || id >= V) {                      // no such table row: the output row is zero and the host hears of it
+    if (lane == 0) note_bad_id(bad, GT_BAD_EMBED_ID, row, id, V);
+    for (int j = lane; j < d; j += WAVE) dst[j] = 0.f;
+    return;
+  }
+  const float *src = W + (size_t)id * d;
   if (d % 4 == 0) {
     for (int j = lane; j < d / 4; j += WAVE) reinterpret_cast<v4f *>(dst)[j] = reinterpret_cast<const v4f *>(src)[j];
   } else {
@@ -61,12 +67,16 @@ __global__ __launch_bounds__(256) void scatter_ids_k(int n, const int *__restric
 
 // one workgroup per sorted slot; only the first slot of each id does work: it sums that id's gradient rows in
 // position order (eight row loads in flight per thread) and adds the sum to the id's dW row
-__global__ __launch_bounds__(256) void embedding_bwd_k(int n, int d, const int *__restrict__ order,
+__global__ __launch_bounds__(256) void embedding_bwd_k(int n, int d, int V, const int *__restrict__ order,
                                                        const int *__restrict__ sorted, const float *__restrict__ g,
-                                                       float *dW) {
+                                                       float *dW, int *bad) {
   int p = blockIdx.x;
   int id = sorted[p];
   if (p > 0 && sorted[p - 1] == id) return;
+  if (id < 0 || id >= V) {                      // no such dW row: nothing is added
+    if (threadIdx.x == 0) note_bad_id(bad, GT_BAD_EMBED_ID, order[p], id, V);
+    return;
+  }
   int e = p + 1;
   while (e < n && sorted[e] == id) e++;
   float *dst = dW + (size_t)id * d;
@@ -170,13 +180,13 @@ __global__ __launch_bounds__(256) void rope_vec_k(unsigned nunits, int T, int H,
 }
 
 extern "C" {
-int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, gt_buf ids, gt_buf W, gt_buf out) {
+int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf W, gt_buf out) {
   GT_ENTER(ctx);
-  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && ids && W && out, "gt_embedding_fwd: bad arguments");
+  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && V >= 1 && ids && W && out, "gt_embedding_fwd: bad arguments");
   if (rows == 0) return 0;
   ProfScope ps(ctx, "embedding");
-  hipLaunchKernelGGL(embedding_fwd_k, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, rows, d, P<const int>(ids),
-                     P<const float>(W), P<float>(out));
+  hipLaunchKernelGGL(embedding_fwd_k, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, ctx->stream, rows, d, V, P<const int>(ids),
+                     P<const float>(W), P<float>(out), ctx->bad_dev);
   GT_LAUNCHED(ctx);
   return 0;
 }
@@ -199,8 +209,8 @@ int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, 
   GT_LAUNCHED(ctx);
   hipLaunchKernelGGL(scatter_ids_k, dim3((unsigned)cdiv(rows, 256)), dim3(256), 0, ctx->stream, rows, P<const int>(ids), pos, order, sorted);
   GT_LAUNCHED(ctx);
-  hipLaunchKernelGGL(embedding_bwd_k, dim3((unsigned)rows), dim3(256), 0, ctx->stream, rows, d, order, sorted,
-                     P<const float>(g), P<float>(dW));
+  hipLaunchKernelGGL(embedding_bwd_k, dim3((unsigned)rows), dim3(256), 0, ctx->stream, rows, d, V, order, sorted,
+                     P<const float>(g), P<float>(dW), ctx->bad_dev);
   GT_LAUNCHED(ctx);
   return 0;
 }

@@ -802,7 +802,7 @@ class HipBackend:
         wd = self._data(weight)
         idb = self._upload(ids32)
         out, e = self._make_out([T, d], [weight])
-        check(self._ctx, lib.gt_embedding_fwd(self._ctx, T, d, idb, wd, e.data), "embedding")
+        check(self._ctx, lib.gt_embedding_fwd(self._ctx, T, d, V, idb, wd, e.data), "embedding")
         wants_dw = weight.requires_grad
 
         def bw():

@@ -10,7 +10,10 @@
  *     Asynchronous HIP errors are sticky: the next call (or gt_sync) reports them.
  *   - gt_buf is a device address (64-bit). Offsets into a buffer are plain additions, which is how
  *     a vocab span of the readout matrix or one sequence of a batch is addressed.
- *   - tensors are f32, row-major; ids / targets are int32 with -1 as the ignore marker.
+ *   - tensors are f32, row-major; ids / targets are int32 with -1 as the ignore marker. They are device buffers,
+ *     so their range cannot be checked before a launch: it is a precondition of each entry point that takes them, and
+ *     a kernel that meets a value outside it skips that row instead of indexing with it; gt_sync, gt_d2h and
+ *     gt_prof_end then return an error once ("... is outside [0, V): that row was skipped").
  *   - "acc" arguments: 0 = the kernel stores its result (the destination need not be cleared),
  *     1 = it adds to what the destination holds. The reference zeroes every gradient buffer and
  *     always adds (src/backend/webgpu.ts:21-26, 1397-1429); a host that knows a gradient's first
@@ -145,8 +148,12 @@ int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, g
 int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
                         gt_buf dw, int acc_dw);
 
-/* ---- embedding: srcEmbeddingFwd / Bwd (wgsl.ts:305-344) ------------------------------------- */
-int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, gt_buf ids, gt_buf W, gt_buf out);
+/* ---- embedding: srcEmbeddingFwd / Bwd (wgsl.ts:305-344) -------------------------------------
+ * Precondition: every id is in [0, V) (the reference checks this above the dispatch, autograd.ts:324-346; ids live on
+ * the device here, so the library cannot look before it launches). A kernel that meets an id outside the range does not
+ * touch memory for it: the forward writes a zero row, the backward adds nothing, and the next gt_sync / gt_d2h /
+ * gt_prof_end fails once, naming the row and the id. */
+int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf W, gt_buf out);
 int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, gt_buf dW, int acc);
 
 /* ---- RoPE: srcRope (wgsl.ts:346-384), NeoX pairing (j, j+hd/2); position of row r is
@@ -179,7 +186,11 @@ int gt_attn_bwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int w
  * max(kept_s, 1) (autograd.ts:938), passed as inv_denom[s] = 1/denominator (f32, device).
  * fwd writes loss[s] = inv_denom[s] * sum over kept rows of (logsumexp - z_target) and lse[rows].
  * bwd: dlogits[r,:] (+)= seed * inv_denom[s] * (softmax - onehot); ignored rows get 0 (acc = 0)
- * or are left alone (acc = 1). */
+ * or are left alone (acc = 1).
+ * Precondition: every target is -1 or in [0, V) (checked above the dispatch in the reference, autograd.ts:875-894).
+ * A target outside that range is never used as an index: gt_ce_fwd counts the row as ignored and the next gt_sync /
+ * gt_d2h / gt_prof_end fails once, naming the row; the chunked kernels and gt_ce_bwd only compare targets with column
+ * numbers. */
 int gt_ce_fwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets, gt_buf inv_denom,
               gt_buf loss, gt_buf lse);
 int gt_ce_bwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets, gt_buf inv_denom,
@@ -192,7 +203,9 @@ int gt_ce_loss_from_stats(gt_ctx *ctx, int rows, int T, gt_buf targets, gt_buf i
                           gt_buf row_max, gt_buf row_sum, gt_buf tgt_logit, gt_buf loss);
 int gt_ce_chunk_grad(gt_ctx *ctx, int rows, int vc, int v0, int T, gt_buf chunk, gt_buf targets,
                      gt_buf inv_denom, gt_buf row_max, gt_buf row_sum, float seed);
-/* sparse-teacher soft CE: srcSoftCeFwd / BwdP / BwdQ (wgsl.ts:1004-1110), webgpu.ts:1331-1378 */
+/* sparse-teacher soft CE: srcSoftCeFwd / BwdP / BwdQ (wgsl.ts:1004-1110), webgpu.ts:1331-1378. teacher_ids[rows*k]:
+ * a row whose first id is -1 is ignored; every other id must be in [0, V) (autograd.ts:974-998 checks it above the
+ * dispatch). An id outside the range is skipped by both kernels and reported by the next gt_sync / gt_d2h / gt_prof_end. */
 int gt_soft_ce_fwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf teacher_ids, gt_buf teacher_probs,
                    float inv_denom, gt_buf loss, gt_buf lse, gt_buf row_mass);
 int gt_soft_ce_bwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf teacher_ids, gt_buf teacher_probs,

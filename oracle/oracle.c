@@ -133,21 +133,39 @@ void or_linear_bwd(const float *x, const float *w, const float *gout, float *gx,
  * or_linear_bwd and a float64 product (tests/test_oracle_torch64.py). */
 void or_linear_bwd_dots(const float *x, const float *w, const float *gout, float *gx, float *gw,
                         int T, int in, int outd) {
+  /* Each output element sums its terms in ascending o (gx) or ascending t (gw) in
+   * a double; the loops are interchanged so that memory is walked along rows. */
+  enum { CH = 512 };
   OR_PAR
   for (int t = 0; t < T; t++) {
-    for (int i = 0; i < in; i++) {
-      double acc = 0;
-      for (int o = 0; o < outd; o++) acc += D(gout[(size_t)t * outd + o]) * D(w[(size_t)o * in + i]);
-      gx[(size_t)t * in + i] = (float)(D(gx[(size_t)t * in + i]) + acc);
+    const float *gr = gout + (size_t)t * outd;
+    for (int i0 = 0; i0 < in; i0 += CH) {
+      int n = in - i0 < CH ? in - i0 : CH;
+      double acc[CH];
+      for (int i = 0; i < n; i++) acc[i] = 0;
+      for (int o = 0; o < outd; o++) {
+        double g = gr[o];
+        const float *wr = w + (size_t)o * in + i0;
+        for (int i = 0; i < n; i++) acc[i] += g * D(wr[i]);
+      }
+      float *gxr = gx + (size_t)t * in + i0;
+      for (int i = 0; i < n; i++) gxr[i] = (float)(D(gxr[i]) + acc[i]);
     }
   }
   if (!gw) return;
   OR_PAR
   for (int o = 0; o < outd; o++) {
-    for (int i = 0; i < in; i++) {
-      double acc = 0;
-      for (int t = 0; t < T; t++) acc += D(gout[(size_t)t * outd + o]) * D(x[(size_t)t * in + i]);
-      gw[(size_t)o * in + i] = (float)(D(gw[(size_t)o * in + i]) + acc);
+    for (int i0 = 0; i0 < in; i0 += CH) {
+      int n = in - i0 < CH ? in - i0 : CH;
+      double acc[CH];
+      for (int i = 0; i < n; i++) acc[i] = 0;
+      for (int t = 0; t < T; t++) {
+        double g = gout[(size_t)t * outd + o];
+        const float *xr = x + (size_t)t * in + i0;
+        for (int i = 0; i < n; i++) acc[i] += g * D(xr[i]);
+      }
+      float *gwr = gw + (size_t)o * in + i0;
+      for (int i = 0; i < n; i++) gwr[i] = (float)(D(gwr[i]) + acc[i]);
     }
   }
 }
