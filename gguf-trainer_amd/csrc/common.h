@@ -41,6 +41,7 @@ struct gt_ctx {
   // Pinned host words a kernel writes when it meets an id / target outside its range (it skips that row):
   // [0] = which check (GT_BAD_*), [1] = row, [2] = the value, [3] = the bound. Read after the stream has drained.
   int *bad_host = nullptr, *bad_dev = nullptr;
+  float *rms_static = nullptr;                  // this device's address of norm.hip's static scratch array
   struct ProfSeen { int64_t n = 0; double work = 0; };
   std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not
 };
@@ -64,6 +65,7 @@ __device__ __forceinline__ void note_bad_id(int *bad, int what, int64_t row, int
   bad[1] = (int)row; bad[2] = value; bad[3] = bound; bad[0] = what;
 }
 int gt_report_bad_id(gt_ctx *ctx);
+int rmsnorm_static_init(gt_ctx *ctx);           // norm.hip: looks up the static scratch array's address on ctx's device
 // gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
 int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc);
 

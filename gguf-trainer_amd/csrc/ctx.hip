@@ -44,6 +44,13 @@ int gt_ctx_create(int device, gt_ctx **out) {
     return 1;
   }
   memset(c->bad_host, 0, 4 * sizeof(int));
+  if (rmsnorm_static_init(c)) {
+    snprintf(g_create_err, sizeof g_create_err, "context setup failed: %s", c->err);
+    hipHostFree(c->bad_host);
+    hipStreamDestroy(c->stream);
+    delete c;
+    return 1;
+  }
   *out = c;
   return 0;
 }

@@ -219,9 +219,24 @@ __global__ __launch_bounds__(256) void rmsnorm_dw_gen(int rows, int d, int slab,
   part[(size_t)blockIdx.y * d + c] = s;
 }
 
+// Scratch of gt_rmsnorm_bwd_static, the entry point that allocates nothing: the per-workgroup dw partial rows, at most
+// two workgroups per CU of up to RMS_STATIC_MAX_D columns. Every GPU the library runs on holds its own copy until the
+// process ends. In host code the name is only a handle for hipGetSymbolAddress; kernels get the address it returns.
+#define RMS_STATIC_MAX_D 2048
+#define RMS_STATIC_FLOATS (512 * RMS_STATIC_MAX_D)          // 4 MiB
+static __device__ __align__(256) float scratch[RMS_STATIC_FLOATS];
+
+int rmsnorm_static_init(gt_ctx *ctx) {
+  void *ptr = nullptr;
+  GT_HIP(ctx, hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));      // this device's copy: the context's device is current
+  GT_REQUIRE(ctx, ptr != nullptr, "hipGetSymbolAddress gave a null address for the static scratch array");
+  ctx->rms_static = static_cast<float *>(ptr);
+  return 0;
+}
+
 template <int LPR, int NJ>
 static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
-                       gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw) {
+                       gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw, float *static_part = nullptr) {
   constexpr int RPB = 4 * (WAVE / LPR);
   int64_t nb = std::min<int64_t>(cdiv(rows, RPB), (int64_t)ctx->num_cu * 2);
   if (!bwd) {
@@ -231,7 +246,11 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
     return 0;
   }
   float *part = nullptr;
-  if (dw) {
+  if (dw && static_part) {
+    GT_REQUIRE(ctx, (size_t)nb * d <= RMS_STATIC_FLOATS, "rmsnorm backward: %lld partial rows of %d columns exceed the static scratch",
+               (long long)nb, d);
+    part = static_part;
+  } else if (dw) {
     void *ws;
     if (gt_ws_reserve(ctx, (size_t)nb * d * sizeof(float), &ws)) return 1;
     part = static_cast<float *>(ws);
@@ -250,11 +269,11 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
 }
 
 static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
-                    gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw) {
+                    gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw, float *static_part = nullptr) {
   bool aligned = (x | w | y_or_g | dx | dx_old) % 16 == 0;
   int d4 = d / 4;
-#define FAST(LPR, NJ) return launch_fast<LPR, NJ>(ctx, bwd, rows, d, eps, x, w, y_or_g, rinv, dx, acc_dx, dx_old, dw, acc_dw)
-  if (d % 4 == 0 && aligned && d <= 2048) {
+#define FAST(LPR, NJ) return launch_fast<LPR, NJ>(ctx, bwd, rows, d, eps, x, w, y_or_g, rinv, dx, acc_dx, dx_old, dw, acc_dw, static_part)
+  if (d % 4 == 0 && aligned && d <= RMS_STATIC_MAX_D) {
     if (d4 <= 16) FAST(16, 1);
     if (d4 <= 32) FAST(32, 1);
     if (d4 <= 64) FAST(64, 1);
@@ -264,6 +283,8 @@ static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x,
     FAST(64, 8);
   }
 #undef FAST
+  GT_REQUIRE(ctx, !static_part, "gt_rmsnorm_bwd_static: d = %d must be a multiple of 4, at most %d, and every operand 16-byte aligned",
+             d, RMS_STATIC_MAX_D);
   unsigned nb = (unsigned)cdiv(rows, 4);
   if (!bwd) {
     hipLaunchKernelGGL(rmsnorm_fwd_gen, dim3(nb), dim3(256), 0, ctx->stream, rows, d, eps, P<const float>(x),
@@ -306,6 +327,27 @@ int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, g
   }
   ProfScope ps(ctx, "rmsnorm.bwd", 12.0 * rows * d);   // read x, g; write dx
   return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dx, dw, acc_dw);
+}
+__global__ __launch_bounds__(256) void fill_zero_k(int n, float *p) {
+  int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+// gt_rmsnorm_bwd for callers that cannot allocate: the same kernels with the dw partials in the static array above.
+// No hipMalloc, no workspace growth, no profiling events, no memset node (a fill kernel clears dw for rows = 0).
+int gt_rmsnorm_bwd_static(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx, int acc_dx,
+                          gt_buf dw, int acc_dw) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && d >= 1 && x && w && g && rinv && dx, "gt_rmsnorm_bwd_static: bad arguments (rows %d, d %d)", rows, d);
+  GT_REQUIRE(ctx, d <= RMS_STATIC_MAX_D, "gt_rmsnorm_bwd_static: d = %d is more than the static scratch is sized for (%d)", d, RMS_STATIC_MAX_D);
+  GT_REQUIRE(ctx, ctx->rms_static, "gt_rmsnorm_bwd_static: the static scratch array has no device address");
+  if (rows == 0) {
+    if (dw && !acc_dw) {
+      hipLaunchKernelGGL(fill_zero_k, dim3((unsigned)cdiv(d, 256)), dim3(256), 0, ctx->stream, d, P<float>(dw));
+      GT_LAUNCHED(ctx);
+    }
+    return 0;
+  }
+  return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dx, dw, acc_dw, ctx->rms_static);
 }
 int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
                         gt_buf dw, int acc_dw) {

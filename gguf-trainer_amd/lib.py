@@ -59,6 +59,7 @@ _SIG = {
     "gt_glu_bwd": [ctxp, i32, i64, buf, buf, buf, buf, i32, buf, i32],
     "gt_rmsnorm_fwd": [ctxp, i32, i32, f32, buf, buf, buf, buf],
     "gt_rmsnorm_bwd": [ctxp, i32, i32, buf, buf, buf, buf, buf, i32, buf, i32],
+    "gt_rmsnorm_bwd_static": [ctxp, i32, i32, buf, buf, buf, buf, buf, i32, buf, i32],
     "gt_rmsnorm_bwd_from": [ctxp, i32, i32, buf, buf, buf, buf, buf, buf, buf, i32],
     "gt_embedding_fwd": [ctxp, i32, i32, i32, buf, buf, buf],
     "gt_embedding_bwd": [ctxp, i32, i32, i32, buf, buf, buf, i32],

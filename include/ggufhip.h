@@ -148,6 +148,17 @@ int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, g
 int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
                         gt_buf dw, int acc_dw);
 
+/* gt_rmsnorm_bwd for callers that cannot allocate device memory: code under HIP graph capture, tight loops of a serving
+ * process, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments and bit-identical
+ * results; the per-workgroup dw partials go to a 4 MiB array that is part of the library's code object (one copy per GPU,
+ * held until the process ends) instead of the context's grow-only workspace, and the call makes no hipMalloc / hipFree,
+ * creates no events (it is not seen by gt_prof_begin / gt_prof_end) and records no memset node. Limits: d a multiple of
+ * 4 and at most 2048, every operand 16-byte aligned; anything else is refused with an error. All calls on one GPU share
+ * that GPU's array: two calls that overlap in time on one GPU (two contexts, i.e. two streams) race on it; calls on one
+ * context are ordered by its stream. */
+int gt_rmsnorm_bwd_static(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv,
+                          gt_buf dx, int acc_dx, gt_buf dw, int acc_dw);
+
 /* ---- embedding: srcEmbeddingFwd / Bwd (wgsl.ts:305-344) -------------------------------------
  * Precondition: every id is in [0, V) (the reference checks this above the dispatch, autograd.ts:324-346; ids live on
  * the device here, so the library cannot look before it launches). A kernel that meets an id outside the range does not
