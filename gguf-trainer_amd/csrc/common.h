@@ -31,6 +31,7 @@ struct gt_ctx {
     if (T != o.T) return T < o.T; if (hd != o.hd) return hd < o.hd; if (pos != o.pos) return pos < o.pos; return base < o.base; } };
   std::map<RopeKey, float *> rope_tables;
   int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1, opt_gemm_staged = 0;
+  int opt_gemm_group = 1;                       // 0: gt_gemm_group launches its products one by one
   int opt_attn_keep_ds = 1, opt_attn_ds_limit_mb = 8192, opt_gemm_sum_min_tiles = -1;
   bool prof_on = false;
   std::string prof_prefix;

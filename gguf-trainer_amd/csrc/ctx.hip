@@ -5,6 +5,13 @@ thread_local char g_create_err[512] = {0};
 
 extern "C" {
 
+static void ctx_release(gt_ctx *c) {
+  if (c->ws) hipFree(c->ws);
+  if (c->bad_host) hipHostFree(c->bad_host);
+  if (c->stream) hipStreamDestroy(c->stream);
+  delete c;
+}
+
 int gt_ctx_create(int device, gt_ctx **out) {
   if (!out) return 1;
   *out = nullptr;
@@ -21,34 +28,30 @@ int gt_ctx_create(int device, gt_ctx **out) {
   gt_ctx *c = new gt_ctx();
   c->device = device;
   hipDeviceProp_t p;
-  if ((e = hipSetDevice(device)) != hipSuccess || (e = hipGetDeviceProperties(&p, device)) != hipSuccess ||
-      (e = hipStreamCreate(&c->stream)) != hipSuccess) {
+  if ((e = hipSetDevice(device)) != hipSuccess || (e = hipGetDeviceProperties(&p, device)) != hipSuccess) {
     snprintf(g_create_err, sizeof g_create_err, "context setup failed: %s", hipGetErrorString(e));
-    delete c;
+    ctx_release(c);
     return 1;
   }
   snprintf(c->name, sizeof c->name, "%s (%s, %d CUs)", p.name, p.gcnArchName, p.multiProcessorCount);
   c->num_cu = p.multiProcessorCount;
   if (strncmp(p.gcnArchName, "gfx950", 6) != 0) {
     snprintf(g_create_err, sizeof g_create_err, "libggufhip is built for gfx950 only; device is %s", p.gcnArchName);
-    hipStreamDestroy(c->stream);
-    delete c;
+    ctx_release(c);
     return 1;
   }
-  if ((e = hipHostMalloc(reinterpret_cast<void **>(&c->bad_host), 4 * sizeof(int), hipHostMallocMapped)) != hipSuccess ||
+  // the stream, and the pinned words kernels note an out-of-range id in
+  if ((e = hipStreamCreate(&c->stream)) != hipSuccess ||
+      (e = hipHostMalloc(reinterpret_cast<void **>(&c->bad_host), 4 * sizeof(int), hipHostMallocMapped)) != hipSuccess ||
       (e = hipHostGetDevicePointer(reinterpret_cast<void **>(&c->bad_dev), c->bad_host, 0)) != hipSuccess) {
     snprintf(g_create_err, sizeof g_create_err, "context setup failed: %s", hipGetErrorString(e));
-    if (c->bad_host) hipHostFree(c->bad_host);
-    hipStreamDestroy(c->stream);
-    delete c;
+    ctx_release(c);
     return 1;
   }
   memset(c->bad_host, 0, 4 * sizeof(int));
   if (rmsnorm_static_init(c)) {
     snprintf(g_create_err, sizeof g_create_err, "context setup failed: %s", c->err);
-    hipHostFree(c->bad_host);
-    hipStreamDestroy(c->stream);
-    delete c;
+    ctx_release(c);
     return 1;
   }
   *out = c;
@@ -61,11 +64,8 @@ int gt_ctx_destroy(gt_ctx *ctx) {
   hipStreamSynchronize(ctx->stream);
   for (auto &kv : ctx->allocs) hipFree(reinterpret_cast<void *>(kv.first));
   for (auto &kv : ctx->rope_tables) hipFree(kv.second);
-  if (ctx->ws) hipFree(ctx->ws);
-  if (ctx->bad_host) hipHostFree(ctx->bad_host);
   for (auto &e : ctx->prof) { hipEventDestroy(e.a); hipEventDestroy(e.b); }
-  hipStreamDestroy(ctx->stream);
-  delete ctx;
+  ctx_release(ctx);
   return 0;
 }
 
@@ -150,6 +150,7 @@ int gt_set_option(gt_ctx *ctx, const char *key, int value) {
   else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
   else if (!strcmp(key, "gemm.splitk")) ctx->opt_gemm_splitk = value;
   else if (!strcmp(key, "gemm.staged")) ctx->opt_gemm_staged = value;
+  else if (!strcmp(key, "gemm.group")) ctx->opt_gemm_group = value;
   else if (!strcmp(key, "gemm.sum_min_tiles")) ctx->opt_gemm_sum_min_tiles = value;
   else GT_FAIL(ctx, "gt_set_option: unknown key '%s'", key);
   return 0;

@@ -350,8 +350,9 @@ struct DirectTile {
   }
 };
 
+// The work of one workgroup on output tile (pm, pn) and K split or batch member z
 template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2, bool BAND = false, bool MSEG = false>
-__global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
+__device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm, const int pn, const int z) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   using TA = DirectTile<BM, KIND != GT_TN, NT, BK>;
@@ -360,17 +361,6 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
   constexpr int STAGE = (TA::CH + TB::CH) * 4;                // floats per stage
   if (a.M < 0) smem[threadIdx.x] = 0.f;                       // never taken: keeps the LDS array "written" for the compiler
 
-  int pm, pn, z;
-  if (BAND) {
-    // Row tiles differ in K range (128 ... T keys). The grid is (batch members, 1, row tiles): dispatch order runs over
-    // the batch members of the longest row tile first, then the next shorter one, so the long workgroups start first and
-    // the short ones fill the gaps at the end, and the 8 XCDs (fed round-robin in dispatch order) get equal lengths.
-    z = blockIdx.x;
-    pn = blockIdx.z % a.nbn;
-    pm = a.nbm - 1 - (int)(blockIdx.z / a.nbn);
-  } else {
-    tile_of_workgroup(a, pm, pn, z);
-  }
   const int m0 = pm * BM, n0 = pn * BN;
   const float *A = a.A, *B = a.B;
   int k0 = 0, kend = a.K;
@@ -532,6 +522,62 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
     }
 }
 
+template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2, bool BAND = false, bool MSEG = false>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
+  int pm, pn, z;
+  if (BAND) {
+    // Row tiles differ in K range (128 ... T keys). The grid is (batch members, 1, row tiles): dispatch order runs over
+    // the batch members of the longest row tile first, then the next shorter one, so the long workgroups start first and
+    // the short ones fill the gaps at the end, and the 8 XCDs (fed round-robin in dispatch order) get equal lengths.
+    z = blockIdx.x;
+    pn = blockIdx.z % a.nbn;
+    pm = a.nbm - 1 - (int)(blockIdx.z / a.nbn);
+  } else {
+    tile_of_workgroup(a, pm, pn, z);
+  }
+  gemm_direct_tile<BM, BN, WM, WN, KIND, BK, NSTG, SEG2, BAND, MSEG>(a, pm, pn, z);
+}
+
+// Several independent TN products with the same K in one launch: the weight gradients dW_i = dY_i^T . X_i of consecutive
+// linears of a layer, whose outputs are too small to fill the chip one at a time. The output tiles of all problems form
+// one list (problem after problem, N fastest inside a problem); with K splits the (split, tile) pairs are numbered
+// split-major and dealt to the XCDs in contiguous ranges, exactly as for a single product. A workgroup looks up its
+// problem, points the argument block at that problem's operands, and runs the ordinary tile loop.
+#define GT_GROUP_MAX 8
+struct GroupProb { const float *A, *B; float *C; int M, N, acc, tile0, nbn; int64_t e0; };   // e0: elements of the problems before it
+struct GroupArgs { GroupProb p[GT_GROUP_MAX]; int n, ntiles; };
+
+template <int BM, int BN, int WM, int WN, int BK, int NSTG>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_group_tn(GemmArgs a, GroupArgs g) {
+  const int total = g.ntiles * a.splits, lin = blockIdx.x;
+  const int xcd = lin % 8, idx = lin / 8, base = total / 8, rem = total % 8;
+  const int w = xcd * base + (xcd < rem ? xcd : rem) + idx;
+  const int z = w / g.ntiles, pid = w % g.ntiles;
+  int i = 0;
+#pragma unroll
+  for (int q = 1; q < GT_GROUP_MAX; q++) if (q < g.n && pid >= g.p[q].tile0) i = q;
+  const GroupProb &p = g.p[i];
+  const int lp = pid - p.tile0;
+  a.A = p.A; a.B = p.B; a.C = p.C;
+  a.M = p.M; a.N = p.N; a.lda = p.M; a.ldb = p.N; a.ldc = p.N; a.acc = p.acc;
+  a.Pp += (size_t)a.splits * p.e0;
+  gemm_direct_tile<BM, BN, WM, WN, GT_TN, BK, NSTG, false>(a, lp / p.nbn, lp % p.nbn, z);
+}
+// C_i (+)= sum over splits of the group's partials, in split order; one thread per output element of the whole group
+__global__ __launch_bounds__(256) void group_reduce(GroupArgs g, const float *__restrict__ Pp, int64_t total, int splits) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  int i = 0;
+#pragma unroll
+  for (int q = 1; q < GT_GROUP_MAX; q++) if (q < g.n && e >= g.p[q].e0) i = q;
+  const GroupProb &p = g.p[i];
+  const int64_t n = (int64_t)p.M * p.N, l = e - p.e0;
+  const float *pp = Pp + (size_t)splits * p.e0 + l;
+  float s = pp[0];
+  for (int z = 1; z < splits; z++) s += pp[(size_t)z * n];
+  p.C[l] = p.acc ? p.C[l] + s : s;
+}
+
 template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2>
 static int launch_direct_kind(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   constexpr int smem = NSTG * (BM + BN) * BK * 4;
@@ -601,6 +647,54 @@ static const TileCfg kTiles[] = {{64, 64, 16}, {128, 64, 16}, {128, 128, 16}, {1
                                  {128, 128, 32}, {128, 192, 32}, {128, 96, 32}, {256, 128, 32}, {64, 192, 16}, {128, 64, 32}, {64, 192, 32}};
 #define NCFG ((int)(sizeof(kTiles) / sizeof(kTiles[0])))
 
+// Tile and split-K choice by a small cost model over the tile shapes that measured best on MI355X:
+// time ~ flops / (tile efficiency x edge utilisation x wave quantisation) + the cost of the split-K reduction pass,
+// for one product (batched `count` times) or a group of `np` products with a common K launched together.
+struct Cand { int cfg; double eff; };
+static void pick_tile(gt_ctx *ctx, int kind, bool direct_ok, int np, const int *Ms, const int *Ns, int K, int count, bool two_seg,
+                      int *cfg_out, int *splits_out, int fixed_splits = 0) {
+  // relative tile efficiencies as measured (asymptotic rate of each tile over the best one's)
+  static const Cand cand_nn[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
+  static const Cand cand_tn[] = {{8, 1.00}, {11, 0.99}, {10, 0.92}, {6, 0.90}, {7, 0.78}, {0, 0.72}};
+  static const Cand cand_nn_direct[] = {{7, 1.00}, {8, 1.00}, {6, 0.98}, {12, 0.97}, {11, 0.92}, {10, 0.85}, {0, 0.72}};
+  static const Cand cand_tn_direct[] = {{8, 1.00}, {12, 1.00}, {7, 0.98}, {11, 0.96}, {6, 0.88}, {10, 0.85}, {0, 0.68}};
+  const Cand *cand = direct_ok ? (kind == GT_TN ? cand_tn_direct : cand_nn_direct) : (kind == GT_TN ? cand_tn : cand_nn);
+  const int ncand = direct_ok ? 7 : 6;
+  int cfg = 0, splits = 1;
+  double elems = 0;
+  for (int i = 0; i < np; i++) elems += (double)Ms[i] * Ns[i];
+  const double flops = 2.0 * elems * K * count;
+  const double t0 = flops / (direct_ok ? 132e12 : 125e12);   // seconds at the best tile's asymptotic rate
+  double best = 1e30;
+  for (int ci = 0; ci < ncand; ci++) {
+    const Cand &c = cand[ci];
+    const TileCfg &tc = kTiles[c.cfg];
+    if (np > 1 && !(c.cfg == 6 || c.cfg == 7 || c.cfg == 8 || c.cfg == 11 || c.cfg == 12)) continue;   // group launches: direct tiles only
+    int64_t tiles = 0;
+    for (int i = 0; i < np; i++) tiles += cdiv(Ms[i], tc.bm) * cdiv(Ns[i], tc.bn);
+    const double util = elems / ((double)tiles * tc.bm * tc.bn);
+    // any split count, not only powers of two: 72 output tiles x 14 splits is 3.94 workgroups per CU, x 16 is 4.5,
+    // and with workgroups of equal length the CUs that get the fifth one set the time
+    for (int sp = fixed_splits > 0 ? fixed_splits : 1; sp <= (fixed_splits > 0 ? fixed_splits : 64); sp++) {
+      // split only when the output tiles alone cannot give every CU a workgroup (a group's split count is given)
+      if (!fixed_splits && sp > 1 && (count > 1 || two_seg || tiles >= ctx->num_cu || K / sp < 8 * tc.bk)) break;
+      const double waves = (double)tiles * sp * count / ctx->num_cu;
+      const double quant = waves / ceil(waves);
+      // a CU with few workgroups over the whole launch overlaps their fills and write-backs less (fitted on the
+      // dW shapes: 1 workgroup per CU runs 15 % and 2 run 6 % below the rate reached from 4 per CU on)
+      const double conc = std::min(1.0, 1.0625 * waves / (waves + 0.25));
+      // short K per workgroup pays the prologue/epilogue more: ~2 K-steps of overhead
+      const double ksteps = (double)K / sp / tc.bk;
+      const double depth = ksteps / (ksteps + 2.0);
+      double t = t0 / (c.eff * util * quant * depth * conc);
+      if (sp > 1) t += ((double)(sp + 2) * elems * 4.0) / 3.5e12 + 4e-6;
+      if (t < best) { best = t; cfg = c.cfg; splits = sp; }
+    }
+  }
+  *cfg_out = cfg;
+  *splits_out = splits;
+}
+
 static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
                      gt_buf C, int64_t sC, int count, int K2 = 0, gt_buf A2 = 0, gt_buf B2 = 0, gt_buf D = 0) {
   GT_ENTER(ctx);
@@ -624,52 +718,15 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   a.ldb2 = (kind == GT_NT) ? K2 : N;
   if (K2 > 0) vec = vec && (a.lda2 % 4 == 0) && (a.ldb2 % 4 == 0) && (A2 % 16 == 0) && (B2 % 16 == 0);
 
-  // Tile and split-K choice by a small cost model over the tile shapes that measured best on
-  // MI355X: time ~ flops / (tile efficiency x edge utilisation x wave quantisation) + the cost of
-  // the split-K reduction pass. N = 576 (SmolLM2) is 3x192 = 6x96; dW has a 1536x576 output and
+  // Tile and split-K choice: pick_tile. N = 576 (SmolLM2) is 3x192 = 6x96; dW has a 1536x576 output and
   // K = 16384 rows, which only fills 256 CUs when K is split.
-  // relative tile efficiencies as measured (asymptotic rate of each tile over the best one's)
   // Tiles with a K step of 32 have a variant that loads operands straight into LDS (gemm_direct); it wants whole K
   // steps and whole 16-byte chunks along the contiguous index of every operand. Where it applies it is 2-8 % faster
   // than the register-staged kernel of the same tile and changes which tile is best, hence two tables.
   const bool direct_ok = vec && K % 32 == 0 && (kind != GT_TN || (M % 4 == 0 && M >= 4)) && (kind == GT_NT || (N % 4 == 0 && N >= 4)) &&
                          (K2 == 0 || (kind != GT_TN && K2 % 8 == 0 && K2 <= 32));   // a short second segment rides in one more stage
-  struct Cand { int cfg; double eff; };
-  static const Cand cand_nn[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
-  static const Cand cand_tn[] = {{8, 1.00}, {11, 0.99}, {10, 0.92}, {6, 0.90}, {7, 0.78}, {0, 0.72}};
-  static const Cand cand_nn_direct[] = {{7, 1.00}, {8, 1.00}, {6, 0.98}, {12, 0.97}, {11, 0.92}, {10, 0.85}, {0, 0.72}};
-  static const Cand cand_tn_direct[] = {{8, 1.00}, {12, 1.00}, {7, 0.98}, {11, 0.96}, {6, 0.88}, {10, 0.85}, {0, 0.68}};
-  const Cand *cand = direct_ok ? (kind == GT_TN ? cand_tn_direct : cand_nn_direct) : (kind == GT_TN ? cand_tn : cand_nn);
-  const int ncand = direct_ok ? 7 : 6;
   int cfg = 0, splits = 1;
-  {
-    const double flops = 2.0 * M * N * K * count;
-    const double t0 = flops / (direct_ok ? 132e12 : 125e12);   // seconds at the best tile's asymptotic rate
-    double best = 1e30;
-    for (int ci = 0; ci < ncand; ci++) {
-      const Cand &c = cand[ci];
-      const TileCfg &tc = kTiles[c.cfg];
-      const int64_t tiles = cdiv(M, tc.bm) * cdiv(N, tc.bn);
-      const double util = (double)M * N / ((double)tiles * tc.bm * tc.bn);
-      // any split count, not only powers of two: 72 output tiles x 14 splits is 3.94 workgroups per CU, x 16 is 4.5,
-      // and with workgroups of equal length the CUs that get the fifth one set the time
-      for (int sp = 1; sp <= 64; sp++) {
-        // split only when the output tiles alone cannot give every CU a workgroup
-        if (sp > 1 && (count > 1 || K2 > 0 || tiles >= ctx->num_cu || K / sp < 8 * tc.bk)) break;
-        const double waves = (double)tiles * sp * count / ctx->num_cu;
-        const double quant = waves / ceil(waves);
-        // a CU with few workgroups over the whole launch overlaps their fills and write-backs less (fitted on the
-        // dW shapes: 1 workgroup per CU runs 15 % and 2 run 6 % below the rate reached from 4 per CU on)
-        const double conc = std::min(1.0, 1.0625 * waves / (waves + 0.25));
-        // short K per workgroup pays the prologue/epilogue more: ~2 K-steps of overhead
-        const double ksteps = (double)K / sp / tc.bk;
-        const double depth = ksteps / (ksteps + 2.0);
-        double t = t0 / (c.eff * util * quant * depth * conc);
-        if (sp > 1) t += ((double)(sp + 2) * M * N * 4.0) / 3.5e12 + 4e-6;
-        if (t < best) { best = t; cfg = c.cfg; splits = sp; }
-      }
-    }
-  }
+  pick_tile(ctx, kind, direct_ok, 1, &M, &N, K, count, K2 > 0, &cfg, &splits);
   if (ctx->opt_gemm_tile >= 0 && ctx->opt_gemm_tile < NCFG) cfg = ctx->opt_gemm_tile;
   const int bm = kTiles[cfg].bm, bn = kTiles[cfg].bn, bk = kTiles[cfg].bk;
   if (count == 1 && K2 == 0 && ctx->opt_gemm_splitk >= 1) splits = ctx->opt_gemm_splitk;
@@ -769,6 +826,101 @@ static int launch_multi(gt_ctx *ctx, GemmArgs &a, int slot) {
                      ctx->stream, a);
   GT_LAUNCHED(ctx);
   return 0;
+}
+
+template <int BM, int BN, int WM, int WN>
+static int launch_group(gt_ctx *ctx, GemmArgs &a, GroupArgs &g, int slot) {
+  constexpr int BK = 32, NSTG = 2, smem = NSTG * (BM + BN) * BK * 4;
+  if (!(ctx->gemm_direct_set & (1ull << slot))) {
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_group_tn<BM, BN, WM, WN, BK, NSTG>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    ctx->gemm_direct_set |= 1ull << slot;
+  }
+  int tiles = 0;
+  for (int i = 0; i < g.n; i++) {
+    g.p[i].tile0 = tiles;
+    g.p[i].nbn = (int)cdiv(g.p[i].N, BN);
+    tiles += (int)cdiv(g.p[i].M, BM) * g.p[i].nbn;
+  }
+  g.ntiles = tiles;
+  hipLaunchKernelGGL((gemm_group_tn<BM, BN, WM, WN, BK, NSTG>), dim3((unsigned)tiles * a.splits), dim3(WM * WN * 64), smem, ctx->stream, a, g);
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+extern "C" {
+int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, int K, const gt_buf *A, const gt_buf *B,
+                  const gt_buf *C, const int *acc) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, kind >= 0 && kind <= 2 && count >= 1 && M && N && A && B && C && acc && K >= 1,
+             "gt_gemm_group: kind %d, %d products, K %d, or a null table", kind, count, K);
+  // What a product's result is, bit for bit, must not depend on which other products it shares a launch with (the host
+  // groups what happens to be pending: with and without recomputed regions those are different sets). The tile shape
+  // does not enter the arithmetic of an output element (every direct tile walks K in the same order); the K split does.
+  // So the split is a function of K alone: ranges of max(512, K/8) rows, at most eight partials per output. A product
+  // that fills the chip on its own (at least one 128 x 96 tile per CU) is not split and goes as its own launch.
+  const int64_t big = (int64_t)ctx->num_cu * 128 * 96;
+  int idx[GT_GROUP_MAX], ng = 0;
+  bool eligible = kind == GT_TN && K % 32 == 0 && !ctx->opt_gemm_staged && ctx->opt_gemm_group;
+  for (int i = 0; i < count; i++) {
+    GT_REQUIRE(ctx, M[i] >= 1 && N[i] >= 1 && A[i] && B[i] && C[i], "gt_gemm_group: product %d has M %d, N %d or a null operand", i, M[i], N[i]);
+    for (int j = 0; j < i; j++) GT_REQUIRE(ctx, C[i] != C[j], "gt_gemm_group: products %d and %d write the same output", j, i);
+  }
+  if (count > GT_GROUP_MAX) {
+    for (int i = 0; i < count; i += GT_GROUP_MAX)
+      if (gt_gemm_group(ctx, kind, std::min(GT_GROUP_MAX, count - i), M + i, N + i, K, A + i, B + i, C + i, acc + i)) return 1;
+    return 0;
+  }
+  for (int i = 0; i < count; i++) {
+    const bool fits = eligible && M[i] % 4 == 0 && N[i] % 4 == 0 && (A[i] | B[i] | C[i]) % 16 == 0 && (int64_t)M[i] * N[i] < big;
+    if (fits) idx[ng++] = i;
+    else if (gemm_impl(ctx, kind, acc[i], M[i], N[i], K, A[i], 0, B[i], 0, C[i], 0, 1)) return 1;
+  }
+  if (ng == 0) return 0;
+  GemmArgs a;
+  memset(&a, 0, sizeof a);
+  a.K = K; a.kchunk = K; a.splits = 1; a.zdiv = a.zgroup = 1;
+  GroupArgs g;
+  memset(&g, 0, sizeof g);
+  g.n = ng;
+  int64_t elems = 0;
+  int gm[GT_GROUP_MAX], gn[GT_GROUP_MAX];
+  for (int q = 0; q < ng; q++) {
+    const int i = idx[q];
+    g.p[q].A = P<const float>(A[i]); g.p[q].B = P<const float>(B[i]); g.p[q].C = P<float>(C[i]);
+    g.p[q].M = gm[q] = M[i]; g.p[q].N = gn[q] = N[i]; g.p[q].acc = acc[i]; g.p[q].e0 = elems;
+    elems += (int64_t)M[i] * N[i];
+  }
+  int64_t kc = std::max<int64_t>(512, cdiv(cdiv(K, 8), 32) * 32);
+  if (ctx->opt_gemm_splitk >= 1) kc = cdiv(cdiv(K, ctx->opt_gemm_splitk), 32) * 32;
+  int splits = (int)cdiv(K, kc), cfg = 0, unused = 0;
+  pick_tile(ctx, GT_TN, true, ng, gm, gn, K, 1, false, &cfg, &unused, splits);
+  if (ctx->opt_gemm_tile == 6 || ctx->opt_gemm_tile == 7 || ctx->opt_gemm_tile == 8 || ctx->opt_gemm_tile == 11 || ctx->opt_gemm_tile == 12)
+    cfg = ctx->opt_gemm_tile;
+  if (splits > 1) {
+    a.kchunk = (int)kc;
+    void *ws;
+    if (gt_ws_reserve(ctx, (size_t)splits * elems * sizeof(float), &ws)) return 1;
+    a.splits = splits; a.Pp = static_cast<float *>(ws);
+  }
+  char label[32];
+  snprintf(label, sizeof label, "gemm.tn.group.%dx%d%s", kTiles[cfg].bm, kTiles[cfg].bn, splits > 1 ? ".splitk" : "");
+  ProfScope ps(ctx, label, 2.0 * elems * K);
+  int rc;
+  switch (cfg) {
+    case 6: rc = launch_group<128, 128, 2, 2>(ctx, a, g, 40); break;
+    case 7: rc = launch_group<128, 192, 2, 2>(ctx, a, g, 41); break;
+    case 8: rc = launch_group<128, 96, 4, 1>(ctx, a, g, 42); break;
+    case 11: rc = launch_group<128, 64, 2, 2>(ctx, a, g, 43); break;
+    default: rc = launch_group<64, 192, 2, 2>(ctx, a, g, 44); break;
+  }
+  if (rc) return rc;
+  if (splits > 1) {
+    hipLaunchKernelGGL(group_reduce, dim3((unsigned)cdiv(elems, 256)), dim3(256), 0, ctx->stream, g, a.Pp, elems, splits);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
 }
 
 extern "C" {

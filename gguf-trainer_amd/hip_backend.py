@@ -21,11 +21,12 @@ What differs from the reference, on purpose:
   * Launches are held back where the next op can ride them. A linear's forward waits one op: a second linear of the
     same shape over the same input joins it as a batch of two (k and v, gate and up), an add of its output is written
     by the product's own write-back (the residual add). A linear's input gradient waits until that gradient is next
-    touched: sibling projections then leave as one summed product. add's backward launches nothing where it is the
+    touched: sibling projections then leave as one summed product. A linear's weight gradient waits for up to seven more:
+    consecutive ones leave as one grouped launch. add's backward launches nothing where it is the
     first writer: the operand's gradient points at the upstream buffer until somebody adds to it.
   * attention keeps its raw scores from the forward to the backward where a backward can come and a byte budget allows,
     as the reference's small-T path keeps its probabilities (webgpu.ts:1176-1189).
-  Each of these has a switch (batch_linears, fuse_residual_add, fuse_sibling_dx, alias_add_grads, attn_keep_scores) and
+  Each of these has a switch (batch_linears, fuse_residual_add, fuse_sibling_dx, group_dw, alias_add_grads, attn_keep_scores) and
   gives the same gradients as the one-launch-per-op form: bit for bit, or to rounding where a sum changes its order.
 """
 from __future__ import annotations
@@ -91,6 +92,14 @@ class HipBackend:
         # touches x's gradient next, and every point where buffers can change hands, sends what is held first.
         self._pend_dx: dict = {}
         self.fuse_sibling_dx = True
+        # weight gradients of linears held back in the backward: [(rows, dY, x data, dW, acc, out, in)]. Up to eight
+        # consecutive ones over the same number of rows leave as ONE grouped launch (gt_gemm_group): the dW of a layer's
+        # seven projections are each too small an output to fill the chip, together they are not. Sent when the group is
+        # full, when a weight in it is touched again (its gradient read or written: tied matrices, a weight used twice),
+        # and at every point where buffers can change hands.
+        self._pend_dw: list = []
+        self._pend_dw_ids: set = set()
+        self.group_dw = True
         self.fuse_residual_add = True
         # add's backward hands its upstream gradient on instead of copying it: an operand whose gradient has no writer yet
         # points at the upstream buffer (grad_src). A reader takes that buffer as it is; the first later writer adds to its
@@ -119,8 +128,35 @@ class HipBackend:
             self._pend = None
             check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, p[1], p[2], p[3], p[4], p[5], p[6]), "linear")
 
+    def _flush_dw(self):
+        """Launch the held-back weight-gradient products as one group."""
+        pend = self._pend_dw
+        if not pend:
+            return
+        self._pend_dw = []
+        self._pend_dw_ids = set()
+        n = len(pend)           # a single one goes the same way: its K split must not depend on the company it has
+        ms = (C.c_int * n)(*[p[5] for p in pend])
+        ns = (C.c_int * n)(*[p[6] for p in pend])
+        gs = (c_buf * n)(*[p[1] for p in pend])
+        xs = (c_buf * n)(*[p[2] for p in pend])
+        ds = (c_buf * n)(*[p[3] for p in pend])
+        accs = (C.c_int * n)(*[p[4] for p in pend])
+        check(self._ctx, lib.gt_gemm_group(self._ctx, TN, n, ms, ns, pend[0][0], gs, xs, ds, accs), "linear.dw")
+
+    def _hold_dw(self, w: Tensor, rows, g, xd, dw, accw, outd, ind):
+        if self._pend_dw and self._pend_dw[0][0] != rows:
+            self._flush_dw()
+        self._pend_dw.append((rows, g, xd, dw, accw, outd, ind))
+        self._pend_dw_ids.add(id(w))
+        if len(self._pend_dw) == 8:
+            self._flush_dw()
+
     def _flush_dx(self, t: Tensor = None):
-        """Launch the held-back input-gradient products: those into t's gradient, or all of them."""
+        """Launch the held-back input-gradient products: those into t's gradient, or all of them (then the held-back
+        weight-gradient products go too)."""
+        if t is None and self._pend_dw:
+            self._flush_dw()
         if not self._pend_dx:
             return
         if t is None:
@@ -263,6 +299,8 @@ class HipBackend:
         self._flush()
         if self._pend_dx:
             self._flush_dx(t)       # products held back for this gradient go first: the order of its writers is kept
+        if self._pend_dw and id(t) in self._pend_dw_ids:
+            self._flush_dw()
         e = self._entries.get(t)
         if e is None:
             e = self._entry_for(t)
@@ -318,6 +356,8 @@ class HipBackend:
         self._flush()
         if self._pend_dx:
             self._flush_dx(t)
+        if self._pend_dw and id(t) in self._pend_dw_ids:
+            self._flush_dw()
         e = self._entries.get(t)
         if e is None:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
@@ -357,6 +397,7 @@ class HipBackend:
     def grads_consumed(self, tensors):
         """The optimizer has read these accumulators: the next backward write stores instead of adding
         (the reference's deferred per-step clear, src/backend/muon-gpu.ts:8-16)."""
+        self._flush_dx()
         for t in tensors:
             e = self._entries.get(t)
             if e is not None:
@@ -364,6 +405,8 @@ class HipBackend:
 
     def ensure_grads_defined(self, tensors):
         """An accumulator no kernel wrote since it was last consumed holds zero, as a cleared one would."""
+        self._flush()
+        self._flush_dx()
         for t in tensors:
             e = self._entry_for(t)
             if e.grad == 0:
@@ -493,6 +536,7 @@ class HipBackend:
     def destroy(self):
         self._pend = None
         self._pend_dx = {}
+        self._pend_dw = []
         if not self._destroyed:
             self._destroyed = True
             lib.gt_ctx_destroy(self._ctx)
@@ -587,7 +631,10 @@ class HipBackend:
             if wants_dw:
                 dw, accw = self._gdst(w)
                 if dw:
-                    check(self._ctx, lib.gt_gemm(self._ctx, TN, accw, outd, ind, T, g, xd, dw), "linear.dw")
+                    if self.group_dw:
+                        self._hold_dw(w, T, g, xd, dw, accw, outd, ind)
+                    else:
+                        check(self._ctx, lib.gt_gemm(self._ctx, TN, accw, outd, ind, T, g, xd, dw), "linear.dw")
 
         out._backward = bw
         return out

@@ -42,6 +42,7 @@ _SIG = {
     "gt_set_option": [ctxp, C.c_char_p, i32],
     "gt_gemm": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf],
     "gt_gemm_pair": [ctxp, i32, i32, i32, i32, i32, buf, buf, i32, buf, buf, buf],
+    "gt_gemm_group": [ctxp, i32, i32, C.POINTER(i32), C.POINTER(i32), i32, C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(i32)],
     "gt_gemm_batched": [ctxp, i32, i32, i32, i32, i32, buf, i64, buf, i64, buf, i64, i32],
     "gt_rank_down": [ctxp, i32, i32, i32, buf, buf, i32, f32, buf],
     "gt_rank_grad": [ctxp, i32, i32, i32, buf, buf, i32, i32, buf],

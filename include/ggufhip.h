@@ -66,6 +66,7 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
  *   "attn.generic" 1 = always take the shape-generic attention kernels, 0 = MFMA kernels where they apply
  *   "gemm.tile"    -1 = heuristic, 0..12 = pin the GEMM tile configuration (tests and tuning)
  *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor
+ *   "gemm.group"   1 (default) = gt_gemm_group runs its TN products as one launch; 0 = one launch per product
  *   "gemm.staged"  1 = always stage GEMM operands through registers (0: aligned shapes load straight into LDS)
  *   "gemm.sum_min_tiles" gt_gemm_sum chains its products in one loop from this many 128-row output tiles on
  *                  (-1 = one per CU, the default; 0 = always, for tests of the chained kernel on small shapes)
@@ -112,6 +113,17 @@ int gt_gemm_add(gt_ctx *ctx, int kind, int M, int N, int K, gt_buf A, gt_buf B, 
  * the one before. */
 int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const int *K, const gt_buf *A, const gt_buf *B,
                 gt_buf C);
+/* `count` independent products of one kind with a common K, each with its own M, N, operands, output and acc flag
+ * (host arrays of `count` entries; operand i is laid out as for gt_gemm with M[i], N[i], K): the weight gradients
+ * dW_i = dY_i^T . X_i of consecutive linears over the same rows (webgpu.ts:900 issues one GEMM per linear), whose outputs
+ * are too small to fill the chip one at a time. TN products with K a multiple of 32, M and N multiples of 4 and 16-byte
+ * aligned operands run as ONE launch over the tiles of all of them (groups of up to 8) with one ordered reduction for the
+ * group; anything else, and a product large enough to fill the chip alone, is one gt_gemm per product. K is split into
+ * ranges of max(512, K/8) rows whatever the group holds, and no tile shape changes the order in which an output element
+ * sums over K, so a product's result does not depend, bit for bit, on what it shares the launch with. Outputs must be
+ * distinct buffers. */
+int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, int K, const gt_buf *A, const gt_buf *B,
+                  const gt_buf *C, const int *acc);
 /* batch of `count` independent products with element strides between consecutive problems
  * (Newton-Schulz over same-shaped matrices; no counterpart call in the reference, which loops). */
 int gt_gemm_batched(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t strideA,

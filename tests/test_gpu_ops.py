@@ -69,6 +69,71 @@ def test_gemm_every_tile_shape_and_kind(gpu, M, N, K):
         gpu.set_option("gemm.staged", 0)
 
 
+@pytest.mark.parametrize("K,shapes", [(16384, [(576, 1536), (1536, 576), (1536, 576), (576, 576), (576, 576), (192, 576), (192, 576)]),
+                                      (2048, [(576, 1536), (1536, 576), (1536, 576), (576, 576), (576, 576), (192, 576), (192, 576), (576, 1536)]),
+                                      (256, [(64, 64), (8, 12)]), (96, [(200, 152), (4, 4), (132, 100)]),
+                                      (100, [(64, 64), (32, 96)]), (64, [(30, 64), (64, 64)]),
+                                      (128, [(64, 96)] * 11)])
+@pytest.mark.parametrize("splitk", [-1, 1, 3])
+def test_gemm_group_equals_the_products_one_by_one(gpu, K, shapes, splitk):
+    """gt_gemm_group: the weight gradients of consecutive linears as one launch, against one gt_gemm per product (same
+    tile arithmetic per output element when the K split is the same: compared at 1e-5 / 1e-4 since the split of a
+    grouped product follows K alone and a single gt_gemm's follows its shape), against each product alone through the
+    same entry point (bit for bit: what a product shares its launch with does not enter its result) and against float64. The seven dW shapes of a SmolLM2 layer at 16384 and at
+    2048 rows (a full group of eight), tiny and ragged outputs next to large ones, and the cases that go product by
+    product: K not a multiple of 32, M not a multiple of 4, more than eight products. Store and accumulate mixed in one
+    group; every tile shape a group can take."""
+    lib = mod("lib")
+    rs = np.random.RandomState(K + len(shapes))
+    n = len(shapes)
+    As = [rs.standard_normal((K, M)).astype(np.float32) for M, N in shapes]
+    Bs = [rs.standard_normal((K, N)).astype(np.float32) for M, N in shapes]
+    C0 = [rs.standard_normal((M, N)).astype(np.float32) for M, N in shapes]
+    accs = [i % 2 for i in range(n)]
+    da = [gpu.create_state_buffer(a_.nbytes) for a_ in As]
+    db = [gpu.create_state_buffer(b_.nbytes) for b_ in Bs]
+    dc = [gpu.create_state_buffer(c_.nbytes) for c_ in C0]
+    for b_, a_ in zip(da + db, As + Bs):
+        gpu.write_state_buffer(b_, a_)
+    want = [a_.astype(np.float64).T @ b_.astype(np.float64) + (c_ if acc else 0) for a_, b_, c_, acc in zip(As, Bs, C0, accs)]
+    Ms, Ns = (C.c_int * n)(*[m for m, _ in shapes]), (C.c_int * n)(*[n_ for _, n_ in shapes])
+    aa, bb, cc, ac = (C.c_uint64 * n)(*da), (C.c_uint64 * n)(*db), (C.c_uint64 * n)(*dc), (C.c_int * n)(*accs)
+    gpu.set_option("gemm.splitk", splitk)
+    try:
+        for tile in ((-1, 6, 7, 8, 11, 12) if K == 256 or K == 96 else (-1,)):
+            gpu.set_option("gemm.tile", tile)
+            for b_, c_ in zip(dc, C0):
+                gpu.write_state_buffer(b_, c_)
+            lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, n, Ms, Ns, K, aa, bb, cc, ac), "gt_gemm_group")
+            got = [gpu.read_state_buffer(b_, c_.size).copy() for b_, c_ in zip(dc, C0)]
+            for i in range(n):
+                assert_close(got[i], want[i], f"group member {i} {shapes[i]} tile {tile} vs float64")
+        gpu.set_option("gemm.tile", -1)
+        # a product's bits do not depend on the company it has in the launch: each one alone, through the same entry point
+        for i in range(n):
+            gpu.write_state_buffer(dc[i], C0[i])
+            lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, 1, (C.c_int * 1)(shapes[i][0]), (C.c_int * 1)(shapes[i][1]), K,
+                                                     (C.c_uint64 * 1)(da[i]), (C.c_uint64 * 1)(db[i]), (C.c_uint64 * 1)(dc[i]),
+                                                     (C.c_int * 1)(accs[i])), "gt_gemm_group")
+            assert np.array_equal(gpu.read_state_buffer(dc[i], C0[i].size), got[i]), f"member {i} alone vs in the group"
+        gpu.set_option("gemm.group", 0)
+        for b_, c_ in zip(dc, C0):
+            gpu.write_state_buffer(b_, c_)
+        lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, n, Ms, Ns, K, aa, bb, cc, ac), "gt_gemm_group")
+        single = [gpu.read_state_buffer(b_, c_.size).copy() for b_, c_ in zip(dc, C0)]
+        for i in range(n):
+            assert_close(got[i], single[i], f"group member {i} vs its own launch")
+        if splitk == 1:          # no K split on either side: the same arithmetic per output element
+            assert all(np.array_equal(g_, s_) for g_, s_ in zip(got, single))
+    finally:
+        gpu.set_option("gemm.group", 1)
+        gpu.set_option("gemm.tile", -1)
+        gpu.set_option("gemm.splitk", -1)
+    with pytest.raises(lib.HipError, match="write the same output"):
+        cc2 = (C.c_uint64 * n)(*([dc[0]] * n))
+        lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, n, Ms, Ns, K, aa, bb, cc2, ac), "gt_gemm_group")
+
+
 @pytest.mark.parametrize("rows,K,r", [(16, 64, 16), (100, 192, 16), (257, 1024, 16), (333, 128, 8), (64, 64, 3), (129, 256, 32),
                                       (200, 320, 20), (70, 48, 16), (50, 64, 40), (90, 100, 16), (2100, 576, 16)])
 def test_rank_products(gpu, rows, K, r):
@@ -734,7 +799,7 @@ def test_unknown_option_is_an_error(gpu):
     assert rc != 0 and b"gemm.no_such_switch" in L.lib.gt_last_error(gpu.ctx)
     with pytest.raises(RuntimeError, match="no_such_switch"):
         gpu.set_option("attn.no_such_switch", 0)
-    for key, default in (("gemm.tile", -1), ("gemm.splitk", -1), ("gemm.staged", 0), ("attn.generic", 0), ("attn.splits", -1),
+    for key, default in (("gemm.tile", -1), ("gemm.splitk", -1), ("gemm.staged", 0), ("gemm.group", 1), ("attn.generic", 0), ("attn.splits", -1),
                          ("prof.sample", 1)):
         gpu.set_option(key, default)
 
