@@ -223,6 +223,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
+    ap.add_argument("--streams", type=int, default=4,
+                    help="HIP streams the backend deals consecutive micro-batches to (matters for --sequential; 1 = one stream)")
+    ap.add_argument("--no-call-pattern", action="store_true",
+                    help="skip the short extra leg that runs the step the way the reference's trainer calls the backend")
     ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (benchmark configs[1] shapes)")
     ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
     ap.add_argument("--no-keep-scores", action="store_true",
@@ -255,7 +259,7 @@ def main():
     cfg = arch.ModelConfig(**wl["model"])
     model = arch.Model(cfg, synth_weights(arch, cfg))
     n_params = sum(p.size for p in model.params())
-    gpu = hb.require_gpu("bench.py")
+    gpu = hb.require_gpu("bench.py", streams=a.streams)
     gpu.batch_linears = not a.no_pair
     gpu.attn_keep_scores = not a.no_keep_scores
     gpu.fuse_sibling_dx = "sibling_dx" not in a.no_fuse
@@ -287,12 +291,12 @@ def main():
         toks = [np.random.RandomState(100 + i).randint(0, cfg.vocab, (BATCH, SEQ + 1)).astype(np.int64) for i in range(total)]
     masks = [np.random.RandomState(500 + i).rand(BATCH, SEQ) < wl["mask"] for i in range(total)] if wl.get("mask") else None
 
-    def step(i):
+    def step(i, sequential=a.sequential):
         t = toks[i]
         tgt = t[:, 1:].copy()
         if masks is not None:
             tgt[~masks[i]] = -1                 # loss mask: only the kept positions carry a target
-        if a.sequential:
+        if sequential:
             losses = []
             for b in range(BATCH):
                 loss = arch.sequence_loss(model, t[b, :-1], tgt[b], 0)
@@ -330,6 +334,25 @@ def main():
         gpu.start_profile("adamw")           # the AdamW kernels alone, outside the timed region
         step(total - 1)
         opt_prof = gpu.stop_profile().get("adamw")
+        # The same step the way the reference's trainer calls a backend (src/backend/train-gpu.ts:200-219): one sequence's
+        # forward and backward at a time, B graphs of 2048 rows per step, gradients accumulated, then the optimizer. A short
+        # leg outside the headline's timed region; the backend deals the micro-batches to its streams.
+        call_pattern = None
+        if not a.sequential and not a.no_call_pattern:
+            nseq = max(2, min(6, a.steps))
+            for i in range(2):
+                step(i % total, True)
+            gpu.sync([])
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for i in range(nseq):
+                step((2 + i) % total, True)
+            gpu.sync([])
+            torch.cuda.synchronize()
+            w1 = time.perf_counter() - t1
+            call_pattern = {"graph": f"{BATCH} graphs of {SEQ} rows per step, one sequence at a time, as src/backend/train-gpu.ts:200-219 calls the backend",
+                            "streams": a.streams, "steps": nseq, "value": round(nseq * BATCH * SEQ / w1, 1), "unit": "tokens/s",
+                            "ms_per_step": round(1e3 * w1 / nseq, 2)}
     finally:
         gpu.uninstall()
         ag.set_checkpointing(False)
@@ -374,9 +397,10 @@ def main():
         "dtype": "f32", "data": "synthetic (weights N(0,0.02) random init, tokens Zipf(1.1) over the vocab)",
         "config": {"workload": wl["name"],
                    "params": n_params, "global_batch": BATCH, "seq_len": SEQ,
-                   "graph": "sequential micro-batches" if a.sequential else "8 sequences stacked into one 16384-row graph",
+                   "graph": f"sequential micro-batches on {a.streams} stream(s)" if a.sequential else f"{BATCH} sequences stacked into one {BATCH * SEQ}-row graph",
                    "device": gpu.adapter_name},
         "loss_first": round(losses[0], 4), "loss_last": round(losses[-1], 4),
+        "reference_call_pattern": call_pattern,
         "roofline": roof,
         "kernels": kernels,
         "cpu_baseline": None if a.no_cpu else cpu_baseline(),

@@ -135,6 +135,39 @@ __global__ __launch_bounds__(256) void adamw_update_k(const Chunk *__restrict__ 
   for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) adam1(g[i] * sc, m[i], v[i], w[i], h);
 }
 
+
+// ---- gradient fold ------------------------------------------------------------------------------------
+// dst_i (+)= src_i0 + src_i1 + ... for a list of tensors in one launch: the accumulators that micro-batches recorded on
+// different streams kept apart, summed in stream order into the accumulator the optimizer reads.
+#define FOLD_CHUNK 8192
+#define FOLD_MAX_SRC 7
+struct FoldPtrs { float *dst; const float *src[FOLD_MAX_SRC]; int acc, nsrc; };
+__global__ __launch_bounds__(256) void grad_fold_k(const Chunk *__restrict__ chunks, const FoldPtrs *__restrict__ ptrs) {
+  const Chunk c = chunks[blockIdx.x];
+  const FoldPtrs p = ptrs[c.tensor];
+  float *dst = p.dst + c.off;
+  bool vec = (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+  for (int s = 0; s < p.nsrc; s++) vec = vec && (reinterpret_cast<uintptr_t>(p.src[s] + c.off) & 15) == 0;
+  const int n4 = vec ? c.len / 4 : 0;
+  for (int i = threadIdx.x; i < n4; i += 256) {
+    v4f x[FOLD_MAX_SRC + 1];
+    if (p.acc) x[0] = reinterpret_cast<const v4f *>(dst)[i];
+#pragma unroll
+    for (int s = 0; s < FOLD_MAX_SRC; s++)
+      if (s < p.nsrc) x[s + 1] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p.src[s] + c.off) + i);
+    v4f sum = p.acc ? x[0] + x[1] : x[1];
+#pragma unroll
+    for (int s = 1; s < FOLD_MAX_SRC; s++)
+      if (s < p.nsrc) sum += x[s + 1];
+    reinterpret_cast<v4f *>(dst)[i] = sum;
+  }
+  for (int i = n4 * 4 + threadIdx.x; i < c.len; i += 256) {
+    float sum = p.acc ? dst[i] + p.src[0][c.off + i] : p.src[0][c.off + i];
+    for (int s = 1; s < p.nsrc; s++) sum += p.src[s][c.off + i];
+    dst[i] = sum;
+  }
+}
+
 // ---- Muon -------------------------------------------------------------------------------------------
 // Matrices of equal shape form a group that is stepped as one batch: every elementwise stage runs over the
 // group's concatenated work buffers (blockIdx.y = matrix), and each Newton-Schulz product is one batched GEMM
@@ -292,6 +325,42 @@ int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const 
   float one[2] = {1.0f, 0.0f};
   GT_HIP(ctx, hipMemcpy(o->scale, one, 8, hipMemcpyHostToDevice));
   *out = o;
+  return 0;
+}
+
+int gt_grad_fold(gt_ctx *ctx, int n, const gt_buf *dst, const int *dst_acc, int nsrc, const gt_buf *src, const int64_t *sizes) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, n >= 0 && nsrc >= 1 && nsrc <= FOLD_MAX_SRC && (n == 0 || (dst && dst_acc && src && sizes)),
+             "gt_grad_fold: %d tensors with %d sources each (at most %d), or a null table", n, nsrc, FOLD_MAX_SRC);
+  std::vector<Chunk> ch;
+  std::vector<FoldPtrs> tp;
+  double bytes = 0;
+  for (int i = 0; i < n; i++) {
+    FoldPtrs p;
+    memset(&p, 0, sizeof p);
+    p.dst = P<float>(dst[i]); p.acc = dst_acc[i];
+    for (int s = 0; s < nsrc; s++)
+      if (src[(size_t)i * nsrc + s]) p.src[p.nsrc++] = P<const float>(src[(size_t)i * nsrc + s]);     // absent ones are skipped
+    GT_REQUIRE(ctx, dst[i] && sizes[i] >= 0, "gt_grad_fold: tensor %d has a null destination or a negative size", i);
+    if (p.nsrc == 0 || sizes[i] == 0) continue;
+    bytes += 4.0 * sizes[i] * (p.nsrc + 1 + (p.acc ? 1 : 0));
+    const int t = (int)tp.size();
+    tp.push_back(p);
+    for (int64_t off = 0; off < sizes[i]; off += FOLD_CHUNK) ch.push_back({t, (int)std::min<int64_t>(FOLD_CHUNK, sizes[i] - off), off});
+  }
+  if (ch.empty()) return 0;
+  // the tables ride in the context's workspace: the copies and the kernel are ordered on the stream with whatever used it
+  // before and uses it next (the source vectors are pageable, so the copy has staged them when it returns)
+  const size_t cb = (ch.size() * sizeof(Chunk) + 255) & ~(size_t)255, pb = tp.size() * sizeof(FoldPtrs);
+  void *ws;
+  if (gt_ws_reserve(ctx, cb + pb, &ws)) return 1;
+  Chunk *dch = static_cast<Chunk *>(ws);
+  FoldPtrs *dtp = reinterpret_cast<FoldPtrs *>(static_cast<char *>(ws) + cb);
+  GT_HIP(ctx, hipMemcpyAsync(dch, ch.data(), ch.size() * sizeof(Chunk), hipMemcpyHostToDevice, ctx->stream));
+  GT_HIP(ctx, hipMemcpyAsync(dtp, tp.data(), pb, hipMemcpyHostToDevice, ctx->stream));
+  ProfScope ps(ctx, "grad.fold", bytes);
+  hipLaunchKernelGGL(grad_fold_k, dim3((unsigned)ch.size()), dim3(256), 0, ctx->stream, dch, dtp);
+  GT_LAUNCHED(ctx);
   return 0;
 }
 

@@ -26,6 +26,8 @@ What differs from the reference, on purpose:
     first writer: the operand's gradient points at the upstream buffer until somebody adds to it.
   * attention keeps its raw scores from the forward to the backward where a backward can come and a byte budget allows,
     as the reference's small-T path keeps its probabilities (webgpu.ts:1176-1189).
+  * Consecutive micro-batches are recorded on different streams (see __init__), each with its own pool of transient
+    buffers and its own parameter-gradient accumulators, summed in stream order before anything reads them.
   Each of these has a switch (batch_linears, fuse_residual_add, fuse_sibling_dx, group_dw, alias_add_grads, attn_keep_scores) and
   gives the same gradients as the one-launch-per-op form: bit for bit, or to rounding where a sum changes its order.
 """
@@ -46,7 +48,7 @@ _ALIGN = 256
 
 class _Entry:
     __slots__ = ("data", "grad", "nbytes", "external", "grad_init", "lazy_act", "consumers", "fused_uses",
-                 "region", "keep_grad", "extra", "needs_grad", "lazy_lin", "grad_src")
+                 "region", "keep_grad", "extra", "needs_grad", "lazy_lin", "grad_src", "stream", "sgrad")
 
     def __init__(self, nbytes, external):
         self.data = 0
@@ -63,20 +65,38 @@ class _Entry:
         self.needs_grad = False     # an intermediate below a trainable tensor: a backward through it may be asked for
         self.lazy_lin = None        # (rows, out, in, x data, w data) while a linear's output lives only inside a fused add
         self.grad_src = 0           # another tensor's gradient buffer that holds this gradient's value so far (add's backward)
+        self.stream = 0             # the stream whose launches produce and consume this tensor (its buffers come from that stream's pool)
+        self.sgrad = None           # parameters: {stream: [accumulator, written?]} of the streams other than the first
 
 
 class HipBackend:
-    def __init__(self, device: int = 0):
-        self._ctx = C.c_void_p()
-        rc = lib.gt_ctx_create(device, C.byref(self._ctx))
-        if rc != 0:
-            raise HipError("gt_ctx_create: " + (lib.gt_last_error(None) or b"").decode())
+    def __init__(self, device: int = 0, streams: int = 4):
+        """streams: how many HIP streams (library contexts on the one device) consecutive micro-batches are dealt to.
+        The reference's trainer records one sequence's forward and backward at a time (src/backend/train-gpu.ts:200-219);
+        a 2048-row graph cannot fill 256 CUs launch by launch, but micro-batches are independent until their parameter
+        gradients meet, so each goes to the next stream, keeps its own parameter-gradient accumulators there, and the
+        accumulators are summed in stream order (gt_grad_fold) before anything reads them. 1 = everything on one stream."""
+        self._nstreams = max(1, min(int(streams), 8))
+        self._ctxs = []
+        for _ in range(self._nstreams):
+            c = C.c_void_p()
+            if lib.gt_ctx_create(device, C.byref(c)) != 0:
+                msg = (lib.gt_last_error(None) or b"").decode()
+                for made in self._ctxs:
+                    lib.gt_ctx_destroy(made)
+                raise HipError("gt_ctx_create: " + msg)
+            self._ctxs.append(c)
+        self._cur = 0                     # stream of the micro-batch being recorded
+        self._used = set()                # streams other than the first with work queued since the last join
+        self._bw_seen = False             # a backward closure has run since the last switch: the next graph root starts a micro-batch
+        self._s0_barrier = False          # the first stream holds work (uploads, an optimizer step, a fold) another stream must not overtake
+        self._sfold: list = []            # (tensor, entry) of parameters with a written accumulator on another stream
         self.adapter_name = lib.gt_device_name(self._ctx).decode()
         self.attn_flash_min_t = 2048      # kept for interface parity; one kernel family serves every T here
         self.last_sync_readback_bytes = 0
         self.grad_clears_issued = 0
         self.fuse_glu = True
-        self._pool: dict[int, list[int]] = {}
+        self._pools = [dict() for _ in range(self._nstreams)]     # per stream: size class -> free buffers
         self._pool_bytes = 0
         self._state_bytes = 0
         self._entries: "weakref.WeakKeyDictionary[Tensor, _Entry]" = weakref.WeakKeyDictionary()
@@ -118,6 +138,67 @@ class HipBackend:
         self.forward_only_region = False  # set by checkpoint() around a block's first forward, whose interior is never differentiated
         self._profiling = False
         self._destroyed = False
+
+    # ---- streams ------------------------------------------------------------------------------------------------
+    @property
+    def _ctx(self):
+        return self._ctxs[self._cur]
+
+    def _op_begin(self, *inputs):
+        """Called first thing by every forward op. After a backward has run, an op whose inputs are all parameters or
+        host data is the root of the next micro-batch's graph: it goes to the next stream."""
+        if not self._bw_seen:
+            return
+        if self._nstreams == 1:
+            return
+        for t in inputs:
+            e = self._entries.get(t)
+            if e is not None and not e.external:
+                return
+        self._flush()
+        self._flush_dx()
+        if self._s0_barrier:
+            check(self._ctxs[0], lib.gt_sync(self._ctxs[0]), "gt_sync")
+            self._s0_barrier = False
+        self._cur = (self._cur + 1) % self._nstreams
+        if self._cur:
+            self._used.add(self._cur)
+        self._bw_seen = False
+
+    def _join(self):
+        """Everything recorded on the other streams has finished and their parameter-gradient accumulators are summed, in
+        stream order, into the first stream's; recording continues on the first stream."""
+        self._flush()
+        self._flush_dx()
+        self._bw_seen = False
+        if self._cur == 0 and not self._used and not self._sfold:
+            return
+        for s in sorted(self._used):
+            check(self._ctxs[s], lib.gt_sync(self._ctxs[s]), "gt_sync")
+        self._used = set()
+        self._cur = 0
+        self._bw_seen = False
+        if self._sfold:
+            seen, items = set(), []
+            for t, e in self._sfold:
+                if id(e) not in seen:
+                    seen.add(id(e))
+                    items.append((t, e))
+            self._sfold = []
+            n, ns = len(items), self._nstreams - 1
+            dst, acc, src, sizes = (c_buf * n)(), (C.c_int * n)(), (c_buf * (n * ns))(), (C.c_int64 * n)()
+            for i, (t, e) in enumerate(items):
+                if e.grad == 0:
+                    e.grad = self._acquire(e.nbytes, 0)
+                dst[i], acc[i], sizes[i] = e.grad, 1 if e.grad_init else 0, e.nbytes // 4
+                for s_ in range(1, self._nstreams):
+                    slot = e.sgrad.get(s_)
+                    if slot is not None and slot[1]:
+                        src[i * ns + s_ - 1] = slot[0]
+                        slot[1] = False
+                e.grad_init = True
+            check(self._ctxs[0], lib.gt_grad_fold(self._ctxs[0], n, dst, acc, ns, src, sizes), "gt_grad_fold")
+            self._s0_barrier = True
 
     # ---- install (webgpu.ts:393-399) ---------------------------------------------------------------
     # ---- a linear's forward launch is held back by one op: two consecutive linears over the same input with the same
@@ -188,40 +269,45 @@ class HipBackend:
         ag.set_ops_backend(None)
 
     # ---- raw memory ------------------------------------------------------------------------------------
-    def _acquire(self, nbytes: int) -> int:
+    def _acquire(self, nbytes: int, stream: int = None) -> int:
+        """A buffer from the pool of `stream` (default: the one being recorded on). A buffer only ever returns to the pool
+        it came from, so it is only ever reused by launches ordered after its last use."""
+        s_ = self._cur if stream is None else stream
         size = max(_ALIGN, (nbytes + _ALIGN - 1) // _ALIGN * _ALIGN)
-        free = self._pool.get(size)
+        free = self._pools[s_].get(size)
         if free:
             return free.pop()
         out = c_buf()
-        if lib.gt_alloc(self._ctx, size, 0, C.byref(out)) != 0:
+        ctx = self._ctxs[s_]
+        if lib.gt_alloc(ctx, size, 0, C.byref(out)) != 0:
             # device memory is full of free buffers of other size classes (another model shape ran before): give them
             # back and ask again; only then is it an error
             if not self.trim_pool():
-                check(self._ctx, 1, "gt_alloc")
-            check(self._ctx, lib.gt_alloc(self._ctx, size, 0, C.byref(out)), "gt_alloc")
+                check(ctx, 1, "gt_alloc")
+            check(ctx, lib.gt_alloc(ctx, size, 0, C.byref(out)), "gt_alloc")
         self._pool_bytes += size
         return out.value
 
     def trim_pool(self) -> int:
         """Return every free buffer of the pool to the device (buffers in use stay). Gives the bytes freed."""
         freed = 0
-        check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")      # queued kernels may still use a buffer recycled at a region's end
-        for size, free in self._pool.items():
-            for b in free:
-                check(self._ctx, lib.gt_free(self._ctx, b), "gt_free")
-                freed += size
-            free.clear()
+        for ctx, pool in zip(self._ctxs, self._pools):
+            check(ctx, lib.gt_sync(ctx), "gt_sync")      # queued kernels may still use a buffer recycled at a region's end
+            for size, free in pool.items():
+                for b in free:
+                    check(ctx, lib.gt_free(ctx, b), "gt_free")
+                    freed += size
+                free.clear()
         self._pool_bytes -= freed
         return freed
 
-    def _recycle(self, b: int, nbytes: int):
+    def _recycle(self, b: int, nbytes: int, stream: int = None):
         size = max(_ALIGN, (nbytes + _ALIGN - 1) // _ALIGN * _ALIGN)
-        self._pool.setdefault(size, []).append(b)
+        self._pools[self._cur if stream is None else stream].setdefault(size, []).append(b)
 
     def _scratch_buf(self, nbytes: int) -> int:
         b = self._acquire(nbytes)
-        self._scratch.append((b, nbytes))
+        self._scratch.append((b, nbytes, self._cur))
         return b
 
     def _upload(self, arr: np.ndarray) -> int:
@@ -239,8 +325,13 @@ class HipBackend:
             if t._prev:
                 raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's buffers")
             e = _Entry(t.size * 4, True)
-            e.data = self._acquire(e.nbytes)
-            check(self._ctx, lib.gt_h2d(self._ctx, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
+            e.data = self._acquire(e.nbytes, 0)
+            c0 = self._ctxs[0]
+            check(c0, lib.gt_h2d(c0, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
+            if self._cur:
+                check(c0, lib.gt_sync(c0), "gt_sync")       # uploaded on the first stream, read by this one
+            else:
+                self._s0_barrier = True
             self._entries[t] = e
             self._externals.add(t)
         if e.external and t.requires_grad and id(t) not in self._touched_ids:
@@ -252,6 +343,7 @@ class HipBackend:
         out = Tensor(None, shape)
         out._prev = list(prev)
         e = _Entry(out.size * 4, False)
+        e.stream = self._cur
         if alloc:
             e.data = self._acquire(e.nbytes)
         e.region = self._regions_opened
@@ -270,6 +362,9 @@ class HipBackend:
         if launch_held:
             self._flush()
         e = self._entry_for(t)
+        if e.stream != self._cur and not e.external:
+            # an intermediate of another micro-batch: that stream's work must be done before this one reads it
+            check(self._ctxs[e.stream], lib.gt_sync(self._ctxs[e.stream]), "gt_sync")
         e.consumers += 1
         if e.lazy_act is not None:
             self._materialise(t, e)
@@ -281,7 +376,7 @@ class HipBackend:
         self._flush()
         x, act = e.lazy_act
         e.lazy_act = None
-        e.data = self._acquire(e.nbytes)
+        e.data = self._acquire(e.nbytes, e.stream)
         xe = self._entry_for(x)
         fn = lib.gt_silu_fwd if act == 0 else lib.gt_gelu_fwd
         check(self._ctx, fn(self._ctx, t.size, xe.data, e.data), "act.fwd")
@@ -290,7 +385,7 @@ class HipBackend:
         """A linear output that went straight into a residual add is wanted on its own after all: compute it now."""
         rows, outd, ind, xd, wd = e.lazy_lin
         e.lazy_lin = None
-        e.data = self._acquire(e.nbytes)
+        e.data = self._acquire(e.nbytes, e.stream)
         check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, rows, outd, ind, xd, wd, e.data), "linear")
 
     def _gdst(self, t: Tensor) -> tuple:
@@ -304,10 +399,23 @@ class HipBackend:
         e = self._entries.get(t)
         if e is None:
             e = self._entry_for(t)
+        self._bw_seen = True
         if e.external and not t.requires_grad:
             return 0, 0
+        if e.external and self._cur:
+            # a parameter's gradient from a micro-batch on another stream than the first: that stream's own accumulator
+            if e.sgrad is None:
+                e.sgrad = {}
+            slot = e.sgrad.get(self._cur)
+            if slot is None:
+                slot = e.sgrad[self._cur] = [self._acquire(e.nbytes), False]
+            acc = 1 if slot[1] else 0
+            if not slot[1]:
+                slot[1] = True
+                self._sfold.append((t, e))
+            return slot[0], acc
         if e.grad == 0:
-            e.grad = self._acquire(e.nbytes)
+            e.grad = self._acquire(e.nbytes, e.stream)
         if e.grad_src:
             check(self._ctx, lib.gt_d2d(self._ctx, e.grad, e.grad_src, e.nbytes), "gt_d2d")
             e.grad_src = 0
@@ -327,7 +435,7 @@ class HipBackend:
             src = e.grad_src
             e.grad_src = 0
             if e.grad == 0:
-                e.grad = self._acquire(e.nbytes)
+                e.grad = self._acquire(e.nbytes, e.stream)
             return e.grad, 1, src
         dst, acc = self._gdst(t)
         return dst, acc, dst
@@ -346,7 +454,7 @@ class HipBackend:
                 e.grad_init = False
             else:
                 if e.grad == 0:
-                    e.grad = self._acquire(e.nbytes)
+                    e.grad = self._acquire(e.nbytes, e.stream)
                 check(self._ctx, lib.gt_d2d(self._ctx, e.grad, e.grad_src, e.nbytes), "gt_d2d")
                 e.grad_src = 0
         self._aliased = []
@@ -362,12 +470,13 @@ class HipBackend:
         if e is None:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
                                "gradient buffers, so this backward would read pool garbage")
+        self._bw_seen = True
         if e.grad_src:
             return e.grad_src       # handed on by an add's backward and not written since: read it where it is
         if e.grad == 0 or not e.grad_init:
             # nothing downstream wrote it (an output the loss does not depend on): its gradient is zero
             if e.grad == 0:
-                e.grad = self._acquire(e.nbytes)
+                e.grad = self._acquire(e.nbytes, e.stream)
             check(self._ctx, lib.gt_memset0(self._ctx, e.grad, e.nbytes), "gt_memset0")
             self.grad_clears_issued += 1
             e.grad_init = True
@@ -375,18 +484,17 @@ class HipBackend:
 
     # ---- public buffer surface (webgpu.ts:1432-1537) ----------------------------------------------------
     def upload_params(self, tensors):
-        self._flush()
-        self._flush_dx()
+        self._join()
         for t in tensors:
             e = self._entry_for(t)
             check(self._ctx, lib.gt_h2d(self._ctx, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
+        self._s0_barrier = True
 
     def buffers_for(self, t: Tensor) -> dict:
-        self._flush()
-        self._flush_dx()
+        self._join()
         e = self._entry_for(t)
         if t.requires_grad and e.grad == 0:
-            e.grad = self._acquire(e.nbytes)
+            e.grad = self._acquire(e.nbytes, e.stream)
             check(self._ctx, lib.gt_memset0(self._ctx, e.grad, e.nbytes), "gt_memset0")
             self.grad_clears_issued += 1
         return {"data": e.data, "grad": e.grad}
@@ -397,7 +505,8 @@ class HipBackend:
     def grads_consumed(self, tensors):
         """The optimizer has read these accumulators: the next backward write stores instead of adding
         (the reference's deferred per-step clear, src/backend/muon-gpu.ts:8-16)."""
-        self._flush_dx()
+        self._join()
+        self._s0_barrier = True      # the optimizer's launches are on the first stream: no other stream may read weights before them
         for t in tensors:
             e = self._entries.get(t)
             if e is not None:
@@ -405,12 +514,11 @@ class HipBackend:
 
     def ensure_grads_defined(self, tensors):
         """An accumulator no kernel wrote since it was last consumed holds zero, as a cleared one would."""
-        self._flush()
-        self._flush_dx()
+        self._join()
         for t in tensors:
             e = self._entry_for(t)
             if e.grad == 0:
-                e.grad = self._acquire(e.nbytes)
+                e.grad = self._acquire(e.nbytes, e.stream)
             if not e.grad_init:
                 check(self._ctx, lib.gt_memset0(self._ctx, e.grad, e.nbytes), "gt_memset0")
                 self.grad_clears_issued += 1
@@ -423,26 +531,27 @@ class HipBackend:
         if e is None:
             raise RuntimeError("seed_grad_from_host: tensor has no device buffers")
         if e.grad == 0:
-            e.grad = self._acquire(e.nbytes)
+            e.grad = self._acquire(e.nbytes, e.stream)
         check(self._ctx, lib.gt_h2d(self._ctx, e.grad, t.grad.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
         e.grad_init = True
         e.grad_src = 0
 
     def create_state_buffer(self, nbytes: int) -> int:
         out = c_buf()
-        check(self._ctx, lib.gt_alloc(self._ctx, max(4, nbytes), 1, C.byref(out)), "gt_alloc")
+        c0 = self._ctxs[0]
+        check(c0, lib.gt_alloc(c0, max(4, nbytes), 1, C.byref(out)), "gt_alloc")
+        self._s0_barrier = True
         self._state_bytes += max(4, nbytes)
         return out.value
 
     def write_state_buffer(self, b: int, arr: np.ndarray):
-        self._flush()
-        self._flush_dx()
+        self._join()
         arr = np.ascontiguousarray(arr)
         check(self._ctx, lib.gt_h2d(self._ctx, b, arr.ctypes.data_as(C.c_void_p), arr.nbytes), "gt_h2d")
+        self._s0_barrier = True
 
     def read_state_buffer(self, b: int, n: int, dtype=np.float32) -> np.ndarray:
-        self._flush()
-        self._flush_dx()
+        self._join()
         out = np.empty(n, dtype=dtype)
         check(self._ctx, lib.gt_d2h(self._ctx, out.ctypes.data_as(C.c_void_p), b, out.nbytes), "gt_d2h")
         return out
@@ -450,19 +559,24 @@ class HipBackend:
     def set_option(self, key: str, value: int):
         """Kernel-selection switches for tests and tuning: "attn.generic", "attn.splits", "gemm.tile", "gemm.splitk", "gemm.staged",
         and "prof.sample" (time every n-th launch of a label)."""
-        check(self._ctx, lib.gt_set_option(self._ctx, key.encode(), int(value)), "gt_set_option")
+        for c in self._ctxs:
+            check(c, lib.gt_set_option(c, key.encode(), int(value)), "gt_set_option")
 
     def resident_bytes(self) -> int:
-        v = C.c_uint64()
-        lib.gt_resident_bytes(self._ctx, C.byref(v))
-        return int(v.value)
+        total = 0
+        for c in self._ctxs:
+            v = C.c_uint64()
+            lib.gt_resident_bytes(c, C.byref(v))
+            total += int(v.value)
+        return total
 
     def region_count(self) -> int:
         return self._regions_opened
 
     @property
     def ctx(self):
-        return self._ctx
+        """The first stream's library context: state buffers, optimizers and raw calls of tests live there."""
+        return self._ctxs[0]
 
     # ---- sync / reclaim (webgpu.ts:419-636) -------------------------------------------------------------
     def _release_transients(self, keep=()):
@@ -474,26 +588,25 @@ class HipBackend:
                 kept.append((t, e))
                 continue
             if e.data:
-                self._recycle(e.data, e.nbytes)
+                self._recycle(e.data, e.nbytes, e.stream)
             if e.grad:
-                self._recycle(e.grad, e.nbytes)
+                self._recycle(e.grad, e.nbytes, e.stream)
             if e.extra:
-                self._recycle(*e.extra)
+                self._recycle(e.extra[0], e.extra[1], e.stream)
                 self._scores_taken -= e.extra[1]
                 e.extra = None
             e.data = e.grad = 0
             self._entries.pop(t, None)
         self._transients = kept
-        for b, n in self._scratch:
-            self._recycle(b, n)
+        for b, n, s_ in self._scratch:
+            self._recycle(b, n, s_)
         self._scratch = []
 
     def sync(self, reads=()):
         """Wait for the stream; read back `reads` (values) and the accumulated gradients of every
         trainable external tensor touched since the last sync that is not kept on the device; recycle
         all intermediates. The graph is unusable for backward afterwards."""
-        self._flush()
-        self._flush_dx()
+        self._join()
         nbytes = 0
         for t in reads:
             e = self._entries.get(t)
@@ -522,15 +635,20 @@ class HipBackend:
         self._touched = []
         self._touched_ids = set()
         check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")
+        self._s0_barrier = False
         self.last_sync_readback_bytes = nbytes
         self._release_transients()
         self._scores_taken = 0
 
     def reclaim_step_transients(self, keep=()):
-        """Free a finished micro-batch's intermediates mid-step; parameter gradients keep accumulating."""
+        """Free a finished micro-batch's intermediates mid-step; parameter gradients keep accumulating. Every stream is
+        waited for, but the micro-batches keep their streams and accumulators: which stream the next one goes to, and
+        the order in which gradients are summed, are the same with and without this call, so it changes no bit."""
         self._flush()
         self._flush_dx()
-        check(self._ctx, lib.gt_sync(self._ctx), "gt_sync")
+        for c in self._ctxs:
+            check(c, lib.gt_sync(c), "gt_sync")
+        self._s0_barrier = False
         self._release_transients(keep)
 
     def destroy(self):
@@ -539,23 +657,29 @@ class HipBackend:
         self._pend_dw = []
         if not self._destroyed:
             self._destroyed = True
-            lib.gt_ctx_destroy(self._ctx)
+            for c in self._ctxs:
+                lib.gt_ctx_destroy(c)
 
     # ---- profiling (webgpu.ts:830-880) -----------------------------------------------------------------------
     def start_profile(self, prefix: str = ""):
         """Time every launch whose label starts with `prefix` ("" = all) with HIP events on the stream."""
-        self._flush()
-        self._flush_dx()
-        check(self._ctx, lib.gt_prof_begin(self._ctx, prefix.encode()), "gt_prof_begin")
+        self._join()
+        for c in self._ctxs:
+            check(c, lib.gt_prof_begin(c, prefix.encode()), "gt_prof_begin")
 
     def stop_profile(self) -> dict:
         """label -> (total ms, launches, algorithmic work: FLOP or bytes)."""
-        self._flush()
-        self._flush_dx()
-        recs = (ProfRec * 128)()
-        n = C.c_int()
-        check(self._ctx, lib.gt_prof_end(self._ctx, recs, 128, C.byref(n)), "gt_prof_end")
-        return {recs[i].label.decode(): (recs[i].ms, recs[i].count, recs[i].work) for i in range(n.value)}
+        self._join()
+        out = {}
+        for c in self._ctxs:
+            recs = (ProfRec * 128)()
+            n = C.c_int()
+            check(c, lib.gt_prof_end(c, recs, 128, C.byref(n)), "gt_prof_end")
+            for i in range(n.value):
+                k = recs[i].label.decode()
+                ms, cnt, work = out.get(k, (0.0, 0, 0.0))
+                out[k] = (ms + recs[i].ms, cnt + recs[i].count, work + recs[i].work)
+        return out
 
     # ---- RegionBackend (webgpu.ts:639-761) ------------------------------------------------------------------------
     def begin_region(self) -> int:
@@ -574,11 +698,11 @@ class HipBackend:
                 self._transients.append((t, e))
                 continue
             if e.data:
-                self._recycle(e.data, e.nbytes)
+                self._recycle(e.data, e.nbytes, e.stream)
             if e.grad:
-                self._recycle(e.grad, e.nbytes)
+                self._recycle(e.grad, e.nbytes, e.stream)
             if e.extra:
-                self._recycle(*e.extra)
+                self._recycle(e.extra[0], e.extra[1], e.stream)
                 self._scores_taken -= e.extra[1]
                 e.extra = None
             e.data = e.grad = 0
@@ -593,6 +717,7 @@ class HipBackend:
 
     # ---- ops --------------------------------------------------------------------------------------------------------
     def linear(self, x: Tensor, w: Tensor) -> Tensor:
+        self._op_begin(x, w)
         T, ind = x.shape
         outd = w.shape[0]
         p = self._pend
@@ -644,6 +769,7 @@ class HipBackend:
         the rank-r activation h = x.a^T (inside the streaming rank kernels) instead of the [rows, out] product, the adapter product is
         accumulated into the base output by the GEMM itself, and the backward reads the upstream gradient directly:
         no [rows, out] elementwise pass in either direction."""
+        self._op_begin(x, w, a, b)
         T, ind = x.shape
         outd, r = w.shape[0], a.shape[0]
         xd, wd, ad, bd = self._data(x), self._data(w), self._data(a), self._data(b)
@@ -678,6 +804,7 @@ class HipBackend:
         return out
 
     def add(self, a: Tensor, b: Tensor) -> Tensor:
+        self._op_begin(a, b)
         p = self._pend
         lin = None
         if self.fuse_residual_add and p is not None and a is not b:
@@ -697,7 +824,7 @@ class HipBackend:
             check(self._ctx, lib.gt_gemm_add(self._ctx, NT, p[1], p[2], p[3], p[4], p[5], od, e.data), "linear+add")
             le.consumers += 1
             le.lazy_lin = (p[1], p[2], p[3], p[4], p[5])
-            self._recycle(le.data, le.nbytes)
+            self._recycle(le.data, le.nbytes, le.stream)
             le.data = 0
         else:
             ad, bd = self._data(a), self._data(b)
@@ -733,6 +860,7 @@ class HipBackend:
         return out
 
     def mul(self, a: Tensor, b: Tensor) -> Tensor:
+        self._op_begin(a, b)
         ea, eb = self._entry_for(a), self._entry_for(b)
         if self.fuse_glu and a is not b:
             # gate * up with a lazy activation on one side: run the fused kernels on the pre-activation
@@ -772,6 +900,7 @@ class HipBackend:
         return out
 
     def _activation(self, x: Tensor, act: int) -> Tensor:
+        self._op_begin(x)
         xd = self._data(x, launch_held=not self.fuse_glu)
         out, e = self._make_out(x.shape, [x], alloc=not self.fuse_glu)
         if self.fuse_glu:
@@ -803,6 +932,7 @@ class HipBackend:
         return self._activation(x, 1)
 
     def scale(self, x: Tensor, c: float) -> Tensor:
+        self._op_begin(x)
         xd = self._data(x)
         out, e = self._make_out(x.shape, [x])
         check(self._ctx, lib.gt_scale_fwd(self._ctx, out.size, xd, c, e.data), "scale")
@@ -817,6 +947,7 @@ class HipBackend:
         return out
 
     def _rms_rows(self, x, weight, rows, d, eps, shape):
+        self._op_begin(x, weight)
         xd, wd = self._data(x), self._data(weight)
         out, e = self._make_out(shape, [x, weight])
         rinv = self._scratch_buf(rows * 4)
@@ -843,6 +974,7 @@ class HipBackend:
         return self._rms_rows(x, weight, T * H, hd, eps, [T, H * hd])
 
     def embedding(self, weight: Tensor, ids) -> Tensor:
+        self._op_begin(weight)
         V, d = weight.shape
         ids32 = np.ascontiguousarray(ids, dtype=np.int32)
         T = ids32.size
@@ -863,6 +995,7 @@ class HipBackend:
         return out
 
     def rope(self, x, T, H, hd, base, pos_offset=0):
+        self._op_begin(x)
         rows = x.shape[0]
         xd = self._data(x)
         out, e = self._make_out([rows, H * hd], [x])
@@ -877,6 +1010,7 @@ class HipBackend:
         return out
 
     def attention(self, q, k, v, T, Hq, Hkv, hd, window=0):
+        self._op_begin(q, k, v)
         rows = q.shape[0]
         if rows % T:
             raise ValueError(f"attention: {rows} rows are not a whole number of sequences of {T}")
@@ -919,6 +1053,7 @@ class HipBackend:
         return (1.0 / np.maximum(kept, 1)).astype(np.float32)
 
     def cross_entropy(self, logits, targets, kept) -> Tensor:
+        self._op_begin(logits)
         rows, V = logits.shape
         inv = self._inv_denoms(kept)
         nseq = inv.size
@@ -941,6 +1076,7 @@ class HipBackend:
         return loss
 
     def fused_cross_entropy(self, hidden, w, targets, chunk, kept) -> Tensor:
+        self._op_begin(hidden, w)
         rows, H = hidden.shape
         V = w.shape[0]
         inv = self._inv_denoms(kept)
@@ -979,6 +1115,7 @@ class HipBackend:
         return loss
 
     def soft_cross_entropy(self, logits, teacher_ids, teacher_probs, k, kept) -> Tensor:
+        self._op_begin(logits)
         rows, V = logits.shape
         inv = 1.0 / max(int(kept), 1)
         zd = self._data(logits)
@@ -1000,22 +1137,21 @@ class HipBackend:
 
     # ---- raw GEMM for tests and benches (webgpu.ts:1654) --------------------------------------------------------------
     def gemm(self, kind: int, acc: int, M: int, N: int, K: int, a: int, b: int, c: int):
-        self._flush()
-        self._flush_dx()
+        self._join()
         check(self._ctx, lib.gt_gemm(self._ctx, kind, acc, M, N, K, a, b, c), "gemm")
 
 
-def init_hip(device: int = 0):
+def init_hip(device: int = 0, streams: int = 4):
     """initWebGPU analogue (webgpu.ts:1823): a backend, or None when no MI355X is visible."""
     try:
-        return HipBackend(device)
+        return HipBackend(device, streams)
     except HipError:
         return None
 
 
-def require_gpu(purpose: str, device: int = 0) -> HipBackend:
+def require_gpu(purpose: str, device: int = 0, streams: int = 4) -> HipBackend:
     """requireGPU analogue (webgpu.ts:1812)."""
     try:
-        return HipBackend(device)
+        return HipBackend(device, streams)
     except HipError as e:
         raise RuntimeError(f"{purpose} needs an MI355X: {e}") from e

@@ -81,6 +81,7 @@ _SIG = {
     "gt_soft_ce_bwd": [ctxp, i32, i32, i32, buf, buf, buf, f32, buf, buf, f32, buf, i32],
     "gt_adamw_create": [ctxp, i32, C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(i64),
                         f64, f64, f64, f64, f64, C.POINTER(C.c_void_p)],
+    "gt_grad_fold": [ctxp, i32, C.POINTER(buf), C.POINTER(i32), i32, C.POINTER(buf), C.POINTER(i64)],
     "gt_adamw_step": [ctxp, C.c_void_p, f64, f64, f64],
     "gt_adamw_grad_norm": [ctxp, C.c_void_p, C.POINTER(f32)],
     "gt_adamw_destroy": [ctxp, C.c_void_p],

@@ -247,6 +247,12 @@ int gt_adamw_step(gt_ctx *ctx, gt_adamw *opt, double lr, double bc1, double bc2)
 int gt_adamw_grad_norm(gt_ctx *ctx, gt_adamw *opt, float *norm);   /* last step's global norm; waits */
 int gt_adamw_destroy(gt_ctx *ctx, gt_adamw *opt);
 
+/* dst[i] (+)= src[i*nsrc + 0] + src[i*nsrc + 1] + ... (a source of 0 is skipped), i < n, sizes[i] elements each, one
+ * launch for the whole list: parameter-gradient accumulators that micro-batches recorded on different streams kept
+ * apart, summed in a fixed order into the one the optimizer reads. dst_acc[i] = 0 stores, 1 adds to dst's contents.
+ * nsrc <= 7. The reference keeps one accumulator per parameter and one queue (webgpu.ts:21-26); no counterpart there. */
+int gt_grad_fold(gt_ctx *ctx, int n, const gt_buf *dst, const int *dst_acc, int nsrc, const gt_buf *src, const int64_t *sizes);
+
 /* ---- Muon: MuonGpu (muon-gpu.ts:351-470), buildNewtonSchulz (:224-252), spec src/train/muon.ts -
  * Matrices w[i] are [rows[i], cols[i]]; buf[i] is the momentum. step(): buf = mu*buf + g;
  * U = nesterov ? g + mu*buf : buf; X = NS(U); w -= lr*sqrt(max(1, rows/cols))*X. */

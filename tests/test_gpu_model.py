@@ -347,9 +347,9 @@ def test_kept_attention_scores_policy(gpu, ref, recompute):
     taken = []
     acquire = gpu._acquire
 
-    def spy(nbytes):
+    def spy(nbytes, *stream):
         taken.append(nbytes)
-        return acquire(nbytes)
+        return acquire(nbytes, *stream)
 
     gpu._acquire = spy
     res = {}
@@ -580,7 +580,7 @@ def test_trim_pool_returns_free_buffers_and_work_goes_on(gpu, ref):
     before = gpu.resident_bytes()
     freed = gpu.trim_pool()
     assert freed > 0 and gpu.resident_bytes() == before - freed
-    assert all(not free for free in gpu._pool.values())
+    assert all(not free for pool in gpu._pools for free in pool.values())
     l1, g1 = hip_step(gpu, model, seqs, True, 19)
     assert np.array_equal(l0, l1) and all(np.array_equal(g0[n], g1[n]) for n in g0)
 
@@ -658,14 +658,15 @@ def test_empty_sync_recycles_without_corrupting_queued_work(gpu, ref):
 def test_recompute_memory_gate(ref):
     """gpu-parity.ts:1363-1420: the buffer pool (a high-water mark) is flat in the number of steps (sync drains the
     regions' buffers), flat in the number of micro-batches when transients are reclaimed between them, and clearly
-    smaller with recompute than without. A fresh backend per arm, sequential micro-batches of 128 tokens."""
+    smaller with recompute than without. A fresh backend per arm, sequential micro-batches of 128 tokens, on one stream
+    (the reference's one queue) and on four (bounded by four micro-batches in flight)."""
     ag, optim, train, hb = mod("autograd"), mod("optim"), mod("train"), mod("hip_backend")
     kw = dict(arch="gemma3", vocab=64, hidden=64, layers=4, heads=4, kv_heads=2, head_dim=16, ffn=256, rope_base=1e6,
               rope_base_local=1e4, sliding_window=16, swa_pattern=2, rms_eps=1e-6)
     tokens = [(i * 7 + 3) % 64 for i in range(8192)]
 
-    def pool_for(recompute, reclaim, steps, batch):
-        g = hb.HipBackend(0)
+    def pool_for(recompute, reclaim, steps, batch, streams=1):
+        g = hb.HipBackend(0, streams=streams)
         _, model = build_pair(ref, kw, seed=5, std=0.05)
         hm, ha = model.param_groups()
         ag.set_checkpointing(recompute)
@@ -684,6 +685,11 @@ def test_recompute_memory_gate(ref):
     assert b4 <= b2 * 1.05, (b2, b4)
     dense = pool_for(False, True, 3, 2)
     assert b2 < 0.9 * dense, (b2, dense)
+    # micro-batches dealt to four streams: every stream has its own pool, so the mark is that of four micro-batches in
+    # flight, and flat from there on
+    m4, m8 = pool_for(True, True, 3, 4, streams=4), pool_for(True, True, 3, 8, streams=4)
+    assert m8 <= m4 * 1.05, (m4, m8)
+    assert m4 <= 4 * b2 * 1.05, (b2, m4)
 
 
 def test_resident_step_then_sample_readback(gpu, ref):
@@ -736,3 +742,74 @@ def test_checkpoint_input_guard_on_device(gpu, ref):
         ag.set_checkpointing(False)
         gpu.uninstall()
         gpu.sync([])
+
+
+def test_micro_batches_on_several_streams(gpu, ref):
+    """Six sequential micro-batches (the reference's call pattern, train-gpu.ts:200-219) on the backend's four streams:
+    micro-batch i runs on stream i mod 4 with that stream's own parameter-gradient accumulators, summed in stream order
+    before the first reader. Losses equal, and every gradient within the parity bound of, the oracle's sequential
+    accumulation; two runs are bit-identical; a one-stream backend gives the same losses bit for bit and the same
+    gradients up to the order of six additions."""
+    hb = mod("hip_backend")
+    assert gpu._nstreams == 4
+    kw = REAL["smollm2"]
+    rmodel, model = build_pair(ref, kw, seed=31, std=0.05)
+    seqs = batches(ref, kw["vocab"], 150, 6, seed=32, mask_every=9)
+    l1, g1 = hip_step(gpu, model, seqs, False, 150)
+    l2, g2 = hip_step(gpu, model, seqs, False, 150)
+    assert l1.tobytes() == l2.tobytes() and all(g1[n].tobytes() == g2[n].tobytes() for n in g1), "run-to-run"
+    ref.PARALLEL_BWD = True
+    ref.set_threads(min(16, ref.max_threads()))
+    try:
+        lr, gr = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.PARALLEL_BWD = False
+        ref.set_threads(1)
+    compare(l1, g1, lr, gr, "six micro-batches on four streams")
+    one = hb.HipBackend(0, streams=1)
+    try:
+        _, model1 = build_pair(ref, kw, seed=31, std=0.05)
+        ls, gs = hip_step(one, model1, seqs, False, 150)
+    finally:
+        one.destroy()
+    assert ls.tobytes() == l1.tobytes()
+    for n in gs:
+        assert_close(g1[n], gs[n], f"four streams vs one, {n}", rel_l2=2e-6, max_rel=2e-5)
+
+
+def test_grad_fold_sums_in_source_order(gpu):
+    """gt_grad_fold: dst (+)= src0 + src1 + ... per tensor in one launch, bit for bit the f32 sums taken in that order;
+    absent sources skipped, store and accumulate, sizes that are no multiple of four and an unaligned tensor."""
+    import ctypes as C
+    lib = mod("lib")
+    rs = np.random.RandomState(3)
+    sizes = [8192 * 3 + 5, 7, 4096, 100000]
+    ns = 3
+    dst0 = [rs.standard_normal(n).astype(np.float32) for n in sizes]
+    srcs = [[rs.standard_normal(n).astype(np.float32) for _ in range(ns)] for n in sizes]
+    present = [[1, 1, 1], [1, 0, 1], [0, 0, 1], [1, 1, 0]]
+    accs = [1, 0, 1, 0]
+    big = gpu.create_state_buffer(4 * (sizes[1] + 1))               # tensor 1's destination starts 4 bytes into a buffer
+    db = [gpu.create_state_buffer(4 * n) for n in sizes]
+    db[1] = big + 4
+    for b, a in zip(db, dst0):
+        lib.check(gpu.ctx, lib.lib.gt_h2d(gpu.ctx, b, a.ctypes.data_as(C.c_void_p), a.nbytes), "h2d")
+    sb = []
+    for i, n in enumerate(sizes):
+        for s_ in range(ns):
+            if present[i][s_]:
+                b = gpu.create_state_buffer(4 * n)
+                gpu.write_state_buffer(b, srcs[i][s_])
+                sb.append(b)
+            else:
+                sb.append(0)
+    n = len(sizes)
+    lib.check(gpu.ctx, lib.lib.gt_grad_fold(gpu.ctx, n, (C.c_uint64 * n)(*db), (C.c_int * n)(*accs), ns, (C.c_uint64 * (n * ns))(*sb),
+                                            (C.c_int64 * n)(*sizes)), "gt_grad_fold")
+    for i in range(n):
+        want = dst0[i].copy() if accs[i] else None
+        for s_ in range(ns):
+            if present[i][s_]:
+                want = srcs[i][s_].copy() if want is None else (want + srcs[i][s_]).astype(np.float32)
+        got = gpu.read_state_buffer(db[i], sizes[i])
+        assert np.array_equal(got, want), f"tensor {i}"
