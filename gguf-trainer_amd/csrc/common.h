@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <string.h>
 #include <map>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -23,6 +24,7 @@ struct gt_ctx {
   int num_cu = 256;
   uint64_t live_bytes = 0;
   std::map<uint64_t, size_t> allocs;
+  std::set<void *> adamws, muons;              // live optimizer objects: gt_ctx_destroy releases what the caller did not
   // grow-only scratch for kernels that need more than inputs and outputs (split-K partials,
   // per-block dw partials, embedding sort keys). One stream => one user at a time.
   void *ws = nullptr; size_t ws_bytes = 0;
@@ -66,6 +68,7 @@ __device__ __forceinline__ void note_bad_id(int *bad, int what, int64_t row, int
   bad[1] = (int)row; bad[2] = value; bad[3] = bound; bad[0] = what;
 }
 int gt_report_bad_id(gt_ctx *ctx);
+void optim_release_all(gt_ctx *ctx);            // optim.hip
 int rmsnorm_static_init(gt_ctx *ctx);           // norm.hip: looks up the static scratch array's address on ctx's device
 // gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
 int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc);

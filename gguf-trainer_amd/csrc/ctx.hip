@@ -62,6 +62,7 @@ int gt_ctx_destroy(gt_ctx *ctx) {
   if (!ctx) return 0;
   hipSetDevice(ctx->device);
   hipStreamSynchronize(ctx->stream);
+  optim_release_all(ctx);
   for (auto &kv : ctx->allocs) hipFree(reinterpret_cast<void *>(kv.first));
   for (auto &kv : ctx->rope_tables) hipFree(kv.second);
   for (auto &e : ctx->prof) { hipEventDestroy(e.a); hipEventDestroy(e.b); }

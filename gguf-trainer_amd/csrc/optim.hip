@@ -277,25 +277,53 @@ static int newton_schulz_run(gt_ctx *ctx, const MuonGroup &G, int steps, int npa
   return 0;
 }
 
+static void group_release(gt_ctx *ctx, MuonGroup &G) {
+  (void)hipStreamSynchronize(ctx->stream);
+  float *bufs[] = {G.U, G.X, G.BX, G.A, G.AA, G.part};
+  for (float *b : bufs) if (b) (void)hipFree(b);
+  G.U = G.X = G.BX = G.A = G.AA = G.part = nullptr;
+  if (G.w) (void)hipFree(G.w);
+  if (G.g) (void)hipFree(G.g);
+  if (G.buf) (void)hipFree(G.buf);
+  G.w = G.g = G.buf = nullptr;
+  ctx->live_bytes -= G.bytes;
+  G.bytes = 0;
+}
+// all of a group's work buffers, or none (what one failed allocation leaves behind is freed)
 static int group_alloc(gt_ctx *ctx, MuonGroup &G) {
   const size_t elems = (size_t)G.rows * G.cols * G.count, r = std::min(G.rows, G.cols);
-  GT_HIP(ctx, hipMalloc((void **)&G.U, elems * 4));
-  GT_HIP(ctx, hipMalloc((void **)&G.X, elems * 4));
-  GT_HIP(ctx, hipMalloc((void **)&G.BX, elems * 4));
-  GT_HIP(ctx, hipMalloc((void **)&G.A, r * r * G.count * 4));
-  GT_HIP(ctx, hipMalloc((void **)&G.AA, r * r * G.count * 4));
-  GT_HIP(ctx, hipMalloc((void **)&G.part, (size_t)RED_BLOCKS * G.count * 4));
+  float **dst[] = {&G.U, &G.X, &G.BX, &G.A, &G.AA, &G.part};
+  const size_t bytes[] = {elems * 4, elems * 4, elems * 4, r * r * G.count * 4, r * r * G.count * 4, (size_t)RED_BLOCKS * G.count * 4};
+  for (int i = 0; i < 6; i++) {
+    hipError_t e = hipMalloc((void **)dst[i], bytes[i]);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      group_release(ctx, G);
+      GT_FAIL(ctx, "Muon work buffers: hipMalloc of %zu bytes failed: %s", bytes[i], hipGetErrorString(e));
+    }
+  }
   G.bytes = elems * 12 + r * r * G.count * 8 + (size_t)RED_BLOCKS * G.count * 4;
   ctx->live_bytes += G.bytes;
   return 0;
 }
-static void group_release(gt_ctx *ctx, MuonGroup &G) {
-  (void)hipStreamSynchronize(ctx->stream);
-  (void)hipFree(G.U); (void)hipFree(G.X); (void)hipFree(G.BX); (void)hipFree(G.A); (void)hipFree(G.AA); (void)hipFree(G.part);
-  if (G.w) (void)hipFree(G.w);
-  if (G.g) (void)hipFree(G.g);
-  if (G.buf) (void)hipFree(G.buf);
-  ctx->live_bytes -= G.bytes;
+
+static void adamw_release(gt_adamw *o) {
+  if (o->chunks) (void)hipFree(o->chunks);
+  if (o->ptrs) (void)hipFree(o->ptrs);
+  if (o->partial) (void)hipFree(o->partial);
+  if (o->scale) (void)hipFree(o->scale);
+  delete o;
+}
+static void muon_release(gt_ctx *ctx, gt_muon *o) {
+  for (auto &G : o->groups) group_release(ctx, G);
+  delete o;
+}
+// optimizers a caller never destroyed go with their context
+void optim_release_all(gt_ctx *ctx) {
+  for (void *o : ctx->adamws) adamw_release(static_cast<gt_adamw *>(o));
+  for (void *o : ctx->muons) muon_release(ctx, static_cast<gt_muon *>(o));
+  ctx->adamws.clear();
+  ctx->muons.clear();
 }
 
 extern "C" {
@@ -316,14 +344,19 @@ int gt_adamw_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const 
   }
   o->nchunks = (int)ch.size();
   size_t cb = std::max<size_t>(1, ch.size()) * sizeof(Chunk), pb = std::max<size_t>(1, tp.size()) * sizeof(TensorPtrs);
-  GT_HIP(ctx, hipMalloc((void **)&o->chunks, cb));
-  GT_HIP(ctx, hipMalloc((void **)&o->ptrs, pb));
-  GT_HIP(ctx, hipMalloc((void **)&o->partial, std::max<size_t>(1, ch.size()) * 4));
-  GT_HIP(ctx, hipMalloc((void **)&o->scale, 8));
-  if (!ch.empty()) GT_HIP(ctx, hipMemcpy(o->chunks, ch.data(), ch.size() * sizeof(Chunk), hipMemcpyHostToDevice));
-  if (!tp.empty()) GT_HIP(ctx, hipMemcpy(o->ptrs, tp.data(), tp.size() * sizeof(TensorPtrs), hipMemcpyHostToDevice));
   float one[2] = {1.0f, 0.0f};
-  GT_HIP(ctx, hipMemcpy(o->scale, one, 8, hipMemcpyHostToDevice));
+  hipError_t e;
+  if ((e = hipMalloc((void **)&o->chunks, cb)) != hipSuccess || (e = hipMalloc((void **)&o->ptrs, pb)) != hipSuccess ||
+      (e = hipMalloc((void **)&o->partial, std::max<size_t>(1, ch.size()) * 4)) != hipSuccess ||
+      (e = hipMalloc((void **)&o->scale, 8)) != hipSuccess ||
+      (!ch.empty() && (e = hipMemcpy(o->chunks, ch.data(), ch.size() * sizeof(Chunk), hipMemcpyHostToDevice)) != hipSuccess) ||
+      (!tp.empty() && (e = hipMemcpy(o->ptrs, tp.data(), tp.size() * sizeof(TensorPtrs), hipMemcpyHostToDevice)) != hipSuccess) ||
+      (e = hipMemcpy(o->scale, one, 8, hipMemcpyHostToDevice)) != hipSuccess) {
+    (void)hipGetLastError();
+    adamw_release(o);
+    GT_FAIL(ctx, "gt_adamw_create: setting up the chunk tables failed: %s", hipGetErrorString(e));
+  }
+  ctx->adamws.insert(o);
   *out = o;
   return 0;
 }
@@ -399,9 +432,9 @@ int gt_adamw_grad_norm(gt_ctx *ctx, gt_adamw *o, float *norm) {
 int gt_adamw_destroy(gt_ctx *ctx, gt_adamw *o) {
   GT_ENTER(ctx);
   if (!o) return 0;
-  hipStreamSynchronize(ctx->stream);
-  hipFree(o->chunks); hipFree(o->ptrs); hipFree(o->partial); hipFree(o->scale);
-  delete o;
+  GT_REQUIRE(ctx, ctx->adamws.erase(o) == 1, "gt_adamw_destroy: not an optimizer of this context");
+  (void)hipStreamSynchronize(ctx->stream);
+  adamw_release(o);
   return 0;
 }
 
@@ -427,16 +460,18 @@ int gt_muon_create(gt_ctx *ctx, int n, const gt_buf *w, const gt_buf *g, const g
     G.count = (int)pw.size();
     size_t tb = pw.size() * sizeof(float *);
     if (hipMalloc((void **)&G.w, tb) != hipSuccess || hipMalloc((void **)&G.g, tb) != hipSuccess ||
-        hipMalloc((void **)&G.buf, tb) != hipSuccess || group_alloc(ctx, G)) {
-      for (auto &gg : o->groups) group_release(ctx, gg);
-      delete o;
-      GT_FAIL(ctx, "gt_muon_create: out of device memory for the %dx%d group", G.rows, G.cols);
+        hipMalloc((void **)&G.buf, tb) != hipSuccess || group_alloc(ctx, G) ||
+        hipMemcpy(G.w, pw.data(), tb, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(G.g, pg.data(), tb, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(G.buf, pb.data(), tb, hipMemcpyHostToDevice) != hipSuccess) {
+      (void)hipGetLastError();
+      group_release(ctx, G);              // frees whichever of this group's buffers exist
+      muon_release(ctx, o);
+      GT_FAIL(ctx, "gt_muon_create: setting up the %dx%d group failed (out of device memory?)", G.rows, G.cols);
     }
-    (void)hipMemcpy(G.w, pw.data(), tb, hipMemcpyHostToDevice);
-    (void)hipMemcpy(G.g, pg.data(), tb, hipMemcpyHostToDevice);
-    (void)hipMemcpy(G.buf, pb.data(), tb, hipMemcpyHostToDevice);
     o->groups.push_back(G);
   }
+  ctx->muons.insert(o);
   *out = o;
   return 0;
 }
@@ -462,8 +497,8 @@ int gt_muon_step(gt_ctx *ctx, gt_muon *o, double lr) {
 int gt_muon_destroy(gt_ctx *ctx, gt_muon *o) {
   GT_ENTER(ctx);
   if (!o) return 0;
-  for (auto &G : o->groups) group_release(ctx, G);
-  delete o;
+  GT_REQUIRE(ctx, ctx->muons.erase(o) == 1, "gt_muon_destroy: not an optimizer of this context");
+  muon_release(ctx, o);
   return 0;
 }
 
@@ -475,7 +510,11 @@ int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out)
   T.rows = m; T.cols = n; T.count = 1;
   if (group_alloc(ctx, T)) return 1;
   const size_t size = (size_t)m * n;
-  GT_HIP(ctx, hipMemcpyAsync(T.U, P<void>(G), size * 4, hipMemcpyDeviceToDevice, ctx->stream));
+  hipError_t ce = hipMemcpyAsync(T.U, P<void>(G), size * 4, hipMemcpyDeviceToDevice, ctx->stream);
+  if (ce != hipSuccess) {
+    group_release(ctx, T);
+    GT_FAIL(ctx, "gt_newton_schulz: copying the matrix failed: %s", hipGetErrorString(ce));
+  }
   const unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv((int64_t)size, 256));
   // sums of squares of U only (no momentum buffer, no gradient)
   hipLaunchKernelGGL(muon_momentum_k, dim3(nb, 1), dim3(256), 0, ctx->stream, (int64_t)size, (float *const *)nullptr,

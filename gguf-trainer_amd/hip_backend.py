@@ -91,6 +91,7 @@ class HipBackend:
         self._bw_seen = False             # a backward closure has run since the last switch: the next graph root starts a micro-batch
         self._s0_barrier = False          # the first stream holds work (uploads, an optimizer step, a fold) another stream must not overtake
         self._sfold: list = []            # (tensor, entry) of parameters with a written accumulator on another stream
+        self._limbo: list = []            # entries of parameters that were released or collected: their buffers return to the pools at the next sync
         self.adapter_name = lib.gt_device_name(self._ctx).decode()
         self.attn_flash_min_t = 2048      # kept for interface parity; one kernel family serves every T here
         self.last_sync_readback_bytes = 0
@@ -334,6 +335,8 @@ class HipBackend:
                 self._s0_barrier = True
             self._entries[t] = e
             self._externals.add(t)
+            # when the tensor is collected its device buffers go back to the pools (at the next sync: queued work may still read them)
+            weakref.finalize(t, self._limbo.append, e)
         if e.external and t.requires_grad and id(t) not in self._touched_ids:
             self._touched_ids.add(id(t))
             self._touched.append(t)
@@ -499,6 +502,41 @@ class HipBackend:
             self.grad_clears_issued += 1
         return {"data": e.data, "grad": e.grad}
 
+    def release(self, tensors):
+        """Give back the device buffers of parameters that are no longer needed (a model being dropped): values, gradient
+        accumulators on every stream. They return to the pools at the next sync(); a tensor used again after that is
+        uploaded afresh."""
+        self._join()
+        for t in tensors:
+            e = self._entries.get(t)
+            if e is not None and e.external:
+                self._entries.pop(t, None)
+                self._externals.discard(t)
+                self._limbo.append(e)
+
+    def _drain_limbo(self):
+        """Called with every stream idle."""
+        seen = set()
+        while self._limbo:
+            e = self._limbo.pop()
+            if id(e) in seen:
+                continue
+            seen.add(id(e))
+            if e.data:
+                self._recycle(e.data, e.nbytes, 0)
+            if e.grad:
+                self._recycle(e.grad, e.nbytes, 0)
+            for s_, slot in (e.sgrad or {}).items():
+                self._recycle(slot[0], e.nbytes, s_)
+            e.data = e.grad = 0
+            e.sgrad = None
+        self._sfold = [(t, e) for t, e in self._sfold if e.data]
+
+    def free_state_buffer(self, b: int):
+        """Free a buffer made by create_state_buffer (waits for the first stream)."""
+        c0 = self._ctxs[0]
+        check(c0, lib.gt_free(c0, b), "gt_free")
+
     def keep_grad_on_device(self, t: Tensor):
         self._entry_for(t).keep_grad = True
 
@@ -559,6 +597,10 @@ class HipBackend:
     def set_option(self, key: str, value: int):
         """Kernel-selection switches for tests and tuning: "attn.generic", "attn.splits", "gemm.tile", "gemm.splitk", "gemm.staged",
         and "prof.sample" (time every n-th launch of a label)."""
+        if key == "attn.generic" and self._transients:
+            # an attention forward already recorded has chosen its kernel family (and may hold kept scores in that
+            # family's layout); its backward must run in the same one
+            raise RuntimeError("set_option: attn.generic cannot change while a graph is live; sync() first")
         for c in self._ctxs:
             check(c, lib.gt_set_option(c, key.encode(), int(value)), "gt_set_option")
 
@@ -639,6 +681,8 @@ class HipBackend:
         self.last_sync_readback_bytes = nbytes
         self._release_transients()
         self._scores_taken = 0
+        if self._limbo:
+            self._drain_limbo()
 
     def reclaim_step_transients(self, keep=()):
         """Free a finished micro-batch's intermediates mid-step; parameter gradients keep accumulating. Every stream is

@@ -45,6 +45,15 @@ class AdamWHip:
     def set_lr_scale(self, s: float):
         self.lr_scale = s
 
+    def destroy(self):
+        """Release the device-side tables; the moment buffers go back with the backend's state buffers."""
+        if self._h:
+            check(self.gpu.ctx, lib.gt_adamw_destroy(self.gpu.ctx, self._h), "gt_adamw_destroy")
+            self._h = C.c_void_p()
+        for b in self._m + self._v:
+            self.gpu.free_state_buffer(b)
+        self._m, self._v = [], []
+
     def zero_grad(self):
         """No-op: accumulators live on the device and are re-armed when a step has consumed them."""
 
@@ -108,6 +117,16 @@ class MuonHip:
     def set_lr_scale(self, s: float):
         self.lr = self.base_lr * s
         self.aux.set_lr_scale(s)
+
+    def destroy(self):
+        """Release the per-shape work buffers and pointer tables, the momentum buffers and the auxiliary AdamW."""
+        if self._h:
+            check(self.gpu.ctx, lib.gt_muon_destroy(self.gpu.ctx, self._h), "gt_muon_destroy")
+            self._h = C.c_void_p()
+        for b in self._bufs:
+            self.gpu.free_state_buffer(b)
+        self._bufs = []
+        self.aux.destroy()
 
     def zero_grad(self):
         self.aux.zero_grad()

@@ -813,3 +813,53 @@ def test_grad_fold_sums_in_source_order(gpu):
                 want = srcs[i][s_].copy() if want is None else (want + srcs[i][s_]).astype(np.float32)
         got = gpu.read_state_buffer(db[i], sizes[i])
         assert np.array_equal(got, want), f"tensor {i}"
+
+
+def test_parameter_buffers_return_when_released_or_collected(gpu, ref):
+    """Device buffers of parameters (values, gradient accumulators, the per-stream ones too) go back to the pool when the
+    host releases the tensors or drops its last reference to them: the next model of the same shape reuses them and the
+    pool does not grow. Optimizers release their tables and moments with destroy()."""
+    import gc
+    ag, optim = mod("autograd"), mod("optim")
+    kw = SMALL["llama"]
+    seqs = batches(ref, kw["vocab"], 19, 3, seed=5)
+
+    def one_model(explicit):
+        _, model = build_pair(ref, kw, seed=3, std=0.1)
+        opt = optim.AdamWHip(gpu, model.params(), lr=1e-3)
+        hip_step(gpu, model, seqs, False, 19)
+        gpu.install()
+        try:
+            opt.record_step()
+            gpu.sync([])
+        finally:
+            gpu.uninstall()
+        opt.destroy()
+        if explicit:
+            gpu.release(model.params())
+        del model, opt
+        gc.collect()
+        gpu.sync([])
+
+    one_model(True)
+    pool0, res0 = gpu._pool_bytes, gpu.resident_bytes()
+    one_model(True)
+    assert (gpu._pool_bytes, gpu.resident_bytes()) == (pool0, res0), "explicit release"
+    one_model(False)
+    assert (gpu._pool_bytes, gpu.resident_bytes()) == (pool0, res0), "collected tensors"
+
+
+def test_kernel_family_cannot_change_under_a_live_graph(gpu, ref):
+    ag = mod("autograd")
+    r = ref.Mulberry32(4)
+    q, k, v = (ag.Tensor(r.fill_randn([128, 2 * 64], 0.5), [128, 128], True) for _ in range(3))
+    gpu.install()
+    try:
+        out = ag.attention(q, k, v, 128, 2, 2, 64, 0)
+        with pytest.raises(RuntimeError, match="attn.generic cannot change"):
+            gpu.set_option("attn.generic", 1)
+        gpu.sync([out])
+        gpu.set_option("attn.generic", 1)
+        gpu.set_option("attn.generic", 0)
+    finally:
+        gpu.uninstall()
