@@ -78,13 +78,29 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 template <int ROWS> struct TileIO {
   static constexpr int LDT = ROWS + 4;
   static constexpr int PER = (ROWS * HD / 4) / 256;
-  __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ src, size_t stride, int row0, int rmax, int tid) {
+  // Where this thread's float4 units sit inside a tile whose first row is at `base`: computed once per kernel. A stage's
+  // loads are then `base + off[i]` with a wave-uniform base that advances from stage to stage (scalar arithmetic) and a
+  // constant 32-bit lane offset: no per-load index arithmetic, and no bounds test while the whole tile lies inside the
+  // matrix (nvalid >= ROWS, wave-uniform). Only a tile that crosses the last row takes the tested path (zeros beyond it).
+  __device__ static __forceinline__ void offsets(unsigned (&off)[PER], size_t stride, int tid) {
 #pragma unroll
     for (int i = 0; i < PER; i++) {
       int u = tid + i * 256, row = u / (HD / 4), c4 = u % (HD / 4);
-      v4f v = {0.f, 0.f, 0.f, 0.f};
-      if (row0 + row < rmax) v = *reinterpret_cast<const v4f *>(src + (size_t)(row0 + row) * stride + c4 * 4);
-      reg[i] = v;
+      off[i] = (unsigned)(row * stride + c4 * 4);
+    }
+  }
+  __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ base, const unsigned (&off)[PER], int nvalid, int tid) {
+    if (nvalid >= ROWS) {
+#pragma unroll
+      for (int i = 0; i < PER; i++) reg[i] = *reinterpret_cast<const v4f *>(base + off[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < PER; i++) {
+        int row = (tid + i * 256) / (HD / 4);
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (row < nvalid) v = *reinterpret_cast<const v4f *>(base + off[i]);
+        reg[i] = v;
+      }
     }
   }
   __device__ static __forceinline__ void store_rows(const v4f (&reg)[PER], float *lds, int tid) {
@@ -229,20 +245,22 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
   float m = NEG_BIG, l = 0.f;
 
   v4f pk[IO::PER], pv[IO::PER];
-  IO::load(pk, kb, kstr, kt_lo * KT, p.T, tid);
-  IO::load(pv, vb, kstr, kt_lo * KT, p.T, tid);
+  unsigned koffs[IO::PER];
+  IO::offsets(koffs, kstr, tid);
+  IO::load(pk, kb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
+  IO::load(pv, vb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
   for (int kt = kt_lo; kt <= kt_hi; kt++) {
     __syncthreads();
     IO::store_rows(pk, sK, tid);
     IO::store_t(pv, sVt, tid);
     __syncthreads();
     if (kt < kt_hi) {
-      IO::load(pk, kb, kstr, (kt + 1) * KT, p.T, tid);
-      IO::load(pv, vb, kstr, (kt + 1) * KT, p.T, tid);
+      IO::load(pk, kb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
+      IO::load(pv, vb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
     }
     if (tq0 >= p.T) continue;
     float pr[NSUB][16];
-    bool act[NSUB];
+    bool act[NSUB], msk[NSUB];
     bool any_act = false;
     float mx = NEG_BIG;
 #pragma unroll
@@ -258,6 +276,7 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
         for (int r = 0; r < 16; r++) __builtin_nontemporal_store(s[r], sb + acc_row(r, g) * 32);   // read again only in the backward
       }
       const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
+      msk[sub] = need_mask;
       if (need_mask) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -287,12 +306,21 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
     for (int sub = 0; sub < NSUB; sub++) {
       if (!act[sub]) continue;
       float ls = 0.f;
+      if (msk[sub]) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        // a masked score is NEG_BIG; with m still NEG_BIG (no visible key yet) the difference would be 0
-        float e = pr[sub][r] > -1.0e29f ? fast_exp2(pr[sub][r] - m) : 0.f;
-        pr[sub][r] = e;
-        ls += e;
+        for (int r = 0; r < 16; r++) {
+          // a masked score is NEG_BIG; with m still NEG_BIG (no visible key yet) the difference would be 0
+          float e = pr[sub][r] > -1.0e29f ? fast_exp2(pr[sub][r] - m) : 0.f;
+          pr[sub][r] = e;
+          ls += e;
+        }
+      } else {          // every pair of the tile is visible: every score is a number and m is at least their maximum
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float e = fast_exp2(pr[sub][r] - m);
+          pr[sub][r] = e;
+          ls += e;
+        }
       }
       l += ls;
       t_dot_acc<IO::LDT>(oacc, sVt, sub * 32, pr[sub], l32, g);
@@ -361,8 +389,10 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
     for (int r = 0; r < 16; r++) dacc[dt][r] = 0.f;
 
   v4f pk[IO::PER], pv[IO::PER];
-  IO::load(pk, kb, kstr, kt_lo * KT, p.T, tid);
-  IO::load(pv, vb, kstr, kt_lo * KT, p.T, tid);
+  unsigned koffs[IO::PER];
+  IO::offsets(koffs, kstr, tid);
+  IO::load(pk, kb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
+  IO::load(pv, vb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
   for (int kt = kt_lo; kt <= kt_hi; kt++) {
     __syncthreads();
     IO::store_rows(pk, sK, tid);
@@ -370,8 +400,8 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
     IO::store_rows(pv, sV, tid);
     __syncthreads();
     if (kt < kt_hi) {
-      IO::load(pk, kb, kstr, (kt + 1) * KT, p.T, tid);
-      IO::load(pv, vb, kstr, (kt + 1) * KT, p.T, tid);
+      IO::load(pk, kb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
+      IO::load(pv, vb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
     }
     if (tq0 >= p.T) continue;
 #pragma unroll
@@ -458,6 +488,10 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   float pstat = 0.f;
   // this wavefront's block of kept scores for a query stage: lane = key row of the block, queries 8a + 4g + (0..3)
   const float *scw = KS ? sco + (((size_t)b * p.Hq + h) * (p.T / 32) + sk0 / 32) * (p.T / 32) * 1024 + l32 * 32 + 4 * g : nullptr;
+  const float *qb = q + (size_t)b * p.T * qstr + (size_t)h * HD;
+  const float *gb = go + (size_t)b * p.T * qstr + (size_t)h * HD;
+  unsigned qoffs[IO::PER];
+  IO::offsets(qoffs, qstr, tid);
   auto prefetch = [&](int it) {
     int qt = qt_lo + it;
     if (KS) {
@@ -467,10 +501,8 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
         for (int a = 0; a < 4; a++) psc[a] = *reinterpret_cast<const v4f *>(scw + (size_t)qt * 1024 + 8 * a);
       }
     }
-    const float *qb = q + (size_t)b * p.T * qstr + (size_t)h * HD;
-    const float *gb = go + (size_t)b * p.T * qstr + (size_t)h * HD;
-    IO::load(pq, qb, qstr, qt * QT, p.T, tid);
-    IO::load(pg, gb, qstr, qt * QT, p.T, tid);
+    IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, p.T - qt * QT, tid);
+    IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, p.T - qt * QT, tid);
     if (tid < 2 * QT) {
       int tt = qt * QT + (tid % QT);
       size_t si = ((size_t)b * p.Hq + h) * p.T + tt;
