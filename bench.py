@@ -231,6 +231,8 @@ def micro_kernels(gpu, L, reps=10):
         # a plain streaming kernel of known size (read 100.7 MB, write 100.7 MB): the yardstick the FETCH_SIZE /
         # WRITE_SIZE counters are scaled by
         L.check(c, lib.gt_scale_fwd(c, R * F, gate, 1.0, dgate), "scale")
+        # and the same copy over as many bytes as RMSNorm backward moves (113 MB in all): the floor for a launch that small
+        L.check(c, lib.gt_add_fwd(c, R * H, X, g_n, dx_n), "add")
 
     run()
     gpu.start_profile("")
@@ -241,7 +243,8 @@ def micro_kernels(gpu, L, reps=10):
     names = {"gemm.nn": ("dX = dY.W  [16384x576x1536]", "mfma"), "gemm.tn": ("dW = dY^T.X [1536x576x16384]", "mfma"),
              "ce.bwd": ("softmax-CE backward [16384x49152]", "hbm"), "ce": ("CE forward statistics [16384x49152]", "hbm"),
              "rmsnorm.bwd": ("RMSNorm backward [16384x576]", "hbm"), "glu.bwd": ("SwiGLU backward [16384x1536]", "hbm"),
-             "scale": ("copy-like yardstick: out = 1.0*x [16384x1536]", "hbm")}
+             "scale": ("copy-like yardstick: out = 1.0*x [16384x1536]", "hbm"),
+             "add": ("yardstick at the RMSNorm size: out = a + b [16384x576], 113 MB like RMSNorm backward", "hbm")}
     for label, (ms, cnt, work) in prof.items():
         key = next((k for k in sorted(names, key=len, reverse=True) if label == k or label.startswith(k + ".")), None)
         if key is None or cnt == 0:

@@ -99,15 +99,20 @@ __global__ __launch_bounds__(256) void ce_seq_loss(int T, const float *__restric
 // of a row, spans of a row numbered fastest: workgroups that run at the same time then work on neighbouring memory,
 // which the DRAM pages like much better than 2048 rows streamed side by side. Each thread has four float4 loads in
 // flight; z and dz are touched exactly once, so both use streaming (non-temporal) accesses.
+// SOFT: the dense half of the sparse-teacher loss, dz (+)= seed*inv_denom * mass[row] * exp(z - lse): no one-hot term (the
+// teacher terms are subtracted by soft_ce_bwd_q afterwards), the row's scale carries its teacher mass, tgt holds k ids per
+// row and a row is ignored when its first id is -1, inv_denom is one number.
 #define CE_SPAN 4096
+template <bool SOFT>
 __global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, int spans, const float *__restrict__ z,
                                                 const int *__restrict__ tgt, const float *__restrict__ inv_denom,
-                                                const float *__restrict__ lse, float seed, float *dz, int acc) {
+                                                const float *__restrict__ lse, float seed, float *dz, int acc,
+                                                const float *__restrict__ mass, int k) {
   const int64_t row = blockIdx.x / spans;
   const int span = blockIdx.x % spans;
-  int g = tgt[row];
+  int g = SOFT ? (tgt[row * k] == IGN ? IGN : -2) : tgt[row];     // -2: no column matches
   if (g == IGN && acc) return;                         // untouched, as the reference leaves it
-  const float sc = seed * inv_denom[row / T];
+  const float sc = SOFT ? seed * mass[row] : seed * inv_denom[row / T];
   const float ls = lse[row];
   const float *zr = z + row * V;
   float *dr = dz + row * V;
@@ -227,20 +232,8 @@ __global__ __launch_bounds__(256) void sum_scale_k(int n, const float *__restric
   a = block_sum<4>(a, sm);
   if (threadIdx.x == 0) out[0] = a * sc;
 }
-// dense half: dz (+)= sc*mass*softmax; sparse half by one thread per row afterwards (duplicate ids
-// in a row are applied one after another by that thread, so they cannot race: wgsl.ts:1086-1090)
-__global__ __launch_bounds__(256) void soft_ce_bwd_p(int V, int k, const float *__restrict__ z, const int *__restrict__ tid,
-                                                     const float *__restrict__ lse, const float *__restrict__ mass, float sc,
-                                                     float *dz, int acc) {
-  int64_t row = blockIdx.x;
-  bool ign = tid[row * k] == IGN;
-  if (ign && acc) return;
-  const float ls = lse[row], w = sc * mass[row];
-  for (int i = blockIdx.y * 256 + threadIdx.x; i < V; i += gridDim.y * 256) {
-    float o = ign ? 0.f : w * __expf(z[row * V + i] - ls);
-    dz[row * V + i] = acc ? dz[row * V + i] + o : o;
-  }
-}
+// sparse half of the soft loss, one thread per row after the dense half (ce_bwd_k<true>): duplicate ids in a row are
+// applied one after another by that thread, so they cannot race (wgsl.ts:1086-1090)
 __global__ __launch_bounds__(64) void soft_ce_bwd_q(int rows, int V, int k, const int *__restrict__ tid,
                                                     const float *__restrict__ tq, float sc, float *dz, int *bad) {
   int64_t row = (int64_t)blockIdx.x * 64 + threadIdx.x;
@@ -251,8 +244,6 @@ __global__ __launch_bounds__(64) void soft_ce_bwd_q(int rows, int V, int k, cons
     dz[row * V + id] -= sc * tq[row * k + j];
   }
 }
-
-static inline unsigned row_chunks(int V) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>(cdiv(V, 4 * 256 * 4), 64)); }
 
 extern "C" {
 int gt_ce_fwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets, gt_buf inv_denom, gt_buf loss, gt_buf lse) {
@@ -278,8 +269,9 @@ int gt_ce_bwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets
   ProfScope ps(ctx, "ce.bwd", 8.0 * rows * V);          // read z, write dz
   const int spans = (int)cdiv(V, CE_SPAN);
   GT_REQUIRE(ctx, (int64_t)rows * spans < (int64_t)1 << 31, "gt_ce_bwd: %d rows x %d logits is more than one launch covers", rows, V);
-  hipLaunchKernelGGL(ce_bwd_k, dim3((unsigned)((int64_t)rows * spans)), dim3(256), 0, ctx->stream, V, T, spans, P<const float>(logits),
-                     P<const int>(targets), P<const float>(inv_denom), P<const float>(lse), seed, P<float>(dlogits), acc);
+  hipLaunchKernelGGL(ce_bwd_k<false>, dim3((unsigned)((int64_t)rows * spans)), dim3(256), 0, ctx->stream, V, T, spans, P<const float>(logits),
+                     P<const int>(targets), P<const float>(inv_denom), P<const float>(lse), seed, P<float>(dlogits), acc,
+                     (const float *)nullptr, 1);
   GT_LAUNCHED(ctx);
   return 0;
 }
@@ -324,7 +316,7 @@ int gt_soft_ce_fwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf te
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 1 && V >= 1 && k >= 1 && logits && teacher_ids && teacher_probs && loss && lse && row_mass,
              "gt_soft_ce_fwd: bad arguments");
-  ProfScope ps(ctx, "softce");
+  ProfScope ps(ctx, "softce", 4.0 * rows * V);
   void *ws;
   if (gt_ws_reserve(ctx, (size_t)rows * sizeof(float), &ws)) return 1;
   hipLaunchKernelGGL(soft_ce_fwd_rows, dim3(rows), dim3(256), 0, ctx->stream, V, k, P<const float>(logits),
@@ -340,10 +332,13 @@ int gt_soft_ce_bwd(gt_ctx *ctx, int rows, int V, int k, gt_buf logits, gt_buf te
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 1 && V >= 1 && k >= 1 && logits && teacher_ids && teacher_probs && lse && row_mass && dlogits,
              "gt_soft_ce_bwd: bad arguments");
-  ProfScope ps(ctx, "softce.bwd");
+  ProfScope ps(ctx, "softce.bwd", 8.0 * rows * V);
   float sc = seed * inv_denom;
-  hipLaunchKernelGGL(soft_ce_bwd_p, dim3(rows, row_chunks(V)), dim3(256), 0, ctx->stream, V, k, P<const float>(logits),
-                     P<const int>(teacher_ids), P<const float>(lse), P<const float>(row_mass), sc, P<float>(dlogits), acc);
+  const int spans = (int)cdiv(V, CE_SPAN);
+  GT_REQUIRE(ctx, (int64_t)rows * spans < (int64_t)1 << 31, "gt_soft_ce_bwd: %d rows x %d logits is more than one launch covers", rows, V);
+  hipLaunchKernelGGL(ce_bwd_k<true>, dim3((unsigned)((int64_t)rows * spans)), dim3(256), 0, ctx->stream, V, rows, spans, P<const float>(logits),
+                     P<const int>(teacher_ids), (const float *)nullptr, P<const float>(lse), sc, P<float>(dlogits), acc,
+                     P<const float>(row_mass), k);
   GT_LAUNCHED(ctx);
   hipLaunchKernelGGL(soft_ce_bwd_q, dim3((unsigned)cdiv(rows, 64)), dim3(64), 0, ctx->stream, rows, V, k,
                      P<const int>(teacher_ids), P<const float>(teacher_probs), sc, P<float>(dlogits), ctx->bad_dev);
