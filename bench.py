@@ -25,13 +25,15 @@ PKG = "gguf-trainer_amd"
 PEAK_FP32_MFMA = 157.3e12      # MI355X dense FP32 matrix peak, FLOP/s
 PEAK_HBM = 8.0e12              # B/s
 PROF_SAMPLE = 4                # the timed region brackets about 1 in 4 launches of a GEMM label with HIP events
-# L2-miss traffic per launch (bytes) of the two backward GEMM kernels that lead the step, from two rocprofv3 --pmc
-# passes over this file (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the factors read off a plain streaming kernel of known
-# size; see profiles/bench_smollm2_135m_pmc_fetch_write.txt). Averages over the shapes each label serves in the step (the NN label:
-# 60 summed sibling products, the 30 dX of the o projection and the readout's).
-MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (60 * (2 * 110763.7 + 36864.0) + 30 * (2 * 29758.3 + 36864.3) + (2 * 4481555.6 + 36864.3)) / 91 * 1024,
-                    "gemm.tn.128x96x32.splitk": (2 * 91867.3 + 48384.1) * 1024,
-                    "gemm.tn.64x192x32.splitk": (90 * 360.1 + 180 * 126.8 + 180 * 67.0) / 450 * 1048576}
+# L2-miss traffic per launch (bytes) of the backward GEMM labels that lead the step, from two rocprofv3 --pmc passes over
+# this file made separately (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the factors read off a plain streaming kernel of known
+# size; see profiles/bench_smollm2_135m_pmc_fetch_write.txt). Averages over the shapes each label serves in the step: the NN
+# label is 30 summed q+k+v products, 30 summed gate+up products, the 30 dX of the o projection and the readout's; the grouped
+# TN labels include their reduction pass.
+MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (30 * (2 * 50006.6 + 36864.7) + 30 * (2 * 166347.9 + 36864.7) + 30 * (2 * 29994.5 + 36866.5) +
+                                          (2 * 4173488.3 + 36866.5)) / 91 * 1024,
+                    "gemm.tn.group.128x96.splitk": ((24 * 1303.5 + 18 * 1117.2) / 42 + 151.9) * 1048576,
+                    "gemm.tn.group.64x192.splitk": ((21 * 1137.6 + 12 * 1400.9) / 33 + 151.9) * 1048576}
 
 SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                rope_base=100000.0, rms_eps=1e-5, tie=True)
