@@ -44,6 +44,7 @@
 // dQ, query stages in dK/dV) into that many workgroups, which write partial results (unnormalised output with
 // its running maximum and sum; partial dQ; dK/dV slices) that a second kernel folds in split order.
 #include <algorithm>
+#include <type_traits>
 #include "common.h"
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -136,11 +137,12 @@ __device__ __forceinline__ void load_row_regs(float (&reg)[HD / 2], const float 
 
 // acc = Tile(32 rows starting at `rows`) . reg^T : A = rows of the row-major tile, B = this lane's registers.
 // The LDS reads are issued eight b128 at a time, ahead of the MFMAs that consume them.
+template <int NBMAX = 8>
 __device__ __forceinline__ v16f rows_dot_regs(const float *rows, const float (&reg)[HD / 2], int l32, int g) {
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
-  constexpr int NB = HD / 8 < 8 ? HD / 8 : 8;       // b128 reads in flight per batch
+  constexpr int NB = HD / 8 < NBMAX ? HD / 8 : NBMAX;       // b128 reads in flight per batch
 #pragma unroll
   for (int j0 = 0; j0 < HD / 8; j0 += NB) {
     v4f a[NB];
@@ -155,10 +157,10 @@ __device__ __forceinline__ v16f rows_dot_regs(const float *rows, const float (&r
 }
 
 // out[dt] += TileT(cols [col0, col0+32)) . w : A = the transposed tile (stride LDT), B = 16 accumulator-ordered weights
-template <int LDT>
+template <int LDT, int INFLIGHT = 8>
 __device__ __forceinline__ void t_dot_acc(v16f (&out)[HD / 32], const float *ldst, int col0, const float (&w)[16], int l32, int g) {
   constexpr int DT = HD / 32;
-  constexpr int QB = DT <= 2 ? 4 : 2;          // column chunks fetched ahead: 8 b128 reads in flight either way
+  constexpr int QB = INFLIGHT / DT >= 4 ? 4 : (INFLIGHT / DT >= 2 ? 2 : 1);    // column chunks fetched ahead: INFLIGHT b128 reads in flight
 #pragma unroll
   for (int q0 = 0; q0 < 4; q0 += QB) {
     v4f a[DT][QB];
@@ -473,7 +475,9 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   const int qt_hi = t_last / QT;
   const int nqt = qt_hi - qt_lo + 1;
   const int wave_t_hi = p.window > 0 ? sk0 + 31 + p.window - 1 : p.T - 1;   // last query that sees a key of this wave
-  const bool ragged_k = sk0 + 31 >= p.T;
+  // queries that see this lane's key s: s ... min(T - 1, s + window - 1); as an unsigned span from s (none for a key past the end)
+  const unsigned span = sv ? (unsigned)((p.window > 0 ? min(p.T - 1, s + p.window - 1) : p.T - 1) - s) : 0u;
+  const unsigned dead = sv ? 0u : 0x40000000u;      // added to every relative index of a key past the end: beyond any span
 
   v16f kacc[HD / 32], vacc[HD / 32];
 #pragma unroll
@@ -538,32 +542,52 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
       }
       continue;
     }
-    if constexpr (!KS) sc = rows_dot_regs(sQ, kreg, l32, g);
-    v16f dp = rows_dot_regs(sG, vreg, l32, g);
-    // fully visible tile: every query is at or after every key of the wave, inside the window, and in range
-    const bool need_mask = ragged_k || t0 < sk0 + 31 || t0 + 31 >= p.T || (p.window > 0 && t0 + 31 > sk0 + p.window - 1);
+    // at head dim 128 without kept scores both operand rows live in registers (128 of them): four LDS reads in flight
+    // instead of eight keep the kernel inside the register file
+    constexpr int DKV_NB = (HD >= 128 && !KS) ? 4 : 8;
+    if constexpr (!KS) sc = rows_dot_regs<DKV_NB>(sQ, kreg, l32, g);
+    // The stage as straight-line code. A pair (query tq, key s) is live when s <= tq <= last query that sees s: one
+    // unsigned compare per element against this lane's span (computed once per kernel), applied to every tile: a
+    // wave-uniform "does this tile need a mask" test would cut the stage into basic blocks, and the scheduler cannot
+    // move an instruction across those. Order: the probabilities need the scores only, so their exponentials are written
+    // between the issue of the dP contraction and its first use, and the dV contraction (which needs the probabilities
+    // only) between dP and the dS arithmetic: the vector ALU work has independent MFMAs to run under instead of sitting
+    // between two dependent blocks, and the group barriers ask for that interleaving (one MFMA, a few vector
+    // instructions, and again).
+    v16f dp = rows_dot_regs<DKV_NB>(sG, vreg, l32, g);
     float pr[16], ds[16];
+    const unsigned rel0 = (unsigned)(t0 + 4 * g - s) + dead;          // query index relative to this lane's key, element (a, j) adds 8a + j
 #pragma unroll
     for (int a = 0; a < 4; a++) {
-      v4f lv = *reinterpret_cast<const v4f *>(sL + 8 * a + 4 * g), dv4 = *reinterpret_cast<const v4f *>(sD + 8 * a + 4 * g);
+      v4f lv = *reinterpret_cast<const v4f *>(sL + 8 * a + 4 * g);
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        int r = 4 * a + j;
-        float e = fast_exp2(sc[r] - lv[j]);
-        if (need_mask) {
-          int tq = t0 + 8 * a + 4 * g + j;
-          if (!(sv && tq < p.T && s <= tq && (p.window == 0 || s + p.window > tq))) e = 0.f;
-        }
-        pr[r] = e;
-        ds[r] = e * (dp[r] - dv4[j]) * p.scale;
+        float e = fast_exp2(sc[4 * a + j] - lv[j]);
+        pr[4 * a + j] = (rel0 + (unsigned)(8 * a + j)) <= span ? e : 0.f;
       }
+    }
+#pragma unroll
+    for (int i = 0; i < HD / 2; i++) {          // dP with the exponentials
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+    t_dot_acc<IO::LDT, DKV_NB>(vacc, sGt, 0, pr, l32, g);
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+      v4f dv4 = *reinterpret_cast<const v4f *>(sD + 8 * a + 4 * g);
+#pragma unroll
+      for (int j = 0; j < 4; j++) ds[4 * a + j] = pr[4 * a + j] * (dp[4 * a + j] - dv4[j]) * p.scale;
+    }
+#pragma unroll
+    for (int i = 0; i < HD / 2; i++) {          // dV with the dS arithmetic
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
     }
     if (dsb) {
 #pragma unroll
       for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = ds[r];
     }
-    t_dot_acc<IO::LDT>(vacc, sGt, 0, pr, l32, g);
-    t_dot_acc<IO::LDT>(kacc, sQt, 0, ds, l32, g);
+    t_dot_acc<IO::LDT, DKV_NB>(kacc, sQt, 0, ds, l32, g);
   }
   if (sv) {
     if (part) {            // slice (split, head of the group) of the workspace, same [row][Hkv*hd] layout as dk
