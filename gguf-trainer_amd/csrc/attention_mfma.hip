@@ -81,8 +81,10 @@ template <int ROWS> struct TileIO {
   static constexpr int PER = (ROWS * HD / 4) / 256;
   // Where this thread's float4 units sit inside a tile whose first row is at `base`: computed once per kernel. A stage's
   // loads are then `base + off[i]` with a wave-uniform base that advances from stage to stage (scalar arithmetic) and a
-  // constant 32-bit lane offset: no per-load index arithmetic, and no bounds test while the whole tile lies inside the
-  // matrix (nvalid >= ROWS, wave-uniform). Only a tile that crosses the last row takes the tested path (zeros beyond it).
+  // 32-bit lane offset. A row past the end of the matrix (the last tile, when fewer than ROWS rows are left: nvalid < ROWS)
+  // reads the matrix's last row instead: no bounds test and no branch, so the loads can be scheduled among the MFMAs around
+  // them. What such a row holds is finite and every product it enters is masked to zero by the kernels (a query or key
+  // past the end is never live), so the results are those of a zero-filled tile.
   __device__ static __forceinline__ void offsets(unsigned (&off)[PER], size_t stride, int tid) {
 #pragma unroll
     for (int i = 0; i < PER; i++) {
@@ -90,18 +92,13 @@ template <int ROWS> struct TileIO {
       off[i] = (unsigned)(row * stride + c4 * 4);
     }
   }
-  __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ base, const unsigned (&off)[PER], int nvalid, int tid) {
-    if (nvalid >= ROWS) {
+  __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ base, const unsigned (&off)[PER], unsigned stride,
+                                              int nvalid, int tid) {
 #pragma unroll
-      for (int i = 0; i < PER; i++) reg[i] = *reinterpret_cast<const v4f *>(base + off[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < PER; i++) {
-        int row = (tid + i * 256) / (HD / 4);
-        v4f v = {0.f, 0.f, 0.f, 0.f};
-        if (row < nvalid) v = *reinterpret_cast<const v4f *>(base + off[i]);
-        reg[i] = v;
-      }
+    for (int i = 0; i < PER; i++) {
+      int row = (tid + i * 256) / (HD / 4);
+      unsigned back = (unsigned)max(row - (nvalid - 1), 0) * stride;      // 0 inside the matrix
+      reg[i] = *reinterpret_cast<const v4f *>(base + (off[i] - back));
     }
   }
   __device__ static __forceinline__ void store_rows(const v4f (&reg)[PER], float *lds, int tid) {
@@ -249,16 +246,16 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
   v4f pk[IO::PER], pv[IO::PER];
   unsigned koffs[IO::PER];
   IO::offsets(koffs, kstr, tid);
-  IO::load(pk, kb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
-  IO::load(pv, vb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
+  IO::load(pk, kb + (size_t)kt_lo * KT * kstr, koffs, (unsigned)kstr, p.T - kt_lo * KT, tid);
+  IO::load(pv, vb + (size_t)kt_lo * KT * kstr, koffs, (unsigned)kstr, p.T - kt_lo * KT, tid);
   for (int kt = kt_lo; kt <= kt_hi; kt++) {
     __syncthreads();
     IO::store_rows(pk, sK, tid);
     IO::store_t(pv, sVt, tid);
     __syncthreads();
     if (kt < kt_hi) {
-      IO::load(pk, kb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
-      IO::load(pv, vb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
+      IO::load(pk, kb + (size_t)(kt + 1) * KT * kstr, koffs, (unsigned)kstr, p.T - (kt + 1) * KT, tid);
+      IO::load(pv, vb + (size_t)(kt + 1) * KT * kstr, koffs, (unsigned)kstr, p.T - (kt + 1) * KT, tid);
     }
     if (tq0 >= p.T) continue;
     float pr[NSUB][16];
@@ -393,8 +390,8 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
   v4f pk[IO::PER], pv[IO::PER];
   unsigned koffs[IO::PER];
   IO::offsets(koffs, kstr, tid);
-  IO::load(pk, kb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
-  IO::load(pv, vb + (size_t)kt_lo * KT * kstr, koffs, p.T - kt_lo * KT, tid);
+  IO::load(pk, kb + (size_t)kt_lo * KT * kstr, koffs, (unsigned)kstr, p.T - kt_lo * KT, tid);
+  IO::load(pv, vb + (size_t)kt_lo * KT * kstr, koffs, (unsigned)kstr, p.T - kt_lo * KT, tid);
   for (int kt = kt_lo; kt <= kt_hi; kt++) {
     __syncthreads();
     IO::store_rows(pk, sK, tid);
@@ -402,8 +399,8 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
     IO::store_rows(pv, sV, tid);
     __syncthreads();
     if (kt < kt_hi) {
-      IO::load(pk, kb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
-      IO::load(pv, vb + (size_t)(kt + 1) * KT * kstr, koffs, p.T - (kt + 1) * KT, tid);
+      IO::load(pk, kb + (size_t)(kt + 1) * KT * kstr, koffs, (unsigned)kstr, p.T - (kt + 1) * KT, tid);
+      IO::load(pv, vb + (size_t)(kt + 1) * KT * kstr, koffs, (unsigned)kstr, p.T - (kt + 1) * KT, tid);
     }
     if (tq0 >= p.T) continue;
 #pragma unroll
@@ -436,16 +433,20 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 // KS: the forward kept its scores (sco: one [key][query] 32 x 32 block per (key sub-tile, query stage) of every
 // (sequence, head), T a multiple of 128). S is then read back, four 16-byte loads per lane and stage issued a stage
 // ahead, instead of recomputed: no key row in registers, no row-major query tile in LDS, three contractions per stage.
-template <bool KS>
+// DS: the score gradients are kept (dsb) for the banded dQ product.
+// The query / dO tiles are double-buffered in LDS: the tile of stage it+1 is written (from the registers its global loads
+// filled during stage it-1) while stage it computes on the other buffer, the loads of stage it+2 follow, and one barrier
+// ends the stage. None of that depends on the stage's MFMAs, and it is straight-line code, so it runs under them.
+#define DKV_BUF (2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT)        // floats per buffer: sQ, sG, sQt, sGt, lse, D
+template <bool KS, bool DS>
 __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
                                                            float *dk, int acc_k, float *dv, int acc_v, float *part,
                                                            float *dsb, const float *__restrict__ sco) {
   using IO = TileIO<QT>;
-  extern __shared__ __attribute__((aligned(16))) float dkv_smem[];      // 35 KB at hd 64, 69 KB at hd 128
-  float *sQ = dkv_smem, *sG = sQ + QT * LD, *sQt = sG + QT * LD, *sGt = sQt + HD * IO::LDT;
-  float *sL = sGt + HD * IO::LDT, *sD = sL + QT;
+  extern __shared__ __attribute__((aligned(16))) float dkv_smem[];      // 2 x 35 KB at hd 64, 2 x 69 KB at hd 128
+  constexpr int O_G = QT * LD, O_QT = 2 * QT * LD, O_GT = O_QT + HD * IO::LDT, O_L = O_GT + HD * IO::LDT, O_D = O_L + QT;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
   // 1-D grid, key tile slowest: the first key tiles are seen by the most queries and go first. One workgroup
   // per QUERY head: with a kv group larger than one, each head's dK/dV goes to its own slice of the workspace
@@ -494,100 +495,113 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const fl
   const float *scw = KS ? sco + (((size_t)b * p.Hq + h) * (p.T / 32) + sk0 / 32) * (p.T / 32) * 1024 + l32 * 32 + 4 * g : nullptr;
   const float *qb = q + (size_t)b * p.T * qstr + (size_t)h * HD;
   const float *gb = go + (size_t)b * p.T * qstr + (size_t)h * HD;
+  // row statistics of a stage: threads 0..31 fetch lse, 32..63 fetch D (the other threads fetch the same words again: no branch)
+  const float *statp = ((tid & QT) ? Dr : lse) + ((size_t)b * p.Hq + h) * p.T;
   unsigned qoffs[IO::PER];
   IO::offsets(qoffs, qstr, tid);
-  auto prefetch = [&](int it) {
-    int qt = qt_lo + it;
-    if (KS) {
-      const int t0n = qt * QT;
-      if (!(t0n + 31 < sk0 || t0n > wave_t_hi || sk0 >= p.T)) {           // only blocks the forward has written
-#pragma unroll
-        for (int a = 0; a < 4; a++) psc[a] = *reinterpret_cast<const v4f *>(scw + (size_t)qt * 1024 + 8 * a);
-      }
-    }
-    IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, p.T - qt * QT, tid);
-    IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, p.T - qt * QT, tid);
-    if (tid < 2 * QT) {
-      int tt = qt * QT + (tid % QT);
-      size_t si = ((size_t)b * p.Hq + h) * p.T + tt;
-      pstat = tt < p.T ? (tid < QT ? lse[si] : Dr[si]) : 0.f;
-    }
+  // Stage indices past the end are clamped to the last stage: its tile is loaded, and written to the idle buffer, again,
+  // which nobody reads; the loop body has no test for "is there a next stage".
+  auto load_tiles = [&](int it) {
+    const int qt = qt_lo + min(it, niter - 1);
+    IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
+    IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
+    pstat = statp[min(qt * QT + (tid % QT), p.T - 1)];
   };
-  prefetch(it_lo);
+  auto load_scores = [&](int it) {          // blocks the forward has not written hold anything: their stage is skipped
+    const int qt = qt_lo + min(it, niter - 1);
+#pragma unroll
+    for (int a = 0; a < 4; a++) psc[a] = *reinterpret_cast<const v4f *>(scw + (size_t)qt * 1024 + 8 * a);
+  };
+  auto store_tiles = [&](float *buf) {
+    if (!KS) IO::store_rows(pq, buf, tid);
+    IO::store_t(pq, buf + O_QT, tid);
+    IO::store_rows(pg, buf + O_G, tid);
+    IO::store_t(pg, buf + O_GT, tid);
+    if (tid < 2 * QT) buf[O_L + tid] = pstat;           // lse, then D
+  };
+  if (it_lo < niter) {
+    load_tiles(it_lo);
+    if (KS) load_scores(it_lo);
+    store_tiles(dkv_smem);
+    load_tiles(it_lo + 1);
+    __syncthreads();
+  }
   for (int it = it_lo; it < niter; it++) {
-    __syncthreads();
-    if (!KS) IO::store_rows(pq, sQ, tid);
-    IO::store_t(pq, sQt, tid);
-    IO::store_rows(pg, sG, tid);
-    IO::store_t(pg, sGt, tid);
-    if (tid < QT) sL[tid] = pstat;
-    else if (tid < 2 * QT) sD[tid - QT] = pstat;
-    __syncthreads();
+    const float *cur = dkv_smem + ((it - it_lo) & 1) * DKV_BUF;
+    float *nxt = dkv_smem + (((it - it_lo) & 1) ^ 1) * DKV_BUF;
+    const float *sQ = cur, *sG = cur + O_G, *sQt = cur + O_QT, *sGt = cur + O_GT, *sL = cur + O_L, *sD = cur + O_D;
     v16f sc;
-    if (KS) {            // out of the prefetch registers before the next stage's loads overwrite them
+    if (KS) {            // out of the prefetch registers, which the next stage's scores then fill
 #pragma unroll
       for (int r = 0; r < 16; r++) sc[r] = psc[r / 4][r % 4];
+      load_scores(it + 1);
     }
-    if (it + 1 < niter) prefetch(it + 1);
     const int t0 = (qt_lo + it) * QT;
     // this lane's column of the dS block of (query stage, keys of this wavefront): rows t0 + 8a + 4g + j. The matrix of a
     // (sequence, head) is kept as [row tile of 128][key step of 32][128 rows][32 keys]: a wavefront's block is 4 KB in one piece
-    float *dsc = dsb ? dsb + ((((size_t)b * p.Hq + h) * (p.T / 128) + t0 / 128) * (p.T / 32) + sk0 / 32) * 4096 +
-                           (t0 % 128 + 4 * g) * 32 + l32
-                     : nullptr;
+    float *dsc = DS ? dsb + ((((size_t)b * p.Hq + h) * (unsigned)(p.T / 128) + (unsigned)t0 / 128) * (unsigned)(p.T / 32) + (unsigned)sk0 / 32) * 4096 +
+                          ((unsigned)t0 % 128 + 4 * g) * 32 + l32
+                    : nullptr;
     if (t0 + 31 < sk0 || t0 > wave_t_hi || sk0 >= p.T) {             // wave-uniform: no (query, key) pair of this tile is live
-      if (dsb) {
+      if (DS) {
 #pragma unroll
         for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = 0.f;
       }
-      continue;
-    }
-    // at head dim 128 without kept scores both operand rows live in registers (128 of them): four LDS reads in flight
-    // instead of eight keep the kernel inside the register file
-    constexpr int DKV_NB = (HD >= 128 && !KS) ? 4 : 8;
-    if constexpr (!KS) sc = rows_dot_regs<DKV_NB>(sQ, kreg, l32, g);
-    // The stage as straight-line code. A pair (query tq, key s) is live when s <= tq <= last query that sees s: one
-    // unsigned compare per element against this lane's span (computed once per kernel), applied to every tile: a
-    // wave-uniform "does this tile need a mask" test would cut the stage into basic blocks, and the scheduler cannot
-    // move an instruction across those. Order: the probabilities need the scores only, so their exponentials are written
-    // between the issue of the dP contraction and its first use, and the dV contraction (which needs the probabilities
-    // only) between dP and the dS arithmetic: the vector ALU work has independent MFMAs to run under instead of sitting
-    // between two dependent blocks, and the group barriers ask for that interleaving (one MFMA, a few vector
-    // instructions, and again).
-    v16f dp = rows_dot_regs<DKV_NB>(sG, vreg, l32, g);
-    float pr[16], ds[16];
-    const unsigned rel0 = (unsigned)(t0 + 4 * g - s) + dead;          // query index relative to this lane's key, element (a, j) adds 8a + j
+      store_tiles(nxt);
+      load_tiles(it + 2);
+    } else {
+      // at head dim 128 without kept scores both operand rows live in registers (128 of them): four LDS reads in flight
+      // instead of eight keep the kernel inside the register file
+      constexpr int DKV_NB = (HD >= 128 && !KS) ? 4 : 8;
+      if constexpr (!KS) sc = rows_dot_regs<DKV_NB>(sQ, kreg, l32, g);
+      // The stage as straight-line code. A pair (query tq, key s) is live when s <= tq <= last query that sees s: one
+      // unsigned compare per element against this lane's span (computed once per kernel), applied to every tile: a
+      // wave-uniform "does this tile need a mask" test would cut the stage into basic blocks, and the scheduler cannot
+      // move an instruction across those. Order: the probabilities need the scores only, so their exponentials are written
+      // between the issue of the dP contraction and its first use, and the dV contraction (which needs the probabilities
+      // only) between dP and the dS arithmetic: the vector ALU work has independent MFMAs to run under instead of sitting
+      // between two dependent blocks, and the group barriers ask for that interleaving (one MFMA, a few vector
+      // instructions, and again).
+      v16f dp = rows_dot_regs<DKV_NB>(sG, vreg, l32, g);
+      float pr[16], ds[16];
+      const unsigned rel0 = (unsigned)(t0 + 4 * g - s) + dead;          // query index relative to this lane's key, element (a, j) adds 8a + j
 #pragma unroll
-    for (int a = 0; a < 4; a++) {
-      v4f lv = *reinterpret_cast<const v4f *>(sL + 8 * a + 4 * g);
+      for (int a = 0; a < 4; a++) {
+        v4f lv = *reinterpret_cast<const v4f *>(sL + 8 * a + 4 * g);
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        float e = fast_exp2(sc[4 * a + j] - lv[j]);
-        pr[4 * a + j] = (rel0 + (unsigned)(8 * a + j)) <= span ? e : 0.f;
+        for (int j = 0; j < 4; j++) {
+          float e = fast_exp2(sc[4 * a + j] - lv[j]);
+          pr[4 * a + j] = (rel0 + (unsigned)(8 * a + j)) <= span ? e : 0.f;
+        }
       }
-    }
 #pragma unroll
-    for (int i = 0; i < HD / 2; i++) {          // dP with the exponentials
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-    }
-    t_dot_acc<IO::LDT, DKV_NB>(vacc, sGt, 0, pr, l32, g);
+      for (int i = 0; i < HD / 2; i++) {          // dP with the exponentials
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      }
+      t_dot_acc<IO::LDT, DKV_NB>(vacc, sGt, 0, pr, l32, g);
 #pragma unroll
-    for (int a = 0; a < 4; a++) {
-      v4f dv4 = *reinterpret_cast<const v4f *>(sD + 8 * a + 4 * g);
+      for (int a = 0; a < 4; a++) {
+        v4f dv4 = *reinterpret_cast<const v4f *>(sD + 8 * a + 4 * g);
 #pragma unroll
-      for (int j = 0; j < 4; j++) ds[4 * a + j] = pr[4 * a + j] * (dp[4 * a + j] - dv4[j]) * p.scale;
-    }
+        for (int j = 0; j < 4; j++) ds[4 * a + j] = pr[4 * a + j] * (dp[4 * a + j] - dv4[j]) * p.scale;
+      }
 #pragma unroll
-    for (int i = 0; i < HD / 2; i++) {          // dV with the dS arithmetic
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-    }
-    if (dsb) {
+      for (int i = 0; i < HD / 2; i++) {          // dV with the dS arithmetic
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      }
+      // next stage's tile into the idle buffer (its loads were issued a stage ago), this stage's dS out, the loads of the
+      // stage after next: all independent of the dK contraction that follows
+      store_tiles(nxt);
+      if (DS) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = ds[r];
+        for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = ds[r];
+      }
+      load_tiles(it + 2);
+      t_dot_acc<IO::LDT, DKV_NB>(kacc, sQt, 0, ds, l32, g);
     }
-    t_dot_acc<IO::LDT, DKV_NB>(kacc, sQt, 0, ds, l32, g);
+    __syncthreads();
   }
   if (sv) {
     if (part) {            // slice (split, head of the group) of the workspace, same [row][Hkv*hd] layout as dk
@@ -615,7 +629,7 @@ __global__ __launch_bounds__(256) void FN(attn_group_sum)(const float *__restric
   *ov = acc_v ? *ov + sv : sv;
 }
 
-#define DKV_SMEM ((2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT) * sizeof(float))
+#define DKV_SMEM (2 * DKV_BUF * sizeof(float))
 
 // fpart: workspace for the split partials (splits x output, then splits x rows maxima, splits x rows sums), or null
 // sco: where to keep the raw scores for the backward (B*Hq*T*T floats, T a multiple of 128), or null
@@ -642,9 +656,13 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
              "attention: split backward without a workspace");
   GT_REQUIRE(ctx, !sco || (p.T % 128 == 0 && HD >= 64), "attention: kept scores with an unsupported shape");
   if (!(ctx->attn_smem_set & HD)) {   // once per context (device): more than the 64 KB a kernel gets by default at hd 128
-    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false>),
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false, false>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
-    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true>),
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
     ctx->attn_smem_set |= HD;
   }
@@ -659,12 +677,12 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
   {
     ProfScope ps(ctx, "attention.bwd.dkv");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
-    if (sco)
-      hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k)<true>, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
-                         P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco);
-    else
-      hipLaunchKernelGGL(FN(attn_bwd_dkv_mfma_k)<false>, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
-                         P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco);
+    auto launch = [&](auto kern) {
+      hipLaunchKernelGGL(kern, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k), P<const float>(v),
+                         P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco);
+    };
+    if (sco) dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false>);
+    else dsb ? launch(FN(attn_bwd_dkv_mfma_k)<false, true>) : launch(FN(attn_bwd_dkv_mfma_k)<false, false>);
     GT_LAUNCHED(ctx);
     if (part) {
       size_t n4 = (size_t)p.B * p.T * p.Hkv * HD / 4;

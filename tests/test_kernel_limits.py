@@ -74,7 +74,7 @@ def test_every_kernel_family_is_in_the_library(kernels):
                    "rmsnorm", "rope_vec_k", "adamw", "colsum"):
         assert family in names, family
     # the kept-scores variant of dK/dV (template argument true) and the banded dQ product (last template argument true)
-    assert any("attn_bwd_dkv_mfma_k64ILb1E" in k["name"] for k in kernels)
+    assert any("attn_bwd_dkv_mfma_k64ILb1ELb1E" in k["name"] for k in kernels)
     assert any("gemm_direct" in k["name"] and k["name"].endswith("Lb0ELb1EEv8GemmArgs") for k in kernels)
 
 
