@@ -30,7 +30,7 @@
 // dK/dV loops over the query heads of the kv group inside the workgroup and over query tiles in
 // increasing order, so the GQA sum has a fixed order and needs no atomics.
 //
-// Kept scores. With a scores buffer (T a multiple of 128) the forward stores its raw scores, one [key][query] 32 x 32
+// Kept scores. With a scores buffer (T a multiple of 128) the forward stores its scores, one [key][query] 32 x 32
 // block per (key sub-tile, query stage) of every (sequence, head), and dK/dV reads them back instead of recomputing
 // Q.K^T: three contractions per stage there instead of four.
 //
@@ -85,11 +85,11 @@ template <int ROWS> struct TileIO {
   // reads the matrix's last row instead: no bounds test and no branch, so the loads can be scheduled among the MFMAs around
   // them. What such a row holds is finite and every product it enters is masked to zero by the kernels (a query or key
   // past the end is never live), so the results are those of a zero-filled tile.
-  __device__ static __forceinline__ void offsets(unsigned (&off)[PER], size_t stride, int tid) {
+  __device__ static __forceinline__ void offsets(unsigned (&off)[PER], size_t stride, int tid) {      // in bytes
 #pragma unroll
     for (int i = 0; i < PER; i++) {
       int u = tid + i * 256, row = u / (HD / 4), c4 = u % (HD / 4);
-      off[i] = (unsigned)(row * stride + c4 * 4);
+      off[i] = (unsigned)((row * stride + c4 * 4) * sizeof(float));
     }
   }
   __device__ static __forceinline__ void load(v4f (&reg)[PER], const float *__restrict__ base, const unsigned (&off)[PER], unsigned stride,
@@ -97,8 +97,8 @@ template <int ROWS> struct TileIO {
 #pragma unroll
     for (int i = 0; i < PER; i++) {
       int row = (tid + i * 256) / (HD / 4);
-      unsigned back = (unsigned)max(row - (nvalid - 1), 0) * stride;      // 0 inside the matrix
-      reg[i] = *reinterpret_cast<const v4f *>(base + (off[i] - back));
+      unsigned back = (unsigned)max(row - (nvalid - 1), 0) * (stride * (unsigned)sizeof(float));      // 0 inside the matrix
+      reg[i] = *reinterpret_cast<const v4f *>(reinterpret_cast<const char *>(base) + (off[i] - back));   // uniform base + 32-bit lane offset
     }
   }
   __device__ static __forceinline__ void store_rows(const v4f (&reg)[PER], float *lds, int tid) {
@@ -199,15 +199,26 @@ __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32]
 }  // namespace
 
 #define KT (HD <= 64 ? 64 : 32)      // keys per LDS stage in forward and dQ
+// forward and dK/dV are held to the registers of two wavefronts per SIMD up to head dim 64 (two workgroups per CU); at 128 one
+#define WAVES_PER_SIMD (HD <= 64 ? 2 : 1)
 #define NSUB (KT / 32)
 
 // ---- forward --------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+// KEEP: the scores are stored for dK/dV (sco).
+// The K and V^T tiles are double-buffered in LDS: the tile of stage kt+1 is written (from the registers its global loads
+// filled during stage kt-1) while stage kt computes on the other buffer, the loads of stage kt+2 follow, and one barrier
+// ends the stage. A stage in which every 32-key sub-tile has a visible pair for this wavefront (all but the stages at the
+// diagonal and at a window's edge) is straight-line code, masks applied by one unsigned compare per element, so that the
+// scheduler can run the softmax of one sub-tile, the LDS stores and the loads under the MFMAs of another.
+#define FWD_BUF (KT * LD + HD * (KT + 4))        // floats per buffer: K rows, V transposed
+#define FWD_SMEM (2 * FWD_BUF * sizeof(float))
+template <bool KEEP>
+__global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, float *__restrict__ out,
                                                        float *__restrict__ lse, float *__restrict__ fpart, float *sco) {
   using IO = TileIO<KT>;
-  __shared__ __attribute__((aligned(16))) float sK[KT * LD];
-  __shared__ __attribute__((aligned(16))) float sVt[HD * IO::LDT];
+  constexpr int FWD_NB = 8;          // LDS reads in flight per contraction
+  extern __shared__ __attribute__((aligned(16))) float fwd_smem[];      // 2 x 35 KB at hd 64 and 128
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
   // 1-D grid ordered by work: every (head, sequence) pair's longest query tile is dispatched before any shorter
   // one, so the causal triangle packs onto the CUs without a long tail
@@ -243,87 +254,143 @@ __global__ __launch_bounds__(256) void FN(attn_fwd_mfma_k)(AttnP p, const float 
     for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
   float m = NEG_BIG, l = 0.f;
 
-  v4f pk[IO::PER], pv[IO::PER];
+  // One set of staging registers serves both tiles: the K tile of the next stage is loaded at the top of a stage and
+  // written to the idle buffer in its middle, the V tile is loaded there and written at the stage's end. A stage index past
+  // the last one is clamped to it (its tiles are loaded, and written to the idle buffer, once more, which nobody reads):
+  // the loop body has no test for "is there a next stage".
+  v4f pt[IO::PER];
   unsigned koffs[IO::PER];
   IO::offsets(koffs, kstr, tid);
-  IO::load(pk, kb + (size_t)kt_lo * KT * kstr, koffs, (unsigned)kstr, p.T - kt_lo * KT, tid);
-  IO::load(pv, vb + (size_t)kt_lo * KT * kstr, koffs, (unsigned)kstr, p.T - kt_lo * KT, tid);
+  auto load_tile = [&](const float *base, int kt) {
+    kt = min(kt, kt_hi);
+    IO::load(pt, base + (size_t)kt * KT * kstr, koffs, (unsigned)kstr, p.T - kt * KT, tid);
+  };
+  if (kt_lo <= kt_hi) {
+    load_tile(kb, kt_lo);
+    IO::store_rows(pt, fwd_smem, tid);
+    load_tile(vb, kt_lo);
+    IO::store_t(pt, fwd_smem + KT * LD, tid);
+    __syncthreads();
+  }
   for (int kt = kt_lo; kt <= kt_hi; kt++) {
-    __syncthreads();
-    IO::store_rows(pk, sK, tid);
-    IO::store_t(pv, sVt, tid);
-    __syncthreads();
-    if (kt < kt_hi) {
-      IO::load(pk, kb + (size_t)(kt + 1) * KT * kstr, koffs, (unsigned)kstr, p.T - (kt + 1) * KT, tid);
-      IO::load(pv, vb + (size_t)(kt + 1) * KT * kstr, koffs, (unsigned)kstr, p.T - (kt + 1) * KT, tid);
-    }
-    if (tq0 >= p.T) continue;
-    float pr[NSUB][16];
-    bool act[NSUB], msk[NSUB];
-    bool any_act = false;
-    float mx = NEG_BIG;
+    const float *sK = fwd_smem + ((kt - kt_lo) & 1) * FWD_BUF, *sVt = sK + KT * LD;
+    float *nxt = fwd_smem + (((kt - kt_lo) & 1) ^ 1) * FWD_BUF;
+    load_tile(kb, kt + 1);
+    bool act[NSUB];
+    bool plain = tq0 < p.T, any_act = false;      // plain: every pair of every sub-tile is visible to this wavefront
 #pragma unroll
     for (int sub = 0; sub < NSUB; sub++) {
       const int k0 = kt * KT + sub * 32;
-      act[sub] = !(k0 > tq1 || k0 + 31 < wave_lo);           // wave-uniform: some (query, key) pair is visible
-      if (!act[sub]) continue;
-      any_act = true;
-      v16f s = rows_dot_regs(sK + sub * 32 * LD, qreg, l32, g);
-      if (sco) {      // keep the raw scores (log2 domain, unmasked) of this 32 x 32 block for dK/dV: [key][query], 4 KB in one piece
-        float *sb = sco + ((((size_t)b * p.Hq + h) * (p.T / 32) + k0 / 32) * (p.T / 32) + tq0 / 32) * 1024 + l32;
+      act[sub] = tq0 < p.T && !(k0 > tq1 || k0 + 31 < wave_lo);           // wave-uniform: some (query, key) pair is visible
+      plain = plain && !(ragged || k0 + 31 > tq0 || k0 < wave_lo_last);
+      any_act = any_act || act[sub];
+    }
+    // where the scores (log2 domain; -1e30 where masked, which dK/dV masks again) of a 32 x 32 block go for dK/dV: [key][query], 4 KB in one piece
+    float *sb = KEEP ? sco + ((((size_t)b * p.Hq + h) * (unsigned)(p.T / 32) + (unsigned)(kt * KT) / 32) * (unsigned)(p.T / 32) + (unsigned)tq0 / 32) * 1024 + l32
+                     : nullptr;
+    float pr[NSUB][16];
+    if (plain) {
+      float mx = NEG_BIG;
 #pragma unroll
-        for (int r = 0; r < 16; r++) __builtin_nontemporal_store(s[r], sb + acc_row(r, g) * 32);   // read again only in the backward
-      }
-      const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
-      msk[sub] = need_mask;
-      if (need_mask) {
+      for (int sub = 0; sub < NSUB; sub++) {
+        v16f s = rows_dot_regs<FWD_NB>(sK + sub * 32 * LD, qreg, l32, g);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          int key = k0 + acc_row(r, g);
-          pr[sub][r] = (tv && key <= t && key >= lo_t) ? s[r] : NEG_BIG;
+          pr[sub][r] = s[r];
+          mx = fmaxf(mx, s[r]);
         }
-      } else {
+        if (KEEP) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) pr[sub][r] = s[r];
+          for (int r = 0; r < 16; r++)                // read again only in the backward
+            __builtin_nontemporal_store(pr[sub][r], sb + (size_t)sub * (p.T / 32) * 1024 + acc_row(r, g) * 32);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      if (__any(mx > m)) {                                      // rare after the first tiles
+        const float mn = fmaxf(m, mx);
+        const float alpha = fast_exp2(m - mn);
+        l *= alpha;
+        m = mn;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
       }
 #pragma unroll
-      for (int r = 0; r < 16; r++) mx = fmaxf(mx, pr[sub][r]);
-    }
-    if (!any_act) continue;
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    if (__any(mx > m)) {                                      // rare after the first tiles
-      const float mn = fmaxf(m, mx);
-      const float alpha = fast_exp2(m - mn);
-      l *= alpha;
-      m = mn;
-#pragma unroll
-      for (int dt = 0; dt < HD / 32; dt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
-    }
-#pragma unroll
-    for (int sub = 0; sub < NSUB; sub++) {
-      if (!act[sub]) continue;
-      float ls = 0.f;
-      if (msk[sub]) {
+      for (int sub = 0; sub < NSUB; sub++) {
+        float ls = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          // a masked score is NEG_BIG; with m still NEG_BIG (no visible key yet) the difference would be 0
-          float e = pr[sub][r] > -1.0e29f ? fast_exp2(pr[sub][r] - m) : 0.f;
+          float e = fast_exp2(pr[sub][r] - m);          // every score is a number and m is at least their maximum
           pr[sub][r] = e;
           ls += e;
         }
-      } else {          // every pair of the tile is visible: every score is a number and m is at least their maximum
+        l += ls;
+        if (sub == 0) {           // independent of the MFMAs around them
+          IO::store_rows(pt, nxt, tid);
+          load_tile(vb, kt + 1);
+        }
+        t_dot_acc<IO::LDT, FWD_NB>(oacc, sVt, sub * 32, pr[sub], l32, g);
+      }
+    } else {
+      IO::store_rows(pt, nxt, tid);
+      load_tile(vb, kt + 1);
+      if (any_act) {
+        bool msk[NSUB];
+        float mx = NEG_BIG;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float e = fast_exp2(pr[sub][r] - m);
-          pr[sub][r] = e;
-          ls += e;
+        for (int sub = 0; sub < NSUB; sub++) {
+          if (!act[sub]) continue;
+          const int k0 = kt * KT + sub * 32;
+          v16f s = rows_dot_regs<FWD_NB>(sK + sub * 32 * LD, qreg, l32, g);
+          const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
+          msk[sub] = need_mask;
+          if (need_mask) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              int key = k0 + acc_row(r, g);
+              pr[sub][r] = (tv && key <= t && key >= lo_t) ? s[r] : NEG_BIG;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) pr[sub][r] = s[r];
+          }
+#pragma unroll
+          for (int r = 0; r < 16; r++) mx = fmaxf(mx, pr[sub][r]);
+          if (KEEP) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) __builtin_nontemporal_store(pr[sub][r], sb + (size_t)sub * (p.T / 32) * 1024 + acc_row(r, g) * 32);
+          }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (__any(mx > m)) {
+          const float mn = fmaxf(m, mx);
+          const float alpha = fast_exp2(m - mn);
+          l *= alpha;
+          m = mn;
+#pragma unroll
+          for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
+        }
+#pragma unroll
+        for (int sub = 0; sub < NSUB; sub++) {
+          if (!act[sub]) continue;
+          float ls = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            // a masked score is NEG_BIG; with m still NEG_BIG (no visible key yet) the difference would be 0
+            float e = (!msk[sub] || pr[sub][r] > -1.0e29f) ? fast_exp2(pr[sub][r] - m) : 0.f;
+            pr[sub][r] = e;
+            ls += e;
+          }
+          l += ls;
+          t_dot_acc<IO::LDT, FWD_NB>(oacc, sVt, sub * 32, pr[sub], l32, g);
         }
       }
-      l += ls;
-      t_dot_acc<IO::LDT>(oacc, sVt, sub * 32, pr[sub], l32, g);
     }
+    IO::store_t(pt, nxt + KT * LD, tid);
+    __syncthreads();
   }
   const float lt = l + __shfl_xor(l, 32, 64);
   if (!tv) return;
@@ -439,7 +506,7 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 // ends the stage. None of that depends on the stage's MFMAs, and it is straight-line code, so it runs under them.
 #define DKV_BUF (2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT)        // floats per buffer: sQ, sG, sQt, sGt, lse, D
 template <bool KS, bool DS>
-__global__ __launch_bounds__(256) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
+__global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
                                                            float *dk, int acc_k, float *dv, int acc_v, float *part,
@@ -636,9 +703,20 @@ __global__ __launch_bounds__(256) void FN(attn_group_sum)(const float *__restric
 int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco) {
   GT_REQUIRE(ctx, (q | k | v | out) % 16 == 0, "attention: buffers must be 16-byte aligned");
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || fpart), "attention: split forward without a workspace");
+  if (!(ctx->attn_smem_set & (HD << 8))) {   // once per context (device): more than the 64 KB a kernel gets by default
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_fwd_mfma_k)<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)FWD_SMEM));
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_fwd_mfma_k)<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)FWD_SMEM));
+    ctx->attn_smem_set |= HD << 8;
+  }
   dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
-  hipLaunchKernelGGL(FN(attn_fwd_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
-                     P<const float>(v), P<float>(out), P<float>(lse), fpart, sco);
+  if (sco)
+    hipLaunchKernelGGL(FN(attn_fwd_mfma_k)<true>, grid, dim3(256), FWD_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
+                       P<const float>(v), P<float>(out), P<float>(lse), fpart, sco);
+  else
+    hipLaunchKernelGGL(FN(attn_fwd_mfma_k)<false>, grid, dim3(256), FWD_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
+                       P<const float>(v), P<float>(out), P<float>(lse), fpart, sco);
   GT_LAUNCHED(ctx);
   return 0;
 }

@@ -38,7 +38,7 @@ struct gt_ctx {
   bool prof_on = false;
   std::string prof_prefix;
   std::vector<ProfEvent> prof;
-  unsigned attn_smem_set = 0;                   // head dims (bits 32 | 64 | 128) whose dK/dV kernel has its LDS size attribute set
+  unsigned attn_smem_set = 0;                   // head dims whose attention kernels have their LDS size attribute set: bits 32 | 64 | 128 dK/dV, the same << 8 forward
   uint64_t gemm_direct_set = 0;                 // direct-to-LDS GEMM variants whose LDS size attribute is set
   int opt_prof_sample = 1;                      // events around every n-th launch of a label
   // Pinned host words a kernel writes when it meets an id / target outside its range (it skips that row):
