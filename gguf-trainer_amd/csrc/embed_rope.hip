@@ -179,6 +179,54 @@ __global__ __launch_bounds__(256) void rope_vec_k(unsigned nunits, int T, int H,
   }
 }
 
+// The same rotation over two tensors that share rows, T, hd and the table (q and k of a layer) in one launch: units
+// [0, n1) belong to the first, [n1, n1 + n2) to the second. Per element the arithmetic is rope_vec_k's.
+struct RopeT { const float *in; float *out; int H, acc; };
+template <bool BWD>
+__global__ __launch_bounds__(256) void rope_vec2_k(unsigned n1, unsigned n2, int T, int hd, const float *__restrict__ tab, RopeT A, RopeT B) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const unsigned q = (unsigned)hd / 8;                    // float4 units per half head
+  const unsigned stride = gridDim.x * 256, nunits = n1 + n2;
+  for (unsigned i0 = blockIdx.x * 256 + threadIdx.x; i0 < nunits; i0 += 2 * stride) {
+    f4 a0[2], a1[2], c0[2], c1[2], o0[2], o1[2];
+    float *op[2];
+    bool ac[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const unsigned ig = min(i0 + u * stride, nunits - 1);
+      const bool second = ig >= n1;
+      const unsigned i = second ? ig - n1 : ig;
+      const unsigned H = (unsigned)(second ? B.H : A.H);
+      const float *in = second ? B.in : A.in;
+      ac[u] = (second ? B.acc : A.acc) != 0;
+      const unsigned rh = i / q, j4 = i - rh * q;           // rh = row*H + h
+      const unsigned row = rh / H, t = row % (unsigned)T;
+      const size_t off = (size_t)rh * hd + 4 * j4;
+      op[u] = (second ? B.out : A.out) + off;
+      const f4 *tp = reinterpret_cast<const f4 *>(tab + ((size_t)t * (hd / 2) + 4 * j4) * 2);
+      a0[u] = *reinterpret_cast<const f4 *>(in + off);
+      a1[u] = *reinterpret_cast<const f4 *>(in + off + hd / 2);
+      c0[u] = tp[0];                                        // cos, sin of pairs j, j+1
+      c1[u] = tp[1];                                        // and of pairs j+2, j+3
+      if (ac[u]) {
+        o0[u] = *reinterpret_cast<const f4 *>(op[u]);
+        o1[u] = *reinterpret_cast<const f4 *>(op[u] + hd / 2);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      if (i0 + u * stride >= nunits) continue;
+      const f4 cs = {c0[u][0], c0[u][2], c1[u][0], c1[u][2]}, sn = {c0[u][1], c0[u][3], c1[u][1], c1[u][3]};
+      f4 r0, r1;
+      if (!BWD) { r0 = a0[u] * cs - a1[u] * sn; r1 = a0[u] * sn + a1[u] * cs; }
+      else { r0 = cs * a0[u] + sn * a1[u]; r1 = -sn * a0[u] + cs * a1[u]; }
+      if (ac[u]) { r0 += o0[u]; r1 += o1[u]; }
+      *reinterpret_cast<f4 *>(op[u]) = r0;
+      *reinterpret_cast<f4 *>(op[u] + hd / 2) = r1;
+    }
+  }
+}
+
 extern "C" {
 int gt_embedding_fwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf W, gt_buf out) {
   GT_ENTER(ctx);
@@ -215,22 +263,28 @@ int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, 
   return 0;
 }
 
+static int rope_table(gt_ctx *ctx, int T, int hd, double base, int pos, float **out) {
+  gt_ctx::RopeKey key{T, hd, pos, base};
+  auto it = ctx->rope_tables.find(key);
+  if (it != ctx->rope_tables.end()) { *out = it->second; return 0; }
+  float *tab;
+  int n = T * (hd / 2);
+  GT_HIP(ctx, hipMalloc(reinterpret_cast<void **>(&tab), (size_t)n * 2 * sizeof(float)));
+  hipLaunchKernelGGL(rope_table_k, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, T, hd, base, pos, tab);
+  GT_LAUNCHED(ctx);
+  ctx->rope_tables[key] = tab;
+  *out = tab;
+  return 0;
+}
+
 int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, int backward, gt_buf in, gt_buf out, int acc) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 0 && T >= 1 && H >= 1 && hd >= 2 && hd % 2 == 0 && in && out, "gt_rope: bad arguments (hd %d)", hd);
   GT_REQUIRE(ctx, rows % T == 0, "gt_rope: rows %d is not a whole number of sequences of %d", rows, T);
   if (rows == 0) return 0;
   ProfScope ps(ctx, backward ? "rope.bwd" : "rope", 8.0 * rows * H * hd);
-  gt_ctx::RopeKey key{T, hd, pos, base};
-  auto it = ctx->rope_tables.find(key);
   float *tab;
-  if (it == ctx->rope_tables.end()) {
-    int n = T * (hd / 2);
-    GT_HIP(ctx, hipMalloc(reinterpret_cast<void **>(&tab), (size_t)n * 2 * sizeof(float)));
-    hipLaunchKernelGGL(rope_table_k, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, T, hd, base, pos, tab);
-    GT_LAUNCHED(ctx);
-    ctx->rope_tables[key] = tab;
-  } else tab = it->second;
+  if (rope_table(ctx, T, hd, base, pos, &tab)) return 1;
   int64_t npairs = (int64_t)rows * H * (hd / 2);
   if (hd % 8 == 0 && npairs / 4 < ((int64_t)1 << 31) && (in | out) % 16 == 0) {
     const unsigned nunits = (unsigned)(npairs / 4);
@@ -249,6 +303,29 @@ int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, i
   else
     hipLaunchKernelGGL((rope_k<false>), dim3(nb), dim3(256), 0, ctx->stream, npairs, T, H, hd, reinterpret_cast<const float2 *>(tab),
                        P<const float>(in), P<float>(out), acc);
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+int gt_rope_pair(gt_ctx *ctx, int rows, int T, int hd, double base, int pos, int backward, int H1, gt_buf in1, gt_buf out1, int acc1, int H2,
+                 gt_buf in2, gt_buf out2, int acc2) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 0 && T >= 1 && H1 >= 1 && H2 >= 1 && hd >= 2 && hd % 2 == 0 && in1 && out1 && in2 && out2,
+             "gt_rope_pair: bad arguments (hd %d)", hd);
+  GT_REQUIRE(ctx, rows % T == 0, "gt_rope_pair: rows %d is not a whole number of sequences of %d", rows, T);
+  if (rows == 0) return 0;
+  const int64_t u1 = (int64_t)rows * H1 * (hd / 2) / 4, u2 = (int64_t)rows * H2 * (hd / 2) / 4;
+  if (!(hd % 8 == 0 && u1 + u2 < ((int64_t)1 << 31) && (in1 | out1 | in2 | out2) % 16 == 0)) {     // the shapes the one-tensor kernels take
+    if (gt_rope(ctx, rows, T, H1, hd, base, pos, backward, in1, out1, acc1)) return 1;
+    return gt_rope(ctx, rows, T, H2, hd, base, pos, backward, in2, out2, acc2);
+  }
+  ProfScope ps(ctx, backward ? "rope.bwd" : "rope", 8.0 * rows * (H1 + H2) * hd);
+  float *tab;
+  if (rope_table(ctx, T, hd, base, pos, &tab)) return 1;
+  const unsigned nbv = (unsigned)std::min<int64_t>(cdiv(u1 + u2, 512), (int64_t)ctx->num_cu * 16);
+  RopeT A{P<const float>(in1), P<float>(out1), H1, acc1}, B{P<const float>(in2), P<float>(out2), H2, acc2};
+  if (backward) hipLaunchKernelGGL((rope_vec2_k<true>), dim3(nbv), dim3(256), 0, ctx->stream, (unsigned)u1, (unsigned)u2, T, hd, tab, A, B);
+  else hipLaunchKernelGGL((rope_vec2_k<false>), dim3(nbv), dim3(256), 0, ctx->stream, (unsigned)u1, (unsigned)u2, T, hd, tab, A, B);
   GT_LAUNCHED(ctx);
   return 0;
 }

@@ -108,6 +108,8 @@ class HipBackend:
         self._scratch: list = []          # (buf, nbytes) raw transients: id uploads, saved statistics
         self._regions_opened = 0
         self._pend = None                 # (x, T, out, in, x data, w data, out data) of a held-back linear launch
+        self._pend_rope = None            # ((rows, T, hd, base, pos, backward), H, source, destination, accumulate) of a held-back rotation
+        self.pair_ropes = True
         # input gradients of linears held back in the backward, by input tensor: id(x) -> (x, rows, in, [(dY, W, out), ...]).
         # Sibling projections of one activation (q/k/v, gate/up) then leave as ONE product dX = sum of dY_i.W_i; whoever
         # touches x's gradient next, and every point where buffers can change hands, sends what is held first.
@@ -209,6 +211,36 @@ class HipBackend:
         if p is not None:
             self._pend = None
             check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, p[1], p[2], p[3], p[4], p[5], p[6]), "linear")
+        r = self._pend_rope
+        if r is not None:
+            self._pend_rope = None
+            self._launch_rope(r)
+
+    # ---- a forward rotation is held back by one op as well: the q and k of a layer (same rows, T, head dim, base and
+    # offset) then leave as ONE launch. Anything that reads or writes a buffer goes through _flush first.
+    def _launch_rope(self, r, other=None):
+        (rows, T, hd, base, pos, bwd), H, src, dst, acc = r
+        if other is None:
+            check(self._ctx, lib.gt_rope(self._ctx, rows, T, H, hd, base, pos, bwd, src, dst, acc), "rope.bwd" if bwd else "rope")
+        else:
+            _, H2, src2, dst2, acc2 = other
+            check(self._ctx, lib.gt_rope_pair(self._ctx, rows, T, hd, base, pos, bwd, H, src, dst, acc, H2, src2, dst2, acc2),
+                  "rope.bwd" if bwd else "rope")
+
+    def _rope(self, r):
+        """Launch r with the held-back rotation if they match, else launch that one and hold r. The caller has already
+        taken self._pend_rope (as `held`, passed inside r's call) so that its own buffer lookups did not flush it."""
+        held, r = r
+        if not self.pair_ropes:
+            if held is not None:
+                self._launch_rope(held)
+            self._launch_rope(r)
+        elif held is not None and held[0] == r[0]:
+            self._launch_rope(held, r)
+        else:
+            if held is not None:
+                self._launch_rope(held)
+            self._pend_rope = r
 
     def _flush_dw(self):
         """Launch the held-back weight-gradient products as one group."""
@@ -697,6 +729,7 @@ class HipBackend:
 
     def destroy(self):
         self._pend = None
+        self._pend_rope = None
         self._pend_dx = {}
         self._pend_dw = []
         if not self._destroyed:
@@ -1041,14 +1074,16 @@ class HipBackend:
     def rope(self, x, T, H, hd, base, pos_offset=0):
         self._op_begin(x)
         rows = x.shape[0]
+        held, self._pend_rope = self._pend_rope, None
         xd = self._data(x)
         out, e = self._make_out([rows, H * hd], [x])
-        check(self._ctx, lib.gt_rope(self._ctx, rows, T, H, hd, base, pos_offset, 0, xd, e.data, 0), "rope")
+        self._rope((held, ((rows, T, hd, float(base), pos_offset, 0), H, xd, e.data, 0)))
 
-        def bw():
+        def bw():           # the two backward rotations are never neighbours in the tape's order (k's linear sits between them)
             g = self._gsrc(out)
             dx, acc = self._gdst(x)
-            check(self._ctx, lib.gt_rope(self._ctx, rows, T, H, hd, base, pos_offset, 1, g, dx, acc), "rope.bwd")
+            if dx:
+                check(self._ctx, lib.gt_rope(self._ctx, rows, T, H, hd, base, pos_offset, 1, g, dx, acc), "rope.bwd")
 
         out._backward = bw
         return out

@@ -65,6 +65,7 @@ _SIG = {
     "gt_embedding_fwd": [ctxp, i32, i32, i32, buf, buf, buf],
     "gt_embedding_bwd": [ctxp, i32, i32, i32, buf, buf, buf, i32],
     "gt_rope": [ctxp, i32, i32, i32, i32, f64, i32, i32, buf, buf, i32],
+    "gt_rope_pair": [ctxp, i32, i32, i32, f64, i32, i32, i32, buf, buf, i32, i32, buf, buf, i32],
     "gt_attn_fwd": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf],
     "gt_attn_bwd": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, buf, buf, i32, buf, i32, buf, i32],
     "gt_gemm_add": [ctxp, i32, i32, i32, i32, buf, buf, buf, buf],

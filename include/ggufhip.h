@@ -183,6 +183,10 @@ int gt_embedding_bwd(gt_ctx *ctx, int rows, int d, int V, gt_buf ids, gt_buf g, 
  * (r mod T) + pos. backward = 1 applies the transposed rotation. */
 int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, int backward,
             gt_buf in, gt_buf out, int acc);
+/* The same rotation over two tensors that share rows, T, hd, base and pos (the q and k of a layer: two srcRope dispatches,
+ * webgpu.ts:1110-1121) as one launch; H1 and H2 heads per row. Results are those of two gt_rope calls. */
+int gt_rope_pair(gt_ctx *ctx, int rows, int T, int hd, double base, int pos, int backward, int H1, gt_buf in1, gt_buf out1, int acc1,
+                 int H2, gt_buf in2, gt_buf out2, int acc2);
 
 /* ---- attention: srcAttnFwd / BwdD / BwdDq / BwdDkv (wgsl.ts:657-918), webgpu.ts:1142-1189 -----
  * q[B*T, Hq*hd], k,v[B*T, Hkv*hd], causal, window > 0 keeps keys [t-window+1, t]; GQA head h reads

@@ -467,6 +467,33 @@ def test_residual_add_rides_the_linear_launch(gpu, ref):
         assert np.array_equal(res[True][1][n], res[False][1][n]), n
 
 
+@pytest.mark.parametrize("arch_name", ["llama", "gemma3"])
+@pytest.mark.parametrize("recompute", [False, True])
+def test_q_and_k_rotations_leave_as_one_launch(gpu, ref, arch_name, recompute):
+    """rope(q), rope(k) of a layer go out as one forward launch: every bit of the loss and of every gradient is what one
+    launch per rotation gives, with half the forward rotation launches; stacked and one sequence at a time (four streams),
+    with and without recomputed layers."""
+    kw = dict(arch="llama", vocab=64, hidden=128, layers=2, heads=4, kv_heads=2, head_dim=32, ffn=256, rope_base=1e4, rms_eps=1e-5)
+    if arch_name == "gemma3":
+        kw = dict(REAL["gemma3-window"], layers=3, vocab=256)
+    _, model = build_pair(ref, kw, seed=51, std=0.05)
+    seqs = batches(ref, kw["vocab"], 48, 3, seed=52, mask_every=5)
+    for stacked in (True, False):
+        res, n = {}, {}
+        try:
+            for pair in (True, False):
+                gpu.pair_ropes = pair
+                gpu.start_profile("rope")
+                res[pair] = hip_step(gpu, model, seqs, stacked, 48, recompute=recompute)
+                n[pair] = {k: v[1] for k, v in gpu.stop_profile().items()}
+        finally:
+            gpu.pair_ropes = True
+        assert n[False]["rope"] == 2 * n[True]["rope"] > 0 and n[False]["rope.bwd"] == n[True]["rope.bwd"], n
+        assert np.array_equal(res[True][0], res[False][0])
+        for name in res[True][1]:
+            assert np.array_equal(res[True][1][name], res[False][1][name]), name
+
+
 def test_linear_output_used_again_after_its_fused_add(gpu, ref):
     """The product that went straight into an add is computed after all when something else wants it: a later op, a
     readback. Against the oracle."""

@@ -284,6 +284,35 @@ def test_rope_far_positions(gpu, ref):
     op_case(gpu, ref, [r(T, H * hd)], lambda ag, x: ag.rope(x, T, H, hd, 1e5, 0), lambda rf, x: rf.rope(x, T, H, hd, 1e5, 0), "rope T=2048")
 
 
+@pytest.mark.parametrize("T,B,H1,H2,hd,pos", [(64, 2, 9, 3, 64, 0), (33, 1, 4, 4, 128, 5), (7, 3, 5, 1, 32, 0), (16, 1, 2, 3, 6, 2), (2048, 1, 9, 3, 64, 0)])
+@pytest.mark.parametrize("backward", [0, 1])
+def test_rope_pair_equals_two_single_launches(gpu, ref, T, B, H1, H2, hd, pos, backward):
+    """gt_rope_pair: the q and k of a layer in one launch give, bit for bit, what two gt_rope calls give: storing and
+    accumulating, the vector kernel's shapes and one it does not take (hd 6: the call falls back to two launches)."""
+    lib = mod("lib")
+    r = R(ref, T + H1 + hd)
+    rows = T * B
+    a1, a2 = r(rows, H1 * hd), r(rows, H2 * hd)
+    o1, o2 = r(rows, H1 * hd), r(rows, H2 * hd)            # old contents of the outputs, for the accumulating calls
+    bufs = [gpu.create_state_buffer(x.nbytes) for x in (a1, a2, o1, o2, o1, o2)]
+    i1, i2, p1, p2, s1, s2 = bufs
+    gpu.write_state_buffer(i1, a1)
+    gpu.write_state_buffer(i2, a2)
+    try:
+        for acc1, acc2 in ((0, 0), (1, 0), (1, 1)):
+            for b, o in ((p1, o1), (p2, o2), (s1, o1), (s2, o2)):
+                gpu.write_state_buffer(b, o)
+            lib.check(gpu.ctx, lib.lib.gt_rope_pair(gpu.ctx, rows, T, hd, 10000.0, pos, backward, H1, i1, p1, acc1, H2, i2, p2, acc2), "pair")
+            lib.check(gpu.ctx, lib.lib.gt_rope(gpu.ctx, rows, T, H1, hd, 10000.0, pos, backward, i1, s1, acc1), "single")
+            lib.check(gpu.ctx, lib.lib.gt_rope(gpu.ctx, rows, T, H2, hd, 10000.0, pos, backward, i2, s2, acc2), "single")
+            for pb, sb, n in ((p1, s1, a1.size), (p2, s2, a2.size)):
+                got, want = gpu.read_state_buffer(pb, n), gpu.read_state_buffer(sb, n)
+                assert np.array_equal(got, want), (acc1, acc2)
+    finally:
+        for b in bufs:
+            gpu.free_state_buffer(b)
+
+
 @pytest.mark.parametrize("kind,M,N,K", [(0, 300, 576, 576), (0, 257, 576, 1536), (0, 70, 83, 75), (0, 64, 64, 4096), (1, 130, 96, 64),
                                         (2, 96, 64, 2048), (0, 1, 5, 3)])
 @pytest.mark.parametrize("in_place", [False, True])
