@@ -556,7 +556,12 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   // this workgroup's share of the query stages
   const int it_lo = p.splits > 1 ? sp * nqt / p.splits : 0;
   const int niter = p.splits > 1 ? (sp + 1) * nqt / p.splits : nqt;
-  v4f pq[IO::PER], pg[IO::PER], psc[KS ? 4 : 1];
+  // ONE_SET (head dim 128 without kept scores, where both operand rows sit in registers): one set of staging registers
+  // serves the Q and the dO tile in turn, which keeps the kernel inside the register file. The Q tile of stage it+1 is
+  // in flight from the end of stage it-1 and written in the middle of stage it; the dO tile is loaded there and written
+  // at the stage's end, where the Q tile of stage it+2 is asked for.
+  constexpr bool ONE_SET = HD >= 128 && !KS;
+  v4f pq[IO::PER], pg[ONE_SET ? 1 : IO::PER], psc[KS ? 4 : 1];
   float pstat = 0.f;
   // this wavefront's block of kept scores for a query stage: lane = key row of the block, queries 8a + 4g + (0..3)
   const float *scw = KS ? sco + (((size_t)b * p.Hq + h) * (p.T / 32) + sk0 / 32) * (p.T / 32) * 1024 + l32 * 32 + 4 * g : nullptr;
@@ -568,10 +573,14 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   IO::offsets(qoffs, qstr, tid);
   // Stage indices past the end are clamped to the last stage: its tile is loaded, and written to the idle buffer, again,
   // which nobody reads; the loop body has no test for "is there a next stage".
-  auto load_tiles = [&](int it) {
+  auto load_q = [&](int it) {
     const int qt = qt_lo + min(it, niter - 1);
     IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
-    IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
+  };
+  auto load_g = [&](int it) {          // dO and the row statistics
+    const int qt = qt_lo + min(it, niter - 1);
+    if constexpr (ONE_SET) IO::load(pq, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
+    else IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
     pstat = statp[min(qt * QT + (tid % QT), p.T - 1)];
   };
   auto load_scores = [&](int it) {          // blocks the forward has not written hold anything: their stage is skipped
@@ -579,18 +588,47 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
 #pragma unroll
     for (int a = 0; a < 4; a++) psc[a] = *reinterpret_cast<const v4f *>(scw + (size_t)qt * 1024 + 8 * a);
   };
-  auto store_tiles = [&](float *buf) {
+  auto store_q = [&](float *buf) {
     if (!KS) IO::store_rows(pq, buf, tid);
     IO::store_t(pq, buf + O_QT, tid);
-    IO::store_rows(pg, buf + O_G, tid);
-    IO::store_t(pg, buf + O_GT, tid);
+  };
+  auto store_g = [&](float *buf) {
+    if constexpr (ONE_SET) {
+      IO::store_rows(pq, buf + O_G, tid);
+      IO::store_t(pq, buf + O_GT, tid);
+    } else {
+      IO::store_rows(pg, buf + O_G, tid);
+      IO::store_t(pg, buf + O_GT, tid);
+    }
     if (tid < 2 * QT) buf[O_L + tid] = pstat;           // lse, then D
   };
+  // the middle of a stage: the next stage's tile(s) into the idle buffer; its end: what is left of them, and the next loads
+  auto stage_middle = [&](float *nxt, int it) {
+    store_q(nxt);
+    if constexpr (ONE_SET) load_g(it + 1);
+    else store_g(nxt);
+  };
+  auto stage_end = [&](float *nxt, int it) {
+    if constexpr (ONE_SET) {
+      store_g(nxt);
+      load_q(it + 2);
+    }
+  };
   if (it_lo < niter) {
-    load_tiles(it_lo);
-    if (KS) load_scores(it_lo);
-    store_tiles(dkv_smem);
-    load_tiles(it_lo + 1);
+    load_q(it_lo);
+    if constexpr (ONE_SET) {
+      store_q(dkv_smem);
+      load_g(it_lo);
+      store_g(dkv_smem);
+      load_q(it_lo + 1);
+    } else {
+      load_g(it_lo);
+      if (KS) load_scores(it_lo);
+      store_q(dkv_smem);
+      store_g(dkv_smem);
+      load_q(it_lo + 1);
+      load_g(it_lo + 1);
+    }
     __syncthreads();
   }
   for (int it = it_lo; it < niter; it++) {
@@ -614,8 +652,11 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
 #pragma unroll
         for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = 0.f;
       }
-      store_tiles(nxt);
-      load_tiles(it + 2);
+      stage_middle(nxt, it);
+      if constexpr (!ONE_SET) {
+        load_q(it + 2);
+        load_g(it + 2);
+      }
     } else {
       // at head dim 128 without kept scores both operand rows live in registers (128 of them): four LDS reads in flight
       // instead of eight keep the kernel inside the register file
@@ -660,14 +701,18 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
       }
       // next stage's tile into the idle buffer (its loads were issued a stage ago), this stage's dS out, the loads of the
       // stage after next: all independent of the dK contraction that follows
-      store_tiles(nxt);
+      stage_middle(nxt, it);
       if (DS) {
 #pragma unroll
         for (int r = 0; r < 16; r++) dsc[(8 * (r / 4) + r % 4) * 32] = ds[r];
       }
-      load_tiles(it + 2);
+      if constexpr (!ONE_SET) {
+        load_q(it + 2);
+        load_g(it + 2);
+      }
       t_dot_acc<IO::LDT, DKV_NB>(kacc, sQt, 0, ds, l32, g);
     }
+    stage_end(nxt, it);
     __syncthreads();
   }
   if (sv) {

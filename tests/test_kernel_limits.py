@@ -3,7 +3,7 @@
 After tests/kernel-limits.ts: that file sums the workgroup arrays each emitted shader declares and holds them to the
 device's portable floor, independently of the formulas the host sizes tiles with. Here the compiler's per-kernel
 metadata plays that part: fixed LDS against the 64 KiB a launch may use without opting in, scratch (register spills)
-against zero apart from the one kernel known to spill, and the register budget of a wavefront. A kernel that starts
+against zero, and the register budget of a wavefront. A kernel that starts
 spilling or grows its LDS past the limit fails here, before any GPU run."""
 import os
 import re
@@ -20,8 +20,7 @@ READELF = shutil.which("llvm-readelf") or "/opt/rocm/llvm/bin/llvm-readelf"
 
 LDS_STATIC_LIMIT = 64 * 1024          # beyond this a kernel must take dynamic LDS and raise its attribute
 REGS_PER_LANE = 512                   # unified VGPR + AGPR file of a gfx950 wavefront at one wave per SIMD
-# hd-128 dK/dV holds a 128 x 128 accumulator pair per wave and spills a few registers; known and documented
-SPILL_ALLOWED = {"attn_bwd_dkv_mfma_k128": 128}
+SPILL_ALLOWED = {}                    # kernel name fragment -> bytes of scratch it may use: none does
 
 
 def code_objects(blob):
@@ -87,7 +86,7 @@ def test_fixed_lds_fits_without_opt_in(kernels):
     assert not over, over
 
 
-def test_no_kernel_spills_except_the_known_one(kernels):
+def test_no_kernel_spills(kernels):
     bad = []
     for k in kernels:
         allowed = max([v for n, v in SPILL_ALLOWED.items() if n in k["name"]], default=0)
