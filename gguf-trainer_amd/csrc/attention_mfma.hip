@@ -744,7 +744,7 @@ __global__ __launch_bounds__(256) void FN(attn_group_sum)(const float *__restric
 #define DKV_SMEM (2 * DKV_BUF * sizeof(float))
 
 // fpart: workspace for the split partials (splits x output, then splits x rows maxima, splits x rows sums), or null
-// sco: where to keep the raw scores for the backward (B*Hq*T*T floats, T a multiple of 128), or null
+// sco: where to keep the scores for the backward (B*Hq*T*T floats, T a multiple of 128), or null
 int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco) {
   GT_REQUIRE(ctx, (q | k | v | out) % 16 == 0, "attention: buffers must be 16-byte aligned");
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || fpart), "attention: split forward without a workspace");

@@ -24,7 +24,7 @@ What differs from the reference, on purpose:
     touched: sibling projections then leave as one summed product. A linear's weight gradient waits for up to seven more:
     consecutive ones leave as one grouped launch. add's backward launches nothing where it is the
     first writer: the operand's gradient points at the upstream buffer until somebody adds to it.
-  * attention keeps its raw scores from the forward to the backward where a backward can come and a byte budget allows,
+  * attention keeps its scores from the forward to the backward where a backward can come and a byte budget allows,
     as the reference's small-T path keeps its probabilities (webgpu.ts:1176-1189).
   * Consecutive micro-batches are recorded on different streams (see __init__), each with its own pool of transient
     buffers and its own parameter-gradient accumulators, summed in stream order before anything reads them.
@@ -131,7 +131,7 @@ class HipBackend:
         self.alias_add_grads = True
         self._aliased: list = []
         self.batch_linears = True
-        # attention keeps its raw scores from the forward to the backward (one [T, T] matrix per sequence and head) when a
+        # attention keeps its scores from the forward to the backward (one [T, T] matrix per sequence and head) when a
         # gradient will be asked for, one call's matrices fit attn_scores_max_bytes and the live ones together stay
         # within attn_scores_budget_bytes: memory spent to take one of four contractions out of dK/dV
         self.attn_keep_scores = True

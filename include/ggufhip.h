@@ -196,11 +196,11 @@ int gt_attn_fwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
 int gt_attn_bwd(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
                 gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf dout, gt_buf lse,
                 gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
-/* The same pair with the raw scores kept from the forward to the backward, as the reference's small-T path keeps its
+/* The same pair with the scores kept from the forward to the backward, as the reference's small-T path keeps its
  * probabilities and score gradients ([Hq,T,T] transients of srcAttnProbs / srcAttnDScore, wgsl.ts:492-583, webgpu.ts:1176-1189): the backward then reads S instead of recomputing
  * Q.K^T for dK/dV. gt_attn_scores_bytes gives the size of the scores buffer for a shape (B*Hq*T*T*4), or 0 where scores
  * are not kept (T not a multiple of 128, head dims other than 64 and 128, "attn.generic"); the buffer belongs to the
- * caller and must live until the backward call. Results equal gt_attn_fwd / gt_attn_bwd up to rounding. */
+ * caller, must live until the backward call and holds the library's own layout (32 x 32 blocks, masked pairs marked). Results equal gt_attn_fwd / gt_attn_bwd up to rounding. */
 int gt_attn_scores_bytes(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, uint64_t *bytes);
 int gt_attn_fwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
                        gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, gt_buf scores);
