@@ -601,6 +601,36 @@ def test_attention_mfma_shapes(gpu, ref, B, T, Hq, Hkv, hd, window, splits):
         ref.set_threads(1)
 
 
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 1, 2, 1, 64, 0), (2, 31, 4, 2, 64, 0), (1, 33, 2, 2, 32, 0), (1, 65, 2, 1, 64, 0),
+                                                  (1, 97, 3, 1, 64, 40), (1, 127, 2, 2, 128, 0), (1, 128, 2, 1, 64, 1),
+                                                  (1, 129, 2, 1, 128, 128), (2, 160, 4, 4, 64, 1000), (3, 95, 2, 1, 32, 7)])
+def test_attention_mfma_tile_edges(gpu, ref, B, T, Hq, Hkv, hd, window):
+    """Sequences that end one row before, on and one row after a tile or a 32- / 64-key stage, a single row, windows of
+    one key, of exactly a tile and longer than the sequence: the last stage's rows past the end are read from the last
+    row and must leave no trace. Against the oracle, every sequence of the stack."""
+    ag = mod("autograd")
+    r = R(ref, 7 * T + Hq + window + hd)
+    q, k, v = r(B * T, Hq * hd), r(B * T, Hkv * hd), r(B * T, Hkv * hd)
+    up = ref.Mulberry32(2).fill_uniform([B * T * Hq * hd])
+    hq, hk, hv = (ag.Tensor(a, list(a.shape), True) for a in (q, k, v))
+    gpu.install()
+    try:
+        out = ag.attention(hq, hk, hv, T, Hq, Hkv, hd, window)
+        backward_from(gpu, ag, out, up)
+        gpu.sync([out])
+    finally:
+        gpu.uninstall()
+    for b in range(B):
+        s = slice(b * T, (b + 1) * T)
+        rq, rk, rv = (ref.Tensor(a[s], [T, a.shape[1]], True) for a in (q, k, v))
+        o = ref.attention(rq, rk, rv, T, Hq, Hkv, hd, window)
+        ref.backward_from(o, up.reshape(B, -1)[b])
+        floor = 1.0 if window == 1 else 0.0          # one key per query: dq and dk are exactly zero up to rounding
+        assert_close(out.data.reshape(B, -1)[b], o.data, f"out[{b}]")
+        for h, rr, nm in ((hq, rq, "q"), (hk, rk, "k"), (hv, rv, "v")):
+            assert_close(h.grad.reshape(B, -1)[b], rr.grad, f"d{nm}[{b}]", floor=floor)
+
+
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 512, 2, 1, 64, 128),
                                                   (1, 512, 2, 1, 64, 127), (1, 640, 2, 2, 64, 129), (1, 256, 3, 1, 64, 1),
                                                   (3, 128, 2, 2, 64, 0), (1, 768, 2, 1, 64, 300), (2, 256, 4, 2, 128, 0),
