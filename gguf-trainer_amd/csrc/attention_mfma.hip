@@ -20,8 +20,11 @@
 // Strides of 4 mod 32 words keep every 8-lane group of a b128 access on distinct banks, and the
 // global->LDS copy assigns consecutive lanes to consecutive rows so both stores are conflict-free.
 // The operand that stays fixed for the whole loop (this lane's query / key row) lives in registers.
-// Global loads of the next tile are issued into registers before the MFMAs of the current one, and
-// all LDS reads of a contraction are issued before its first MFMA.
+// Forward and dK/dV keep two LDS buffers for the changing tile: while a stage computes on one, the next stage's
+// tile is written to the other from the registers its global loads filled earlier, and one barrier ends the
+// stage. Those loads take rows past the end of a sequence from its last row instead of testing bounds, so a
+// stage has no branch between its MFMAs and the scheduler can lay the loads, LDS stores and softmax arithmetic
+// under them. All LDS reads of a contraction are issued before its first MFMA.
 //
 // The running maximum of the online softmax is only raised, and the output accumulators rescaled,
 // when some lane of the wavefront actually sees a larger score (after the first few tiles it almost
