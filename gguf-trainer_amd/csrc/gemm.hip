@@ -320,15 +320,21 @@ struct DirectTile {
   __device__ static __forceinline__ int load_index(int wave, int i) { return (wave + i * NW) % WL; }
   // XOR swizzle of a row's chunks: any 16 consecutive rows put a given chunk on 16 different bank groups
   __device__ static __forceinline__ int sw(int row) { return CPR == 8 ? (row & 7) : ((row & 3) ^ ((row >> 2) & 3)); }
-  // source of this lane's chunk in load i of its wavefront, for the stage that starts at k = 0
-  __device__ static __forceinline__ const float *src(const float *p, int ld, int r0, int Rtot, int wave, int i, int lane) {
+  // Source of this lane's chunk in load i of its wavefront, for the stage that starts at k = 0, as a wave-uniform origin
+  // (the tile's first row or column) plus this lane's byte offset from it, which fits 32 bits and never changes: a
+  // stage's loads are then "scalar base + lane offset" and moving on by a stage is scalar arithmetic.
+  __device__ static __forceinline__ const float *origin(const float *p, int ld, int r0) { return KC ? p + (size_t)r0 * ld : p + r0; }
+  __device__ static __forceinline__ unsigned off(int ld, int r0, int Rtot, int wave, int i, int lane) {
     const int slot = load_index(wave, i) * 64 + lane;
     if (KC) {
       const int row = slot / CPR, c = (slot % CPR) ^ sw(row);
-      return p + (size_t)min(r0 + row, Rtot - 1) * ld + 4 * c;
+      return (unsigned)(((size_t)(min(r0 + row, Rtot - 1) - r0) * ld + 4 * c) * sizeof(float));
     }
     const int k = slot / (R / 4), c4 = slot % (R / 4);
-    return p + (size_t)k * ld + min(r0 + 4 * c4, Rtot - 4);
+    return (unsigned)(((size_t)k * ld + (min(r0 + 4 * c4, Rtot - 4) - r0)) * sizeof(float));
+  }
+  __device__ static __forceinline__ const float *src(const float *p, int ld, int r0, int Rtot, int wave, int i, int lane) {
+    return reinterpret_cast<const float *>(reinterpret_cast<const char *>(origin(p, ld, r0)) + off(ld, r0, Rtot, wave, i, lane));
   }
   // The same for a second K segment of K2 <= BKD (a multiple of 8) that fills one stage partly: chunks past K2 repeat
   // valid ones (they are loaded but never fed to an MFMA), so nothing is read outside the operand.
@@ -373,25 +379,39 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
     kend = min(a.K, m0 + BM);
   } else if (a.splits > 1) { k0 = z * a.kchunk; kend = min(a.K, k0 + a.kchunk); }
   else { A += z * a.sA; B += z * a.sB; }
-  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  const int wm = wave / WN, wn = wave % WN;
+  // The wavefront's index as a scalar for the loads (which of a stage's loads are its own, and their LDS addresses, are then
+  // scalar arithmetic instead of vector instructions among the MFMAs); its part of the tile stays derived from the thread
+  // index (with a scalar there the 4 x 1 wave layouts ran 10-20 % slower). Measured exception: the NN product on the 4 x 1
+  // layout at K = 1536 loses 9 % with the scalar form (its seven loads then leave in one burst) and keeps the vector one.
+  constexpr bool SCALAR_WAVE = !(KIND == GT_NN && WN == 1);
+  const int tid = threadIdx.x, lane = tid % 64, wave = SCALAR_WAVE ? __builtin_amdgcn_readfirstlane(tid / 64) : tid / 64;
+  const int wm = (tid / 64) / WN, wn = (tid / 64) % WN;
   const int g = lane / 32, l32 = lane % 32;
 
-  const float *pa[TA::PER], *pb[TB::PER];
+  // wave-uniform source of the next stage to issue (bytes), and this lane's fixed offsets from it
+  const char *ba = reinterpret_cast<const char *>(BAND ? A + (size_t)(k0 / BK) * 4096
+                                                       : TA::origin(A, a.lda, m0) + (size_t)(k0 / BK) * TA::stage_step(a.lda));
+  const char *bb = reinterpret_cast<const char *>(TB::origin(B, a.ldb, n0) + (size_t)(k0 / BK) * TB::stage_step(a.ldb));
+  unsigned oa[TA::PER], ob[TB::PER];
 #pragma unroll
-  for (int i = 0; i < TA::PER; i++)
-    pa[i] = BAND ? TA::src(A, 32, 0, BM, wave, i, lane) + (size_t)(k0 / BK) * 4096
-                 : TA::src(A, a.lda, m0, a.M, wave, i, lane) + (size_t)(k0 / BK) * TA::stage_step(a.lda);
+  for (int i = 0; i < TA::PER; i++) oa[i] = BAND ? TA::off(32, 0, BM, wave, i, lane) : TA::off(a.lda, m0, a.M, wave, i, lane);
 #pragma unroll
-  for (int i = 0; i < TB::PER; i++) pb[i] = TB::src(B, a.ldb, n0, a.N, wave, i, lane) + (size_t)(k0 / BK) * TB::stage_step(a.ldb);
-  size_t sta = BAND ? (size_t)4096 : TA::stage_step(a.lda), stb = TB::stage_step(a.ldb);
+  for (int i = 0; i < TB::PER; i++) ob[i] = TB::off(a.ldb, n0, a.N, wave, i, lane);
+  size_t sta = (BAND ? (size_t)4096 : TA::stage_step(a.lda)) * sizeof(float), stb = TB::stage_step(a.ldb) * sizeof(float);
   // MSEG: stages of the current segment still to be issued, and the segment after it (wave-uniform)
   int seg_left = MSEG ? a.K / BK : 0, seg_next = 0;
 #define ISSUE(buf_)                                                                                              \
   {                                                                                                              \
     float *sa_ = smem + (buf_) * STAGE, *sb_ = sa_ + TA::CH * 4;                                                 \
-    _Pragma("unroll") for (int i = 0; i < TA::PER; i++) { load_to_lds16(pa[i], sa_ + TA::load_index(wave, i) * 256); pa[i] += sta; } \
-    _Pragma("unroll") for (int i = 0; i < TB::PER; i++) { load_to_lds16(pb[i], sb_ + TB::load_index(wave, i) * 256); pb[i] += stb; } \
+    _Pragma("unroll") for (int i = 0; i < TA::PER; i++) {                                                        \
+      asm volatile("" : "+v"(oa[i]));  /* keeps the offset a 32-bit register: scalar base + lane offset */        \
+      load_to_lds16(reinterpret_cast<const float *>(ba + oa[i]), sa_ + TA::load_index(wave, i) * 256);           \
+    }                                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < TB::PER; i++) {                                                        \
+      asm volatile("" : "+v"(ob[i]));                                                                            \
+      load_to_lds16(reinterpret_cast<const float *>(bb + ob[i]), sb_ + TB::load_index(wave, i) * 256);           \
+    }                                                                                                            \
+    ba += sta; bb += stb;                                                                                        \
   }
   // the stage of the second segment (SEG2): its sources are computed when it is issued, once per workgroup
 #define ISSUE2(buf_)                                                                                             \
@@ -407,9 +427,11 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
   {                                                                                                              \
     const float *A_ = a.xA[seg_next], *B_ = a.xB[seg_next];                                                      \
     const int lda_ = a.xlda[seg_next], ldb_ = a.xldb[seg_next];                                                  \
-    _Pragma("unroll") for (int i = 0; i < TA::PER; i++) pa[i] = TA::src(A_, lda_, m0, a.M, wave, i, lane);       \
-    _Pragma("unroll") for (int i = 0; i < TB::PER; i++) pb[i] = TB::src(B_, ldb_, n0, a.N, wave, i, lane);       \
-    sta = TA::stage_step(lda_); stb = TB::stage_step(ldb_);                                                      \
+    ba = reinterpret_cast<const char *>(TA::origin(A_, lda_, m0));                                               \
+    bb = reinterpret_cast<const char *>(TB::origin(B_, ldb_, n0));                                               \
+    _Pragma("unroll") for (int i = 0; i < TA::PER; i++) oa[i] = TA::off(lda_, m0, a.M, wave, i, lane);           \
+    _Pragma("unroll") for (int i = 0; i < TB::PER; i++) ob[i] = TB::off(ldb_, n0, a.N, wave, i, lane);           \
+    sta = TA::stage_step(lda_) * sizeof(float); stb = TB::stage_step(ldb_) * sizeof(float);                      \
     seg_left = a.xK[seg_next] / BK; seg_next++;                                                                  \
   }
 #define ISSUE_STAGE(buf_, st_)                                                                                   \
