@@ -30,10 +30,10 @@ PROF_SAMPLE = 4                # the timed region brackets about 1 in 4 launches
 # size; see profiles/bench_smollm2_135m_pmc_fetch_write.txt). Averages over the shapes each label serves in the step: the NN
 # label is 30 summed q+k+v products, 30 summed gate+up products, the 30 dX of the o projection and the readout's; the grouped
 # TN labels include their reduction pass.
-MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (30 * (2 * 50006.6 + 36864.7) + 30 * (2 * 166347.9 + 36864.7) + 30 * (2 * 29994.5 + 36866.5) +
-                                          (2 * 4173488.3 + 36866.5)) / 91 * 1024,
-                    "gemm.tn.group.128x96.splitk": ((24 * 1303.5 + 18 * 1117.2) / 42 + 151.9) * 1048576,
-                    "gemm.tn.group.64x192.splitk": ((21 * 1137.6 + 12 * 1400.9) / 33 + 151.9) * 1048576}
+MEASURED_TRAFFIC = {"gemm.nn.128x96x32": (30 * (2 * 50010.9 + 36864.5) + 30 * (2 * 174988.0 + 36864.5) + 30 * (2 * 29882.9 + 36865.5) +
+                                          (2 * 3508313.8 + 36865.5)) / 91 * 1024,
+                    "gemm.tn.group.128x96.splitk": ((24 * 1200.5 + 18 * 943.5) / 42 + 151.9) * 1048576,
+                    "gemm.tn.group.64x192.splitk": ((21 * 959.7 + 12 * 1193.4) / 33 + 151.9) * 1048576}
 
 SMOLLM2 = dict(arch="llama", vocab=49152, hidden=576, layers=30, heads=9, kv_heads=3, head_dim=64, ffn=1536,
                rope_base=100000.0, rms_eps=1e-5, tie=True)
