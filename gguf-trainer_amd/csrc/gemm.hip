@@ -566,6 +566,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_direct(GemmArgs a) {
 // split-major and dealt to the XCDs in contiguous ranges, exactly as for a single product. A workgroup looks up its
 // problem, points the argument block at that problem's operands, and runs the ordinary tile loop.
 #define GT_GROUP_MAX 8
+#define GT_DIRECT_LD_MAX (1 << 22)     // largest leading dimension (floats) the direct kernels address: 192 rows x 4 B x this < 2^32
 struct GroupProb { const float *A, *B; float *C; int M, N, acc, tile0, nbn; int64_t e0; };   // e0: elements of the problems before it
 struct GroupArgs { GroupProb p[GT_GROUP_MAX]; int n, ntiles; };
 
@@ -745,7 +746,9 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   // Tiles with a K step of 32 have a variant that loads operands straight into LDS (gemm_direct); it wants whole K
   // steps and whole 16-byte chunks along the contiguous index of every operand. Where it applies it is 2-8 % faster
   // than the register-staged kernel of the same tile and changes which tile is best, hence two tables.
+  // a lane's byte offset inside a tile (up to 192 rows of ld floats) must fit the 32 bits the direct kernels keep it in
   const bool direct_ok = vec && K % 32 == 0 && (kind != GT_TN || (M % 4 == 0 && M >= 4)) && (kind == GT_NT || (N % 4 == 0 && N >= 4)) &&
+                         std::max(std::max(a.lda, a.ldb), K2 > 0 ? std::max(a.lda2, a.ldb2) : 0) <= GT_DIRECT_LD_MAX &&
                          (K2 == 0 || (kind != GT_TN && K2 % 8 == 0 && K2 <= 32));   // a short second segment rides in one more stage
   int cfg = 0, splits = 1;
   pick_tile(ctx, kind, direct_ok, 1, &M, &N, K, count, K2 > 0, &cfg, &splits);
@@ -883,7 +886,7 @@ int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, 
   // that fills the chip on its own (at least one 128 x 96 tile per CU) is not split and goes as its own launch.
   const int64_t big = (int64_t)ctx->num_cu * 128 * 96;
   int idx[GT_GROUP_MAX], ng = 0;
-  bool eligible = kind == GT_TN && K % 32 == 0 && !ctx->opt_gemm_staged && ctx->opt_gemm_group;
+  bool eligible = kind == GT_TN && K % 32 == 0 && !ctx->opt_gemm_staged && ctx->opt_gemm_group;      // (TN: ld = M, N, below GT_DIRECT_LD_MAX for any grouped size)
   for (int i = 0; i < count; i++) {
     GT_REQUIRE(ctx, M[i] >= 1 && N[i] >= 1 && A[i] && B[i] && C[i], "gt_gemm_group: product %d has M %d, N %d or a null operand", i, M[i], N[i]);
     for (int j = 0; j < i; j++) GT_REQUIRE(ctx, C[i] != C[j], "gt_gemm_group: products %d and %d write the same output", j, i);
@@ -894,7 +897,8 @@ int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, 
     return 0;
   }
   for (int i = 0; i < count; i++) {
-    const bool fits = eligible && M[i] % 4 == 0 && N[i] % 4 == 0 && (A[i] | B[i] | C[i]) % 16 == 0 && (int64_t)M[i] * N[i] < big;
+    const bool fits = eligible && M[i] % 4 == 0 && N[i] % 4 == 0 && (A[i] | B[i] | C[i]) % 16 == 0 && (int64_t)M[i] * N[i] < big &&
+                      M[i] <= GT_DIRECT_LD_MAX && N[i] <= GT_DIRECT_LD_MAX;
     if (fits) idx[ng++] = i;
     else if (gemm_impl(ctx, kind, acc[i], M[i], N[i], K, A[i], 0, B[i], 0, C[i], 0, 1)) return 1;
   }
@@ -953,8 +957,9 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
   bool fused = count > 1 && kind != GT_TN && !ctx->opt_gemm_staged && C % 16 == 0 && N % 4 == 0 && (kind == GT_NT || N >= 4);
   for (int i = 0; i < count; i++) {
     GT_REQUIRE(ctx, K[i] >= 1 && A[i] && B[i], "gt_gemm_sum: product %d has K %d or a null operand", i, K[i]);
-    fused = fused && K[i] % 32 == 0 && A[i] % 16 == 0 && B[i] % 16 == 0;
+    fused = fused && K[i] % 32 == 0 && A[i] % 16 == 0 && B[i] % 16 == 0 && K[i] <= GT_DIRECT_LD_MAX;
   }
+  fused = fused && N <= GT_DIRECT_LD_MAX;
   // the chained loop has one tile shape and no K split: below one workgroup per CU the single products, which pick
   // smaller tiles and split K, fill the chip better
   const bool t96 = N % 96 == 0;
