@@ -405,9 +405,12 @@ void or_attention_bwd(const float *q, const float *k, const float *v, const floa
   free(dP);
 }
 
-/* Parallel-safe attention backward for the timed CPU baseline only: the same
- * per-(h,t) arithmetic, with dK/dV accumulated per kv-head in f64 scratch and
- * rounded once. or_attention_bwd stays the parity oracle. */
+/* Parallel-safe attention backward: the same per-(h,t) arithmetic as or_attention_bwd,
+ * with dK/dV accumulated per kv-head in f64 scratch and rounded once (so it differs from
+ * the serial form by f32 rounding of the running dK/dV sums only). It is the checker of the
+ * GPU comparisons at T = 2048 and of the real-width layer test, where the serial form takes
+ * minutes, and the attention backward of the timed CPU baseline. Pinned against float64
+ * autograd directly (window 0 and > 0, GQA group 3) and against the serial form. */
 void or_attention_bwd_par(const float *q, const float *k, const float *v, const float *probs,
                           const float *gout, float *gq, float *gk, float *gv,
                           int T, int Hq, int Hkv, int hd, int window) {

@@ -39,6 +39,44 @@ def test_mulberry32_known_first_output(ref):
     assert ref.Mulberry32(0)() == 0.26642920868471265
 
 
+def test_randn_and_fills_match_box_muller_over_the_js_generator(ref):
+    """autograd.ts:54-66: randn = sqrt(-2 ln u) cos(2 pi v) with u, v the next two non-zero uniforms; param() /
+    randTensor() store randn * std as f32; the uniform fill is lo + (hi - lo) * u. Replayed on the big-int generator
+    with math.sqrt/log/cos. libm and Python's math share the platform's log/cos, so the f64 values agree to the last
+    bit or one ulp; the f32 stores are compared exactly except where an f64 ulp straddles an f32 rounding tie."""
+    for seed in (0, 7, 0xBEEF):
+        js = js_mulberry32(seed)
+        def js_randn():
+            u = v = 0.0
+            while u == 0.0:
+                u = js()
+            while v == 0.0:
+                v = js()
+            return math.sqrt(-2.0 * math.log(u)) * math.cos(2.0 * math.pi * v)
+        a = ref.Mulberry32(seed)
+        for _ in range(500):
+            got, want = a.randn(), js_randn()
+            assert abs(got - want) <= 4e-16 * max(1.0, abs(want))
+        # the generator state stays in step (two uniforms per normal): the fills continue the same stream
+        got = ref.Mulberry32(seed).fill_randn([1000], 0.02)
+        js = js_mulberry32(seed)
+        want = np.array([js_randn() * 0.02 for _ in range(1000)])
+        assert np.count_nonzero(got != want.astype(np.float32)) <= 1
+        assert np.all(np.abs(got.astype(np.float64) - want) <= 2.0 ** -24 * np.abs(want) + 1e-45)
+        # sample moments of N(0, 0.02^2): a dropped factor 2 or a sine for the cosine would still pass these,
+        # the replay above would not; a wrong std or a uniform in place of a normal fails here
+        big = ref.Mulberry32(seed).fill_randn([200000], 0.02).astype(np.float64)
+        assert abs(big.mean()) < 2e-4 and abs(big.std() - 0.02) < 2e-4
+        assert abs(np.mean(big ** 4) / big.var() ** 2 - 3.0) < 0.05
+        gotu = ref.Mulberry32(seed).fill_uniform([1000], -1.0, 1.0)
+        js = js_mulberry32(seed)
+        wantu = np.array([-1.0 + 2.0 * js() for _ in range(1000)]).astype(np.float32)
+        assert np.array_equal(gotu, wantu)
+        gotu = ref.Mulberry32(seed).fill_uniform([64], 0.25, 3.0)
+        js = js_mulberry32(seed)
+        assert np.array_equal(gotu, np.array([0.25 + 2.75 * js() for _ in range(64)]).astype(np.float32))
+
+
 def test_ce_closed_form_big_gaps(ref):
     """tests/gradcheck.ts:321-335: rows [gap,0,0,-3], target 3, tolerance 1e-4, hard and soft (q=0.6)."""
     for gap in [1, 10, 30, 60, 90]:

@@ -93,19 +93,27 @@ def test_attention_vs_torch64(ref, T, Hq, Hkv, hd, window):
           floor=1.0 if window == 1 else 1e-6)
 
 
-def test_attention_parallel_bwd_variant_matches(ref):
-    """The OpenMP-safe backward used only for the timed CPU baseline computes the same gradients."""
-    rng = ref.Mulberry32(9)
-    T, Hq, Hkv, hd = 40, 6, 2, 16
+@pytest.mark.parametrize("T,Hq,Hkv,hd,window", [(40, 6, 2, 16, 9), (33, 6, 2, 16, 0), (64, 9, 3, 64, 0), (50, 9, 3, 8, 16),
+                                                (21, 4, 4, 8, 5)])
+def test_attention_parallel_bwd_variant_matches(ref, T, Hq, Hkv, hd, window):
+    """or_attention_bwd_par (dK/dV summed per kv head in f64 and rounded once) is the checker of the GPU attention
+    comparisons at T = 2048 and the attention backward of the timed CPU baseline: pinned against torch float64
+    autograd directly, with and without a window and with a GQA group of 3, and against the serial form."""
+    rng = ref.Mulberry32(9 + T)
     arrs = [rng.fill_randn([T, n * hd], 0.8) for n in (Hq, Hkv, Hkv)]
+    up = ref.Mulberry32(1).fill_uniform([T * Hq * hd])
     res = []
     for par in (False, True):
         q, k, v = (ref.Tensor(a, list(a.shape), True) for a in arrs)
-        o = ref.attention(q, k, v, T, Hq, Hkv, hd, 9, parallel_bwd=par)
-        ref.backward_from(o, ref.Mulberry32(1).fill_uniform([o.size]))
+        o = ref.attention(q, k, v, T, Hq, Hkv, hd, window, parallel_bwd=par)
+        ref.backward_from(o, up)
         res.append([q.grad, k.grad, v.grad])
     for a, b in zip(*res):
         assert relerr(a, b) < 1e-6
+    tq, tk, tv = (t64(a, list(a.shape)) for a in arrs)
+    torch_attention(tq, tk, tv, T, Hq, Hkv, hd, window).backward(torch.tensor(up.astype(np.float64)).reshape(T, Hq * hd))
+    for a, t in zip(res[1], (tq, tk, tv)):
+        assert relerr(a, t.grad.numpy()) < 2e-6
 
 
 @pytest.mark.parametrize("T,ind,outd,frozen", [(7, 12, 9, False), (33, 17, 5, False), (1, 3, 40, False), (19, 31, 23, True)])
