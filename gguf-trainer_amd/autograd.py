@@ -128,12 +128,28 @@ def _topo(root, seen):
     return topo
 
 
+class _backward_scope:
+    """Tells a backend that keeps a `backward_depth` counter that closures are being walked: forward ops recorded
+    meanwhile (a checkpoint's replay) belong to the graph being differentiated, not to a new one."""
+
+    def __enter__(self):
+        self.be = _backend if _backend is not None and hasattr(_backend, "backward_depth") else None
+        if self.be is not None:
+            self.be.backward_depth += 1
+
+    def __exit__(self, *exc):
+        if self.be is not None:
+            self.be.backward_depth -= 1
+        return False
+
+
 def backward(loss: Tensor, seed: float = 1.0):
     """autograd.ts:81-93. A per-sequence loss vector gets the same seed in every slot."""
     topo = _topo(loss, set())
     loss.grad[:] = seed
-    for t in reversed(topo):
-        t._backward()
+    with _backward_scope():
+        for t in reversed(topo):
+            t._backward()
 
 
 # ---- backend dispatch (autograd.ts:95-169, 275-279) -----------------------------------------------
@@ -204,17 +220,18 @@ def checkpoint(inputs, fn):
     out._prev = inputs
 
     def bw():
-        mark2 = rb.begin_region() if rb else 0
-        replay = fn()
-        if rb:
-            rb.seed_grad_from(replay, out)
-        else:
-            replay.grad[:] = out.grad
-        topo = _topo(replay, {id(t) for t in inputs})
-        for t in reversed(topo):
-            t._backward()
-        if rb:
-            rb.end_region(mark2, [])
+        with _backward_scope():         # also when the closure is walked by hand (a test seeding a non-scalar output)
+            mark2 = rb.begin_region() if rb else 0
+            replay = fn()
+            if rb:
+                rb.seed_grad_from(replay, out)
+            else:
+                replay.grad[:] = out.grad
+            topo = _topo(replay, {id(t) for t in inputs})
+            for t in reversed(topo):
+                t._backward()
+            if rb:
+                rb.end_region(mark2, [])
 
     out._backward = bw
     return out

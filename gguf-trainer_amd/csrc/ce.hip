@@ -111,6 +111,7 @@ __global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, int spans, const f
   const int64_t row = blockIdx.x / spans;
   const int span = blockIdx.x % spans;
   int g = SOFT ? (tgt[row * k] == IGN ? IGN : -2) : tgt[row];     // -2: no column matches
+  if (!SOFT && (g < IGN || g >= V)) g = IGN;           // no such logit: ignored, as the forward counted it (and reported it)
   if (g == IGN && acc) return;                         // untouched, as the reference leaves it
   const float sc = SOFT ? seed * mass[row] : seed * inv_denom[row / T];
   const float ls = lse[row];
@@ -151,9 +152,9 @@ __global__ __launch_bounds__(256) void ce_bwd_k(int V, int T, int spans, const f
 }
 
 // ---- chunked: per-row running (max, sum, target logit) across vocab spans ------------------------
-__global__ __launch_bounds__(256) void ce_chunk_stats_k(int vc, int v0, int first, const float *__restrict__ chunk,
+__global__ __launch_bounds__(256) void ce_chunk_stats_k(int V, int vc, int v0, int first, const float *__restrict__ chunk,
                                                         const int *__restrict__ tgt, float *row_max, float *row_sum,
-                                                        float *tgt_logit) {
+                                                        float *tgt_logit, int *bad) {
   __shared__ float sm[8];
   int64_t row = blockIdx.x;
   const float *zr = chunk + row * vc;
@@ -165,11 +166,14 @@ __global__ __launch_bounds__(256) void ce_chunk_stats_k(int vc, int v0, int firs
     row_max[row] = m0;
     row_sum[row] = l0;
     int g = tgt[row];
-    if (first) tgt_logit[row] = 0.f;
-    if (g >= v0 && g < v0 + vc) tgt_logit[row] = zr[g - v0];
+    if (first) {
+      tgt_logit[row] = 0.f;
+      if (g < IGN || g >= V) note_bad_id(bad, GT_BAD_TARGET, row, g, V);    // once per row; every kernel below ignores the row
+    }
+    if (g >= v0 && g < v0 + vc && g < V) tgt_logit[row] = zr[g - v0];
   }
 }
-__global__ __launch_bounds__(256) void ce_loss_from_stats_k(int T, const int *__restrict__ tgt, const float *__restrict__ inv_denom,
+__global__ __launch_bounds__(256) void ce_loss_from_stats_k(int V, int T, const int *__restrict__ tgt, const float *__restrict__ inv_denom,
                                                             const float *__restrict__ row_max, const float *__restrict__ row_sum,
                                                             const float *__restrict__ tgt_logit, float *__restrict__ loss) {
   __shared__ float sm[4];
@@ -177,19 +181,21 @@ __global__ __launch_bounds__(256) void ce_loss_from_stats_k(int T, const int *__
   float a = 0;
   for (int t = threadIdx.x; t < T; t += 256) {
     size_t r = (size_t)s * T + t;
-    if (tgt[r] != IGN) a += logf(row_sum[r]) + row_max[r] - tgt_logit[r];
+    const int g = tgt[r];
+    if (g >= 0 && g < V) a += logf(row_sum[r]) + row_max[r] - tgt_logit[r];
   }
   a = block_sum<4>(a, sm);
   if (threadIdx.x == 0) loss[s] = a * inv_denom[s];
 }
 // in place: chunk logits -> chunk dlogits; ignored rows zeroed (wgsl.ts:1242)
-__global__ __launch_bounds__(256) void ce_chunk_grad_k(int vc, int v0, int T, int spans, float *chunk,
+__global__ __launch_bounds__(256) void ce_chunk_grad_k(int V, int vc, int v0, int T, int spans, float *chunk,
                                                        const int *__restrict__ tgt, const float *__restrict__ inv_denom,
                                                        const float *__restrict__ row_max, const float *__restrict__ row_sum,
                                                        float seed) {
   const int64_t row = blockIdx.x / spans;        // spans of a row are numbered fastest, as in ce_bwd_k
   const int span = blockIdx.x % spans;
   int g = tgt[row];
+  if (g < IGN || g >= V) g = IGN;
   const float sc = seed * inv_denom[row / T];
   const float m = row_max[row], il = 1.0f / row_sum[row];
   float *zr = chunk + row * vc;
@@ -275,37 +281,38 @@ int gt_ce_bwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets
   GT_LAUNCHED(ctx);
   return 0;
 }
-int gt_ce_chunk_stats(gt_ctx *ctx, int rows, int vc, int v0, int first, gt_buf chunk, gt_buf targets, gt_buf row_max,
+int gt_ce_chunk_stats(gt_ctx *ctx, int rows, int V, int vc, int v0, int first, gt_buf chunk, gt_buf targets, gt_buf row_max,
                       gt_buf row_sum, gt_buf tgt_logit) {
   GT_ENTER(ctx);
-  GT_REQUIRE(ctx, rows >= 1 && vc >= 1 && v0 >= 0 && chunk && targets && row_max && row_sum && tgt_logit, "gt_ce_chunk_stats: bad arguments");
+  GT_REQUIRE(ctx, rows >= 1 && vc >= 1 && v0 >= 0 && (int64_t)v0 + vc <= V && chunk && targets && row_max && row_sum && tgt_logit,
+             "gt_ce_chunk_stats: bad arguments (span [%d, %d) of %d logits)", v0, v0 + vc, V);
   ProfScope ps(ctx, "ce.chunk");
-  hipLaunchKernelGGL(ce_chunk_stats_k, dim3(rows), dim3(256), 0, ctx->stream, vc, v0, first, P<const float>(chunk),
-                     P<const int>(targets), P<float>(row_max), P<float>(row_sum), P<float>(tgt_logit));
+  hipLaunchKernelGGL(ce_chunk_stats_k, dim3(rows), dim3(256), 0, ctx->stream, V, vc, v0, first, P<const float>(chunk),
+                     P<const int>(targets), P<float>(row_max), P<float>(row_sum), P<float>(tgt_logit), ctx->bad_dev);
   GT_LAUNCHED(ctx);
   return 0;
 }
-int gt_ce_loss_from_stats(gt_ctx *ctx, int rows, int T, gt_buf targets, gt_buf inv_denom, gt_buf row_max, gt_buf row_sum,
+int gt_ce_loss_from_stats(gt_ctx *ctx, int rows, int V, int T, gt_buf targets, gt_buf inv_denom, gt_buf row_max, gt_buf row_sum,
                           gt_buf tgt_logit, gt_buf loss) {
   GT_ENTER(ctx);
-  GT_REQUIRE(ctx, rows >= 1 && T >= 1 && rows % T == 0 && targets && inv_denom && row_max && row_sum && tgt_logit && loss,
+  GT_REQUIRE(ctx, rows >= 1 && V >= 1 && T >= 1 && rows % T == 0 && targets && inv_denom && row_max && row_sum && tgt_logit && loss,
              "gt_ce_loss_from_stats: bad arguments");
   ProfScope ps(ctx, "ce.chunk");
-  hipLaunchKernelGGL(ce_loss_from_stats_k, dim3(rows / T), dim3(256), 0, ctx->stream, T, P<const int>(targets),
+  hipLaunchKernelGGL(ce_loss_from_stats_k, dim3(rows / T), dim3(256), 0, ctx->stream, V, T, P<const int>(targets),
                      P<const float>(inv_denom), P<const float>(row_max), P<const float>(row_sum), P<const float>(tgt_logit),
                      P<float>(loss));
   GT_LAUNCHED(ctx);
   return 0;
 }
-int gt_ce_chunk_grad(gt_ctx *ctx, int rows, int vc, int v0, int T, gt_buf chunk, gt_buf targets, gt_buf inv_denom,
+int gt_ce_chunk_grad(gt_ctx *ctx, int rows, int V, int vc, int v0, int T, gt_buf chunk, gt_buf targets, gt_buf inv_denom,
                      gt_buf row_max, gt_buf row_sum, float seed) {
   GT_ENTER(ctx);
-  GT_REQUIRE(ctx, rows >= 1 && vc >= 1 && T >= 1 && rows % T == 0 && chunk && targets && inv_denom && row_max && row_sum,
+  GT_REQUIRE(ctx, rows >= 1 && vc >= 1 && v0 >= 0 && (int64_t)v0 + vc <= V && T >= 1 && rows % T == 0 && chunk && targets && inv_denom && row_max && row_sum,
              "gt_ce_chunk_grad: bad arguments");
   ProfScope ps(ctx, "ce.chunk.bwd");
   const int spans = (int)cdiv(vc, CE_SPAN);
   GT_REQUIRE(ctx, (int64_t)rows * spans < (int64_t)1 << 31, "gt_ce_chunk_grad: %d rows x %d logits is more than one launch covers", rows, vc);
-  hipLaunchKernelGGL(ce_chunk_grad_k, dim3((unsigned)((int64_t)rows * spans)), dim3(256), 0, ctx->stream, vc, v0, T, spans,
+  hipLaunchKernelGGL(ce_chunk_grad_k, dim3((unsigned)((int64_t)rows * spans)), dim3(256), 0, ctx->stream, V, vc, v0, T, spans,
                      P<float>(chunk), P<const int>(targets), P<const float>(inv_denom), P<const float>(row_max),
                      P<const float>(row_sum), seed);
   GT_LAUNCHED(ctx);

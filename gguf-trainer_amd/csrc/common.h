@@ -45,6 +45,8 @@ struct gt_ctx {
   // [0] = which check (GT_BAD_*), [1] = row, [2] = the value, [3] = the bound. Read after the stream has drained.
   int *bad_host = nullptr, *bad_dev = nullptr;
   float *rms_static = nullptr;                  // this device's address of norm.hip's static scratch array
+  bool rms_static_pending = false;              // a gt_rmsnorm_bwd_static call is queued on this stream and the stream has not been waited for since
+  hipEvent_t mark = nullptr;                    // gt_stream_mark records it, another context's gt_stream_wait waits for it
   struct ProfSeen { int64_t n = 0; double work = 0; };
   std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not
 };
@@ -70,6 +72,7 @@ __device__ __forceinline__ void note_bad_id(int *bad, int what, int64_t row, int
 int gt_report_bad_id(gt_ctx *ctx);
 void optim_release_all(gt_ctx *ctx);            // optim.hip
 int rmsnorm_static_init(gt_ctx *ctx);           // norm.hip: looks up the static scratch array's address on ctx's device
+void rmsnorm_static_forget(gt_ctx *ctx);        // norm.hip: ctx is going away and must not be remembered as the array's last user
 // gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
 int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc);
 

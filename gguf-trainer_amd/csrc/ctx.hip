@@ -8,6 +8,7 @@ extern "C" {
 static void ctx_release(gt_ctx *c) {
   if (c->ws) hipFree(c->ws);
   if (c->bad_host) hipHostFree(c->bad_host);
+  if (c->mark) hipEventDestroy(c->mark);
   if (c->stream) hipStreamDestroy(c->stream);
   delete c;
 }
@@ -42,6 +43,7 @@ int gt_ctx_create(int device, gt_ctx **out) {
   }
   // the stream, and the pinned words kernels note an out-of-range id in
   if ((e = hipStreamCreate(&c->stream)) != hipSuccess ||
+      (e = hipEventCreateWithFlags(&c->mark, hipEventDisableTiming)) != hipSuccess ||
       (e = hipHostMalloc(reinterpret_cast<void **>(&c->bad_host), 4 * sizeof(int), hipHostMallocMapped)) != hipSuccess ||
       (e = hipHostGetDevicePointer(reinterpret_cast<void **>(&c->bad_dev), c->bad_host, 0)) != hipSuccess) {
     snprintf(g_create_err, sizeof g_create_err, "context setup failed: %s", hipGetErrorString(e));
@@ -62,6 +64,7 @@ int gt_ctx_destroy(gt_ctx *ctx) {
   if (!ctx) return 0;
   hipSetDevice(ctx->device);
   hipStreamSynchronize(ctx->stream);
+  rmsnorm_static_forget(ctx);
   optim_release_all(ctx);
   for (auto &kv : ctx->allocs) hipFree(reinterpret_cast<void *>(kv.first));
   for (auto &kv : ctx->rope_tables) hipFree(kv.second);
@@ -119,6 +122,7 @@ int gt_d2h(gt_ctx *ctx, void *dst, gt_buf src, size_t bytes) {
   GT_ENTER(ctx);
   if (bytes) GT_HIP(ctx, hipMemcpyAsync(dst, P<void>(src), bytes, hipMemcpyDeviceToHost, ctx->stream));
   GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  ctx->rms_static_pending = false;
   return gt_report_bad_id(ctx);
 }
 
@@ -132,7 +136,23 @@ int gt_d2d(gt_ctx *ctx, gt_buf dst, gt_buf src, size_t bytes) {
 int gt_sync(gt_ctx *ctx) {
   GT_ENTER(ctx);
   GT_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  ctx->rms_static_pending = false;
   return gt_report_bad_id(ctx);
+}
+
+// Ordering between two contexts' streams without the host waiting: everything queued on `ctx` so far ...
+int gt_stream_mark(gt_ctx *ctx) {
+  GT_ENTER(ctx);
+  GT_HIP(ctx, hipEventRecord(ctx->mark, ctx->stream));
+  return 0;
+}
+// ... is finished before anything queued on `ctx` after this call starts, where `other` is the context that was marked.
+int gt_stream_wait(gt_ctx *ctx, gt_ctx *other) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, other && other->device == ctx->device, "gt_stream_wait: the other context is null or on another device");
+  if (other == ctx) return 0;
+  GT_HIP(ctx, hipStreamWaitEvent(ctx->stream, other->mark, 0));
+  return 0;
 }
 
 int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes) {

@@ -889,8 +889,13 @@ int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, 
   bool eligible = kind == GT_TN && K % 32 == 0 && !ctx->opt_gemm_staged && ctx->opt_gemm_group;      // (TN: ld = M, N, below GT_DIRECT_LD_MAX for any grouped size)
   for (int i = 0; i < count; i++) {
     GT_REQUIRE(ctx, M[i] >= 1 && N[i] >= 1 && A[i] && B[i] && C[i], "gt_gemm_group: product %d has M %d, N %d or a null operand", i, M[i], N[i]);
-    for (int j = 0; j < i; j++) GT_REQUIRE(ctx, C[i] != C[j], "gt_gemm_group: products %d and %d write the same output", j, i);
+    for (int j = 0; j < i; j++)
+      GT_REQUIRE(ctx, C[i] + (uint64_t)M[i] * N[i] * 4 <= C[j] || C[j] + (uint64_t)M[j] * N[j] * 4 <= C[i],
+                 "gt_gemm_group: the outputs of products %d and %d overlap", j, i);
   }
+  const int pin = ctx->opt_gemm_tile;
+  GT_REQUIRE(ctx, !(eligible && pin >= 0 && pin != 6 && pin != 7 && pin != 8 && pin != 11 && pin != 12),
+             "gt_gemm_group: \"gemm.tile\" pins tile %d, which the grouped launch does not have (6, 7, 8, 11 or 12; -1 = choose)", pin);
   if (count > GT_GROUP_MAX) {
     for (int i = 0; i < count; i += GT_GROUP_MAX)
       if (gt_gemm_group(ctx, kind, std::min(GT_GROUP_MAX, count - i), M + i, N + i, K, A + i, B + i, C + i, acc + i)) return 1;

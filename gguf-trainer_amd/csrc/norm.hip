@@ -226,6 +226,16 @@ __global__ __launch_bounds__(256) void rmsnorm_dw_gen(int rows, int d, int slab,
 #define RMS_STATIC_FLOATS (512 * RMS_STATIC_MAX_D)          // 4 MiB
 static __device__ __align__(256) float scratch[RMS_STATIC_FLOATS];
 
+// The array is one per device and every context on the device shares it. The last context that queued a static call on
+// each device is remembered: a call from another context while that one's stream has not been waited for since would race
+// on the partials and is refused.
+#define RMS_STATIC_MAX_DEV 64
+static gt_ctx *g_static_last[RMS_STATIC_MAX_DEV];
+
+void rmsnorm_static_forget(gt_ctx *ctx) {
+  if (ctx->device >= 0 && ctx->device < RMS_STATIC_MAX_DEV && g_static_last[ctx->device] == ctx) g_static_last[ctx->device] = nullptr;
+}
+
 int rmsnorm_static_init(gt_ctx *ctx) {
   void *ptr = nullptr;
   GT_HIP(ctx, hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));      // this device's copy: the context's device is current
@@ -340,6 +350,10 @@ int gt_rmsnorm_bwd_static(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_b
   GT_REQUIRE(ctx, rows >= 0 && d >= 1 && x && w && g && rinv && dx, "gt_rmsnorm_bwd_static: bad arguments (rows %d, d %d)", rows, d);
   GT_REQUIRE(ctx, d <= RMS_STATIC_MAX_D, "gt_rmsnorm_bwd_static: d = %d is more than the static scratch is sized for (%d)", d, RMS_STATIC_MAX_D);
   GT_REQUIRE(ctx, ctx->rms_static, "gt_rmsnorm_bwd_static: the static scratch array has no device address");
+  GT_REQUIRE(ctx, ctx->device < RMS_STATIC_MAX_DEV, "gt_rmsnorm_bwd_static: device %d is beyond the %d this entry point keeps track of", ctx->device, RMS_STATIC_MAX_DEV);
+  gt_ctx *last = g_static_last[ctx->device];
+  GT_REQUIRE(ctx, !dw || !last || last == ctx || !last->rms_static_pending,
+             "gt_rmsnorm_bwd_static: another context's call on this device is still queued and shares the scratch array; gt_sync that context first");
   if (rows == 0) {
     if (dw && !acc_dw) {
       hipLaunchKernelGGL(fill_zero_k, dim3((unsigned)cdiv(d, 256)), dim3(256), 0, ctx->stream, d, P<float>(dw));
@@ -347,6 +361,7 @@ int gt_rmsnorm_bwd_static(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_b
     }
     return 0;
   }
+  if (dw) { g_static_last[ctx->device] = ctx; ctx->rms_static_pending = true; }      // without dw the array is not touched
   return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dx, dw, acc_dw, ctx->rms_static);
 }
 int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,

@@ -89,7 +89,12 @@ class HipBackend:
         self._cur = 0                     # stream of the micro-batch being recorded
         self._used = set()                # streams other than the first with work queued since the last join
         self._bw_seen = False             # a backward closure has run since the last switch: the next graph root starts a micro-batch
-        self._s0_barrier = False          # the first stream holds work (uploads, an optimizer step, a fold) another stream must not overtake
+        self.backward_depth = 0           # raised by autograd while closures are walked: a checkpoint's replay is not a new graph
+        # the first stream holds work (uploads, an optimizer step, a fold) another stream must not overtake: the point is
+        # marked on the first stream when that work is queued, and a stream that starts a micro-batch afterwards waits for
+        # the mark on the device (the host does not wait, and the first stream's own micro-batch is not waited for)
+        self._s0_barrier = False
+        self._s0_waited: set = set()
         self._sfold: list = []            # (tensor, entry) of parameters with a written accumulator on another stream
         self._limbo: list = []            # entries of parameters that were released or collected: their buffers return to the pools at the next sync
         self.adapter_name = lib.gt_device_name(self._ctx).decode()
@@ -150,23 +155,27 @@ class HipBackend:
     def _op_begin(self, *inputs):
         """Called first thing by every forward op. After a backward has run, an op whose inputs are all parameters or
         host data is the root of the next micro-batch's graph: it goes to the next stream."""
-        if not self._bw_seen:
-            return
-        if self._nstreams == 1:
-            return
+        if not self._bw_seen or self._nstreams == 1 or self.backward_depth:
+            return                  # (a forward op inside a backward is a checkpoint replaying its block: same micro-batch)
         for t in inputs:
             e = self._entries.get(t)
             if e is not None and not e.external:
                 return
         self._flush()
         self._flush_dx()
-        if self._s0_barrier:
-            check(self._ctxs[0], lib.gt_sync(self._ctxs[0]), "gt_sync")
-            self._s0_barrier = False
         self._cur = (self._cur + 1) % self._nstreams
         if self._cur:
             self._used.add(self._cur)
+            if self._s0_barrier and self._cur not in self._s0_waited:
+                check(self._ctx, lib.gt_stream_wait(self._ctx, self._ctxs[0]), "gt_stream_wait")
+                self._s0_waited.add(self._cur)
         self._bw_seen = False
+
+    def _barrier0(self):
+        """Work that the other streams must not overtake has just been queued on the first stream."""
+        check(self._ctxs[0], lib.gt_stream_mark(self._ctxs[0]), "gt_stream_mark")
+        self._s0_barrier = True
+        self._s0_waited = set()
 
     def _join(self):
         """Everything recorded on the other streams has finished and their parameter-gradient accumulators are summed, in
@@ -201,7 +210,7 @@ class HipBackend:
                         slot[1] = False
                 e.grad_init = True
             check(self._ctxs[0], lib.gt_grad_fold(self._ctxs[0], n, dst, acc, ns, src, sizes), "gt_grad_fold")
-            self._s0_barrier = True
+            self._barrier0()
 
     # ---- install (webgpu.ts:393-399) ---------------------------------------------------------------
     # ---- a linear's forward launch is held back by one op: two consecutive linears over the same input with the same
@@ -364,7 +373,7 @@ class HipBackend:
             if self._cur:
                 check(c0, lib.gt_sync(c0), "gt_sync")       # uploaded on the first stream, read by this one
             else:
-                self._s0_barrier = True
+                self._barrier0()
             self._entries[t] = e
             self._externals.add(t)
             # when the tensor is collected its device buffers go back to the pools (at the next sync: queued work may still read them)
@@ -423,6 +432,12 @@ class HipBackend:
         e.data = self._acquire(e.nbytes, e.stream)
         check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, rows, outd, ind, xd, wd, e.data), "linear")
 
+    def _same_stream(self, e: _Entry):
+        """An intermediate made by another micro-batch's stream is about to have its gradient read or written here
+        (a closure walked after the recording moved on): that stream's queued work goes first."""
+        if e.stream != self._cur and not e.external:
+            check(self._ctxs[e.stream], lib.gt_sync(self._ctxs[e.stream]), "gt_sync")
+
     def _gdst(self, t: Tensor) -> tuple:
         """(gradient buffer, acc) for a backward kernel about to contribute to t's gradient;
         (0, 0) when t takes no gradient (a frozen parameter)."""
@@ -435,6 +450,7 @@ class HipBackend:
         if e is None:
             e = self._entry_for(t)
         self._bw_seen = True
+        self._same_stream(e)
         if e.external and not t.requires_grad:
             return 0, 0
         if e.external and self._cur:
@@ -506,6 +522,7 @@ class HipBackend:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
                                "gradient buffers, so this backward would read pool garbage")
         self._bw_seen = True
+        self._same_stream(e)
         if e.grad_src:
             return e.grad_src       # handed on by an add's backward and not written since: read it where it is
         if e.grad == 0 or not e.grad_init:
@@ -523,7 +540,7 @@ class HipBackend:
         for t in tensors:
             e = self._entry_for(t)
             check(self._ctx, lib.gt_h2d(self._ctx, e.data, t.data.ctypes.data_as(C.c_void_p), e.nbytes), "gt_h2d")
-        self._s0_barrier = True
+        self._barrier0()
 
     def buffers_for(self, t: Tensor) -> dict:
         self._join()
@@ -576,7 +593,7 @@ class HipBackend:
         """The optimizer has read these accumulators: the next backward write stores instead of adding
         (the reference's deferred per-step clear, src/backend/muon-gpu.ts:8-16)."""
         self._join()
-        self._s0_barrier = True      # the optimizer's launches are on the first stream: no other stream may read weights before them
+        self._barrier0()             # the optimizer's launches are on the first stream: no other stream may read weights before them
         for t in tensors:
             e = self._entries.get(t)
             if e is not None:
@@ -610,7 +627,7 @@ class HipBackend:
         out = c_buf()
         c0 = self._ctxs[0]
         check(c0, lib.gt_alloc(c0, max(4, nbytes), 1, C.byref(out)), "gt_alloc")
-        self._s0_barrier = True
+        self._barrier0()
         self._state_bytes += max(4, nbytes)
         return out.value
 
@@ -618,7 +635,7 @@ class HipBackend:
         self._join()
         arr = np.ascontiguousarray(arr)
         check(self._ctx, lib.gt_h2d(self._ctx, b, arr.ctypes.data_as(C.c_void_p), arr.nbytes), "gt_h2d")
-        self._s0_barrier = True
+        self._barrier0()
 
     def read_state_buffer(self, b: int, n: int, dtype=np.float32) -> np.ndarray:
         self._join()
@@ -1170,9 +1187,9 @@ class HipBackend:
         spans = [(v0, min(v0 + chunk, V) - v0) for v0 in range(0, V, chunk)]
         for i, (v0, vc) in enumerate(spans):
             check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, rows, vc, H, hd_, wd + v0 * H * 4, cb), "fusedCE.logits")
-            check(self._ctx, lib.gt_ce_chunk_stats(self._ctx, rows, vc, v0, 1 if i == 0 else 0, cb, tg, rmax, rsum, tl), "fusedCE.stats")
+            check(self._ctx, lib.gt_ce_chunk_stats(self._ctx, rows, V, vc, v0, 1 if i == 0 else 0, cb, tg, rmax, rsum, tl), "fusedCE.stats")
         loss, e = self._make_out([nseq], [hidden, w])
-        check(self._ctx, lib.gt_ce_loss_from_stats(self._ctx, rows, T, tg, invb, rmax, rsum, tl, e.data), "fusedCE.loss")
+        check(self._ctx, lib.gt_ce_loss_from_stats(self._ctx, rows, V, T, tg, invb, rmax, rsum, tl, e.data), "fusedCE.loss")
         wants_dw = w.requires_grad
 
         def bw():
@@ -1183,7 +1200,7 @@ class HipBackend:
             dw, accw = self._gdst(w) if wants_dw else (0, 0)
             for v0, vc in spans:
                 check(self._ctx, lib.gt_gemm(self._ctx, NT, 0, rows, vc, H, hd_, wd + v0 * H * 4, cb), "fusedCE.logits")
-                check(self._ctx, lib.gt_ce_chunk_grad(self._ctx, rows, vc, v0, T, cb, tg, invb, rmax, rsum, seed), "fusedCE.grad")
+                check(self._ctx, lib.gt_ce_chunk_grad(self._ctx, rows, V, vc, v0, T, cb, tg, invb, rmax, rsum, seed), "fusedCE.grad")
                 check(self._ctx, lib.gt_gemm(self._ctx, NN, acch, rows, H, vc, cb, wd + v0 * H * 4, dh), "fusedCE.dh")
                 acch = 1
                 if dw:

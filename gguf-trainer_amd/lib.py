@@ -38,6 +38,8 @@ _SIG = {
     "gt_d2h": [ctxp, C.c_void_p, buf, sz],
     "gt_d2d": [ctxp, buf, buf, sz],
     "gt_sync": [ctxp],
+    "gt_stream_mark": [ctxp],
+    "gt_stream_wait": [ctxp, ctxp],
     "gt_resident_bytes": [ctxp, C.POINTER(C.c_uint64)],
     "gt_set_option": [ctxp, C.c_char_p, i32],
     "gt_gemm": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf],
@@ -75,9 +77,9 @@ _SIG = {
     "gt_attn_bwd_scores": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, buf, buf, buf, i32, buf, i32, buf, i32],
     "gt_ce_fwd": [ctxp, i32, i32, i32, buf, buf, buf, buf, buf],
     "gt_ce_bwd": [ctxp, i32, i32, i32, buf, buf, buf, buf, f32, buf, i32],
-    "gt_ce_chunk_stats": [ctxp, i32, i32, i32, i32, buf, buf, buf, buf, buf],
-    "gt_ce_loss_from_stats": [ctxp, i32, i32, buf, buf, buf, buf, buf, buf],
-    "gt_ce_chunk_grad": [ctxp, i32, i32, i32, i32, buf, buf, buf, buf, buf, f32],
+    "gt_ce_chunk_stats": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf],
+    "gt_ce_loss_from_stats": [ctxp, i32, i32, i32, buf, buf, buf, buf, buf, buf],
+    "gt_ce_chunk_grad": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, f32],
     "gt_soft_ce_fwd": [ctxp, i32, i32, i32, buf, buf, buf, f32, buf, buf, buf],
     "gt_soft_ce_bwd": [ctxp, i32, i32, i32, buf, buf, buf, f32, buf, buf, f32, buf, i32],
     "gt_adamw_create": [ctxp, i32, C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(buf), C.POINTER(i64),

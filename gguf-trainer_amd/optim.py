@@ -47,6 +47,9 @@ class AdamWHip:
 
     def destroy(self):
         """Release the device-side tables; the moment buffers go back with the backend's state buffers."""
+        if self.gpu._destroyed:             # the library context is gone and took the tables and the buffers with it
+            self._h, self._m, self._v = C.c_void_p(), [], []
+            return
         if self._h:
             check(self.gpu.ctx, lib.gt_adamw_destroy(self.gpu.ctx, self._h), "gt_adamw_destroy")
             self._h = C.c_void_p()
@@ -120,6 +123,10 @@ class MuonHip:
 
     def destroy(self):
         """Release the per-shape work buffers and pointer tables, the momentum buffers and the auxiliary AdamW."""
+        if self.gpu._destroyed:
+            self._h, self._bufs = C.c_void_p(), []
+            self.aux.destroy()
+            return
         if self._h:
             check(self.gpu.ctx, lib.gt_muon_destroy(self.gpu.ctx, self._h), "gt_muon_destroy")
             self._h = C.c_void_p()

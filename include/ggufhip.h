@@ -60,6 +60,13 @@ int gt_h2d(gt_ctx *ctx, gt_buf dst, const void *src, size_t bytes);   /* enqueue
 int gt_d2h(gt_ctx *ctx, void *dst, gt_buf src, size_t bytes);         /* waits for the stream */
 int gt_d2d(gt_ctx *ctx, gt_buf dst, gt_buf src, size_t bytes);
 int gt_sync(gt_ctx *ctx);
+/* Ordering between the streams of two contexts on one device without the host waiting (no reference counterpart: a
+ * WebGPU device has one queue, webgpu.ts:129-141; a host that records independent micro-batches on several contexts needs
+ * it where they meet: weights written by an optimizer step on one stream and read by forward passes on the others).
+ * gt_stream_mark(a) notes the point a's stream has reached; gt_stream_wait(b, a) makes everything queued on b afterwards
+ * start only when a's work up to its latest mark has finished. Neither call blocks the host or allocates. */
+int gt_stream_mark(gt_ctx *ctx);
+int gt_stream_wait(gt_ctx *ctx, gt_ctx *marked);
 int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt_alloc bytes + workspace */
 /* Kernel-selection switches for tests and tuning (no reference counterpart; WebGPUBackend exposes
  * attnFlashMinT as a public field for the same purpose, webgpu.ts:305):
@@ -215,20 +222,20 @@ int gt_attn_bwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int w
  * bwd: dlogits[r,:] (+)= seed * inv_denom[s] * (softmax - onehot); ignored rows get 0 (acc = 0)
  * or are left alone (acc = 1).
  * Precondition: every target is -1 or in [0, V) (checked above the dispatch in the reference, autograd.ts:875-894).
- * A target outside that range is never used as an index: gt_ce_fwd counts the row as ignored and the next gt_sync /
- * gt_d2h / gt_prof_end fails once, naming the row; the chunked kernels and gt_ce_bwd only compare targets with column
- * numbers. */
+ * A target outside that range is never used as an index: every kernel, forward and backward, dense and chunked, treats
+ * the row as ignored; gt_ce_fwd (dense) and the first gt_ce_chunk_stats of a pass (chunked) note it and the next gt_sync /
+ * gt_d2h / gt_prof_end fails once, naming the row. */
 int gt_ce_fwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets, gt_buf inv_denom,
               gt_buf loss, gt_buf lse);
 int gt_ce_bwd(gt_ctx *ctx, int rows, int V, int T, gt_buf logits, gt_buf targets, gt_buf inv_denom,
               gt_buf lse, float seed, gt_buf dlogits, int acc);
 /* chunked path: srcCeChunkStats / CeLossFromStats / CeChunkGrad (wgsl.ts:1153-1247),
- * fusedCrossEntropy (webgpu.ts:1214-1278). `chunk` holds logits of vocab span [v0, v0+vc). */
-int gt_ce_chunk_stats(gt_ctx *ctx, int rows, int vc, int v0, int first, gt_buf chunk, gt_buf targets,
+ * fusedCrossEntropy (webgpu.ts:1214-1278). `chunk` holds logits of vocab span [v0, v0+vc) of the V-wide vocabulary. */
+int gt_ce_chunk_stats(gt_ctx *ctx, int rows, int V, int vc, int v0, int first, gt_buf chunk, gt_buf targets,
                       gt_buf row_max, gt_buf row_sum, gt_buf tgt_logit);
-int gt_ce_loss_from_stats(gt_ctx *ctx, int rows, int T, gt_buf targets, gt_buf inv_denom,
+int gt_ce_loss_from_stats(gt_ctx *ctx, int rows, int V, int T, gt_buf targets, gt_buf inv_denom,
                           gt_buf row_max, gt_buf row_sum, gt_buf tgt_logit, gt_buf loss);
-int gt_ce_chunk_grad(gt_ctx *ctx, int rows, int vc, int v0, int T, gt_buf chunk, gt_buf targets,
+int gt_ce_chunk_grad(gt_ctx *ctx, int rows, int V, int vc, int v0, int T, gt_buf chunk, gt_buf targets,
                      gt_buf inv_denom, gt_buf row_max, gt_buf row_sum, float seed);
 /* sparse-teacher soft CE: srcSoftCeFwd / BwdP / BwdQ (wgsl.ts:1004-1110), webgpu.ts:1331-1378. teacher_ids[rows*k]:
  * a row whose first id is -1 is ignored; every other id must be in [0, V) (autograd.ts:974-998 checks it above the

@@ -5,7 +5,7 @@ import math
 import numpy as np
 import pytest
 
-from gpu_common import LOSS_REL, assert_close, mod
+from gpu_common import LOSS_REL, assert_close, backward_from, mod
 
 pytestmark = pytest.mark.gpu
 
@@ -890,3 +890,73 @@ def test_kernel_family_cannot_change_under_a_live_graph(gpu, ref):
         gpu.set_option("attn.generic", 0)
     finally:
         gpu.uninstall()
+
+
+def test_checkpoint_over_leaf_inputs_after_an_earlier_backward(gpu, ref):
+    """A checkpointed block whose declared inputs are parameters (the gradcheck-style use, gradcheck.ts:770-806), differentiated
+    after another graph's backward has already run: the block's replay records forward ops in the middle of a backward,
+    all of whose inputs are leaves. That replay belongs to the graph being differentiated: it must not start a micro-batch
+    on another stream (the replayed output's gradient, the seed copy and the rest of the tape would then run on two
+    streams with nothing ordering them). Gradients against the oracle and against a one-stream backend, bit for bit."""
+    hb, ag = mod("hip_backend"), mod("autograd")
+    assert gpu._nstreams == 4
+    r = ref.Mulberry32(77)
+    T, d = 96, 64
+    xs, w1s, w2s, w0s = r.fill_randn([T, d], 0.8), r.fill_randn([d, d], 0.3), r.fill_randn([d, d], 0.3), r.fill_randn([d, d], 0.3)
+    up = ref.Mulberry32(5).fill_uniform([T * d])
+
+    def run(be):
+        x, w1, w2, w0 = (ag.Tensor(a, list(a.shape), True) for a in (xs, w1s, w2s, w0s))
+        be.install()
+        ag.set_checkpointing(True)
+        try:
+            first = ag.linear(x, w0)                             # an earlier graph and its backward
+            backward_from(be, ag, first, up)
+            streams_seen = []
+            def block():
+                o = ag.linear(ag.silu(ag.linear(x, w1)), w2)
+                streams_seen.append(be._cur)                     # the stream the block's ops were recorded on
+                return o
+            out = ag.checkpoint([x, w1, w2], block)              # every declared input is a leaf
+            y = ag.add(out, ag.linear(x, w0))
+            cur = be._cur
+            backward_from(be, ag, y, up)
+            assert be._cur == cur, "the replay inside the backward moved the recording to another stream"
+            assert streams_seen == [cur, cur]
+            be.sync([y])
+        finally:
+            ag.set_checkpointing(False)
+            be.uninstall()
+        return y.data.copy(), [t.grad.copy() for t in (x, w1, w2, w0)]
+
+    y4, g4 = run(gpu)
+    one = hb.HipBackend(0, streams=1)
+    try:
+        y1, g1 = run(one)
+    finally:
+        one.destroy()
+    assert y4.tobytes() == y1.tobytes()
+    for a, b, n in zip(g4, g1, "x w1 w2 w0".split()):
+        assert_close(a, b, f"four streams vs one, d{n}", rel_l2=2e-6, max_rel=2e-5)
+    rx, rw1, rw2, rw0 = (ref.Tensor(a, list(a.shape), True) for a in (xs, w1s, w2s, w0s))
+    ref.backward_from(ref.linear(rx, rw0), up)
+    ry = ref.add(ref.linear(ref.silu(ref.linear(rx, rw1)), rw2), ref.linear(rx, rw0))
+    ref.backward_from(ry, up)
+    assert_close(y4, ry.data, "checkpointed block over leaf inputs, forward")
+    for a, t, n in zip(g4, (rx, rw1, rw2, rw0), "x w1 w2 w0".split()):
+        assert_close(a, t.grad, f"checkpointed block over leaf inputs, d{n}")
+
+
+def test_optimizer_destroy_after_the_backend_is_gone(ref):
+    """gt_ctx_destroy releases every live optimizer of the context; an optimizer object destroyed after its backend must
+    not hand the freed handles back to the library."""
+    hb, optim, ag = mod("hip_backend"), mod("optim"), mod("autograd")
+    be = hb.HipBackend(0, streams=2)
+    r = ref.Mulberry32(3)
+    ps = [ag.Tensor(r.fill_randn([8, 8], 0.1), [8, 8], True), ag.Tensor(r.fill_randn([8], 0.1), [8], True)]
+    mu = optim.MuonHip(be, ps[:1], ps[1:], lr=0.01)
+    ad = optim.AdamWHip(be, ps, lr=1e-3)
+    be.destroy()
+    mu.destroy()
+    ad.destroy()
+    assert not ad._h and not mu._h and ad._m == [] and mu._bufs == []

@@ -129,9 +129,20 @@ def test_gemm_group_equals_the_products_one_by_one(gpu, K, shapes, splitk):
         gpu.set_option("gemm.group", 1)
         gpu.set_option("gemm.tile", -1)
         gpu.set_option("gemm.splitk", -1)
-    with pytest.raises(lib.HipError, match="write the same output"):
+    with pytest.raises(lib.HipError, match="overlap"):
         cc2 = (C.c_uint64 * n)(*([dc[0]] * n))
         lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, n, Ms, Ns, K, aa, bb, cc2, ac), "gt_gemm_group")
+    if n >= 2 and shapes[0][0] * shapes[0][1] > 4:
+        with pytest.raises(lib.HipError, match="overlap"):      # the second output starts inside the first
+            cc3 = (C.c_uint64 * n)(*([dc[0], dc[0] + 16] + dc[2:]))
+            lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, n, Ms, Ns, K, aa, bb, cc3, ac), "gt_gemm_group")
+    if K % 32 == 0:
+        gpu.set_option("gemm.tile", 3)                           # a register-staged tile: the grouped launch has none such
+        try:
+            with pytest.raises(lib.HipError, match="pins tile 3"):
+                lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, n, Ms, Ns, K, aa, bb, cc, ac), "gt_gemm_group")
+        finally:
+            gpu.set_option("gemm.tile", -1)
 
 
 @pytest.mark.parametrize("rows,K,r", [(16, 64, 16), (100, 192, 16), (257, 1024, 16), (333, 128, 8), (64, 64, 3), (129, 256, 32),

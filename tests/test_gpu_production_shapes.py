@@ -300,7 +300,31 @@ def test_out_of_range_ids_are_skipped_and_reported(gpu):
     want = 0.5 * ((lse[0] - z64[0, 5]) + (lse[3] - z64[3, 0]))
     assert abs(gpu.read_state_buffer(bloss, 1)[0] - want) <= 1e-5 * abs(want)
     lib.check(gpu.ctx, L.gt_ce_bwd(gpu.ctx, rows, Vc, rows, bz, btg, binv, blse, 1.0, bdz, 0), "ce.bwd")
-    assert sync_error() == ""                                    # the backward only compares targets with column numbers
+    assert sync_error() == ""                                    # reported once, by the forward
+    dzb = gpu.read_state_buffer(bdz, rows * Vc).reshape(rows, Vc)
+    pz = np.exp(z64 - lse[:, None])
+    wantb = 0.5 * pz
+    wantb[0, 5] -= 0.5
+    wantb[3, 0] -= 0.5
+    wantb[1] = 0
+    wantb[2] = 0                                                 # the bad row is ignored in the backward as in the forward
+    assert_close(dzb, wantb, "dense CE backward with an out-of-range target")
+    # the chunked path (two spans of 6): the first statistics pass notes the row, loss and gradient ignore it
+    brm, brs, btl = (gpu.create_state_buffer(rows * 4) for _ in range(3))
+    bl2 = gpu.create_state_buffer(4)
+    chunks = [np.ascontiguousarray(z[:, v0:v0 + 6]) for v0 in (0, 6)]
+    bch = [dev(gpu, c) for c in chunks]
+    for i, v0 in enumerate((0, 6)):
+        lib.check(gpu.ctx, L.gt_ce_chunk_stats(gpu.ctx, rows, Vc, 6, v0, 1 if i == 0 else 0, bch[i], btg, brm, brs, btl), "stats")
+    lib.check(gpu.ctx, L.gt_ce_loss_from_stats(gpu.ctx, rows, Vc, rows, btg, binv, brm, brs, btl, bl2), "loss")
+    assert "cross-entropy target 12 at row 2 is outside [-1, 12)" in sync_error()
+    assert abs(gpu.read_state_buffer(bl2, 1)[0] - want) <= 1e-5 * abs(want)
+    for i, v0 in enumerate((0, 6)):
+        lib.check(gpu.ctx, L.gt_ce_chunk_grad(gpu.ctx, rows, Vc, 6, v0, rows, bch[i], btg, binv, brm, brs, 1.0), "grad")
+        assert_close(gpu.read_state_buffer(bch[i], rows * 6).reshape(rows, 6), wantb[:, v0:v0 + 6], f"chunked CE gradient, span {i}")
+    assert sync_error() == ""
+    rc = L.gt_ce_chunk_stats(gpu.ctx, rows, Vc, 8, 6, 0, bch[1], btg, brm, brs, btl)      # span [6, 14) of 12 logits
+    assert rc != 0 and "span [6, 14) of 12" in L.gt_last_error(gpu.ctx).decode()
 
     k = 2
     tid = np.array([1, 2, -1, 0, 3, 40, 4, 4], np.int32)         # row 2: second teacher id 40 >= V

@@ -62,3 +62,39 @@ def test_static_scratch_rmsnorm_backward_refuses_what_it_cannot_hold(gpu):
     dw = dev(gpu, np.ones(64, np.float32))
     lib.check(gpu.ctx, L.gt_rmsnorm_bwd_static(gpu.ctx, 0, 64, b, b, b, b, b, 0, dw, 0), "bwd")
     assert not np.any(gpu.read_state_buffer(dw, 64))
+
+
+def test_static_scratch_is_not_shared_by_two_contexts_at_once(gpu):
+    """The scratch array is one per device. A second context's call while the first one's is still queued would race on
+    it: refused until the first context has been waited for."""
+    lib, hb = mod("lib"), mod("hip_backend")
+    L = lib.lib
+    other = hb.HipBackend(0, streams=1)
+    try:
+        rows, d = 4096, 256
+        rs = np.random.RandomState(9)
+        x = rs.standard_normal((rows, d)).astype(np.float32)
+        w = np.ones(d, np.float32)
+
+        def bufs(be):
+            bx, bw = dev(be, x), dev(be, w)
+            br, bdx, bdw = be.create_state_buffer(rows * 4), be.create_state_buffer(x.nbytes), be.create_state_buffer(d * 4)
+            lib.check(be.ctx, L.gt_rmsnorm_fwd(be.ctx, rows, d, 1e-5, bx, bw, bdx, br), "fwd")
+            return bx, bw, br, bdx, bdw
+        a, b = bufs(gpu), bufs(other)
+        lib.check(gpu.ctx, L.gt_sync(gpu.ctx), "sync")
+        lib.check(other.ctx, L.gt_sync(other.ctx), "sync")
+        lib.check(gpu.ctx, L.gt_rmsnorm_bwd_static(gpu.ctx, rows, d, a[0], a[1], a[0], a[2], a[3], 0, a[4], 0), "bwd")
+        rc = L.gt_rmsnorm_bwd_static(other.ctx, rows, d, b[0], b[1], b[0], b[2], b[3], 0, b[4], 0)
+        assert rc != 0 and "gt_sync that context first" in L.gt_last_error(other.ctx).decode()
+        # without dw the array is not touched: allowed
+        lib.check(other.ctx, L.gt_rmsnorm_bwd_static(other.ctx, rows, d, b[0], b[1], b[0], b[2], b[3], 0, 0, 0), "bwd")
+        lib.check(gpu.ctx, L.gt_sync(gpu.ctx), "sync")
+        lib.check(other.ctx, L.gt_rmsnorm_bwd_static(other.ctx, rows, d, b[0], b[1], b[0], b[2], b[3], 0, b[4], 0), "bwd")
+        got_a, got_b = gpu.read_state_buffer(a[4], d), other.read_state_buffer(b[4], d)
+        assert np.array_equal(got_a, got_b)
+    finally:
+        other.destroy()
+    # the context that last used the array is gone: the next caller is not held up by it
+    lib.check(gpu.ctx, L.gt_rmsnorm_bwd_static(gpu.ctx, rows, d, a[0], a[1], a[0], a[2], a[3], 0, a[4], 0), "bwd")
+    lib.check(gpu.ctx, L.gt_sync(gpu.ctx), "sync")
