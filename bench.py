@@ -104,6 +104,13 @@ def cpu_baseline():
     ids = zipf_tokens(cfg.vocab, T + 1, 1)
     ref.set_threads(cores)
     ref.PARALLEL_BWD = True
+    REPS = 3
+
+    def stats(fn):
+        """one untimed warm-up, then REPS timed runs: (min, median, all)"""
+        fn()
+        ts = sorted(timed(fn) for _ in range(REPS))
+        return ts[0], ts[len(ts) // 2], ts
     try:
         # (1) one layer, whole sequence
         h0 = ref.Tensor((0.5 * rs.standard_normal((T, cfg.hidden))).astype(np.float32), [T, cfg.hidden], True)
@@ -112,7 +119,7 @@ def cpu_baseline():
         def layer():
             o = model._block(h0, model.layers[0], 0, T)()
             ref.backward_from(o, up)
-        t_layer = timed(layer)
+        layer_min, layer_med, layer_all = stats(layer)
         # (2) readout + loss on a quarter of the rows
         RS = 512
         hs = ref.Tensor((0.5 * rs.standard_normal((RS, cfg.hidden))).astype(np.float32), [RS, cfg.hidden], True)
@@ -120,14 +127,19 @@ def cpu_baseline():
         def head():
             loss = ref.cross_entropy(ref.linear(ref.rms_norm(hs, model.outputNorm, cfg.rms_eps), model.tokenEmbd), ids[1:RS + 1].tolist())
             ref.backward(loss, 1.0)
-        t_head = timed(head) * (T / RS)
+        head_min, head_med, head_all = stats(head)
         # (3) AdamW over the layer + table + final norm
         opt = ref.AdamW(model.params(), lr=1e-3, beta2=0.95, weight_decay=0.1)
-        t_opt = timed(opt.step)
+        opt_min, opt_med, opt_all = stats(opt.step)
         n_layer = sum(p.size for p in model.layers[0].values())
         n_head = model.tokenEmbd.size + model.outputNorm.size
-        t_opt_full = t_opt * (n_head + 30 * n_layer) / (n_head + n_layer)
-        per_token = (30 * t_layer + t_head) / T + t_opt_full / (BATCH * SEQ)
+        opt_scale = (n_head + 30 * n_layer) / (n_head + n_layer)
+
+        def per_token_of(tl, th, to):
+            return (30 * tl + th * (T / RS)) / T + to * opt_scale / (BATCH * SEQ)
+        per_token = per_token_of(layer_med, head_med, opt_med)          # `value`: the median run
+        per_token_best = per_token_of(layer_min, head_min, opt_min)
+        t_layer, t_head, t_opt = layer_med, head_med * (T / RS), opt_med
         # (4) configs[1]: isolated backward kernels on 1024 of 16384 rows
         R1, H, F, V = 1024, 576, 1536, 49152
         x = ref.Tensor(rs.standard_normal((R1, H)).astype(np.float32), [R1, H], True)
@@ -171,7 +183,11 @@ def cpu_baseline():
     t_tiny = timed(tiny_step)
     slowdown = t_small_1t / max(t_small_mt, 1e-9)
     return {"value": round(1.0 / per_token, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"oracle (C restatement of the reference's CPU ops) under OpenMP: one SmolLM2 layer fwd+bwd on a whole "
+            "runs": {"warmup": 1, "timed": REPS, "median_tokens_per_s": round(1.0 / per_token, 2), "best_tokens_per_s": round(1.0 / per_token_best, 2),
+                     "layer_s": [round(t, 3) for t in layer_all], "readout_s": [round(t, 3) for t in head_all],
+                     "adamw_s": [round(t, 4) for t in opt_all]},
+            "sample": f"oracle (C restatement of the reference's CPU ops) under OpenMP, each part run once untimed and then {REPS} times "
+                      f"(value = from the medians): one SmolLM2 layer fwd+bwd on a whole "
                       f"{T}-token sequence {t_layer:.2f} s (x30), tied readout + cross-entropy fwd+bwd on {RS} of {T} rows "
                       f"{t_head * RS / T:.2f} s (x{T // RS}), AdamW over one layer + table {t_opt:.2f} s (scaled to 134.5 M parameters, once per "
                       f"{BATCH * SEQ} tokens)",
@@ -186,11 +202,15 @@ def cpu_baseline():
                               "seconds": round(t_tiny, 3), "tokens/s": round(512 / t_tiny, 1)}}
 
 
-def micro_kernels(gpu, L, reps=10):
+def micro_kernels(gpu, L, reps=10, sustained=30):
     """benchmark configs[1]: the isolated backward kernels at the SmolLM2 MLP shape, timed with HIP events on the
     library's stream. fp32 dX = dY.W and dW = dY^T.X with X [16384x576], W [1536x576], dY [16384x1536]; softmax-CE
     backward over logits [16384x49152] with 10% of the targets masked; RMSNorm backward on [16384x576]; SwiGLU
-    backward on [16384x1536]. Rates are algorithmic work (FLOP, or bytes each tensor is touched once) over time."""
+    backward on [16384x1536]. Rates are algorithmic work (FLOP, or bytes each tensor is touched once) over time.
+    Two figures per GEMM: `frac` is a single launch between other kernels (each round puts the 6.4 GB cross-entropy
+    pass and four streaming kernels between two launches of the same product: cold caches, clocks and power ramping up
+    from memory-bound work), `sustained_frac` is `sustained` launches back to back inside one pair of events, which is
+    how the products run inside a training step."""
     import ctypes as C
     rs = np.random.RandomState(7)
     R, H, F, V = 16384, 576, 1536, 49152
@@ -241,6 +261,20 @@ def micro_kernels(gpu, L, reps=10):
     for _ in range(reps):
         run()
     prof = gpu.stop_profile()
+
+    def sustained_rate(fn, flop):
+        """`sustained` launches of one product back to back inside one event pair, after a few untimed ones"""
+        for _ in range(5):
+            fn()
+        ms = C.c_double()
+        L.check(c, lib.gt_timer_start(c), "gt_timer_start")
+        for _ in range(sustained):
+            fn()
+        L.check(c, lib.gt_timer_stop(c, C.byref(ms)), "gt_timer_stop")
+        return ms.value / sustained, flop * sustained / (ms.value * 1e-3)
+    flop = 2.0 * R * H * F
+    sus = {"gemm.nn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.NN, 0, R, H, F, dY, W, dX), "dX"), flop),
+           "gemm.tn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.TN, 0, F, H, R, dY, X, dW), "dW"), flop)}
     out = {}
     names = {"gemm.nn": ("dX = dY.W  [16384x576x1536]", "mfma"), "gemm.tn": ("dW = dY^T.X [1536x576x16384]", "mfma"),
              "ce.bwd": ("softmax-CE backward [16384x49152]", "hbm"), "ce": ("CE forward statistics [16384x49152]", "hbm"),
@@ -257,51 +291,36 @@ def micro_kernels(gpu, L, reps=10):
         out[desc] = {"kernel": label, "bound": bound, "us_per_launch": round(1e3 * ms / cnt, 1),
                      "achieved": round(rate / 1e12, 3), "unit": "TFLOP/s" if bound == "mfma" else "TB/s",
                      "frac": round(rate / peak, 4)}
+        if key in sus:
+            out[desc]["launch"] = "single launches, each between a 6.4 GB cross-entropy pass and four streaming kernels (cold)"
+            out[desc]["sustained_us_per_launch"] = round(1e3 * sus[key][0], 1)
+            out[desc]["sustained_achieved"] = round(sus[key][1] / 1e12, 3)
+            out[desc]["sustained_frac"] = round(sus[key][1] / PEAK_FP32_MFMA, 4)
+            out[desc]["sustained"] = f"{sustained} launches back to back inside one event pair (the reduction pass of a split-K product included)"
     for b in (X, W, dY, dX, dW, gate, up, dgate, dup, g_n, w_n, rinv, y_n, dx_n, dw_n, z, dz, tgb, inv, loss, lse):
         L.check(c, lib.gt_free(c, b), "gt_free")
     return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
-    ap.add_argument("--streams", type=int, default=4,
-                    help="HIP streams the backend deals consecutive micro-batches to (matters for --sequential; 1 = one stream)")
-    ap.add_argument("--no-call-pattern", action="store_true",
-                    help="skip the short extra leg that runs the step the way the reference's trainer calls the backend")
-    ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (benchmark configs[1] shapes)")
-    ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
-    ap.add_argument("--no-keep-scores", action="store_true",
-                    help="attention recomputes Q.K^T in the backward instead of keeping the forward's scores (saves B*Hq*T*T*4 bytes per layer)")
-    ap.add_argument("--no-fuse", action="append", default=[], choices=["sibling_dx", "residual_add", "add_grads"],
-                    help="switch one of the host-side launch fusions off for an A/B run (repeatable)")
-    ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
-                    help="library option for an A/B run, e.g. attn.keep_ds=0 (dQ recomputes the scores) or gemm.staged=1")
-    ap.add_argument("--profile-all", action="store_true",
-                    help="time every kernel label (not only the GEMMs) over the timed region and print the table to stderr")
-    ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS),
-                    help="index into BASELINE.json configs (default 3, the headline SmolLM2 shape)")
-    a = ap.parse_args()
-    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-              "(no collectives are part of it: the path would shard over sequences with one gradient sum per step)", file=sys.stderr)
-        sys.exit(2)
+def muon_flop(model):
+    """Newton-Schulz work of one Muon step: 5 iterations of A = X X^T (2 r^2 c), A^2 (2 r^3) and (bA + cA^2) X (2 r^2 c)
+    per matrix, r = min(rows, cols), c = max(rows, cols)."""
+    mu, _ = model.param_groups()
+    tot = 0.0
+    for p in mu:
+        r, c = min(p.shape), max(p.shape)
+        tot += 5.0 * (4.0 * r * r * c + 2.0 * r * r * r)
+    return tot
 
-    import torch  # device plumbing only: make sure a GPU is there before touching the library
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    ag = importlib.import_module(f"{PKG}.autograd")
-    hb = importlib.import_module(f"{PKG}.hip_backend")
-    arch = importlib.import_module(f"{PKG}.arch")
-    optim = importlib.import_module(f"{PKG}.optim")
 
-    wl = WORKLOADS[a.config]
-    BATCH = wl["batch"]
+def run_workload(mods, config, steps, warmup, a, headline):
+    """One training workload on its own backend: `warmup` untimed steps, `steps` timed ones (wall clock around them with the
+    device idle on both sides, HIP events on the library's streams around a sample of the GEMM launches), then short legs
+    outside the timed region. Returns the pieces of the JSON line."""
+    import torch
+    ag, hb, arch, optim = mods
+    wl = WORKLOADS[config]
+    batch = wl["batch"]
     cfg = arch.ModelConfig(**wl["model"])
     model = arch.Model(cfg, synth_weights(arch, cfg))
     n_params = sum(p.size for p in model.params())
@@ -330,12 +349,12 @@ def main():
     else:
         opt = optim.AdamWHip(gpu, model.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
     ag.set_checkpointing(bool(wl.get("recompute")))
-    total = a.steps + a.warmup
-    if a.config == 3:
-        toks = [zipf_tokens(cfg.vocab, BATCH * (SEQ + 1), 100 + i).reshape(BATCH, SEQ + 1) for i in range(total)]
+    total = steps + warmup
+    if config == 3:
+        toks = [zipf_tokens(cfg.vocab, batch * (SEQ + 1), 100 + i).reshape(batch, SEQ + 1) for i in range(total)]
     else:
-        toks = [np.random.RandomState(100 + i).randint(0, cfg.vocab, (BATCH, SEQ + 1)).astype(np.int64) for i in range(total)]
-    masks = [np.random.RandomState(500 + i).rand(BATCH, SEQ) < wl["mask"] for i in range(total)] if wl.get("mask") else None
+        toks = [np.random.RandomState(100 + i).randint(0, cfg.vocab, (batch, SEQ + 1)).astype(np.int64) for i in range(total)]
+    masks = [np.random.RandomState(500 + i).rand(batch, SEQ) < wl["mask"] for i in range(total)] if wl.get("mask") else None
 
     def step(i, sequential=a.sequential):
         t = toks[i]
@@ -344,22 +363,33 @@ def main():
             tgt[~masks[i]] = -1                 # loss mask: only the kept positions carry a target
         if sequential:
             losses = []
-            for b in range(BATCH):
+            for b in range(batch):
                 loss = arch.sequence_loss(model, t[b, :-1], tgt[b], 0)
-                ag.backward(loss, 1.0 / BATCH)
+                ag.backward(loss, 1.0 / batch)
                 losses.append(loss)
         else:
             loss = arch.sequence_loss(model, t[:, :-1].reshape(-1), tgt.reshape(-1), 0, SEQ)
-            ag.backward(loss, 1.0 / BATCH)
+            ag.backward(loss, 1.0 / batch)
             losses = [loss]
         gpu.sync(losses)                     # loss scalars back to the host, as train-gpu.ts:221
         opt.record_step()
         gpu.sync([])
         return float(np.mean(np.concatenate([l.data for l in losses])))
 
+    def timed_leg(n, sequential, first=0):
+        gpu.sync([])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(n):
+            step((first + i) % total, sequential)
+        gpu.sync([])
+        torch.cuda.synchronize()
+        return time.perf_counter() - t1
+
+    res = {"wl": wl, "batch": batch, "n_params": n_params, "device": gpu.adapter_name}
     gpu.install()
     try:
-        losses = [step(i) for i in range(a.warmup)]
+        losses = [step(i) for i in range(warmup)]
         gpu.sync([])
         torch.cuda.synchronize()
         # HIP events on the library's stream around the GEMM launches of the timed region. A pair of events delays the
@@ -369,48 +399,162 @@ def main():
         gpu.set_option("prof.sample", 1 if a.profile_all else PROF_SAMPLE)
         gpu.start_profile("" if a.profile_all else "gemm.")
         t0 = time.perf_counter()
-        for i in range(a.warmup, total):
+        for i in range(warmup, total):
             losses.append(step(i))
         gpu.sync([])
         torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        prof = gpu.stop_profile()
+        res["wall"] = time.perf_counter() - t0
+        res["prof"] = gpu.stop_profile()
+        res["losses"] = losses
         gpu.set_option("prof.sample", 1)
-        opt_prof = None
-        gpu.start_profile("adamw")           # the AdamW kernels alone, outside the timed region
+        # the optimizer kernels alone, outside the timed region
+        gpu.start_profile("muon" if wl.get("muon") else "adamw")
         step(total - 1)
-        opt_prof = gpu.stop_profile().get("adamw")
+        op = gpu.stop_profile()
+        res["opt_prof"] = op.get("adamw")
+        if wl.get("muon") and op.get("muon"):
+            ms, cnt, _ = op["muon"]
+            fl = muon_flop(model)
+            res["muon"] = {"ms_per_step": round(ms / cnt, 3), "newton_schulz_TFLOP_per_step": round(fl / 1e12, 4),
+                           "achieved": round(fl / (ms / cnt * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                           "frac": round(fl / (ms / cnt * 1e-3) / PEAK_FP32_MFMA, 4),
+                           "note": "whole gt_muon_step (momentum, normalise, 5 Newton-Schulz iterations, apply) against the "
+                                   "Newton-Schulz FLOP 5*(4 r^2 c + 2 r^3) per matrix"}
         # The same step the way the reference's trainer calls a backend (src/backend/train-gpu.ts:200-219): one sequence's
         # forward and backward at a time, B graphs of 2048 rows per step, gradients accumulated, then the optimizer. A short
         # leg outside the headline's timed region; the backend deals the micro-batches to its streams.
-        call_pattern = None
-        if not a.sequential and not a.no_call_pattern:
-            nseq = max(2, min(6, a.steps))
+        res["call_pattern"] = None
+        if headline and not a.sequential and not a.no_call_pattern:
+            nseq = max(2, min(6, steps))
             for i in range(2):
                 step(i % total, True)
-            gpu.sync([])
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            for i in range(nseq):
-                step((2 + i) % total, True)
-            gpu.sync([])
-            torch.cuda.synchronize()
-            w1 = time.perf_counter() - t1
-            call_pattern = {"graph": f"{BATCH} graphs of {SEQ} rows per step, one sequence at a time, as src/backend/train-gpu.ts:200-219 calls the backend",
-                            "streams": a.streams, "steps": nseq, "value": round(nseq * BATCH * SEQ / w1, 1), "unit": "tokens/s",
-                            "ms_per_step": round(1e3 * w1 / nseq, 2)}
+            w1 = timed_leg(nseq, True, 2)
+            res["call_pattern"] = {"graph": f"{batch} graphs of {SEQ} rows per step, one sequence at a time, as src/backend/train-gpu.ts:200-219 calls the backend",
+                                   "streams": a.streams, "steps": nseq, "value": round(nseq * batch * SEQ / w1, 1), "unit": "tokens/s",
+                                   "ms_per_step": round(1e3 * w1 / nseq, 2)}
     finally:
         gpu.uninstall()
         ag.set_checkpointing(False)
         if wl.get("lora"):
             arch.clear_lora(model)
+    res["gpu"] = gpu
+    res["model"] = model
+    res["step"] = step
+    res["timed_leg"] = timed_leg
+    res["total"] = total
+    return res
+
+
+def naive_host_leg(mods, a, nsteps=3):
+    """What a literal shim over the C ABI gets: the reference's call pattern (one sequence per graph) on ONE stream with
+    every host-side hold-back and fusion of HipBackend switched off, so that each autograd op issues its own gt_* call
+    in tape order (separate k/v and gate/up products, one dX and one dW launch per linear, unfused residual adds and
+    gated activations, separate q and k rotations, add's backward as a launch). Attention still keeps its scores:
+    that is a choice inside the attention entry points, not a host fusion."""
+    import torch
+    ag, hb, arch, optim = mods
+    wl = WORKLOADS[3]
+    batch = wl["batch"]
+    cfg = arch.ModelConfig(**wl["model"])
+    model = arch.Model(cfg, synth_weights(arch, cfg))
+    gpu = hb.require_gpu("bench.py", streams=1)
+    gpu.batch_linears = gpu.fuse_sibling_dx = gpu.fuse_residual_add = gpu.alias_add_grads = False
+    gpu.group_dw = gpu.pair_ropes = gpu.fuse_glu = False
+    opt = optim.AdamWHip(gpu, model.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
+    toks = [zipf_tokens(cfg.vocab, batch * (SEQ + 1), 900 + i).reshape(batch, SEQ + 1) for i in range(nsteps + 1)]
+
+    def step(i):
+        t = toks[i]
+        losses = []
+        for b in range(batch):
+            loss = arch.sequence_loss(model, t[b, :-1], t[b, 1:], 0)
+            ag.backward(loss, 1.0 / batch)
+            losses.append(loss)
+        gpu.sync(losses)
+        opt.record_step()
+        gpu.sync([])
+    gpu.install()
+    try:
+        step(0)
+        gpu.sync([])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(nsteps):
+            step(1 + i)
+        gpu.sync([])
+        torch.cuda.synchronize()
+        w = time.perf_counter() - t0
+    finally:
+        gpu.uninstall()
+        gpu.destroy()
+    return {"graph": f"{batch} graphs of {SEQ} rows per step, one stream, one gt_* call per autograd op (no held-back, batched, grouped or fused launches)",
+            "steps": nsteps, "value": round(nsteps * batch * SEQ / w, 1), "unit": "tokens/s", "ms_per_step": round(1e3 * w / nsteps, 2)}
+
+
+def gemm_summary(prof, steps):
+    """Backward GEMM labels of a profiled region: the label with the most time, and all of them together."""
+    bwd = {k: v for k, v in prof.items() if k.startswith("gemm.nn") or k.startswith("gemm.tn")}
+    if not bwd:
+        return None, None, None
+    dom = max(bwd, key=lambda k: bwd[k][0])
+    all_ms = sum(v[0] for v in bwd.values())
+    all_work = sum(v[2] for v in bwd.values())
+    per = {k: {"TFLOP/s": round(v[2] / (v[0] * 1e-3) / 1e12, 2), "ms_per_step": round(v[0] / steps, 2),
+               "launches_per_step": v[1] // steps} for k, v in sorted(prof.items()) if v[0] > 0}
+    allb = {"achieved": round(all_work / (all_ms * 1e-3) / 1e12, 3), "ms_per_step": round(all_ms / steps, 2),
+            "frac": round(all_work / (all_ms * 1e-3) / PEAK_FP32_MFMA, 4)}
+    return dom, allb, per
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sequential", action="store_true", help="one sequence per graph, as the reference accumulates")
+    ap.add_argument("--streams", type=int, default=4,
+                    help="HIP streams the backend deals consecutive micro-batches to (matters for --sequential; 1 = one stream)")
+    ap.add_argument("--no-call-pattern", action="store_true",
+                    help="skip the short extra leg that runs the step the way the reference's trainer calls the backend")
+    ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (benchmark configs[1] shapes)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short legs over benchmark configs[2] (gemma3-style, Muon) and configs[4] (Qwen3-0.6B, LoRA)")
+    ap.add_argument("--naive-host", action="store_true",
+                    help="add a leg that runs the reference's call pattern on one stream with every host-side hold-back and fusion off")
+    ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
+    ap.add_argument("--no-keep-scores", action="store_true",
+                    help="attention recomputes Q.K^T in the backward instead of keeping the forward's scores (saves B*Hq*T*T*4 bytes per layer)")
+    ap.add_argument("--no-fuse", action="append", default=[], choices=["sibling_dx", "residual_add", "add_grads"],
+                    help="switch one of the host-side launch fusions off for an A/B run (repeatable)")
+    ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
+                    help="library option for an A/B run, e.g. attn.keep_ds=0 (dQ recomputes the scores) or gemm.staged=1")
+    ap.add_argument("--profile-all", action="store_true",
+                    help="time every kernel label (not only the GEMMs) over the timed region and print the table to stderr")
+    ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS),
+                    help="index into BASELINE.json configs (default 3, the headline SmolLM2 shape)")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+              "(no collectives are part of it: the path would shard over sequences with one gradient sum per step)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch  # device plumbing only: make sure a GPU is there before touching the library
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    mods = tuple(importlib.import_module(f"{PKG}.{m}") for m in ("autograd", "hip_backend", "arch", "optim"))
     Lmod = importlib.import_module(f"{PKG}.lib")
+
+    r = run_workload(mods, a.config, a.steps, a.warmup, a, headline=True)
+    wl, BATCH, prof, gpu, losses, wall = r["wl"], r["batch"], r["prof"], r["gpu"], r["losses"], r["wall"]
     kernels = None if a.no_micro else micro_kernels(gpu, Lmod)
-    if kernels is not None and opt_prof and a.config == 3:
-        ms, cnt, work = opt_prof
-        kernels[f"AdamW step, {n_params} params, clip on"] = {
+    if kernels is not None and r["opt_prof"] and a.config == 3:
+        ms, cnt, work = r["opt_prof"]
+        kernels[f"AdamW step, {r['n_params']} params, clip on"] = {
             "kernel": "adamw", "bound": "hbm", "us_per_launch": round(1e3 * ms / cnt, 1),
             "achieved": round(work / (ms * 1e-3) / 1e12, 3), "unit": "TB/s", "frac": round(work / (ms * 1e-3) / PEAK_HBM, 4)}
+    gpu.destroy()
 
     if a.profile_all:
         print(f"{'label':30s} {'ms/step':>9s} {'launches/step':>14s} {'T(FLOP|B)/s':>12s}", file=sys.stderr)
@@ -418,14 +562,11 @@ def main():
             print(f"{k:30s} {v[0] / a.steps:9.2f} {v[1] / a.steps:14.1f} {v[2] / (v[0] * 1e-3) / 1e12 if v[0] else 0:12.2f}", file=sys.stderr)
     tokens = a.steps * BATCH * SEQ
     # dominant kernel: the backward GEMMs (NN = dX, TN = dW); the one tile shape with the most time stands for it
-    bwd = {k: v for k, v in prof.items() if k.startswith("gemm.nn") or k.startswith("gemm.tn")}
-    dom = max(bwd, key=lambda k: bwd[k][0]) if bwd else None
+    dom, allb, per = gemm_summary(prof, a.steps)
     roof = None
     if dom:
-        ms, cnt, work = bwd[dom]
+        ms, cnt, work = prof[dom]
         ach = work / (ms * 1e-3)
-        all_ms = sum(v[0] for v in bwd.values())
-        all_work = sum(v[2] for v in bwd.values())
         roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach / 1e12, 3), "peak": PEAK_FP32_MFMA / 1e12,
                 "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA, 4),
                 "traffic": MEASURED_TRAFFIC.get(dom) if a.config == 3 else None,
@@ -433,10 +574,30 @@ def main():
                                   "this file, made separately; not measured by this run" if a.config == 3 and MEASURED_TRAFFIC.get(dom) else None,
                 "launches": int(cnt), "avg_launch_ms": round(ms / cnt, 4),
                 "timed_launches": "all" if a.profile_all else f"1 in {PROF_SAMPLE} of each label",
-                "all_bwd_gemms": {"achieved": round(all_work / (all_ms * 1e-3) / 1e12, 3), "ms_per_step": round(all_ms / a.steps, 2),
-                                  "frac": round(all_work / (all_ms * 1e-3) / PEAK_FP32_MFMA, 4)},
-                "per_kernel": {k: {"TFLOP/s": round(v[2] / (v[0] * 1e-3) / 1e12, 2), "ms_per_step": round(v[0] / a.steps, 2),
-                                   "launches_per_step": v[1] // a.steps} for k, v in sorted(prof.items())}}
+                "all_bwd_gemms": allb, "per_kernel": per}
+
+    # The other model-sized benchmark configs, three timed steps each on a backend of their own, outside the headline's
+    # timed region: tokens/s, the backward GEMM label with the most time, and for configs[2] the Muon step.
+    other = None
+    if a.config == 3 and not a.no_other_configs:
+        other = {}
+        for ci in (2, 4):
+            o = run_workload(mods, ci, 3, 2, a, headline=False)
+            o["gpu"].destroy()
+            d2, all2, per2 = gemm_summary(o["prof"], 3)
+            ent = {"workload": o["wl"]["name"], "steps": 3, "warmup": 2, "value": round(3 * o["batch"] * SEQ / o["wall"], 1), "unit": "tokens/s",
+                   "ms_per_step": round(1e3 * o["wall"] / 3, 2), "loss_first": round(o["losses"][0], 4), "loss_last": round(o["losses"][-1], 4)}
+            if d2:
+                ms2, cnt2, work2 = o["prof"][d2]
+                ent["dominant_bwd_gemm"] = {"kernel": d2, "achieved": round(work2 / (ms2 * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                                            "frac": round(work2 / (ms2 * 1e-3) / PEAK_FP32_MFMA, 4), "ms_per_step": round(ms2 / 3, 2),
+                                            "launches_per_step": int(cnt2) // 3}
+                ent["all_bwd_gemms"] = all2
+                ent["per_kernel"] = per2
+            if o.get("muon"):
+                ent["muon_step"] = o["muon"]
+            other[f"configs[{ci}]"] = ent
+    naive = naive_host_leg(mods, a) if a.naive_host or (a.config == 3 and not a.no_call_pattern and not a.sequential) else None
     out = {
         "metric": "train tokens/s (SmolLM2-135M shape, 2048x8); bwd GEMM % FP32 MFMA peak" if a.config == 3 else
                   "train tokens/s (" + wl["name"].split(":")[0] + ")",
@@ -444,16 +605,18 @@ def main():
         "ms_per_step": round(1e3 * wall / a.steps, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic (weights N(0,0.02) random init, tokens Zipf(1.1) over the vocab)",
         "config": {"workload": wl["name"],
-                   "params": n_params, "global_batch": BATCH, "seq_len": SEQ,
+                   "params": r["n_params"], "global_batch": BATCH, "seq_len": SEQ,
                    "graph": f"sequential micro-batches on {a.streams} stream(s)" if a.sequential else f"{BATCH} sequences stacked into one {BATCH * SEQ}-row graph",
-                   "device": gpu.adapter_name},
+                   "device": r["device"]},
         "loss_first": round(losses[0], 4), "loss_last": round(losses[-1], 4),
-        "reference_call_pattern": call_pattern,
+        "reference_call_pattern": r["call_pattern"],
+        "naive_host": naive,
         "roofline": roof,
+        "muon_step": r.get("muon"),
         "kernels": kernels,
+        "other_configs": other,
         "cpu_baseline": None if a.no_cpu else cpu_baseline(),
     }
-    gpu.destroy()
     print(json.dumps(out))
 
 

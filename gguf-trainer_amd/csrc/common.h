@@ -46,6 +46,7 @@ struct gt_ctx {
   int *bad_host = nullptr, *bad_dev = nullptr;
   float *rms_static = nullptr;                  // this device's address of norm.hip's static scratch array
   bool rms_static_pending = false;              // a gt_rmsnorm_bwd_static call is queued on this stream and the stream has not been waited for since
+  hipEvent_t timer_a = nullptr, timer_b = nullptr;   // gt_timer_start / gt_timer_stop
   hipEvent_t mark = nullptr;                    // gt_stream_mark records it, another context's gt_stream_wait waits for it
   struct ProfSeen { int64_t n = 0; double work = 0; };
   std::map<std::string, ProfSeen> prof_seen;    // launches and their work per label since gt_prof_begin, timed or not

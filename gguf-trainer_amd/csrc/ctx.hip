@@ -9,6 +9,8 @@ static void ctx_release(gt_ctx *c) {
   if (c->ws) hipFree(c->ws);
   if (c->bad_host) hipHostFree(c->bad_host);
   if (c->mark) hipEventDestroy(c->mark);
+  if (c->timer_a) hipEventDestroy(c->timer_a);
+  if (c->timer_b) hipEventDestroy(c->timer_b);
   if (c->stream) hipStreamDestroy(c->stream);
   delete c;
 }
@@ -152,6 +154,28 @@ int gt_stream_wait(gt_ctx *ctx, gt_ctx *other) {
   GT_REQUIRE(ctx, other && other->device == ctx->device, "gt_stream_wait: the other context is null or on another device");
   if (other == ctx) return 0;
   GT_HIP(ctx, hipStreamWaitEvent(ctx->stream, other->mark, 0));
+  return 0;
+}
+
+// One pair of events around whatever the caller queues between the two calls: the time of a run of launches as the
+// device sees it, without a pair per launch.
+int gt_timer_start(gt_ctx *ctx) {
+  GT_ENTER(ctx);
+  if (!ctx->timer_a) {
+    GT_HIP(ctx, hipEventCreate(&ctx->timer_a));
+    GT_HIP(ctx, hipEventCreate(&ctx->timer_b));
+  }
+  GT_HIP(ctx, hipEventRecord(ctx->timer_a, ctx->stream));
+  return 0;
+}
+int gt_timer_stop(gt_ctx *ctx, double *ms) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, ms && ctx->timer_a, "gt_timer_stop: no result pointer, or gt_timer_start was not called");
+  GT_HIP(ctx, hipEventRecord(ctx->timer_b, ctx->stream));
+  GT_HIP(ctx, hipEventSynchronize(ctx->timer_b));
+  float t = 0;
+  GT_HIP(ctx, hipEventElapsedTime(&t, ctx->timer_a, ctx->timer_b));
+  *ms = t;
   return 0;
 }
 

@@ -613,18 +613,19 @@ static int launch_direct_kind(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   GT_LAUNCHED(ctx);
   return 0;
 }
-// slot: index of the tile shape (0..4); the bit of (shape, kind, one or two segments) in gemm_direct_set follows from it
+// slot: index of the tile shape (0..5); the bit of (shape, kind, one or two segments) in gemm_direct_set follows from it
 template <int BM, int BN, int WM, int WN, int BK, int NSTG>
 static int launch_direct(gt_ctx *ctx, int kind, GemmArgs &a, int zdim, int slot) {
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
+  const int b1 = slot < 5 ? 3 * slot : 45 + 3 * (slot - 5), b2 = slot < 5 ? 15 + 2 * slot : 54 + 2 * (slot - 5);
   if (a.K2 > 0) {                // two K segments: NT / NN only
-    if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG, true>(ctx, a, zdim, 15 + 2 * slot);
-    return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG, true>(ctx, a, zdim, 15 + 2 * slot + 1);
+    if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG, true>(ctx, a, zdim, b2);
+    return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG, true>(ctx, a, zdim, b2 + 1);
   }
-  if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG, false>(ctx, a, zdim, 3 * slot);
-  if (kind == GT_NN) return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG, false>(ctx, a, zdim, 3 * slot + 1);
-  return launch_direct_kind<BM, BN, WM, WN, GT_TN, BK, NSTG, false>(ctx, a, zdim, 3 * slot + 2);
+  if (kind == GT_NT) return launch_direct_kind<BM, BN, WM, WN, GT_NT, BK, NSTG, false>(ctx, a, zdim, b1);
+  if (kind == GT_NN) return launch_direct_kind<BM, BN, WM, WN, GT_NN, BK, NSTG, false>(ctx, a, zdim, b1 + 1);
+  return launch_direct_kind<BM, BN, WM, WN, GT_TN, BK, NSTG, false>(ctx, a, zdim, b1 + 2);
 }
 
 // C (+)= sum over splits, in split order
@@ -667,7 +668,7 @@ static int reduce_splits(gt_ctx *ctx, const GemmArgs &a, int M, int N, int split
 
 struct TileCfg { int bm, bn, bk; };
 static const TileCfg kTiles[] = {{64, 64, 16}, {128, 64, 16}, {128, 128, 16}, {128, 192, 16}, {128, 96, 16}, {256, 128, 16},
-                                 {128, 128, 32}, {128, 192, 32}, {128, 96, 32}, {256, 128, 32}, {64, 192, 16}, {128, 64, 32}, {64, 192, 32}};
+                                 {128, 128, 32}, {128, 192, 32}, {128, 96, 32}, {256, 128, 32}, {64, 192, 16}, {128, 64, 32}, {64, 192, 32}, {128, 160, 32}};
 #define NCFG ((int)(sizeof(kTiles) / sizeof(kTiles[0])))
 
 // Tile and split-K choice by a small cost model over the tile shapes that measured best on MI355X:
@@ -679,10 +680,10 @@ static void pick_tile(gt_ctx *ctx, int kind, bool direct_ok, int np, const int *
   // relative tile efficiencies as measured (asymptotic rate of each tile over the best one's)
   static const Cand cand_nn[] = {{7, 1.00}, {6, 0.98}, {8, 0.98}, {10, 0.95}, {11, 0.82}, {0, 0.78}};
   static const Cand cand_tn[] = {{8, 1.00}, {11, 0.99}, {10, 0.92}, {6, 0.90}, {7, 0.78}, {0, 0.72}};
-  static const Cand cand_nn_direct[] = {{7, 1.00}, {8, 1.00}, {6, 0.98}, {12, 0.97}, {11, 0.92}, {10, 0.85}, {0, 0.72}};
-  static const Cand cand_tn_direct[] = {{8, 1.00}, {12, 1.00}, {7, 0.98}, {11, 0.96}, {6, 0.88}, {10, 0.85}, {0, 0.68}};
+  static const Cand cand_nn_direct[] = {{7, 1.00}, {8, 1.00}, {13, 1.00}, {6, 0.98}, {12, 0.97}, {11, 0.92}, {10, 0.85}, {0, 0.72}};
+  static const Cand cand_tn_direct[] = {{8, 1.00}, {12, 1.00}, {13, 0.99}, {7, 0.98}, {11, 0.96}, {6, 0.88}, {10, 0.85}, {0, 0.68}};
   const Cand *cand = direct_ok ? (kind == GT_TN ? cand_tn_direct : cand_nn_direct) : (kind == GT_TN ? cand_tn : cand_nn);
-  const int ncand = direct_ok ? 7 : 6;
+  const int ncand = direct_ok ? 8 : 6;
   int cfg = 0, splits = 1;
   double elems = 0;
   for (int i = 0; i < np; i++) elems += (double)Ms[i] * Ns[i];
@@ -692,7 +693,7 @@ static void pick_tile(gt_ctx *ctx, int kind, bool direct_ok, int np, const int *
   for (int ci = 0; ci < ncand; ci++) {
     const Cand &c = cand[ci];
     const TileCfg &tc = kTiles[c.cfg];
-    if (np > 1 && !(c.cfg == 6 || c.cfg == 7 || c.cfg == 8 || c.cfg == 11 || c.cfg == 12)) continue;   // group launches: direct tiles only
+    if (np > 1 && !(c.cfg == 6 || c.cfg == 7 || c.cfg == 8 || c.cfg == 11 || c.cfg == 12 || c.cfg == 13)) continue;   // group launches: direct tiles only
     int64_t tiles = 0;
     for (int i = 0; i < np; i++) tiles += cdiv(Ms[i], tc.bm) * cdiv(Ns[i], tc.bn);
     const double util = elems / ((double)tiles * tc.bm * tc.bn);
@@ -777,6 +778,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
       case 8: return launch_direct<128, 96, 4, 1, 32, 2>(ctx, kind, a, zdim, 2) || reduce_splits(ctx, a, M, N, splits, acc);
       case 11: return launch_direct<128, 64, 2, 2, 32, 2>(ctx, kind, a, zdim, 3) || reduce_splits(ctx, a, M, N, splits, acc);
       case 12: return launch_direct<64, 192, 2, 2, 32, 2>(ctx, kind, a, zdim, 4) || reduce_splits(ctx, a, M, N, splits, acc);
+      case 13: return launch_direct<128, 160, 4, 1, 32, 2>(ctx, kind, a, zdim, 5) || reduce_splits(ctx, a, M, N, splits, acc);
       default: break;
     }
   }
@@ -793,6 +795,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
     case 9: rc = launch_cfg<256, 128, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
     case 10: rc = launch_cfg<64, 192, 2, 2, 16>(ctx, kind, vec, a, zdim); break;
     case 11: rc = launch_cfg<128, 64, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
+    case 13: rc = launch_cfg<128, 160, 4, 1, 32>(ctx, kind, vec, a, zdim); break;
     default: rc = launch_cfg<64, 192, 2, 2, 32>(ctx, kind, vec, a, zdim); break;
   }
   if (rc) return rc;
@@ -894,8 +897,8 @@ int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, 
                  "gt_gemm_group: the outputs of products %d and %d overlap", j, i);
   }
   const int pin = ctx->opt_gemm_tile;
-  GT_REQUIRE(ctx, !(eligible && pin >= 0 && pin != 6 && pin != 7 && pin != 8 && pin != 11 && pin != 12),
-             "gt_gemm_group: \"gemm.tile\" pins tile %d, which the grouped launch does not have (6, 7, 8, 11 or 12; -1 = choose)", pin);
+  GT_REQUIRE(ctx, !(eligible && pin >= 0 && pin != 6 && pin != 7 && pin != 8 && pin != 11 && pin != 12 && pin != 13),
+             "gt_gemm_group: \"gemm.tile\" pins tile %d, which the grouped launch does not have (6, 7, 8, 11, 12 or 13; -1 = choose)", pin);
   if (count > GT_GROUP_MAX) {
     for (int i = 0; i < count; i += GT_GROUP_MAX)
       if (gt_gemm_group(ctx, kind, std::min(GT_GROUP_MAX, count - i), M + i, N + i, K, A + i, B + i, C + i, acc + i)) return 1;
@@ -926,8 +929,7 @@ int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, 
   if (ctx->opt_gemm_splitk >= 1) kc = cdiv(cdiv(K, ctx->opt_gemm_splitk), 32) * 32;
   int splits = (int)cdiv(K, kc), cfg = 0, unused = 0;
   pick_tile(ctx, GT_TN, true, ng, gm, gn, K, 1, false, &cfg, &unused, splits);
-  if (ctx->opt_gemm_tile == 6 || ctx->opt_gemm_tile == 7 || ctx->opt_gemm_tile == 8 || ctx->opt_gemm_tile == 11 || ctx->opt_gemm_tile == 12)
-    cfg = ctx->opt_gemm_tile;
+  if (pin == 6 || pin == 7 || pin == 8 || pin == 11 || pin == 12 || pin == 13) cfg = pin;
   if (splits > 1) {
     a.kchunk = (int)kc;
     void *ws;
@@ -943,6 +945,7 @@ int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, 
     case 7: rc = launch_group<128, 192, 2, 2>(ctx, a, g, 41); break;
     case 8: rc = launch_group<128, 96, 4, 1>(ctx, a, g, 42); break;
     case 11: rc = launch_group<128, 64, 2, 2>(ctx, a, g, 43); break;
+    case 13: rc = launch_group<128, 160, 4, 1>(ctx, a, g, 58); break;
     default: rc = launch_group<64, 192, 2, 2>(ctx, a, g, 44); break;
   }
   if (rc) return rc;
@@ -967,8 +970,23 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
   fused = fused && N <= GT_DIRECT_LD_MAX;
   // the chained loop has one tile shape and no K split: below one workgroup per CU the single products, which pick
   // smaller tiles and split K, fill the chip better
-  const bool t96 = N % 96 == 0;
-  if (fused && cdiv(M, 128) * cdiv(N, t96 ? 96 : 128) < (ctx->opt_gemm_sum_min_tiles >= 0 ? ctx->opt_gemm_sum_min_tiles : ctx->num_cu)) fused = false;
+  // Tile of the chained loop: 128 x 96, 128 x 160 or 128 x 128, whichever leaves the least idle in edge tiles and in the
+  // last round of workgroups (two are resident per CU). 576 = 6 x 96; 640 = 4 x 160: a 16384-row output is 512 tiles, one
+  // full round, where 128 x 128 makes 640 tiles for 512 slots and a quarter-full second round.
+  int bn_sum = 128;
+  {
+    double best = 0;
+    const int cands[3] = {128, 160, 96};
+    for (int ci = 0; ci < 3; ci++) {
+      const int bn = cands[ci];
+      if (bn != 128 && N % bn != 0) continue;
+      const double tiles = (double)cdiv(M, 128) * cdiv(N, bn), rounds = tiles / (2.0 * ctx->num_cu);
+      const double score = ((double)M * N) / (tiles * 128.0 * bn) * (rounds / ceil(rounds));
+      if (score > best * 1.02) { best = score; bn_sum = bn; }
+    }
+  }
+  const bool t96 = bn_sum == 96, t160 = bn_sum == 160;
+  if (fused && cdiv(M, 128) * cdiv(N, bn_sum) < (ctx->opt_gemm_sum_min_tiles >= 0 ? ctx->opt_gemm_sum_min_tiles : ctx->num_cu)) fused = false;
   if (!fused) {        // one launch per product, each adding to the one before
     for (int i = 0; i < count; i++)
       if (gemm_impl(ctx, kind, i ? 1 : acc, M, N, K[i], A[i], 0, B[i], 0, C, 0, 1)) return 1;
@@ -990,10 +1008,13 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
     ksum += K[i];
   }
   char label[32];
-  snprintf(label, sizeof label, "gemm.%s.128x%dx32", kind == GT_NT ? "nt" : "nn", t96 ? 96 : 128);
+  snprintf(label, sizeof label, "gemm.%s.128x%dx32", kind == GT_NT ? "nt" : "nn", bn_sum);
   ProfScope ps(ctx, label, 2.0 * M * N * ksum);
-  if (kind == GT_NN) return t96 ? launch_multi<128, 96, 4, 1, GT_NN>(ctx, a, 30) : launch_multi<128, 128, 2, 2, GT_NN>(ctx, a, 31);
-  return t96 ? launch_multi<128, 96, 4, 1, GT_NT>(ctx, a, 32) : launch_multi<128, 128, 2, 2, GT_NT>(ctx, a, 33);
+  if (kind == GT_NN)
+    return t96 ? launch_multi<128, 96, 4, 1, GT_NN>(ctx, a, 30) : t160 ? launch_multi<128, 160, 4, 1, GT_NN>(ctx, a, 34)
+                                                                       : launch_multi<128, 128, 2, 2, GT_NN>(ctx, a, 31);
+  return t96 ? launch_multi<128, 96, 4, 1, GT_NT>(ctx, a, 32) : t160 ? launch_multi<128, 160, 4, 1, GT_NT>(ctx, a, 35)
+                                                                     : launch_multi<128, 128, 2, 2, GT_NT>(ctx, a, 33);
 }
 int gt_gemm(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, gt_buf B, gt_buf C) {
   return gemm_impl(ctx, kind, acc, M, N, K, A, 0, B, 0, C, 0, 1);

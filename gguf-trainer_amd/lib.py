@@ -95,6 +95,8 @@ _SIG = {
     "gt_newton_schulz": [ctxp, i32, i32, i32, buf, buf],
     "gt_prof_begin": [ctxp, C.c_char_p],
     "gt_prof_end": [ctxp, C.POINTER(ProfRec), i32, C.POINTER(i32)],
+    "gt_timer_start": [ctxp],
+    "gt_timer_stop": [ctxp, C.POINTER(f64)],
 }
 
 for _name, _args in _SIG.items():

@@ -71,7 +71,7 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
 /* Kernel-selection switches for tests and tuning (no reference counterpart; WebGPUBackend exposes
  * attnFlashMinT as a public field for the same purpose, webgpu.ts:305):
  *   "attn.generic" 1 = always take the shape-generic attention kernels, 0 = MFMA kernels where they apply
- *   "gemm.tile"    -1 = heuristic, 0..12 = pin the GEMM tile configuration (tests and tuning)
+ *   "gemm.tile"    -1 = heuristic, 0..13 = pin the GEMM tile configuration (tests and tuning)
  *   "gemm.splitk"  -1 = heuristic, n >= 1 = pin the split-K factor
  *   "gemm.group"   1 (default) = gt_gemm_group runs its TN products as one launch; 0 = one launch per product
  *   "gemm.staged"  1 = always stage GEMM operands through registers (0: aligned shapes load straight into LDS)
@@ -286,6 +286,11 @@ int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out)
 typedef struct gt_prof_rec { char label[32]; double ms; int64_t count; double work; } gt_prof_rec;
 int gt_prof_begin(gt_ctx *ctx, const char *prefix);
 int gt_prof_end(gt_ctx *ctx, gt_prof_rec *out, int cap, int *n);
+/* One event pair around everything queued between the two calls (the same startProfile / stopProfile surface, for a
+ * run of back-to-back launches as the device sees it, without a pair per launch). gt_timer_stop waits for the stream
+ * and gives the elapsed milliseconds. */
+int gt_timer_start(gt_ctx *ctx);
+int gt_timer_stop(gt_ctx *ctx, double *ms);
 
 #ifdef __cplusplus
 }

@@ -49,7 +49,7 @@ def test_gemm_every_tile_shape_and_kind(gpu, M, N, K):
         for kind, (A, B) in enumerate([(a, b), (a, np.ascontiguousarray(b.T)), (np.ascontiguousarray(a.T), np.ascontiguousarray(b.T))]):
             gpu.write_state_buffer(da, A)
             gpu.write_state_buffer(db, B)
-            for tile in range(13):
+            for tile in range(14):
                 for splitk in ((1, 3) if kind == 2 else (1,)):
                     for acc in (0, 1):
                         # staged = 1 pins the register-staged kernels; 0 lets the aligned shapes (K a multiple of 32, whole
@@ -100,7 +100,7 @@ def test_gemm_group_equals_the_products_one_by_one(gpu, K, shapes, splitk):
     aa, bb, cc, ac = (C.c_uint64 * n)(*da), (C.c_uint64 * n)(*db), (C.c_uint64 * n)(*dc), (C.c_int * n)(*accs)
     gpu.set_option("gemm.splitk", splitk)
     try:
-        for tile in ((-1, 6, 7, 8, 11, 12) if K == 256 or K == 96 else (-1,)):
+        for tile in ((-1, 6, 7, 8, 11, 12, 13) if K == 256 or K == 96 else (-1,)):
             gpu.set_option("gemm.tile", tile)
             for b_, c_ in zip(dc, C0):
                 gpu.write_state_buffer(b_, c_)
@@ -198,7 +198,7 @@ def test_gemm_pair(gpu, M, N, K1, K2):
         for kind, ops in enumerate([(a1, b1, a2, b2), (a1, T(b1), a2, T(b2)), (T(a1), T(b1), T(a2), T(b2))]):
             for buf, arr in zip(bufs, ops):
                 gpu.write_state_buffer(buf, arr)
-            for tile in (-1, 0, 6, 7, 8, 10, 11, 12):
+            for tile in (-1, 0, 6, 7, 8, 10, 11, 12, 13):
                 for acc in (0, 1):
                     gpu.set_option("gemm.tile", tile)
                     gpu.write_state_buffer(bufs[4], c0)
@@ -353,7 +353,7 @@ def test_gemm_add_is_the_product_plus_the_addend(gpu, ref, kind, M, N, K, in_pla
 @pytest.mark.parametrize("kind,M,N,Ks", [(1, 300, 576, (576, 192, 192)), (1, 257, 576, (1536, 1536)), (1, 128, 640, (640, 128, 128)),
                                          (0, 200, 192, (64, 96)), (0, 130, 96, (32, 32, 32)), (1, 64, 576, (576,)),
                                          (1, 100, 576, (576, 190)), (1, 100, 574, (64, 64)), (2, 96, 64, (128, 160)),
-                                         (1, 5600, 576, (576, 192, 192))])
+                                         (1, 5600, 576, (576, 192, 192)), (0, 260, 640, (64, 96)), (1, 300, 320, (2048, 2048))])
 @pytest.mark.parametrize("acc", [0, 1])
 def test_gemm_sum_equals_the_products_one_by_one(gpu, ref, kind, M, N, Ks, acc):
     """gt_gemm_sum: up to three products summed in one launch (the K segments chained in one loop for aligned NT / NN
