@@ -74,6 +74,9 @@ int gt_report_bad_id(gt_ctx *ctx);
 void optim_release_all(gt_ctx *ctx);            // optim.hip
 int rmsnorm_static_init(gt_ctx *ctx);           // norm.hip: looks up the static scratch array's address on ctx's device
 void rmsnorm_static_forget(gt_ctx *ctx);        // norm.hip: ctx is going away and must not be remembered as the array's last user
+// gemm.hip: C_i = dscale * D_i + pscale * A_i.B_i, a batch of `count` products of one kind (strides in elements)
+int gemm_scaled_batched(gt_ctx *ctx, int kind, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB, gt_buf D, int64_t sD,
+                        float dscale, float pscale, gt_buf C, int64_t sC, int count);
 // gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
 int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc);
 

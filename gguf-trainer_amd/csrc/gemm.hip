@@ -55,9 +55,13 @@ struct GemmArgs {
   // K step, same M, N and operand orientation: the dX of sibling projections of one input as one product
   const float *xA[2], *xB[2];
   int xK[2], xlda[2], xldb[2], nx;
-  // C = D + A.B: the matrix the product is added to when it is not C's own old contents (layout of C; null: none).
-  // Single products only (no batch); with K splits the reduce kernel adds it.
+  // C = D + A.B: the matrix the product is added to when it is not C's own old contents (layout of C, batch stride sD;
+  // null: none). With K splits the reduce kernel adds it. scaled: C = dscale * D + pscale * A.B (the Newton-Schulz
+  // combines b A + c A.A and a X + B.X in the products' own write-back).
   const float *D;
+  int64_t sD;
+  int scaled;
+  float dscale, pscale;
 };
 
 // Which output tile (pm, pn) and which K split or batch member (z) a workgroup works on. Workgroups are handed
@@ -268,7 +272,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
   bool add;
   if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
   else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0 || a.D != nullptr; }
-  const float *Cold = (a.D && a.splits == 1) ? a.D : C;
+  const float *Cold = (a.D && a.splits == 1) ? a.D + z * a.sD : C;
+  const bool scaled = a.scaled && a.splits == 1;
   // When accumulating, the sixteen old values of a 32x32 tile are loaded together (from clamped, always valid
   // addresses) before the first store: a load placed after a store to the same array waits for it, and one round trip
   // per element is what an interleaved read-add-write loop would pay.
@@ -288,7 +293,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int row = rbase + 8 * (r / 4) + (r % 4);
-        if (row < a.M) C[(size_t)row * ldc + col] = add ? old[r] + acc[i][j][r] : acc[i][j][r];
+        if (row < a.M) C[(size_t)row * ldc + col] = !add ? acc[i][j][r] : scaled ? a.dscale * old[r] + a.pscale * acc[i][j][r] : old[r] + acc[i][j][r];
       }
     }
 }
@@ -498,7 +503,8 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
   if (BAND) { C = a.C + (z / a.zdiv) * a.sC + (z % a.zdiv) * a.sC2; ldc = a.ldc; add = a.acc != 0; }
   else if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
   else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0 || a.D != nullptr; }
-  const float *Cold = (!BAND && a.D && a.splits == 1) ? a.D : C;
+  const float *Cold = (!BAND && a.D && a.splits == 1) ? a.D + z * a.sD : C;
+  const bool scaled = !BAND && a.scaled && a.splits == 1;
   // The MFMAs above take the B tile as their first operand, so an accumulator holds a C^T tile: lane l32 is the row
   // of C, and registers 4q..4q+3 are four consecutive columns 8q + 4g + (0..3): one 16-byte store (and, when
   // accumulating, one 16-byte load issued before any store) instead of four scalar ones.
@@ -523,7 +529,7 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
           const int col = cbase + 8 * q;
           if (col >= a.N) continue;                       // N is a multiple of 4 here: a chunk is all in or all out
           v4f o = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          if (add) o += old[q];
+          if (add) o = scaled ? a.dscale * old[q] + a.pscale * o : o + old[q];
           *reinterpret_cast<v4f *>(cr + col) = o;
         }
       } else {
@@ -538,7 +544,7 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int col = cbase + 8 * (r / 4) + (r % 4);
-          if (col < a.N) cr[col] = add ? old[r] + acc[i][j][r] : acc[i][j][r];
+          if (col < a.N) cr[col] = !add ? acc[i][j][r] : scaled ? a.dscale * old[r] + a.pscale * acc[i][j][r] : old[r] + acc[i][j][r];
         }
       }
     }
@@ -630,12 +636,13 @@ static int launch_direct(gt_ctx *ctx, int kind, GemmArgs &a, int zdim, int slot)
 
 // C (+)= sum over splits, in split order
 __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ Pp, float *__restrict__ C, int64_t n,
-                                                     int splits, int acc, const float *__restrict__ D) {
+                                                     int splits, int acc, const float *__restrict__ D, int scaled, float dscale,
+                                                     float pscale) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = Pp[i];
   for (int z = 1; z < splits; z++) s += Pp[(size_t)z * n + i];
-  C[i] = D ? D[i] + s : acc ? C[i] + s : s;
+  C[i] = D ? (scaled ? dscale * D[i] + pscale * s : D[i] + s) : acc ? C[i] + s : s;
 }
 
 template <int BM, int BN, int WM, int WN, int BKT>
@@ -660,7 +667,7 @@ static int launch_cfg(gt_ctx *ctx, int kind, bool vec, GemmArgs &a, int zdim) {
 static int reduce_splits(gt_ctx *ctx, const GemmArgs &a, int M, int N, int splits, int acc) {
   if (splits > 1) {
     int64_t n = (int64_t)M * N;
-    hipLaunchKernelGGL(splitk_reduce, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, a.Pp, a.C, n, splits, acc, a.D);
+    hipLaunchKernelGGL(splitk_reduce, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, a.Pp, a.C, n, splits, acc, a.D, a.scaled, a.dscale, a.pscale);
     GT_LAUNCHED(ctx);
   }
   return 0;
@@ -720,7 +727,8 @@ static void pick_tile(gt_ctx *ctx, int kind, bool direct_ok, int np, const int *
 }
 
 static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB,
-                     gt_buf C, int64_t sC, int count, int K2 = 0, gt_buf A2 = 0, gt_buf B2 = 0, gt_buf D = 0) {
+                     gt_buf C, int64_t sC, int count, int K2 = 0, gt_buf A2 = 0, gt_buf B2 = 0, gt_buf D = 0, int64_t sD = 0,
+                     int scaled = 0, float dscale = 1.f, float pscale = 1.f) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, kind >= 0 && kind <= 2, "gt_gemm: kind %d is not NT(0)/NN(1)/TN(2)", kind);
   GT_REQUIRE(ctx, M >= 1 && N >= 1 && K >= 1 && count >= 1, "gt_gemm: M,N,K,count must be >= 1 (got %d,%d,%d,%d)", M, N, K, count);
@@ -734,7 +742,9 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   a.acc = acc; a.kchunk = K; a.splits = 1; a.Pp = nullptr;
   a.sA = sA; a.sB = sB; a.sC = sC;
   a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0; a.nx = 0; a.D = P<const float>(D);
-  GT_REQUIRE(ctx, !D || (count == 1 && K2 == 0), "gt_gemm_add: one single product only");
+  a.sD = sD; a.scaled = scaled; a.dscale = dscale; a.pscale = pscale;
+  GT_REQUIRE(ctx, !D || K2 == 0, "gt_gemm_add: single-segment products only");
+  GT_REQUIRE(ctx, !scaled || D, "scaled write-back needs the matrix it combines the product with");
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
              (sA % 4 == 0) && (sB % 4 == 0);
   a.K2 = K2; a.A2 = P<const float>(A2); a.B2 = P<const float>(B2);
@@ -834,7 +844,7 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.acc = acc; a.kchunk = T; a.splits = 1; a.Pp = nullptr;
   a.sA = (int64_t)T * T; a.sB = (int64_t)T * Hkv * hd; a.sC = (int64_t)T * Hq * hd;
   a.zdiv = Hq; a.zgroup = Hq / Hkv; a.window = window; a.sB2 = hd; a.sC2 = hd;
-  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0; a.nx = 0; a.D = nullptr;
+  a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0; a.nx = 0; a.D = nullptr; a.sD = 0; a.scaled = 0; a.dscale = a.pscale = 1.f;
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
   return hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26);
 }
@@ -957,6 +967,12 @@ int gt_gemm_group(gt_ctx *ctx, int kind, int count, const int *M, const int *N, 
 }
 }
 
+// C_i = dscale * D_i + pscale * A_i.B_i for a batch of `count` products (strides in elements; D laid out as C)
+int gemm_scaled_batched(gt_ctx *ctx, int kind, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB, gt_buf D, int64_t sD,
+                        float dscale, float pscale, gt_buf C, int64_t sC, int count) {
+  return gemm_impl(ctx, kind, 0, M, N, K, A, sA, B, sB, C, sC, count, 0, 0, 0, D, sD, 1, dscale, pscale);
+}
+
 extern "C" {
 int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const int *K, const gt_buf *A, const gt_buf *B, gt_buf C) {
   GT_ENTER(ctx);
@@ -1000,7 +1016,7 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
   a.sA = a.sB = a.sC = 0;
   a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0;
   a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0;
-  a.nx = count - 1; a.D = nullptr;
+  a.nx = count - 1; a.D = nullptr; a.sD = 0; a.scaled = 0; a.dscale = a.pscale = 1.f;
   double ksum = K[0];
   for (int i = 1; i < count; i++) {
     a.xA[i - 1] = P<const float>(A[i]); a.xB[i - 1] = P<const float>(B[i]);

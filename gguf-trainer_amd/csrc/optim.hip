@@ -8,10 +8,14 @@
 // clip scale, and the fused element update. The fold runs in chunk order, so the norm and
 // everything downstream is identical from run to run.
 //
-// Muon. Per matrix: momentum + Nesterov + sum of squares, normalise (transposing tall matrices so
-// the Gram matrix is the small one), five quintic Newton-Schulz iterations as three MFMA GEMMs and
-// two fused elementwise combines each, then the scaled descent. Matrices of equal shape are stepped
-// together as one batch (see below).
+// Muon. Per matrix: momentum + Nesterov + sum of squares, normalise, five quintic Newton-Schulz
+// iterations of three MFMA GEMMs each, then the scaled descent. The reference transposes a tall matrix
+// so that the Gram matrix is the small one (muon.ts:137-158); here a tall matrix stays as it lies and
+// its iteration is written on the other side (A = X^T X, X <- a X + X B), which is the same
+// arithmetic without the two transposing passes. The two combines of an iteration, b A + c A.A and
+// a X + B.X, are the write-backs of the products that feed them (C = dscale*D + pscale*A.B), so an
+// iteration is three launches and no elementwise pass. Matrices of equal shape are stepped together
+// as one batch (see below).
 #include <algorithm>
 #include <vector>
 #include "common.h"
@@ -188,7 +192,7 @@ struct gt_muon {
 #define NS_A 3.4445f
 #define NS_B (-4.7750f)
 #define NS_C 2.0315f
-#define RED_BLOCKS 64
+#define RED_BLOCKS 256
 
 // buf = mu*buf + g; U = nesterov ? g + mu*buf : buf; per-workgroup sum of U^2 (muon-gpu.ts:51-92).
 // With null tables (Newton-Schulz on a caller's matrix) U is only read.
@@ -200,80 +204,93 @@ __global__ __launch_bounds__(256) void muon_momentum_k(int64_t n, float *const *
   const float *g = gt ? gt[mi] : nullptr;
   float *buf = bt ? bt[mi] : nullptr;
   float s = 0;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    float u;
-    if (buf) {
-      float gi = g[i];
-      float b = mu * buf[i] + gi;
-      buf[i] = b;
-      u = nesterov ? gi + mu * b : b;
-      U[i] = u;
-    } else u = U[i];
-    s += u * u;
+  const bool vec = (n % 4 == 0) && (((reinterpret_cast<uintptr_t>(U) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(buf)) & 15) == 0);
+  if (vec) {
+    // every array is touched once: float4 per lane, the partial sum of a workgroup taken in a fixed order
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n / 4; i += (int64_t)gridDim.x * 256) {
+      v4f u;
+      if (buf) {
+        const v4f gi = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(g) + i);
+        const v4f b = reinterpret_cast<const v4f *>(buf)[i] * mu + gi;
+        reinterpret_cast<v4f *>(buf)[i] = b;
+        u = nesterov ? gi + b * mu : b;
+        reinterpret_cast<v4f *>(U)[i] = u;
+      } else u = reinterpret_cast<const v4f *>(U)[i];
+      s += (u[0] * u[0] + u[1] * u[1]) + (u[2] * u[2] + u[3] * u[3]);
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+      float u;
+      if (buf) {
+        float gi = g[i];
+        float b = mu * buf[i] + gi;
+        buf[i] = b;
+        u = nesterov ? gi + mu * b : b;
+        U[i] = u;
+      } else u = U[i];
+      s += u * u;
+    }
   }
   s = block_sum<4>(s, sm);
   if (threadIdx.x == 0) part[(size_t)mi * gridDim.x + blockIdx.x] = s;
 }
-// X = (flip ? U^T : U) / (sqrt(sum part) + 1e-7); U is [m,n], X is [r,c] with r = min(m,n)
-__global__ __launch_bounds__(256) void muon_normalize_k(int m, int n, int flip, const float *__restrict__ Uall,
+// X = U / (sqrt(sum part) + 1e-7), one matrix of `total` elements per blockIdx.y (muon.ts:137-144 without the transpose)
+__global__ __launch_bounds__(256) void muon_normalize_k(int64_t total, const float *__restrict__ Uall,
                                                         const float *__restrict__ part, int nparts, float *__restrict__ Xall) {
   __shared__ float sm[4];
   const int mi = blockIdx.y;
-  const int64_t total = (int64_t)m * n;
   const float *U = Uall + (size_t)mi * total;
   float *X = Xall + (size_t)mi * total;
   float s = 0;
   for (int i = threadIdx.x; i < nparts; i += 256) s += part[(size_t)mi * nparts + i];
   s = block_sum<4>(s, sm);
   const float inv = 1.0f / (sqrtf(s) + 1e-7f);
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    float u;
-    if (flip) { int64_t xr = i / m, xc = i % m; u = U[xc * n + xr]; }   // X[xr,xc] = U[xc,xr], X is [n,m]
-    else u = U[i];
-    X[i] = u * inv;
+  const bool vec = (total % 4 == 0) && (((reinterpret_cast<uintptr_t>(U) | reinterpret_cast<uintptr_t>(X)) & 15) == 0);
+  if (vec) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total / 4; i += (int64_t)gridDim.x * 256)
+      reinterpret_cast<v4f *>(X)[i] = reinterpret_cast<const v4f *>(U)[i] * inv;
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) X[i] = U[i] * inv;
   }
 }
-__global__ __launch_bounds__(256) void muon_combine_a_k(int64_t n, float *A, const float *__restrict__ AA) {
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) A[i] = NS_B * A[i] + NS_C * AA[i];
-}
-__global__ __launch_bounds__(256) void muon_combine_x_k(int64_t n, float *X, const float *__restrict__ BX) {
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) X[i] = NS_A * X[i] + BX[i];
-}
-// W[m,n] -= f * (flip ? X^T : X), one matrix per blockIdx.y
-__global__ __launch_bounds__(256) void muon_apply_k(int m, int n, int flip, float *const *__restrict__ wt, float *Wone,
+// W -= f * X, one matrix per blockIdx.y
+__global__ __launch_bounds__(256) void muon_apply_k(int64_t total, float *const *__restrict__ wt, float *Wone,
                                                     const float *__restrict__ Xall, float f) {
   const int mi = blockIdx.y;
-  const int64_t total = (int64_t)m * n;
   float *W = wt ? wt[mi] : Wone;
   const float *X = Xall + (size_t)mi * total;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    float x;
-    if (flip) { int64_t wr = i / n, wc = i % n; x = X[wc * m + wr]; }    // X is [n,m]
-    else x = X[i];
-    W[i] -= f * x;
+  const bool vec = (total % 4 == 0) && (((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(X)) & 15) == 0);
+  if (vec) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total / 4; i += (int64_t)gridDim.x * 256)
+      reinterpret_cast<v4f *>(W)[i] -= reinterpret_cast<const v4f *>(X)[i] * f;
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) W[i] -= f * X[i];
   }
 }
 
 static inline unsigned sgrid(gt_ctx *ctx, int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>(cdiv(n, 256), (int64_t)ctx->num_cu * 8)); }
 
-// Leaves NS(U) in X ([count][r,c]); U holds the inputs, part their per-workgroup sums of squares.
-static int newton_schulz_run(gt_ctx *ctx, const MuonGroup &G, int steps, int nparts) {
+// Leaves NS(U), laid out as U ([count][m,n]), in *result (G.X or G.BX); U holds the inputs, part their per-workgroup
+// sums of squares. Per iteration (muon.ts:146-156 with A the r x r Gram matrix, r = min(m, n)):
+//   wide (m <= n):  A = X X^T          B = b A + c A.A      X <- a X + B.X
+//   tall (m >  n):  A = X^T X          B = b A + c A.A      X <- a X + X.B
+static int newton_schulz_run(gt_ctx *ctx, const MuonGroup &G, int steps, int nparts, float **result) {
   const int m = G.rows, n = G.cols, cnt = G.count;
-  const int flip = m > n;
-  const int r = flip ? n : m, c = flip ? m : n;
+  const bool tall = m > n;
+  const int r = tall ? n : m;
   const int64_t size = (int64_t)m * n, rr = (int64_t)r * r;
-  hipLaunchKernelGGL(muon_normalize_k, dim3(sgrid(ctx, size), cnt), dim3(256), 0, ctx->stream, m, n, flip, G.U, G.part, nparts, G.X);
+  hipLaunchKernelGGL(muon_normalize_k, dim3(sgrid(ctx, size / 4 + 1), cnt), dim3(256), 0, ctx->stream, size, G.U, G.part, nparts, G.X);
   GT_LAUNCHED(ctx);
-  gt_buf bX = reinterpret_cast<gt_buf>(G.X), bA = reinterpret_cast<gt_buf>(G.A), bAA = reinterpret_cast<gt_buf>(G.AA), bBX = reinterpret_cast<gt_buf>(G.BX);
+  gt_buf bX = reinterpret_cast<gt_buf>(G.X), bY = reinterpret_cast<gt_buf>(G.BX), bA = reinterpret_cast<gt_buf>(G.A), bB = reinterpret_cast<gt_buf>(G.AA);
   for (int s = 0; s < steps; s++) {
-    if (gt_gemm_batched(ctx, GT_NT, 0, r, r, c, bX, size, bX, size, bA, rr, cnt)) return 1;       // A = X X^T
-    if (gt_gemm_batched(ctx, GT_NN, 0, r, r, r, bA, rr, bA, rr, bAA, rr, cnt)) return 1;         // AA = A^2
-    hipLaunchKernelGGL(muon_combine_a_k, dim3(sgrid(ctx, rr * cnt)), dim3(256), 0, ctx->stream, rr * cnt, G.A, G.AA);
-    GT_LAUNCHED(ctx);
-    if (gt_gemm_batched(ctx, GT_NN, 0, r, c, r, bA, rr, bX, size, bBX, size, cnt)) return 1;     // BX = (bA + cA^2) X
-    hipLaunchKernelGGL(muon_combine_x_k, dim3(sgrid(ctx, size * cnt)), dim3(256), 0, ctx->stream, size * cnt, G.X, G.BX);
-    GT_LAUNCHED(ctx);
+    if (tall) { if (gt_gemm_batched(ctx, GT_TN, 0, r, r, m, bX, size, bX, size, bA, rr, cnt)) return 1; }       // A = X^T X
+    else if (gt_gemm_batched(ctx, GT_NT, 0, r, r, n, bX, size, bX, size, bA, rr, cnt)) return 1;               // A = X X^T
+    if (gemm_scaled_batched(ctx, GT_NN, r, r, r, bA, rr, bA, rr, bA, rr, NS_B, NS_C, bB, rr, cnt)) return 1;   // B = b A + c A.A
+    if (tall) { if (gemm_scaled_batched(ctx, GT_NN, m, n, n, bX, size, bB, rr, bX, size, NS_A, 1.f, bY, size, cnt)) return 1; }   // a X + X.B
+    else if (gemm_scaled_batched(ctx, GT_NN, m, n, m, bB, rr, bX, size, bX, size, NS_A, 1.f, bY, size, cnt)) return 1;          // a X + B.X
+    std::swap(bX, bY);
   }
+  *result = reinterpret_cast<float *>(bX);
   return 0;
 }
 
@@ -482,13 +499,13 @@ int gt_muon_step(gt_ctx *ctx, gt_muon *o, double lr) {
   ProfScope ps(ctx, "muon");
   for (auto &G : o->groups) {
     const int64_t size = (int64_t)G.rows * G.cols;
-    const unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv(size, 256));
+    const unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv(size, 1024));
     hipLaunchKernelGGL(muon_momentum_k, dim3(nb, G.count), dim3(256), 0, ctx->stream, size, G.g, G.buf, G.U, o->momentum, o->nesterov, G.part);
     GT_LAUNCHED(ctx);
-    if (newton_schulz_run(ctx, G, o->ns_steps, (int)nb)) return 1;
+    float *X = nullptr;
+    if (newton_schulz_run(ctx, G, o->ns_steps, (int)nb, &X)) return 1;
     const float f = (float)(lr * sqrt(std::max(1.0, (double)G.rows / (double)G.cols)));
-    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, size), G.count), dim3(256), 0, ctx->stream, G.rows, G.cols, G.rows > G.cols ? 1 : 0,
-                       G.w, (float *)nullptr, G.X, f);
+    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, size / 4 + 1), G.count), dim3(256), 0, ctx->stream, size, G.w, (float *)nullptr, X, f);
     GT_LAUNCHED(ctx);
   }
   return 0;
@@ -515,18 +532,14 @@ int gt_newton_schulz(gt_ctx *ctx, int m, int n, int steps, gt_buf G, gt_buf out)
     group_release(ctx, T);
     GT_FAIL(ctx, "gt_newton_schulz: copying the matrix failed: %s", hipGetErrorString(ce));
   }
-  const unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv((int64_t)size, 256));
+  const unsigned nb = (unsigned)std::min<int64_t>(RED_BLOCKS, cdiv((int64_t)size, 1024));
   // sums of squares of U only (no momentum buffer, no gradient)
   hipLaunchKernelGGL(muon_momentum_k, dim3(nb, 1), dim3(256), 0, ctx->stream, (int64_t)size, (float *const *)nullptr,
                      (float *const *)nullptr, T.U, 0.f, 0, T.part);
   int rc = hipGetLastError() != hipSuccess;
-  if (!rc) rc = newton_schulz_run(ctx, T, steps, (int)nb);
-  if (!rc) {
-    // out = 0 - (-1) * X(^T): the apply kernel on a cleared destination
-    (void)hipMemsetAsync(P<void>(out), 0, size * 4, ctx->stream);
-    hipLaunchKernelGGL(muon_apply_k, dim3(sgrid(ctx, (int64_t)size), 1), dim3(256), 0, ctx->stream, m, n, m > n ? 1 : 0,
-                       (float *const *)nullptr, P<float>(out), T.X, -1.0f);
-  }
+  float *X = nullptr;
+  if (!rc) rc = newton_schulz_run(ctx, T, steps, (int)nb, &X);
+  if (!rc) rc = hipMemcpyAsync(P<void>(out), X, size * 4, hipMemcpyDeviceToDevice, ctx->stream) != hipSuccess;
   group_release(ctx, T);
   return rc;
 }
