@@ -249,13 +249,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
 // attention_mfma.hip, compiled once per head dim
 int attn_fwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_bwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                    float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                    float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v,
+                    const float *rot_q, const float *rot_k);
 int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_bwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                    float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                    float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v,
+                    const float *rot_q, const float *rot_k);
 int attn_bwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
-                     float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+                     float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v,
+                     const float *rot_q, const float *rot_k);
 static int attn_mfma_supported(int hd) { return hd == 32 || hd == 64 || hd == 128; }
 
 // A launch with fewer 128-row tiles than three per CU is cut further (measured at T = 2048, 9 heads: 1 sequence runs
@@ -329,10 +332,10 @@ static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
 }
 static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
                          float *part, float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv,
-                         int acc_v) {
-  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v)
-      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v)
-                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v))
+                         int acc_v, const float *rot_q, const float *rot_k) {
+  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k)
+      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k)
+                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k))
     return 1;
   if (p.splits > 1 && !dsb) {
     const size_t n4 = (size_t)p.B * p.T * p.Hq * p.hd / 4;
@@ -381,8 +384,12 @@ static int attn_fwd_impl(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int
   return 0;
 }
 
+// rope: with rot_q / rot_k set, q / k are rows that went through the rotation (base, pos) and dq / dk receive the gradients
+// with respect to the rows BEFORE it (MFMA kernels only: the caller has checked that)
+struct RopeBack { double base = 0; int pos = 0, rot_q = 0, rot_k = 0; };
 static int attn_bwd_impl(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
-                         gt_buf dout, gt_buf lse, gt_buf scores, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+                         gt_buf dout, gt_buf lse, gt_buf scores, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v,
+                         const RopeBack &rope = RopeBack()) {
   GT_ENTER(ctx);
   if (check(ctx, "gt_attn_bwd", B, T, Hq, Hkv, hd, window)) return 1;
   GT_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, "gt_attn_bwd: null operand");
@@ -430,7 +437,13 @@ static int attn_bwd_impl(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int
     }
     GT_LAUNCHED(ctx);
   }
-  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, P<const float>(scores), dq, acc_q, dk, acc_k, dv, acc_v);
+  float *rot = nullptr;
+  if (rope.rot_q || rope.rot_k) {
+    GT_REQUIRE(ctx, mfma, "gt_attn_bwd_scores_rope: the rotation's backward rides the matrix-core kernels only");
+    if (rope_table_get(ctx, T, hd, rope.base, rope.pos, &rot)) return 1;
+  }
+  if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, P<const float>(scores), dq, acc_q, dk, acc_k, dv, acc_v,
+                                 rope.rot_q ? rot : nullptr, rope.rot_k ? rot : nullptr);
   {
     ProfScope ps(ctx, "attention.bwd.dq");
     size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);
@@ -474,5 +487,14 @@ int gt_attn_bwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int w
                        gt_buf dout, gt_buf lse, gt_buf scores, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
   if (ctx && !scores) GT_FAIL(ctx, "gt_attn_bwd_scores: null scores buffer");
   return attn_bwd_impl(ctx, B, T, Hq, Hkv, hd, window, q, k, v, out, dout, lse, scores, dq, acc_q, dk, acc_k, dv, acc_v);
+}
+int gt_attn_bwd_scores_rope(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, gt_buf q, gt_buf k, gt_buf v, gt_buf out,
+                            gt_buf dout, gt_buf lse, gt_buf scores, double rope_base, int rope_pos, int rot_q, int rot_k,
+                            gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v) {
+  if (ctx && !scores) GT_FAIL(ctx, "gt_attn_bwd_scores_rope: null scores buffer");
+  if (ctx && hd % 8 != 0) GT_FAIL(ctx, "gt_attn_bwd_scores_rope: head dim %d is not a multiple of 8", hd);
+  RopeBack r;
+  r.base = rope_base; r.pos = rope_pos; r.rot_q = rot_q != 0; r.rot_k = rot_k != 0;
+  return attn_bwd_impl(ctx, B, T, Hq, Hkv, hd, window, q, k, v, out, dout, lse, scores, dq, acc_q, dk, acc_k, dv, acc_v, r);
 }
 }

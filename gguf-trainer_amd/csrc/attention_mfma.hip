@@ -199,6 +199,47 @@ __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32]
     }
 }
 
+// store_row for a gradient with respect to ROTATED rows (q or k after rope) whose caller wants the gradient with respect
+// to the rows before the rotation: (lo, hi) = (c lo + s hi, -s lo + c hi) per pair (j, j + HD/2), srcRope's backward
+// (wgsl.ts:346-384), applied to the accumulators on their way out. A lane holds whole rows, so both halves of every pair
+// are its own registers. cs: this row's (cos, sin) pairs, HD floats. Two float4 units of the low half at a time.
+__device__ __forceinline__ void store_row_rot(float *row, const v16f (&acc)[HD / 32], int g, float mul, int add, const float *__restrict__ cs) {
+  constexpr int NU = HD / 16;                    // float4 units in the low half of a row
+#pragma unroll
+  for (int u0 = 0; u0 < NU; u0 += 2) {
+    v4f lo[2], hi[2], c0[2], c1[2], olo[2], ohi[2];
+    int col[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+      const int u = u0 + q;
+      const int dt = HD >= 64 ? u / 4 : 0, a = HD >= 64 ? u % 4 : u;
+      const int dth = HD >= 64 ? dt + HD / 64 : 0, ah = HD >= 64 ? a : a + 2;
+      col[q] = dt * 32 + 8 * a + 4 * g;
+      lo[q] = v4f{acc[dt][4 * a], acc[dt][4 * a + 1], acc[dt][4 * a + 2], acc[dt][4 * a + 3]} * mul;
+      hi[q] = v4f{acc[dth][4 * ah], acc[dth][4 * ah + 1], acc[dth][4 * ah + 2], acc[dth][4 * ah + 3]} * mul;
+      c0[q] = *reinterpret_cast<const v4f *>(cs + 2 * col[q]);
+      c1[q] = *reinterpret_cast<const v4f *>(cs + 2 * col[q] + 4);
+      if (add) {
+        olo[q] = *reinterpret_cast<const v4f *>(row + col[q]);
+        ohi[q] = *reinterpret_cast<const v4f *>(row + col[q] + HD / 2);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+      const v4f c = {c0[q][0], c0[q][2], c1[q][0], c1[q][2]}, sn = {c0[q][1], c0[q][3], c1[q][1], c1[q][3]};
+      v4f r0 = c * lo[q] + sn * hi[q], r1 = -sn * lo[q] + c * hi[q];
+      if (add) { r0 += olo[q]; r1 += ohi[q]; }
+      *reinterpret_cast<v4f *>(row + col[q]) = r0;
+      *reinterpret_cast<v4f *>(row + col[q] + HD / 2) = r1;
+    }
+  }
+}
+// rot: the rotation table ([T][HD/2] (cos, sin) pairs) when the destination wants the gradient before the rotation, else null
+__device__ __forceinline__ void store_grad_row(float *row, const v16f (&acc)[HD / 32], int g, float mul, int add, const float *rot, int t) {
+  if (rot) store_row_rot(row, acc, g, mul, add, rot + (size_t)t * HD);
+  else store_row(row, acc, g, mul, add);
+}
+
 }  // namespace
 
 #define KT (HD <= 64 ? 64 : 32)      // keys per LDS stage in forward and dQ
@@ -416,7 +457,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP
 __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                           const float *__restrict__ v, const float *__restrict__ go,
                                                           const float *__restrict__ lse, const float *__restrict__ Dr,
-                                                          float *dq, int acc_q, float *__restrict__ dqpart) {
+                                                          float *dq, int acc_q, float *__restrict__ dqpart, const float *__restrict__ rot) {
   using IO = TileIO<KT>;
   __shared__ __attribute__((aligned(16))) float sK[KT * LD];
   __shared__ __attribute__((aligned(16))) float sV[KT * LD];
@@ -494,8 +535,9 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
     }
   }
   if (!tv) return;
-  if (p.splits > 1) store_row(dqpart + sp * ((size_t)p.B * p.T * qstr) + qoff, dacc, g, 1.0f, 0);
-  else store_row(dq + qoff, dacc, g, 1.0f, acc_q);
+  // (the rotation is linear: rotating every split's partial and summing them is the rotated sum)
+  if (p.splits > 1) store_grad_row(dqpart + sp * ((size_t)p.B * p.T * qstr) + qoff, dacc, g, 1.0f, 0, rot, t);
+  else store_grad_row(dq + qoff, dacc, g, 1.0f, acc_q, rot, t);
 }
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------
@@ -513,7 +555,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
                                                            float *dk, int acc_k, float *dv, int acc_v, float *part,
-                                                           float *dsb, const float *__restrict__ sco) {
+                                                           float *dsb, const float *__restrict__ sco, const float *__restrict__ rot) {
   using IO = TileIO<QT>;
   extern __shared__ __attribute__((aligned(16))) float dkv_smem[];      // 2 x 35 KB at hd 64, 2 x 69 KB at hd 128
   constexpr int O_G = QT * LD, O_QT = 2 * QT * LD, O_GT = O_QT + HD * IO::LDT, O_L = O_GT + HD * IO::LDT, O_D = O_L + QT;
@@ -722,10 +764,10 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
     if (part) {            // slice (split, head of the group) of the workspace, same [row][Hkv*hd] layout as dk
       const size_t slice = (size_t)p.B * p.T * kstr;
       const int nslice = p.splits * group, mine = sp * group + hh;
-      store_row(part + (size_t)mine * slice + koff, kacc, g, 1.0f, 0);
+      store_grad_row(part + (size_t)mine * slice + koff, kacc, g, 1.0f, 0, rot, s);      // every slice rotated: their sum is the rotated sum
       store_row(part + (size_t)(nslice + mine) * slice + koff, vacc, g, 1.0f, 0);
     } else {
-      store_row(dk + koff, kacc, g, 1.0f, acc_k);
+      store_grad_row(dk + koff, kacc, g, 1.0f, acc_k, rot, s);
       store_row(dv + koff, vacc, g, 1.0f, acc_v);
     }
   }
@@ -775,7 +817,7 @@ int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
 // product dS.K afterwards (5 contractions in all); without it dQ recomputes S and dP in its own kernel (7).
 int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
                       float *part, float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv,
-                      int acc_v) {
+                      int acc_v, const float *rot_q, const float *rot_k) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
   const int group = p.Hq / p.Hkv;
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart || dsb) && (p.splits * group == 1 || part),
@@ -797,7 +839,7 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
     ProfScope ps(ctx, "attention.bwd.dq");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
     hipLaunchKernelGGL(FN(attn_bwd_dq_mfma_k), grid, dim3(256), 0, ctx->stream, p, P<const float>(q), P<const float>(k),
-                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q, dqpart);
+                       P<const float>(v), P<const float>(dout), P<const float>(lse), Dr, P<float>(dq), acc_q, dqpart, rot_q);
     GT_LAUNCHED(ctx);
   }
   {
@@ -805,7 +847,7 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
     auto launch = [&](auto kern) {
       hipLaunchKernelGGL(kern, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k), P<const float>(v),
-                         P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco);
+                         P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco, rot_k);
     };
     if (sco) dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false>);
     else dsb ? launch(FN(attn_bwd_dkv_mfma_k)<false, true>) : launch(FN(attn_bwd_dkv_mfma_k)<false, false>);
@@ -819,7 +861,7 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
   }
   if (dsb) {
     ProfScope ps(ctx, "attention.bwd.dq");
-    if (gemm_band_dq(ctx, p.B, p.T, p.Hq, p.Hkv, HD, p.window, dsb, P<const float>(k), P<float>(dq), acc_q)) return 1;
+    if (gemm_band_dq(ctx, p.B, p.T, p.Hq, p.Hkv, HD, p.window, dsb, P<const float>(k), P<float>(dq), acc_q, rot_q)) return 1;
   }
   return 0;
 }

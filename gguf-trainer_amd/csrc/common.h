@@ -78,7 +78,12 @@ void rmsnorm_static_forget(gt_ctx *ctx);        // norm.hip: ctx is going away a
 int gemm_scaled_batched(gt_ctx *ctx, int kind, int M, int N, int K, gt_buf A, int64_t sA, gt_buf B, int64_t sB, gt_buf D, int64_t sD,
                         float dscale, float pscale, gt_buf C, int64_t sC, int count);
 // gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
-int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc);
+// rot: the rotation table of the rope the query rows went through ([T][hd/2] (cos, sin) pairs), when dQ is wanted with respect
+// to the rows before that rotation (the write-back then applies the rotation's backward), else null
+int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc,
+                 const float *rot = nullptr);
+// embed_rope.hip: the (cos, sin) table of a rotation, built once per (T, hd, base, pos) and kept with the context
+int rope_table_get(gt_ctx *ctx, int T, int hd, double base, int pos, float **out);
 
 // Brackets the launches made during its lifetime with a pair of events when profiling is on.
 struct ProfScope {

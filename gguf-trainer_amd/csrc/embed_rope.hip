@@ -277,6 +277,10 @@ static int rope_table(gt_ctx *ctx, int T, int hd, double base, int pos, float **
   return 0;
 }
 
+}
+int rope_table_get(gt_ctx *ctx, int T, int hd, double base, int pos, float **out) { return rope_table(ctx, T, hd, base, pos, out); }
+extern "C" {
+
 int gt_rope(gt_ctx *ctx, int rows, int T, int H, int hd, double base, int pos, int backward, gt_buf in, gt_buf out, int acc) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 0 && T >= 1 && H >= 1 && hd >= 2 && hd % 2 == 0 && in && out, "gt_rope: bad arguments (hd %d)", hd);

@@ -62,6 +62,9 @@ struct GemmArgs {
   int64_t sD;
   int scaled;
   float dscale, pscale;
+  // banded batch only: the (cos, sin) table ([M][N/2] pairs) of the rotation the rows of the other operand's source went
+  // through; the write-back then applies that rotation's backward to each row of C (pairs (j, j + N/2)). Null: none.
+  const float *rope;
 };
 
 // Which output tile (pm, pn) and which K split or batch member (z) a workgroup works on. Workgroups are handed
@@ -509,6 +512,41 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
   // of C, and registers 4q..4q+3 are four consecutive columns 8q + 4g + (0..3): one 16-byte store (and, when
   // accumulating, one 16-byte load issued before any store) instead of four scalar ones.
   const bool vec_c = (ldc % 4 == 0) && (((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(Cold)) & 15) == 0);
+  if constexpr (BAND) {
+    if (a.rope) {
+      // dQ with respect to the rows before their rotation: a pair (j, j + BN/2) of a row sits in two wavefronts' accumulators
+      // (WN = 2), so the tile goes through LDS once (the pipeline's buffers are idle now) and every thread then rotates
+      // float4 pairs of whole rows: (lo, hi) -> (c lo + s hi, -s lo + c hi), the reference's srcRope backward (wgsl.ts:346-384)
+      static_assert(!BAND || NSTG * (BM + BN) * BK >= BM * (BN + 4), "the tile must fit the pipeline's LDS");
+      constexpr int LDS_C = BN + 4;            // = 4 mod 32 words: 8 lanes of a b128 access cover all banks
+      __syncthreads();                         // everybody is done reading the last stage
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+            *reinterpret_cast<v4f *>(smem + (wm * (TM * 32) + i * 32 + l32) * LDS_C + wn * (TN * 32) + j * 32 + 8 * q + 4 * g) =
+                v4f{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+      __syncthreads();
+      constexpr int UPR = BN / 8;              // float4 pairs per row
+      for (int u = tid; u < BM * UPR; u += NT) {
+        const int rl = u / UPR, c = 4 * (u % UPR), row = m0 + rl;
+        const v4f lo = *reinterpret_cast<const v4f *>(smem + rl * LDS_C + c), hi = *reinterpret_cast<const v4f *>(smem + rl * LDS_C + BN / 2 + c);
+        const float *tp = a.rope + ((size_t)row * (BN / 2) + c) * 2;
+        const v4f c0 = *reinterpret_cast<const v4f *>(tp), c1 = *reinterpret_cast<const v4f *>(tp + 4);
+        const v4f cs = {c0[0], c0[2], c1[0], c1[2]}, sn = {c0[1], c0[3], c1[1], c1[3]};
+        float *cr = C + (size_t)row * ldc + c;
+        v4f r0 = cs * lo + sn * hi, r1 = -sn * lo + cs * hi;
+        if (add) { r0 += *reinterpret_cast<const v4f *>(cr); r1 += *reinterpret_cast<const v4f *>(cr + BN / 2); }
+        if (row < a.M) {
+          *reinterpret_cast<v4f *>(cr) = r0;
+          *reinterpret_cast<v4f *>(cr + BN / 2) = r1;
+        }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -742,7 +780,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   a.acc = acc; a.kchunk = K; a.splits = 1; a.Pp = nullptr;
   a.sA = sA; a.sB = sB; a.sC = sC;
   a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0; a.nx = 0; a.D = P<const float>(D);
-  a.sD = sD; a.scaled = scaled; a.dscale = dscale; a.pscale = pscale;
+  a.sD = sD; a.scaled = scaled; a.dscale = dscale; a.pscale = pscale; a.rope = nullptr;
   GT_REQUIRE(ctx, !D || K2 == 0, "gt_gemm_add: single-segment products only");
   GT_REQUIRE(ctx, !scaled || D, "scaled write-back needs the matrix it combines the product with");
   bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (A % 16 == 0) && (B % 16 == 0) &&
@@ -833,7 +871,8 @@ static int launch_band(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   return 0;
 }
 
-int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc) {
+int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc,
+                 const float *rot) {
   GT_REQUIRE(ctx, T % 128 == 0 && (hd == 64 || hd == 128), "banded dQ product: T %d must be a multiple of 128 and hd %d 64 or 128", T, hd);
   GT_REQUIRE(ctx, ((reinterpret_cast<uintptr_t>(dS) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(dQ)) & 15) == 0,
              "banded dQ product: operands must be 16-byte aligned");
@@ -845,6 +884,8 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.sA = (int64_t)T * T; a.sB = (int64_t)T * Hkv * hd; a.sC = (int64_t)T * Hq * hd;
   a.zdiv = Hq; a.zgroup = Hq / Hkv; a.window = window; a.sB2 = hd; a.sC2 = hd;
   a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0; a.nx = 0; a.D = nullptr; a.sD = 0; a.scaled = 0; a.dscale = a.pscale = 1.f;
+  a.rope = rot;
+  GT_REQUIRE(ctx, !rot || (Hq * hd) % 4 == 0, "banded dQ product: rotated rows need 16-byte aligned output rows");
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
   return hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26);
 }
@@ -1016,7 +1057,7 @@ int gt_gemm_sum(gt_ctx *ctx, int kind, int acc, int M, int N, int count, const i
   a.sA = a.sB = a.sC = 0;
   a.zdiv = a.zgroup = 1; a.window = 0; a.sB2 = a.sC2 = 0;
   a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0;
-  a.nx = count - 1; a.D = nullptr; a.sD = 0; a.scaled = 0; a.dscale = a.pscale = 1.f;
+  a.nx = count - 1; a.D = nullptr; a.sD = 0; a.scaled = 0; a.dscale = a.pscale = 1.f; a.rope = nullptr;
   double ksum = K[0];
   for (int i = 1; i < count; i++) {
     a.xA[i - 1] = P<const float>(A[i]); a.xB[i - 1] = P<const float>(B[i]);

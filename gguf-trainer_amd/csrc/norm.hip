@@ -150,10 +150,10 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_k(int rows, int d, const floa
 // the group sums added in group order. Narrow workgroups because the launch is latency-bound: d = 576 gives 36 of them.
 #define CS_COLS 16
 #define CS_GRPS 16
-__global__ __launch_bounds__(256) void colsum_reduce(const float *__restrict__ part, int nparts, int d, float *dw, int acc) {
+__device__ __forceinline__ void colsum_body(const float *__restrict__ part, int nparts, int d, float *dw, int acc, int blk) {
   __shared__ float sm[CS_GRPS][CS_COLS];
   const int cl = threadIdx.x % CS_COLS, grp = threadIdx.x / CS_COLS;
-  const int c = blockIdx.x * CS_COLS + cl;
+  const int c = blk * CS_COLS + cl;
   const int cr = min(c, d - 1);
   float s = 0;
   int p = grp;
@@ -173,6 +173,21 @@ __global__ __launch_bounds__(256) void colsum_reduce(const float *__restrict__ p
     for (int q = 1; q < CS_GRPS; q++) t += sm[q][cl];
     dw[c] = acc ? dw[c] + t : t;
   }
+}
+__global__ __launch_bounds__(256) void colsum_reduce(const float *__restrict__ part, int nparts, int d, float *dw, int acc) {
+  colsum_body(part, nparts, d, dw, acc, blockIdx.x);
+}
+// The column sums of several normalisations' partials in one launch (the dw of every norm a backward pass went through,
+// summed when somebody is about to read them instead of once per norm): workgroup -> (entry, 16-column block) through the
+// table in the kernel arguments, then colsum_reduce's arithmetic, so each dw has the bits its own launch would give it.
+#define CSG_MAX 96
+struct CsEntry { const float *part; float *dw; int nparts, d, acc, blk0; };
+struct CsGroup { CsEntry e[CSG_MAX]; int n; };
+__global__ __launch_bounds__(256) void colsum_group_k(CsGroup G) {
+  int i = 0;
+  for (int q = 1; q < G.n; q++) if ((int)blockIdx.x >= G.e[q].blk0) i = q;
+  const CsEntry &e = G.e[i];
+  colsum_body(e.part, e.nparts, e.d, e.dw, e.acc, (int)blockIdx.x - e.blk0);
 }
 
 // scalar fallback for d % 4 != 0 or very wide rows: one wavefront per row
@@ -246,7 +261,7 @@ int rmsnorm_static_init(gt_ctx *ctx) {
 
 template <int LPR, int NJ>
 static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
-                       gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw, float *static_part = nullptr) {
+                       gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw, float *static_part = nullptr, bool defer = false) {
   constexpr int RPB = 4 * (WAVE / LPR);
   int64_t nb = std::min<int64_t>(cdiv(rows, RPB), (int64_t)ctx->num_cu * 2);
   if (!bwd) {
@@ -256,7 +271,8 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
     return 0;
   }
   float *part = nullptr;
-  if (dw && static_part) {
+  if (defer) part = static_part;                 // the caller's buffer of nb x d floats; it sums the columns later
+  else if (dw && static_part) {
     GT_REQUIRE(ctx, (size_t)nb * d <= RMS_STATIC_FLOATS, "rmsnorm backward: %lld partial rows of %d columns exceed the static scratch",
                (long long)nb, d);
     part = static_part;
@@ -270,19 +286,25 @@ static int launch_fast(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf
                      P<const float>(x), P<const float>(w), P<const float>(y_or_g), P<const float>(rinv), P<float>(dx),
                      acc_dx, P<const float>(dx_old), part);
   GT_LAUNCHED(ctx);
-  if (dw) {
+  if (dw && !defer) {
     hipLaunchKernelGGL(colsum_reduce, dim3((unsigned)cdiv(d, CS_COLS)), dim3(256), 0, ctx->stream, part, (int)nb, d,
                        P<float>(dw), acc_dw);
     GT_LAUNCHED(ctx);
   }
   return 0;
 }
+// partial rows the fast backward kernel writes for (rows, d): one per workgroup
+static int fast_parts_rows(gt_ctx *ctx, int rows, int d) {
+  const int d4 = d / 4;
+  const int lpr = d4 <= 16 ? 16 : d4 <= 32 ? 32 : 64;
+  return (int)std::min<int64_t>(cdiv(rows, 4 * (WAVE / lpr)), (int64_t)ctx->num_cu * 2);
+}
 
 static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x, gt_buf w, gt_buf y_or_g, gt_buf rinv,
-                    gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw, float *static_part = nullptr) {
+                    gt_buf dx, int acc_dx, gt_buf dx_old, gt_buf dw, int acc_dw, float *static_part = nullptr, bool defer = false) {
   bool aligned = (x | w | y_or_g | dx | dx_old) % 16 == 0;
   int d4 = d / 4;
-#define FAST(LPR, NJ) return launch_fast<LPR, NJ>(ctx, bwd, rows, d, eps, x, w, y_or_g, rinv, dx, acc_dx, dx_old, dw, acc_dw, static_part)
+#define FAST(LPR, NJ) return launch_fast<LPR, NJ>(ctx, bwd, rows, d, eps, x, w, y_or_g, rinv, dx, acc_dx, dx_old, dw, acc_dw, static_part, defer)
   if (d % 4 == 0 && aligned && d <= RMS_STATIC_MAX_D) {
     if (d4 <= 16) FAST(16, 1);
     if (d4 <= 32) FAST(32, 1);
@@ -293,8 +315,8 @@ static int dispatch(gt_ctx *ctx, bool bwd, int rows, int d, float eps, gt_buf x,
     FAST(64, 8);
   }
 #undef FAST
-  GT_REQUIRE(ctx, !static_part, "gt_rmsnorm_bwd_static: d = %d must be a multiple of 4, at most %d, and every operand 16-byte aligned",
-             d, RMS_STATIC_MAX_D);
+  GT_REQUIRE(ctx, !static_part, "%s: d = %d must be a multiple of 4, at most %d, and every operand 16-byte aligned",
+             defer ? "gt_rmsnorm_bwd_parts" : "gt_rmsnorm_bwd_static", d, RMS_STATIC_MAX_D);
   unsigned nb = (unsigned)cdiv(rows, 4);
   if (!bwd) {
     hipLaunchKernelGGL(rmsnorm_fwd_gen, dim3(nb), dim3(256), 0, ctx->stream, rows, d, eps, P<const float>(x),
@@ -363,6 +385,40 @@ int gt_rmsnorm_bwd_static(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_b
   }
   if (dw) { g_static_last[ctx->device] = ctx; ctx->rms_static_pending = true; }      // without dw the array is not touched
   return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dx, dw, acc_dw, ctx->rms_static);
+}
+int gt_rmsnorm_parts_rows(gt_ctx *ctx, int rows, int d, int *nparts) {
+  if (!ctx || !nparts) return 1;
+  *nparts = (rows >= 1 && d >= 4 && d % 4 == 0 && d <= RMS_STATIC_MAX_D) ? fast_parts_rows(ctx, rows, d) : 0;
+  return 0;
+}
+int gt_rmsnorm_bwd_parts(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx, int acc_dx,
+                         gt_buf parts) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 1 && d >= 4 && d % 4 == 0 && d <= RMS_STATIC_MAX_D && x && w && g && rinv && dx && dx_old && parts && parts % 16 == 0,
+             "gt_rmsnorm_bwd_parts: bad arguments (rows %d, d %d: rows >= 1, d a multiple of 4 up to %d)", rows, d, RMS_STATIC_MAX_D);
+  ProfScope ps(ctx, "rmsnorm.bwd", 12.0 * rows * d);
+  return dispatch(ctx, true, rows, d, 0.f, x, w, g, rinv, dx, acc_dx, dx_old, parts, 0, P<float>(parts), true);
+}
+int gt_colsum_group(gt_ctx *ctx, int n, const gt_buf *parts, const int *nparts, const int *d, const gt_buf *dw, const int *acc) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, n >= 0 && (n == 0 || (parts && nparts && d && dw && acc)), "gt_colsum_group: %d entries or a null table", n);
+  for (int i0 = 0; i0 < n; i0 += CSG_MAX) {
+    CsGroup G;
+    memset(&G, 0, sizeof G);
+    G.n = std::min(CSG_MAX, n - i0);
+    int blocks = 0;
+    for (int q = 0; q < G.n; q++) {
+      const int i = i0 + q;
+      GT_REQUIRE(ctx, parts[i] && dw[i] && nparts[i] >= 1 && d[i] >= 1, "gt_colsum_group: entry %d is malformed", i);
+      for (int j = i0; j < i; j++) GT_REQUIRE(ctx, dw[j] != dw[i], "gt_colsum_group: entries %d and %d write the same sums", j, i);
+      G.e[q] = {P<const float>(parts[i]), P<float>(dw[i]), nparts[i], d[i], acc[i], blocks};
+      blocks += (int)cdiv(d[i], CS_COLS);
+    }
+    ProfScope ps(ctx, "rmsnorm.colsum");
+    hipLaunchKernelGGL(colsum_group_k, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, G);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
 }
 int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
                         gt_buf dw, int acc_dw) {

@@ -128,6 +128,12 @@ class HipBackend:
         self._pend_dw: list = []
         self._pend_dw_ids: set = set()
         self.group_dw = True
+        # weight gradients of normalisations held back in the backward: the kernel leaves one partial row per workgroup and
+        # the column sums of every pending one leave as ONE launch (gt_colsum_group) when anything is about to read or write
+        # one of those gradients, and wherever buffers can change hands: [(parts, rows of parts, d, dw, acc)]
+        self._pend_cs: list = []
+        self._pend_cs_ids: set = set()
+        self.defer_norm_dw = True
         self.fuse_residual_add = True
         # add's backward hands its upstream gradient on instead of copying it: an operand whose gradient has no writer yet
         # points at the upstream buffer (grad_src). A reader takes that buffer as it is; the first later writer adds to its
@@ -275,11 +281,25 @@ class HipBackend:
         if len(self._pend_dw) == 8:
             self._flush_dw()
 
+    def _flush_cs(self):
+        """The column sums of every held-back normalisation weight gradient, one launch."""
+        pend = self._pend_cs
+        if not pend:
+            return
+        self._pend_cs = []
+        self._pend_cs_ids = set()
+        n = len(pend)
+        check(self._ctx, lib.gt_colsum_group(self._ctx, n, (c_buf * n)(*[p[0] for p in pend]), (C.c_int * n)(*[p[1] for p in pend]),
+                                             (C.c_int * n)(*[p[2] for p in pend]), (c_buf * n)(*[p[3] for p in pend]),
+                                             (C.c_int * n)(*[p[4] for p in pend])), "rmsnorm.dw")
+
     def _flush_dx(self, t: Tensor = None):
         """Launch the held-back input-gradient products: those into t's gradient, or all of them (then the held-back
-        weight-gradient products go too)."""
+        weight-gradient products and column sums go too)."""
         if t is None and self._pend_dw:
             self._flush_dw()
+        if t is None and self._pend_cs:
+            self._flush_cs()
         if not self._pend_dx:
             return
         if t is None:
@@ -446,6 +466,8 @@ class HipBackend:
             self._flush_dx(t)       # products held back for this gradient go first: the order of its writers is kept
         if self._pend_dw and id(t) in self._pend_dw_ids:
             self._flush_dw()
+        if self._pend_cs and id(t) in self._pend_cs_ids:
+            self._flush_cs()
         e = self._entries.get(t)
         if e is None:
             e = self._entry_for(t)
@@ -517,6 +539,8 @@ class HipBackend:
             self._flush_dx(t)
         if self._pend_dw and id(t) in self._pend_dw_ids:
             self._flush_dw()
+        if self._pend_cs and id(t) in self._pend_cs_ids:
+            self._flush_cs()
         e = self._entries.get(t)
         if e is None:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
@@ -749,6 +773,7 @@ class HipBackend:
         self._pend_rope = None
         self._pend_dx = {}
         self._pend_dw = []
+        self._pend_cs = []
         if not self._destroyed:
             self._destroyed = True
             for c in self._ctxs:
@@ -1052,6 +1077,16 @@ class HipBackend:
             g = self._gsrc(out)
             dx, acc, old = self._gdst_from(x)
             dw, accw = self._gdst(weight) if wants_dw else (0, 0)
+            if dw and self.defer_norm_dw:
+                nparts = C.c_int(0)
+                check(self._ctx, lib.gt_rmsnorm_parts_rows(self._ctx, rows, d, C.byref(nparts)), "rmsnorm.bwd")
+                if nparts.value > 0 and (xd | wd | g | dx | old) % 16 == 0:
+                    parts = self._scratch_buf(nparts.value * d * 4)
+                    check(self._ctx, lib.gt_rmsnorm_bwd_parts(self._ctx, rows, d, xd, wd, g, rinv, old, dx, 1 if old != dx else acc, parts),
+                          "rmsnorm.bwd")
+                    self._pend_cs.append((parts, nparts.value, d, dw, accw))
+                    self._pend_cs_ids.add(id(weight))
+                    return
             if old != dx:
                 check(self._ctx, lib.gt_rmsnorm_bwd_from(self._ctx, rows, d, xd, wd, g, rinv, old, dx, dw, accw), "rmsnorm.bwd")
             else:

@@ -64,6 +64,9 @@ _SIG = {
     "gt_rmsnorm_bwd": [ctxp, i32, i32, buf, buf, buf, buf, buf, i32, buf, i32],
     "gt_rmsnorm_bwd_static": [ctxp, i32, i32, buf, buf, buf, buf, buf, i32, buf, i32],
     "gt_rmsnorm_bwd_from": [ctxp, i32, i32, buf, buf, buf, buf, buf, buf, buf, i32],
+    "gt_rmsnorm_parts_rows": [ctxp, i32, i32, C.POINTER(i32)],
+    "gt_rmsnorm_bwd_parts": [ctxp, i32, i32, buf, buf, buf, buf, buf, buf, i32, buf],
+    "gt_colsum_group": [ctxp, i32, C.POINTER(buf), C.POINTER(i32), C.POINTER(i32), C.POINTER(buf), C.POINTER(i32)],
     "gt_embedding_fwd": [ctxp, i32, i32, i32, buf, buf, buf],
     "gt_embedding_bwd": [ctxp, i32, i32, i32, buf, buf, buf, i32],
     "gt_rope": [ctxp, i32, i32, i32, i32, f64, i32, i32, buf, buf, i32],
@@ -75,6 +78,7 @@ _SIG = {
     "gt_attn_scores_bytes": [ctxp, i32, i32, i32, i32, i32, i32, C.POINTER(C.c_uint64)],
     "gt_attn_fwd_scores": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, buf],
     "gt_attn_bwd_scores": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, buf, buf, buf, i32, buf, i32, buf, i32],
+    "gt_attn_bwd_scores_rope": [ctxp, i32, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf, buf, buf, f64, i32, i32, i32, buf, i32, buf, i32, buf, i32],
     "gt_ce_fwd": [ctxp, i32, i32, i32, buf, buf, buf, buf, buf],
     "gt_ce_bwd": [ctxp, i32, i32, i32, buf, buf, buf, buf, f32, buf, i32],
     "gt_ce_chunk_stats": [ctxp, i32, i32, i32, i32, i32, buf, buf, buf, buf, buf],

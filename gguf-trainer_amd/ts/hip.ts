@@ -70,6 +70,9 @@ const SYMBOLS = {
   gt_rmsnorm_bwd:        { parameters: [ptr, i32, i32, u64, u64, u64, u64, u64, i32, u64, i32], result: i32 },
   gt_rmsnorm_bwd_static: { parameters: [ptr, i32, i32, u64, u64, u64, u64, u64, i32, u64, i32], result: i32 },
   gt_rmsnorm_bwd_from:   { parameters: [ptr, i32, i32, u64, u64, u64, u64, u64, u64, u64, i32], result: i32 },
+  gt_rmsnorm_parts_rows: { parameters: [ptr, i32, i32, buf], result: i32 },
+  gt_rmsnorm_bwd_parts:  { parameters: [ptr, i32, i32, u64, u64, u64, u64, u64, u64, i32, u64], result: i32 },
+  gt_colsum_group:       { parameters: [ptr, i32, buf, buf, buf, buf, buf], result: i32 },
   gt_embedding_fwd:      { parameters: [ptr, i32, i32, i32, u64, u64, u64], result: i32 },
   gt_embedding_bwd:      { parameters: [ptr, i32, i32, i32, u64, u64, u64, i32], result: i32 },
   gt_rope:               { parameters: [ptr, i32, i32, i32, i32, f64, i32, i32, u64, u64, i32], result: i32 },
@@ -79,6 +82,7 @@ const SYMBOLS = {
   gt_attn_scores_bytes:  { parameters: [ptr, i32, i32, i32, i32, i32, i32, buf], result: i32 },
   gt_attn_fwd_scores:    { parameters: [ptr, i32, i32, i32, i32, i32, i32, u64, u64, u64, u64, u64, u64], result: i32 },
   gt_attn_bwd_scores:    { parameters: [ptr, i32, i32, i32, i32, i32, i32, u64, u64, u64, u64, u64, u64, u64, u64, i32, u64, i32, u64, i32], result: i32 },
+  gt_attn_bwd_scores_rope: { parameters: [ptr, i32, i32, i32, i32, i32, i32, u64, u64, u64, u64, u64, u64, u64, f64, i32, i32, i32, u64, i32, u64, i32, u64, i32], result: i32 },
   gt_ce_fwd:             { parameters: [ptr, i32, i32, i32, u64, u64, u64, u64, u64], result: i32 },
   gt_ce_bwd:             { parameters: [ptr, i32, i32, i32, u64, u64, u64, u64, f32, u64, i32], result: i32 },
   gt_ce_chunk_stats:     { parameters: [ptr, i32, i32, i32, i32, i32, u64, u64, u64, u64, u64], result: i32 },

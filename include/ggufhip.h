@@ -166,6 +166,19 @@ int gt_rmsnorm_bwd(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, g
  * webgpu.ts:921-937): the copy is skipped and the upstream buffer is read here instead. */
 int gt_rmsnorm_bwd_from(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
                         gt_buf dw, int acc_dw);
+/* The weight gradient's column sums put off. srcRmsNormBwdW (wgsl.ts:286-303) runs once per normalisation; here the backward
+ * kernel already leaves one partial row per workgroup, and a host that knows nobody reads dw before the end of the backward
+ * pass can keep those rows and sum the columns of every normalisation in ONE launch at that point:
+ *   gt_rmsnorm_parts_rows: how many partial rows of d floats gt_rmsnorm_bwd_parts writes for (rows, d); 0 = this shape is
+ *                          not served (d not a multiple of 4 or above 2048: use gt_rmsnorm_bwd)
+ *   gt_rmsnorm_bwd_parts:  dx = (acc_dx ? dx_old : 0) + the normalisation's input gradient (dx_old may be dx itself), and the
+ *                          partial rows into `parts` (the caller's buffer, 16-byte aligned); no dw is written
+ *   gt_colsum_group:       dw_i (+)= the column sums of parts_i, for n entries in one launch (host arrays of n entries);
+ *                          bit for bit what gt_rmsnorm_bwd would have written. Entries must have distinct dw. */
+int gt_rmsnorm_parts_rows(gt_ctx *ctx, int rows, int d, int *nparts);
+int gt_rmsnorm_bwd_parts(gt_ctx *ctx, int rows, int d, gt_buf x, gt_buf w, gt_buf g, gt_buf rinv, gt_buf dx_old, gt_buf dx,
+                         int acc_dx, gt_buf parts);
+int gt_colsum_group(gt_ctx *ctx, int n, const gt_buf *parts, const int *nparts, const int *d, const gt_buf *dw, const int *acc);
 
 /* gt_rmsnorm_bwd for callers that cannot allocate device memory: code under HIP graph capture, tight loops of a serving
  * process, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments and bit-identical
@@ -214,6 +227,15 @@ int gt_attn_fwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int w
 int gt_attn_bwd_scores(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
                        gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf dout, gt_buf lse, gt_buf scores,
                        gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
+/* gt_attn_bwd_scores for q and / or k that are the outputs of a rope (src/arch/llama.ts:196-199 rotates both before attention):
+ * with rot_q (rot_k) set, dq (dk) receives the gradient with respect to the rows BEFORE the rotation (base rope_base,
+ * offset rope_pos, as gt_rope takes them), i.e. what gt_rope(backward = 1) would make of the gradient this call computes, applied
+ * in the write-backs of the dQ product and of dK. The reference runs srcRope's backward as a dispatch of its own per tensor
+ * (webgpu.ts:1117-1121). Same conditions as gt_attn_bwd_scores; the results differ from the two-call form by rounding only. */
+int gt_attn_bwd_scores_rope(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
+                            gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf dout, gt_buf lse, gt_buf scores,
+                            double rope_base, int rope_pos, int rot_q, int rot_k,
+                            gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v);
 
 /* ---- cross-entropy: srcCeFwd / CeReduce / CeBwd (wgsl.ts:936-1133), webgpu.ts:1281-1327 ------
  * rows = n_seq * T. Sequence s owns rows [s*T, (s+1)*T) and its own denominator
