@@ -48,7 +48,7 @@ _ALIGN = 256
 
 class _Entry:
     __slots__ = ("data", "grad", "nbytes", "external", "grad_init", "lazy_act", "consumers", "fused_uses",
-                 "region", "keep_grad", "extra", "needs_grad", "lazy_lin", "grad_src", "stream", "sgrad")
+                 "region", "keep_grad", "extra", "needs_grad", "lazy_lin", "grad_src", "stream", "sgrad", "rope_of", "rope_fused")
 
     def __init__(self, nbytes, external):
         self.data = 0
@@ -67,6 +67,8 @@ class _Entry:
         self.grad_src = 0           # another tensor's gradient buffer that holds this gradient's value so far (add's backward)
         self.stream = 0             # the stream whose launches produce and consume this tensor (its buffers come from that stream's pool)
         self.sgrad = None           # parameters: {stream: [accumulator, written?]} of the streams other than the first
+        self.rope_of = None         # a rotation's output: (input tensor, (T, hd, base, pos))
+        self.rope_fused = False     # an attention backward wrote the rotation's input gradient itself: the rotation's closure has nothing to do
 
 
 class HipBackend:
@@ -134,6 +136,9 @@ class HipBackend:
         self._pend_cs: list = []
         self._pend_cs_ids: set = set()
         self.defer_norm_dw = True
+        # attention's backward applies the backward of the rotations its q and k came through in the write-backs of dQ and
+        # dK (gt_attn_bwd_scores_rope) where q / k are rotation outputs nobody else has read: no rope.bwd launch is left
+        self.fuse_rope_bwd = True
         self.fuse_residual_add = True
         # add's backward hands its upstream gradient on instead of copying it: an operand whose gradient has no writer yet
         # points at the upstream buffer (grad_src). A reader takes that buffer as it is; the first later writer adds to its
@@ -1129,9 +1134,13 @@ class HipBackend:
         held, self._pend_rope = self._pend_rope, None
         xd = self._data(x)
         out, e = self._make_out([rows, H * hd], [x])
+        e.rope_of = (x, (T, hd, float(base), int(pos_offset)))
         self._rope((held, ((rows, T, hd, float(base), pos_offset, 0), H, xd, e.data, 0)))
 
         def bw():           # the two backward rotations are never neighbours in the tape's order (k's linear sits between them)
+            oe = self._entries.get(out)
+            if oe is not None and oe.rope_fused:
+                return      # the attention that consumed this rotation wrote x's gradient in its own write-back
             g = self._gsrc(out)
             dx, acc = self._gdst(x)
             if dx:
@@ -1163,8 +1172,39 @@ class HipBackend:
             check(self._ctx, lib.gt_attn_fwd(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, e.data, lse), "attention")
         od = e.data
 
+        def rope_source(t):
+            """t's rotation (input tensor, parameters) when its backward can ride this attention's write-backs: t is a
+            rotation's output that only this attention has read and whose gradient nobody has touched."""
+            te = self._entries.get(t)
+            if (not self.fuse_rope_bwd or not scores or te is None or te.rope_of is None or te.consumers != 1 or te.grad_init
+                    or te.grad_src or te.keep_grad or te.grad or hd % 8 or id(t) in self._pend_dx):
+                return None
+            src, par = te.rope_of
+            if par[0] != T or par[1] != hd:
+                return None
+            se = self._entries.get(src)
+            if se is None or (se.external and not src.requires_grad):
+                return None
+            return src, par
+
         def bw():
             g = self._gsrc(out)
+            rq, rk = rope_source(q), (rope_source(k) if k is not q else None)
+            if rq and rk and rq[1] != rk[1]:
+                rk = None                           # two different rotations: one table per call
+            if rq or rk:
+                par = (rq or rk)[1]
+                dq, aq = self._gdst(rq[0] if rq else q)
+                dk, ak = self._gdst(rk[0] if rk else k)
+                dv, av = self._gdst(v)
+                if rq:
+                    self._entries[q].rope_fused = True
+                if rk:
+                    self._entries[k].rope_fused = True
+                check(self._ctx, lib.gt_attn_bwd_scores_rope(self._ctx, B, T, Hq, Hkv, hd, window, qd, kd, vd, od, g, lse, scores,
+                                                             par[2], par[3], 1 if rq else 0, 1 if rk else 0,
+                                                             dq, aq, dk, ak, dv, av), "attention.bwd")
+                return
             dq, aq = self._gdst(q)
             dk, ak = self._gdst(k)
             dv, av = self._gdst(v)

@@ -960,3 +960,37 @@ def test_optimizer_destroy_after_the_backend_is_gone(ref):
     mu.destroy()
     ad.destroy()
     assert not ad._h and not mu._h and ad._m == [] and mu._bufs == []
+
+
+@pytest.mark.parametrize("name", ["smollm2", "gemma3-window", "qwen3-hd128"])
+@pytest.mark.parametrize("recompute", [False, True])
+def test_rotation_backward_rides_the_attention_write_backs(gpu, ref, name, recompute):
+    """With kept scores (T a multiple of 128) the backward of rope(q) and rope(k) is applied where attention's backward
+    writes dQ and dK: no rope.bwd launch is left, the loss is bit-identical and every gradient equals the unfused path's to
+    rounding and the oracle's to the parity bound. llama (rotation straight after the projections), gemma-style and qwen3
+    (after the per-head norms), GQA, a window, with and without recomputed layers."""
+    kw = dict(REAL[name], layers=2)
+    rmodel, model = build_pair(ref, kw, seed=61, std=0.05)
+    T = 128
+    seqs = batches(ref, kw["vocab"], T, 2, seed=62, mask_every=7)
+    res, n = {}, {}
+    try:
+        for fuse in (True, False):
+            gpu.fuse_rope_bwd = fuse
+            gpu.start_profile("rope")
+            res[fuse] = hip_step(gpu, model, seqs, True, T, recompute=recompute)
+            n[fuse] = {k: v[1] for k, v in gpu.stop_profile().items()}
+    finally:
+        gpu.fuse_rope_bwd = True
+    assert n[True].get("rope.bwd", 0) == 0 and n[False]["rope.bwd"] == 2 * kw["layers"], n
+    assert np.array_equal(res[True][0], res[False][0])
+    for pname in res[True][1]:
+        assert_close(res[True][1][pname], res[False][1][pname], f"fused vs separate rotations, {pname}", rel_l2=2e-6, max_rel=2e-5)
+    ref.PARALLEL_BWD = True
+    ref.set_threads(min(16, ref.max_threads()))
+    try:
+        lr, gr = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.PARALLEL_BWD = False
+        ref.set_threads(1)
+    compare(res[True][0], res[True][1], lr, gr, f"{name}, rotations' backward in the attention write-backs")

@@ -924,3 +924,61 @@ def test_paired_linear_launches(gpu, ref):
             gpu.uninstall()
             gpu.batch_linears = True
     assert counts == {True: 1, False: 2}, counts
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,keep_ds", [(1, 256, 4, 2, 64, 0, 1), (2, 128, 3, 3, 64, 0, 1), (1, 384, 4, 1, 128, 100, 1),
+                                                        (2, 256, 6, 2, 64, 70, 0), (1, 128, 2, 2, 128, 0, 0), (8, 256, 9, 3, 64, 0, 1)])
+@pytest.mark.parametrize("acc", [0, 1])
+def test_attention_backward_with_the_rotations_backward_in_its_write_backs(gpu, B, T, Hq, Hkv, hd, window, keep_ds, acc):
+    """gt_attn_bwd_scores_rope against gt_attn_bwd_scores followed by gt_rope(backward = 1) on dq and dk: the gradients with
+    respect to q and k before their rotation, by the banded dQ product's write-back (keep_ds = 1) and by the dQ kernel's
+    (keep_ds = 0), dK direct (one head per kv head) and through the per-head slices (GQA, and the split launches of a small
+    batch), head dims 64 and 128, with a window, storing and accumulating; and each of the two rotations alone."""
+    lib = mod("lib")
+    L = lib.lib
+    rs = np.random.RandomState(T + hd + window)
+    rows = B * T
+    mk = lambda n: rs.standard_normal((rows, n)).astype(np.float32)
+    q, k, v, go = mk(Hq * hd), mk(Hkv * hd), mk(Hkv * hd), mk(Hq * hd)
+    dq0, dk0, dv0 = mk(Hq * hd), mk(Hkv * hd), mk(Hkv * hd)
+    c = gpu.ctx
+
+    def dev(a):
+        b = gpu.create_state_buffer(a.nbytes)
+        gpu.write_state_buffer(b, a)
+        return b
+    bq, bk, bv, bgo = dev(q), dev(k), dev(v), dev(go)
+    bout, blse = gpu.create_state_buffer(q.nbytes), gpu.create_state_buffer(B * Hq * T * 4)
+    need = C.c_uint64()
+    lib.check(c, L.gt_attn_scores_bytes(c, B, T, Hq, Hkv, hd, window, C.byref(need)), "bytes")
+    assert need.value > 0
+    bsc = gpu.create_state_buffer(need.value)
+    base, pos = 10000.0, 3
+    gpu.set_option("attn.keep_ds", keep_ds)
+    try:
+        lib.check(c, L.gt_attn_fwd_scores(c, B, T, Hq, Hkv, hd, window, bq, bk, bv, bout, blse, bsc), "fwd")
+        # the two-call form: gradients with respect to the rotated rows, then the rotation's backward
+        tq, tk = gpu.create_state_buffer(q.nbytes), gpu.create_state_buffer(k.nbytes)
+        rq, rk, rv = dev(dq0), dev(dk0), dev(dv0)
+        lib.check(c, L.gt_attn_bwd_scores(c, B, T, Hq, Hkv, hd, window, bq, bk, bv, bout, bgo, blse, bsc, tq, 0, tk, 0, rv, acc), "bwd")
+        lib.check(c, L.gt_rope(c, rows, T, Hq, hd, base, pos, 1, tq, rq, acc), "rope.bwd")
+        lib.check(c, L.gt_rope(c, rows, T, Hkv, hd, base, pos, 1, tk, rk, acc), "rope.bwd")
+        want = [gpu.read_state_buffer(b, n).copy() for b, n in ((rq, q.size), (rk, k.size), (rv, v.size))]
+        plain = [gpu.read_state_buffer(b, n).copy() for b, n in ((tq, q.size), (tk, k.size))]
+        for rot_q, rot_k in ((1, 1), (1, 0), (0, 1)):
+            fq, fk, fv = dev(dq0), dev(dk0), dev(dv0)
+            lib.check(c, L.gt_attn_bwd_scores_rope(c, B, T, Hq, Hkv, hd, window, bq, bk, bv, bout, bgo, blse, bsc, base, pos, rot_q, rot_k,
+                                                   fq, acc, fk, acc, fv, acc), "bwd.rope")
+            got = [gpu.read_state_buffer(b, n).copy() for b, n in ((fq, q.size), (fk, k.size), (fv, v.size))]
+            wq = want[0] if rot_q else plain[0] + (dq0.ravel() if acc else 0)
+            wk = want[1] if rot_k else plain[1] + (dk0.ravel() if acc else 0)
+            assert_close(got[0], wq, f"dq, rotations ({rot_q}, {rot_k})", rel_l2=2e-6, max_rel=2e-5)
+            assert_close(got[1], wk, f"dk, rotations ({rot_q}, {rot_k})", rel_l2=2e-6, max_rel=2e-5)
+            assert np.array_equal(got[2], want[2]), "dv does not depend on the rotations"
+            for b in (fq, fk, fv):
+                gpu.free_state_buffer(b)
+        rc = L.gt_attn_bwd_scores_rope(c, B, T, Hq, Hkv, hd, window, bq, bk, bv, bout, bgo, blse, 0, base, pos, 1, 1, tq, 0, tk, 0, rv, 0)
+        assert rc != 0 and "null scores buffer" in L.gt_last_error(c).decode()
+    finally:
+        gpu.set_option("attn.keep_ds", 1)
+        gpu.sync([])
