@@ -272,6 +272,28 @@ def micro_kernels(gpu, L, reps=10, sustained=30):
             fn()
         L.check(c, lib.gt_timer_stop(c, C.byref(ms)), "gt_timer_stop")
         return ms.value / sustained, flop * sustained / (ms.value * 1e-3)
+    # RMSNorm backward is a 113 MB launch here, 25 us: its ramp and tail weigh as much as for the plain add of the same size
+    # above. The same kernel over eight times the rows (906 MB) shows its rate without them.
+    R8 = 8 * R
+    x8, g8, dx8, rinv8 = zeros(R8 * H), zeros(R8 * H), zeros(R8 * H), zeros(R8)
+    for off in range(0, 4 * R8 * H, blk.nbytes):
+        nb_ = min(blk.nbytes, 4 * R8 * H - off)
+        L.check(c, lib.gt_h2d(c, x8 + off, blk.ctypes.data_as(C.c_void_p), nb_), "h2d")
+        L.check(c, lib.gt_h2d(c, g8 + off, blk.ctypes.data_as(C.c_void_p), nb_), "h2d")
+    L.check(c, lib.gt_rmsnorm_fwd(c, R8, H, 1e-5, x8, w_n, dx8, rinv8), "rmsnorm")
+    big = {}
+    for name, fn in (("rmsnorm.bwd", lambda: L.check(c, lib.gt_rmsnorm_bwd(c, R8, H, x8, w_n, g8, rinv8, dx8, 0, dw_n, 0), "rmsnorm.bwd")),
+                     ("add", lambda: L.check(c, lib.gt_add_fwd(c, R8 * H, x8, g8, dx8), "add"))):
+        for _ in range(3):
+            fn()
+        ms8 = C.c_double()
+        L.check(c, lib.gt_timer_start(c), "gt_timer_start")
+        for _ in range(10):
+            fn()
+        L.check(c, lib.gt_timer_stop(c, C.byref(ms8)), "gt_timer_stop")
+        big[name] = ms8.value / 10
+    for b8 in (x8, g8, dx8, rinv8):
+        L.check(c, lib.gt_free(c, b8), "gt_free")
     flop = 2.0 * R * H * F
     sus = {"gemm.nn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.NN, 0, R, H, F, dY, W, dX), "dX"), flop),
            "gemm.tn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.TN, 0, F, H, R, dY, X, dW), "dW"), flop)}
@@ -297,6 +319,11 @@ def micro_kernels(gpu, L, reps=10, sustained=30):
             out[desc]["sustained_achieved"] = round(sus[key][1] / 1e12, 3)
             out[desc]["sustained_frac"] = round(sus[key][1] / PEAK_FP32_MFMA, 4)
             out[desc]["sustained"] = f"{sustained} launches back to back inside one event pair (the reduction pass of a split-K product included)"
+    for key, desc in (("rmsnorm.bwd", "RMSNorm backward [131072x576] (8x the rows, 10 launches back to back)"),
+                      ("add", "yardstick out = a + b [131072x576] (8x the rows, 10 launches back to back)")):
+        rate = 12.0 * R8 * H / (big[key] * 1e-3)
+        out[desc] = {"kernel": key, "bound": "hbm", "us_per_launch": round(1e3 * big[key], 1), "achieved": round(rate / 1e12, 3), "unit": "TB/s",
+                     "frac": round(rate / PEAK_HBM, 4)}
     for b in (X, W, dY, dX, dW, gate, up, dgate, dup, g_n, w_n, rinv, y_n, dx_n, dw_n, z, dz, tgb, inv, loss, lse):
         L.check(c, lib.gt_free(c, b), "gt_free")
     return out
@@ -412,6 +439,21 @@ def run_workload(mods, config, steps, warmup, a, headline):
         step(total - 1)
         op = gpu.stop_profile()
         res["opt_prof"] = op.get("adamw")
+        res["opt_sustained"] = None
+        if headline and not wl.get("muon") and not wl.get("lora"):
+            # ten AdamW steps back to back inside one event pair (gradients as the last backward left them): the kernel's rate
+            # without the clock and cache state a whole training step leaves behind
+            import ctypes as C
+            Lm = importlib.import_module(f"{PKG}.lib")
+            gpu.ensure_grads_defined(opt.params)
+            ms = C.c_double()
+            for _ in range(2):
+                Lm.check(gpu.ctx, Lm.lib.gt_adamw_step(gpu.ctx, opt._h, 0.0, 0.5, 0.5), "gt_adamw_step")      # lr 0: the weights stay put
+            Lm.check(gpu.ctx, Lm.lib.gt_timer_start(gpu.ctx), "gt_timer_start")
+            for _ in range(10):
+                Lm.check(gpu.ctx, Lm.lib.gt_adamw_step(gpu.ctx, opt._h, 0.0, 0.5, 0.5), "gt_adamw_step")
+            Lm.check(gpu.ctx, Lm.lib.gt_timer_stop(gpu.ctx, C.byref(ms)), "gt_timer_stop")
+            res["opt_sustained"] = ms.value / 10
         if wl.get("muon") and op.get("muon"):
             ms, cnt, _ = op["muon"]
             fl = muon_flop(model)
@@ -553,7 +595,13 @@ def main():
         ms, cnt, work = r["opt_prof"]
         kernels[f"AdamW step, {r['n_params']} params, clip on"] = {
             "kernel": "adamw", "bound": "hbm", "us_per_launch": round(1e3 * ms / cnt, 1),
-            "achieved": round(work / (ms * 1e-3) / 1e12, 3), "unit": "TB/s", "frac": round(work / (ms * 1e-3) / PEAK_HBM, 4)}
+            "achieved": round(work / (ms * 1e-3) / 1e12, 3), "unit": "TB/s", "frac": round(work / (ms * 1e-3) / PEAK_HBM, 4),
+            "launch": "the one step after a training step (three launches: sum of squares, clip scale, update)"}
+        if r.get("opt_sustained"):
+            rate = work / cnt / (r["opt_sustained"] * 1e-3)
+            kernels[f"AdamW step, {r['n_params']} params, clip on"].update(
+                {"sustained_us_per_launch": round(1e3 * r["opt_sustained"], 1), "sustained_achieved": round(rate / 1e12, 3),
+                 "sustained_frac": round(rate / PEAK_HBM, 4), "sustained": "10 steps back to back inside one event pair"})
     gpu.destroy()
 
     if a.profile_all:
