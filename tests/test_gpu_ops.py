@@ -982,3 +982,97 @@ def test_attention_backward_with_the_rotations_backward_in_its_write_backs(gpu, 
     finally:
         gpu.set_option("attn.keep_ds", 1)
         gpu.sync([])
+
+
+def test_deferred_rmsnorm_weight_gradient_sums_equal_the_direct_ones(gpu):
+    """gt_rmsnorm_bwd_parts + gt_colsum_group against gt_rmsnorm_bwd, bit for bit: dx (stored, added to its own contents, added
+    to another buffer's) and dw (stored and accumulated) for several normalisations summed in ONE launch, per-row and per-head
+    shapes, more entries than one launch's table holds (chunked), and the refusals: a shape the fast kernel does not serve
+    reports 0 partial rows, two entries with one destination are an error."""
+    lib = mod("lib")
+    L, c = lib.lib, gpu.ctx
+    rs = np.random.RandomState(5)
+    shapes = [(2048, 576), (4096, 64), (300, 128), (16384, 576), (77, 2048), (1, 4)] + [(64 + i, 32) for i in range(100)]
+
+    def dev(a):
+        b = gpu.create_state_buffer(a.nbytes)
+        gpu.write_state_buffer(b, a)
+        return b
+    want, pend, keep = [], [], []
+    for i, (rows, d) in enumerate(shapes):
+        x, g = rs.standard_normal((rows, d)).astype(np.float32), rs.standard_normal((rows, d)).astype(np.float32)
+        w = (1 + 0.3 * rs.standard_normal(d)).astype(np.float32)
+        dx0, dw0 = rs.standard_normal((rows, d)).astype(np.float32), rs.standard_normal(d).astype(np.float32)
+        mode = i % 3                              # 0: dx stored, 1: dx += , 2: dx = other + ...
+        accw = (i // 3) % 2
+        bx, bg, bw = dev(x), dev(g), dev(w)
+        by, br = gpu.create_state_buffer(x.nbytes), gpu.create_state_buffer(rows * 4)
+        lib.check(c, L.gt_rmsnorm_fwd(c, rows, d, 1e-5, bx, bw, by, br), "fwd")
+        # direct
+        bdx, bdw, bold = dev(dx0), dev(dw0), dev(dx0)
+        if mode == 2:
+            lib.check(c, L.gt_rmsnorm_bwd_from(c, rows, d, bx, bw, bg, br, bold, bdx, bdw, accw), "bwd")
+        else:
+            lib.check(c, L.gt_rmsnorm_bwd(c, rows, d, bx, bw, bg, br, bdx, mode, bdw, accw), "bwd")
+        want.append((gpu.read_state_buffer(bdx, rows * d).copy(), gpu.read_state_buffer(bdw, d).copy()))
+        # deferred
+        n = C.c_int(-1)
+        lib.check(c, L.gt_rmsnorm_parts_rows(c, rows, d, C.byref(n)), "rows")
+        assert n.value >= 1
+        fdx, fdw = dev(dx0), dev(dw0)
+        parts = gpu.create_state_buffer(n.value * d * 4)
+        lib.check(c, L.gt_rmsnorm_bwd_parts(c, rows, d, bx, bw, bg, br, bold if mode == 2 else fdx, fdx, 1 if mode else 0, parts), "parts")
+        pend.append((parts, n.value, d, fdw, accw))
+        keep.append((fdx, fdw, rows, d))
+    n = len(pend)
+    lib.check(c, L.gt_colsum_group(c, n, (C.c_uint64 * n)(*[p[0] for p in pend]), (C.c_int * n)(*[p[1] for p in pend]),
+                                   (C.c_int * n)(*[p[2] for p in pend]), (C.c_uint64 * n)(*[p[3] for p in pend]),
+                                   (C.c_int * n)(*[p[4] for p in pend])), "colsum")
+    for (fdx, fdw, rows, d), (wdx, wdw) in zip(keep, want):
+        assert np.array_equal(gpu.read_state_buffer(fdx, rows * d), wdx), f"dx [{rows}, {d}]"
+        assert np.array_equal(gpu.read_state_buffer(fdw, d), wdw), f"dw [{rows}, {d}]"
+    for rows, d in ((10, 30), (10, 4096), (0, 64)):
+        nn = C.c_int(-1)
+        lib.check(c, L.gt_rmsnorm_parts_rows(c, rows, d, C.byref(nn)), "rows")
+        assert nn.value == 0
+    two = pend[:2]
+    rc = L.gt_colsum_group(c, 2, (C.c_uint64 * 2)(two[0][0], two[1][0]), (C.c_int * 2)(two[0][1], two[1][1]), (C.c_int * 2)(two[0][2], two[0][2]),
+                           (C.c_uint64 * 2)(two[0][3], two[0][3]), (C.c_int * 2)(0, 0))
+    assert rc != 0 and "write the same sums" in L.gt_last_error(c).decode()
+    gpu.sync([])
+
+
+def test_stream_mark_and_wait_order_two_contexts(gpu):
+    """gt_stream_mark / gt_stream_wait: work queued on a second context after the wait sees what the first context had queued
+    before its mark, with no host wait in between; and gt_timer_start / gt_timer_stop bracket queued work."""
+    lib, hb = mod("lib"), mod("hip_backend")
+    L = lib.lib
+    other = hb.HipBackend(0, streams=1)
+    try:
+        a, b = gpu.ctx, other.ctx
+        n = 1 << 24
+        x = gpu.create_state_buffer(n * 4)
+        y = other.create_state_buffer(n * 4)
+        gpu.write_state_buffer(x, np.full(n, 1.0, np.float32))
+        lib.check(a, L.gt_sync(a), "sync")
+        ms = C.c_double(-1)
+        lib.check(a, L.gt_timer_start(a), "timer")
+        for _ in range(200):                      # a long chain on the first stream: x *= 1.01, 200 times
+            lib.check(a, L.gt_scale_fwd(a, n, x, 1.01, x), "scale")
+        lib.check(a, L.gt_stream_mark(a), "mark")
+        lib.check(b, L.gt_stream_wait(b, a), "wait")
+        lib.check(b, L.gt_scale_fwd(b, n, x, 1.0, y), "copy")          # reads x on the second stream: must see all 200 updates
+        got = other.read_state_buffer(y, n)
+        lib.check(a, L.gt_timer_stop(a, C.byref(ms)), "timer")
+        want = np.float32(1.0)
+        for _ in range(200):
+            want = np.float32(want * np.float32(1.01))
+        assert np.all(got == want), (got[:4], want)
+        assert ms.value > 0.5                                          # 200 passes over 64 MB took measurable time
+        rc = L.gt_stream_wait(b, None)
+        assert rc != 0 and "other context" in L.gt_last_error(b).decode()
+        rc = L.gt_timer_stop(b, C.byref(ms))
+        assert rc != 0 and "gt_timer_start" in L.gt_last_error(b).decode()
+    finally:
+        other.destroy()
+    gpu.sync([])
