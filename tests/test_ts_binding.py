@@ -113,3 +113,63 @@ def test_backend_class_has_the_reference_surface():
     for a, b in ("()", "[]", "{}"):
         stripped = re.sub(r"//[^\n]*|`[^`]*`|\"[^\"\n]*\"", "", src)
         assert stripped.count(a) == stripped.count(b), (a, stripped.count(a), stripped.count(b))
+
+
+def _calls(src: str):
+    """(name, [argument texts]) of every direct call `….gt_name(…)` in the TypeScript source, arguments split at top-level commas."""
+    src = re.sub(r"//[^\n]*", "", src)
+    out = []
+    for m in re.finditer(r"\.(gt_[a-z0-9_]+)\(", src):
+        i, depth, args, cur, quote = m.end(), 1, [], "", None
+        while depth:
+            ch = src[i]
+            if quote:
+                cur += ch
+                if ch == quote and src[i - 1] != "\\":
+                    quote = None
+            elif ch in "\"'`":
+                quote = ch
+                cur += ch
+            elif ch in "([{":
+                depth += 1
+                cur += ch
+            elif ch in ")]}":
+                depth -= 1
+                if depth:
+                    cur += ch
+            elif ch == "," and depth == 1:
+                args.append(cur.strip())
+                cur = ""
+            else:
+                cur += ch
+            i += 1
+        if cur.strip():
+            args.append(cur.strip())
+        out.append((m.group(1), args))
+    return out
+
+
+def test_every_call_in_the_binding_passes_what_the_header_declares():
+    """Deno.dlopen checks nothing until a call is made, and the binding cannot be run here: every direct call of a library
+    symbol in hip.ts must pass exactly as many arguments as the header's prototype has parameters, no BigInt where the
+    parameter is a 32-bit integer or a float, and no float literal or array where it is an integer."""
+    protos = header_prototypes()
+    calls = _calls(open(TS).read())
+    assert len(calls) >= 70
+    seen = set()
+    for name, args in calls:
+        ret, params = protos[name]
+        assert len(args) == len(params), f"{name}: called with {len(args)} arguments {args}, the header declares {len(params)}"
+        seen.add(name)
+        for a, p in zip(args, params):
+            want = ffi_type(p)
+            if want in ("i32", "f32", "f64"):
+                assert not re.fullmatch(r"\d+n", a) and not a.startswith("BigInt("), f"{name}: BigInt {a!r} for {p}"
+            if want in ("i32", "i64", "u64", "usize"):
+                assert not re.fullmatch(r"\d+\.\d+", a) and not a.startswith("["), f"{name}: {a!r} for {p}"
+            if want == "pointer":
+                assert re.fullmatch(r"null|(\w+\.)*(ctx|context|handle)", a), f"{name}: {a!r} where the handle {p} goes"
+    # the binding exercises the whole path: every op's forward and backward entry point, the optimizers, the buffer calls
+    for must in ("gt_gemm", "gt_rmsnorm_fwd", "gt_rmsnorm_bwd", "gt_rope", "gt_attn_fwd_scores", "gt_attn_bwd_scores", "gt_ce_fwd", "gt_ce_bwd",
+                 "gt_embedding_fwd", "gt_embedding_bwd", "gt_glu_fwd", "gt_glu_bwd", "gt_adamw_step", "gt_muon_step", "gt_sync", "gt_h2d", "gt_d2h"):
+        assert must in seen, must
