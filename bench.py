@@ -209,8 +209,8 @@ def micro_kernels(gpu, L, reps=10, sustained=30):
     backward on [16384x1536]. Rates are algorithmic work (FLOP, or bytes each tensor is touched once) over time.
     Two figures per GEMM: `frac` is a single launch between other kernels (each round puts the 6.4 GB cross-entropy
     pass and four streaming kernels between two launches of the same product: cold caches, clocks and power ramping up
-    from memory-bound work), `sustained_frac` is `sustained` launches back to back inside one pair of events, which is
-    how the products run inside a training step."""
+    from memory-bound work), `sustained_frac` is `sustained` launches back to back inside one pair of events once the
+    clocks have settled on matrix work (see sustained_rate)."""
     import ctypes as C
     rs = np.random.RandomState(7)
     R, H, F, V = 16384, 576, 1536, 49152
@@ -262,9 +262,13 @@ def micro_kernels(gpu, L, reps=10, sustained=30):
         run()
     prof = gpu.stop_profile()
 
+    SETTLE = 150
+
     def sustained_rate(fn, flop):
-        """`sustained` launches of one product back to back inside one event pair, after a few untimed ones"""
-        for _ in range(5):
+        """`sustained` launches of one product back to back inside one event pair, after SETTLE untimed ones: coming from
+        memory-bound kernels the chip's clocks take about 25 ms of matrix work to settle (this product: 112-114 TFLOP/s over
+        its first ten launches, 130 from the 110th on, by event pairs around consecutive groups of ten)"""
+        for _ in range(SETTLE):
             fn()
         ms = C.c_double()
         L.check(c, lib.gt_timer_start(c), "gt_timer_start")
@@ -318,7 +322,8 @@ def micro_kernels(gpu, L, reps=10, sustained=30):
             out[desc]["sustained_us_per_launch"] = round(1e3 * sus[key][0], 1)
             out[desc]["sustained_achieved"] = round(sus[key][1] / 1e12, 3)
             out[desc]["sustained_frac"] = round(sus[key][1] / PEAK_FP32_MFMA, 4)
-            out[desc]["sustained"] = f"{sustained} launches back to back inside one event pair (the reduction pass of a split-K product included)"
+            out[desc]["sustained"] = (f"{sustained} launches back to back inside one event pair, after {SETTLE} untimed ones that let the clocks settle "
+                                      f"(the reduction pass of a split-K product included)")
     for key, desc in (("rmsnorm.bwd", "RMSNorm backward [131072x576] (8x the rows, 10 launches back to back)"),
                       ("add", "yardstick out = a + b [131072x576] (8x the rows, 10 launches back to back)")):
         rate = 12.0 * R8 * H / (big[key] * 1e-3)
