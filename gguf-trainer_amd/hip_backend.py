@@ -157,6 +157,7 @@ class HipBackend:
         self.forward_only_region = False  # set by checkpoint() around a block's first forward, whose interior is never differentiated
         self._profiling = False
         self._destroyed = False
+        self._explicit_micro_batches = False     # set by next_micro_batch(): boundaries are told, not inferred
 
     # ---- streams ------------------------------------------------------------------------------------------------
     @property
@@ -166,12 +167,25 @@ class HipBackend:
     def _op_begin(self, *inputs):
         """Called first thing by every forward op. After a backward has run, an op whose inputs are all parameters or
         host data is the root of the next micro-batch's graph: it goes to the next stream."""
-        if not self._bw_seen or self._nstreams == 1 or self.backward_depth:
+        if not self._bw_seen or self._nstreams == 1 or self.backward_depth or self._explicit_micro_batches:
             return                  # (a forward op inside a backward is a checkpoint replaying its block: same micro-batch)
         for t in inputs:
             e = self._entries.get(t)
             if e is not None and not e.external:
                 return
+        self._advance_stream()
+
+    def next_micro_batch(self):
+        """The trainer says where a micro-batch's graph begins: call it at the top of the loop body that builds one
+        sequence's forward and backward (train-gpu.ts:200-219). From the first call on the backend stops inferring the
+        boundary from the ops' inputs (see _op_begin: that inference holds for graphs whose first op takes only parameters
+        and host data, like the three in arch.py, and for nothing else). A call before any backward has run since the last
+        boundary changes nothing, so the first micro-batch of a step stays on the first stream."""
+        self._explicit_micro_batches = True
+        if self._bw_seen and self._nstreams > 1 and not self.backward_depth:
+            self._advance_stream()
+
+    def _advance_stream(self):
         self._flush()
         self._flush_dx()
         self._cur = (self._cur + 1) % self._nstreams

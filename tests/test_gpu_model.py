@@ -804,6 +804,78 @@ def test_micro_batches_on_several_streams(gpu, ref):
         assert_close(g1[n], gs[n], f"four streams vs one, {n}", rel_l2=2e-6, max_rel=2e-5)
 
 
+def test_micro_batch_boundaries_told_by_the_trainer(ref):
+    """next_micro_batch(): the trainer marks where a sequence's graph begins instead of the backend inferring it from the
+    first op's inputs. On the llama graph (where the inference holds) both give the same streams and the same bits; a
+    graph whose every forward op reads an intermediate made before the loop (which the inference takes for the
+    continuation of the previous micro-batch) is dealt to the streams only when told. Gradients against one stream."""
+    hb, ag = mod("hip_backend"), mod("autograd")
+    kw = REAL["smollm2"]
+    seqs = batches(ref, kw["vocab"], 150, 5, seed=41, mask_every=7)
+
+    def run(explicit, streams=4):
+        be = hb.HipBackend(0, streams=streams)
+        arch = mod("arch")
+        try:
+            _, model = build_pair(ref, kw, seed=40, std=0.05)
+            be.install()
+            seen, losses = [], []
+            for ids, tg in seqs:
+                if explicit:
+                    be.next_micro_batch()
+                loss = arch.sequence_loss(model, ids, tg, 0)
+                seen.append(be._cur)
+                ag.backward(loss, 1.0 / len(seqs))
+                losses.append(loss)
+            be.sync(losses)
+            be.uninstall()
+            return seen, np.concatenate([l.data for l in losses]), {n: p.grad.copy() for n, p in model.named_params()}
+        finally:
+            be.destroy()
+
+    s_inf, l_inf, g_inf = run(False)
+    s_exp, l_exp, g_exp = run(True)
+    assert s_inf == s_exp == [0, 1, 2, 3, 0]
+    assert l_inf.tobytes() == l_exp.tobytes() and all(g_inf[n].tobytes() == g_exp[n].tobytes() for n in g_inf)
+
+    # a graph the inference does not cut: every micro-batch starts from one shared, gradient-free feature h0 = x W0^T
+    # computed once (W0 frozen), which the inference takes for the continuation of the graph before it
+    r = ref.Mulberry32(43)
+    xs = r.fill_randn([64, 32], 1.0)
+    w0d, w1d = r.fill_randn([32, 32], 0.3), r.fill_randn([48, 32], 0.3)
+    scales = [0.5, 1.5, -1.0, 2.0]
+
+    def shared_root(explicit, streams):
+        be = hb.HipBackend(0, streams=streams)
+        try:
+            x = ag.Tensor(xs, [64, 32])
+            w0, w1 = ag.Tensor(w0d, [32, 32], False), ag.Tensor(w1d, [48, 32], True)
+            be.install()
+            h0 = ag.linear(x, w0)
+            seen, outs = [], []
+            for c in scales:
+                if explicit:
+                    be.next_micro_batch()
+                y = ag.linear(ag.silu(ag.scale(h0, c)), w1)
+                seen.append(be._cur)
+                ag.backward(y, 0.25)          # seeds dy = 0.25 everywhere
+                outs.append(y)
+            be.sync(outs)
+            be.uninstall()
+            return seen, w1.grad.copy(), [o.data.copy() for o in outs]
+        finally:
+            be.destroy()
+
+    s1, a1, ya = shared_root(False, 4)
+    s2, b1, yb = shared_root(True, 4)
+    s3, c1, yc = shared_root(True, 1)
+    assert s1 == [0, 0, 0, 0], s1                      # inferred: all one micro-batch, one stream
+    assert s2 == [0, 1, 2, 3] and s3 == [0, 0, 0, 0]
+    assert all(u.tobytes() == v.tobytes() == w.tobytes() for u, v, w in zip(ya, yb, yc))
+    assert a1.tobytes() == c1.tobytes()
+    assert_close(b1, c1, "told boundaries on four streams vs one stream, dW1", rel_l2=2e-6, max_rel=2e-5)
+
+
 def test_grad_fold_sums_in_source_order(gpu):
     """gt_grad_fold: dst (+)= src0 + src1 + ... per tensor in one launch, bit for bit the f32 sums taken in that order;
     absent sources skipped, store and accumulate, sizes that are no multiple of four and an unaligned tensor."""
