@@ -307,7 +307,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP
   IO::offsets(koffs, kstr, tid);
   auto load_tile = [&](const float *base, int kt) {
     kt = min(kt, kt_hi);
-    IO::load(pt, base + (size_t)kt * KT * kstr, koffs, (unsigned)kstr, p.T - kt * KT, tid);
+    IO::load(pt, base + (size_t)kt * KT * kstr, koffs, (unsigned)kstr, KEEP ? KT : p.T - kt * KT, tid);      // (kept scores: T is a multiple of 128, no tile is short: no clamp arithmetic; 3 % at head dim 128)
   };
   if (kt_lo <= kt_hi) {
     load_tile(kb, kt_lo);
@@ -618,15 +618,18 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   IO::offsets(qoffs, qstr, tid);
   // Stage indices past the end are clamped to the last stage: its tile is loaded, and written to the idle buffer, again,
   // which nobody reads; the loop body has no test for "is there a next stage".
+  // With kept scores T is a multiple of 128 and no tile is short: telling the loads so takes their clamp arithmetic out of the
+  // stage (measured: 1 % at head dim 128, where the kernel is short of registers; nothing at 64, where it stays as it was).
+  constexpr bool WHOLE = KS && HD >= 128;
   auto load_q = [&](int it) {
     const int qt = qt_lo + min(it, niter - 1);
-    IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
+    IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, WHOLE ? QT : p.T - qt * QT, tid);
   };
   auto load_g = [&](int it) {          // dO and the row statistics
     const int qt = qt_lo + min(it, niter - 1);
     if constexpr (ONE_SET) IO::load(pq, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
-    else IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
-    pstat = statp[min(qt * QT + (tid % QT), p.T - 1)];
+    else IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, WHOLE ? QT : p.T - qt * QT, tid);
+    pstat = statp[WHOLE ? qt * QT + (tid % QT) : min(qt * QT + (tid % QT), p.T - 1)];
   };
   auto load_scores = [&](int it) {          // blocks the forward has not written hold anything: their stage is skipped
     const int qt = qt_lo + min(it, niter - 1);
