@@ -15,6 +15,7 @@
 // Both kernels read every element of the large operand exactly once, straight from global memory into MFMA operand
 // registers (no LDS staging), several loads ahead. Sums over wavefronts and over row slices have a fixed order.
 #include <algorithm>
+#include <cstring>
 #include "common.h"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -158,6 +159,33 @@ __global__ __launch_bounds__(256) void rank_slices_sum(const float *__restrict__
   p[i] = accp ? p[i] + s : s;
 }
 
+// The slice sums of several rank gradients as one launch (the adapter gradients of a whole backward pass are not read
+// before the optimizer, so their sums can wait and go out together): workgroup -> (entry, block of 256 elements) through
+// the table in the kernel arguments, then rank_slices_sum's arithmetic, so every gradient has the bits its own launch gives.
+#define RSG_MAX 96
+struct RsEntry { const float *part; float *p; int slices, n, acc, blk0; };
+struct RsGroup { RsEntry e[RSG_MAX]; int n; };
+__global__ __launch_bounds__(256) void rank_slices_group_k(RsGroup G) {
+  int i = 0;
+  for (int q = 1; q < G.n; q++) if ((int)blockIdx.x >= G.e[q].blk0) i = q;
+  const RsEntry &e = G.e[i];
+  const int k = ((int)blockIdx.x - e.blk0) * 256 + threadIdx.x;
+  if (k >= e.n) return;
+  float s = e.part[k];
+  for (int z = 1; z < e.slices; z++) s += e.part[(size_t)z * e.n + k];
+  e.p[k] = e.acc ? e.p[k] + s : s;
+}
+
+// how the streaming rank-gradient kernel cuts `rows`: slices of rows_per_slice rows (a whole number of workgroup passes)
+static int rank_grad_cut(gt_ctx *ctx, int rows, int K, int *rows_per_slice) {
+  const int colblocks = K / RG_COLS;
+  const int pass = 16 * RG_WAVES * 2;
+  int slices = (int)std::max<int64_t>(1, std::min<int64_t>(cdiv(3 * ctx->num_cu, colblocks), cdiv(rows, pass)));
+  *rows_per_slice = (int)(cdiv(cdiv(rows, slices), pass) * pass);
+  return (int)cdiv(rows, *rows_per_slice);
+}
+static bool rank_grad_streams(int K, int r, gt_buf y) { return !(r > 32 || K % RG_COLS != 0 || y % 16 != 0); }
+
 extern "C" {
 
 int gt_rank_down(gt_ctx *ctx, int rows, int K, int r, gt_buf x, gt_buf s, int s_kmajor, float alpha, gt_buf h) {
@@ -181,16 +209,14 @@ int gt_rank_down(gt_ctx *ctx, int rows, int K, int r, gt_buf x, gt_buf s, int s_
 int gt_rank_grad(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int transpose_out, int acc, gt_buf p) {
   GT_ENTER(ctx);
   GT_REQUIRE(ctx, rows >= 1 && K >= 1 && r >= 1 && h && y && p, "gt_rank_grad: bad arguments (rows %d, K %d, r %d)", rows, K, r);
-  if (r > 32 || K % RG_COLS != 0 || y % 16 != 0) {
+  if (!rank_grad_streams(K, r, y)) {
     return transpose_out ? gt_gemm(ctx, GT_TN, acc, K, r, rows, y, h, p) : gt_gemm(ctx, GT_TN, acc, r, K, rows, h, y, p);
   }
   ProfScope ps(ctx, "rank.grad", 4.0 * ((double)rows * K + (double)rows * r));
   // enough row slices to give every CU a few workgroups; a slice is a whole number of passes of the workgroup
   const int colblocks = K / RG_COLS;
-  const int pass = 16 * RG_WAVES * 2;
-  int slices = (int)std::max<int64_t>(1, std::min<int64_t>(cdiv(3 * ctx->num_cu, colblocks), cdiv(rows, pass)));
-  const int rows_per_slice = (int)(cdiv(cdiv(rows, slices), pass) * pass);
-  slices = (int)cdiv(rows, rows_per_slice);
+  int rows_per_slice;
+  const int slices = rank_grad_cut(ctx, rows, K, &rows_per_slice);
   float *part = nullptr;
   if (slices > 1) {
     void *ws;
@@ -206,6 +232,54 @@ int gt_rank_grad(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int tr
   if (part) {
     const int n = r * K;
     hipLaunchKernelGGL(rank_slices_sum, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, ctx->stream, part, slices, n, P<float>(p), acc);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
+}
+
+int gt_rank_grad_slices(gt_ctx *ctx, int rows, int K, int r, gt_buf y, int *slices) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 1 && K >= 1 && r >= 1 && slices, "gt_rank_grad_slices: bad arguments (rows %d, K %d, r %d)", rows, K, r);
+  int rps;
+  const int n = rank_grad_streams(K, r, y) ? rank_grad_cut(ctx, rows, K, &rps) : 0;
+  *slices = n > 1 ? n : 0;          // one slice is written straight to its destination: nothing to hold back
+  return 0;
+}
+
+int gt_rank_grad_parts(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int transpose_out, gt_buf parts) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, rows >= 1 && K >= 1 && r >= 1 && h && y && parts, "gt_rank_grad_parts: bad arguments (rows %d, K %d, r %d)", rows, K, r);
+  GT_REQUIRE(ctx, rank_grad_streams(K, r, y), "gt_rank_grad_parts: this shape does not take the streaming kernel (ask gt_rank_grad_slices first)");
+  int rows_per_slice;
+  const int slices = rank_grad_cut(ctx, rows, K, &rows_per_slice);
+  GT_REQUIRE(ctx, slices > 1, "gt_rank_grad_parts: a single slice has no partial sums (ask gt_rank_grad_slices first)");
+  ProfScope ps(ctx, "rank.grad", 4.0 * ((double)rows * K + (double)rows * r));
+  dim3 grid((unsigned)(K / RG_COLS), (unsigned)slices), block(RG_WAVES * 64);
+#define GO(NR, TR) hipLaunchKernelGGL((rank_grad_k<NR, TR>), grid, block, 0, ctx->stream, rows, K, r, rows_per_slice, P<const float>(h), P<const float>(y), (float *)nullptr, 0, P<float>(parts))
+  if (r <= 16) { if (transpose_out) GO(1, true); else GO(1, false); }
+  else { if (transpose_out) GO(2, true); else GO(2, false); }
+#undef GO
+  GT_LAUNCHED(ctx);
+  return 0;
+}
+
+int gt_rank_slices_group(gt_ctx *ctx, int n, const gt_buf *parts, const int *slices, const int *len, const gt_buf *p, const int *acc) {
+  GT_ENTER(ctx);
+  GT_REQUIRE(ctx, n >= 0 && (n == 0 || (parts && slices && len && p && acc)), "gt_rank_slices_group: %d entries or a null table", n);
+  for (int i0 = 0; i0 < n; i0 += RSG_MAX) {
+    RsGroup G;
+    memset(&G, 0, sizeof G);
+    G.n = std::min(RSG_MAX, n - i0);
+    int blocks = 0;
+    for (int q = 0; q < G.n; q++) {
+      const int i = i0 + q;
+      GT_REQUIRE(ctx, parts[i] && p[i] && slices[i] >= 1 && len[i] >= 1, "gt_rank_slices_group: entry %d is malformed", i);
+      for (int j = i0; j < i; j++) GT_REQUIRE(ctx, p[j] != p[i], "gt_rank_slices_group: entries %d and %d write the same gradient", j, i);
+      G.e[q] = {P<const float>(parts[i]), P<float>(p[i]), slices[i], len[i], acc[i], blocks};
+      blocks += (int)cdiv(len[i], 256);
+    }
+    ProfScope ps(ctx, "rank.slices");
+    hipLaunchKernelGGL(rank_slices_group_k, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, G);
     GT_LAUNCHED(ctx);
   }
   return 0;

@@ -136,6 +136,9 @@ class HipBackend:
         self._pend_cs: list = []
         self._pend_cs_ids: set = set()
         self.defer_norm_dw = True
+        self._pend_rs: list = []          # held-back slice sums of adapter gradients: (parts, slices, len, destination, acc)
+        self._pend_rs_ids: set = set()
+        self.defer_rank_sums = True
         # attention's backward applies the backward of the rotations its q and k came through in the write-backs of dQ and
         # dK (gt_attn_bwd_scores_rope) where q / k are rotation outputs nobody else has read: no rope.bwd launch is left
         self.fuse_rope_bwd = True
@@ -312,6 +315,32 @@ class HipBackend:
                                              (C.c_int * n)(*[p[2] for p in pend]), (c_buf * n)(*[p[3] for p in pend]),
                                              (C.c_int * n)(*[p[4] for p in pend])), "rmsnorm.dw")
 
+    def _flush_rs(self):
+        """The slice sums of every held-back adapter gradient, one launch."""
+        pend = self._pend_rs
+        if not pend:
+            return
+        self._pend_rs = []
+        self._pend_rs_ids = set()
+        n = len(pend)
+        check(self._ctx, lib.gt_rank_slices_group(self._ctx, n, (c_buf * n)(*[p[0] for p in pend]), (C.c_int * n)(*[p[1] for p in pend]),
+                                                  (C.c_int * n)(*[p[2] for p in pend]), (c_buf * n)(*[p[3] for p in pend]),
+                                                  (C.c_int * n)(*[p[4] for p in pend])), "lora.slices")
+
+    def _rank_grad(self, param, rows, K, r, h, y, transpose_out, acc, dst, label):
+        """dst (+)= the rank-r gradient product; its slice sums are held back for one grouped launch when the library
+        would go through partial sums and nobody can be reading the gradient before the backward ends."""
+        if self.defer_rank_sums:
+            ns = C.c_int(0)
+            check(self._ctx, lib.gt_rank_grad_slices(self._ctx, rows, K, r, y, C.byref(ns)), label)
+            if ns.value > 0:
+                parts = self._scratch_buf(ns.value * r * K * 4)
+                check(self._ctx, lib.gt_rank_grad_parts(self._ctx, rows, K, r, h, y, transpose_out, parts), label)
+                self._pend_rs.append((parts, ns.value, r * K, dst, acc))
+                self._pend_rs_ids.add(id(param))
+                return
+        check(self._ctx, lib.gt_rank_grad(self._ctx, rows, K, r, h, y, transpose_out, acc, dst), label)
+
     def _flush_dx(self, t: Tensor = None):
         """Launch the held-back input-gradient products: those into t's gradient, or all of them (then the held-back
         weight-gradient products and column sums go too)."""
@@ -319,6 +348,8 @@ class HipBackend:
             self._flush_dw()
         if t is None and self._pend_cs:
             self._flush_cs()
+        if t is None and self._pend_rs:
+            self._flush_rs()
         if not self._pend_dx:
             return
         if t is None:
@@ -487,6 +518,8 @@ class HipBackend:
             self._flush_dw()
         if self._pend_cs and id(t) in self._pend_cs_ids:
             self._flush_cs()
+        if self._pend_rs and id(t) in self._pend_rs_ids:
+            self._flush_rs()
         e = self._entries.get(t)
         if e is None:
             e = self._entry_for(t)
@@ -560,6 +593,8 @@ class HipBackend:
             self._flush_dw()
         if self._pend_cs and id(t) in self._pend_cs_ids:
             self._flush_cs()
+        if self._pend_rs and id(t) in self._pend_rs_ids:
+            self._flush_rs()
         e = self._entries.get(t)
         if e is None:
             raise RuntimeError("backward over a graph built before a sync(): that sync recycled the graph's "
@@ -793,6 +828,7 @@ class HipBackend:
         self._pend_dx = {}
         self._pend_dw = []
         self._pend_cs = []
+        self._pend_rs = []
         if not self._destroyed:
             self._destroyed = True
             for c in self._ctxs:
@@ -927,14 +963,14 @@ class HipBackend:
             if wants_db:
                 db, accb = self._gdst(b)
                 if db:
-                    check(self._ctx, lib.gt_rank_grad(self._ctx, T, outd, r, hs, g, 1, accb, db), "lora.db")
+                    self._rank_grad(b, T, outd, r, hs, g, 1, accb, db, "lora.db")
             if dx or wants_da:
                 dh = self._scratch_buf(T * r * 4)
                 check(self._ctx, lib.gt_rank_down(self._ctx, T, outd, r, g, bd, 1, sc, dh), "lora.dh")
                 if wants_da:
                     da, acca = self._gdst(a)
                     if da:
-                        check(self._ctx, lib.gt_rank_grad(self._ctx, T, ind, r, dh, xd, 0, acca, da), "lora.da")
+                        self._rank_grad(a, T, ind, r, dh, xd, 0, acca, da, "lora.da")
                 if dx:      # dX (+)= dY.W + dH.A in one K loop
                     check(self._ctx, lib.gt_gemm_pair(self._ctx, NN, acc, T, ind, outd, g, wd, r, dh, ad, dx), "lora.dx")
 

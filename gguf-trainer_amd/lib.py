@@ -48,6 +48,9 @@ _SIG = {
     "gt_gemm_batched": [ctxp, i32, i32, i32, i32, i32, buf, i64, buf, i64, buf, i64, i32],
     "gt_rank_down": [ctxp, i32, i32, i32, buf, buf, i32, f32, buf],
     "gt_rank_grad": [ctxp, i32, i32, i32, buf, buf, i32, i32, buf],
+    "gt_rank_grad_slices": [ctxp, i32, i32, i32, buf, C.POINTER(i32)],
+    "gt_rank_grad_parts": [ctxp, i32, i32, i32, buf, buf, i32, buf],
+    "gt_rank_slices_group": [ctxp, i32, C.POINTER(buf), C.POINTER(i32), C.POINTER(i32), C.POINTER(buf), C.POINTER(i32)],
     "gt_add_fwd": [ctxp, i64, buf, buf, buf],
     "gt_mul_fwd": [ctxp, i64, buf, buf, buf],
     "gt_silu_fwd": [ctxp, i64, buf, buf],

@@ -50,6 +50,9 @@ const SYMBOLS = {
   gt_gemm_pair:          { parameters: [ptr, i32, i32, i32, i32, i32, u64, u64, i32, u64, u64, u64], result: i32 },
   gt_rank_down:          { parameters: [ptr, i32, i32, i32, u64, u64, i32, f32, u64], result: i32 },
   gt_rank_grad:          { parameters: [ptr, i32, i32, i32, u64, u64, i32, i32, u64], result: i32 },
+  gt_rank_grad_slices:   { parameters: [ptr, i32, i32, i32, u64, buf], result: i32 },
+  gt_rank_grad_parts:    { parameters: [ptr, i32, i32, i32, u64, u64, i32, u64], result: i32 },
+  gt_rank_slices_group:  { parameters: [ptr, i32, buf, buf, buf, buf, buf], result: i32 },
   gt_gemm_add:           { parameters: [ptr, i32, i32, i32, i32, u64, u64, u64, u64], result: i32 },
   gt_gemm_sum:           { parameters: [ptr, i32, i32, i32, i32, i32, buf, buf, buf, u64], result: i32 },
   gt_gemm_group:         { parameters: [ptr, i32, i32, buf, buf, i32, buf, buf, buf, buf], result: i32 },

@@ -108,6 +108,18 @@ int gt_gemm_pair(gt_ctx *ctx, int kind, int acc, int M, int N, int K1, gt_buf A1
  * kernels, everything else the general GEMM. */
 int gt_rank_down(gt_ctx *ctx, int rows, int K, int r, gt_buf x, gt_buf s, int s_kmajor, float alpha, gt_buf h);
 int gt_rank_grad(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int transpose_out, int acc, gt_buf p);
+/* gt_rank_grad in two parts, for a host that holds the sums back: an adapter's gradient is not read before the optimizer
+ * (src/backend/adamw-gpu.ts:131-251), so the partial sums of a whole backward pass can be added up by ONE launch instead
+ * of one small launch per adapter matrix (the reference has no counterpart: its rank-r products are ordinary GEMMs).
+ *   gt_rank_grad_slices:  how many row slices gt_rank_grad would cut this product into; 0 when it would not go through
+ *                         partial sums at all (one slice, or a shape that takes the general GEMM): call gt_rank_grad then.
+ *   gt_rank_grad_parts:   the slices' partial products into parts[slices][r * K] (laid out as p), nothing summed.
+ *   gt_rank_slices_group: p_i (+)= parts_i[0] + parts_i[1] + ... for n gradients at once (host arrays of n entries, len_i =
+ *                         r * K elements each; distinct p_i), in slice order: the bits gt_rank_grad gives. */
+int gt_rank_grad_slices(gt_ctx *ctx, int rows, int K, int r, gt_buf y, int *slices);
+int gt_rank_grad_parts(gt_ctx *ctx, int rows, int K, int r, gt_buf h, gt_buf y, int transpose_out, gt_buf parts);
+int gt_rank_slices_group(gt_ctx *ctx, int n, const gt_buf *parts, const int *slices, const int *len, const gt_buf *p,
+                         const int *acc);
 /* C = D + A.B with D a matrix laid out as C (it may be C itself): a linear whose output is at once added to the residual
  * stream, add(h, linear(x, W)) in the reference's layer bodies (src/arch/llama.ts:131-222), as one launch
  * with no [rows, out] round trip for the product. */

@@ -208,6 +208,71 @@ def test_lora(gpu, ref, recompute):
         assert gpu._entries[p].grad == 0
 
 
+def test_lora_adapter_gradient_sums_held_back(gpu, ref):
+    """Sequences long enough for the rank-r gradient products to go through row slices (300 tokens): the host holds the
+    slice sums of a backward pass back and adds them up in grouped launches. Same bits as summing each at once, parity
+    with the oracle, stacked and one sequence at a time (where the sums go out before the stream changes)."""
+    ag, arch = mod("autograd"), mod("arch")
+    kw = SMALL["qwen3"]
+    rank, alpha = 4, 8.0
+
+    def build():
+        rmodel, model = build_pair(ref, kw, seed=5, std=0.1)
+        rmap, rparams = ref.attach_lora(rmodel, rank, alpha, ref.Mulberry32(11), a_std=0.1)
+        rng = ref.Mulberry32(12)
+        for a, b, _ in rmap.values():
+            b.data[:] = rng.fill_randn([b.size], 0.1)
+        adapters = {}
+        for l, L in enumerate(rmodel.layers):
+            for k in ref.MATRIX_KEYS:
+                a, b, _ = rmap[id(L[k])]
+                adapters[f"L{l}.{k}"] = (a.data.copy(), b.data.copy())
+        return rmodel, model, rmap, rparams, arch.apply_lora(model, rank, alpha, adapters)
+
+    seqs = batches(ref, kw["vocab"], 300, 3, seed=9, mask_every=4)
+    rmodel, model, rmap, rparams, aux = build()
+    ref.set_lora_adapters(rmap)
+    try:
+        lr, _ = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.set_lora_adapters({})
+    want = [r.grad.copy() for r in rparams]
+    held = []
+    flush = gpu._flush_rs
+
+    def counting_flush():
+        if gpu._pend_rs:
+            held.append(len(gpu._pend_rs))
+        flush()
+
+    gpu._flush_rs = counting_flush
+    got = {}
+    try:
+        for stacked in (True, False):
+            for defer in (True, False):
+                _, model, _, _, aux = build()
+                gpu.defer_rank_sums = defer
+                held.clear()
+                try:
+                    lh, _ = hip_step(gpu, model, seqs, stacked, 300)
+                finally:
+                    arch.clear_lora(model)
+                assert (len(held) > 0) == defer, (stacked, defer, held)
+                if defer:
+                    assert sum(held) >= 2 * (1 if stacked else len(seqs)), held      # (the products whose K the streaming kernel takes)
+                got[(stacked, defer)] = [h.grad.copy() for h in aux]
+                if not stacked:
+                    assert np.all(np.abs(lh - lr) <= LOSS_REL * np.abs(lr))
+                for i, (h, w) in enumerate(zip(aux, want)):
+                    assert_close(h.grad, w, f"lora adapter {i}, stacked {stacked}, held back {defer}")
+    finally:
+        gpu.defer_rank_sums = True
+        gpu._flush_rs = flush
+    for stacked in (True, False):
+        for a, b in zip(got[(stacked, True)], got[(stacked, False)]):
+            assert a.tobytes() == b.tobytes(), f"held-back sums change bits (stacked {stacked})"
+
+
 def test_config1_tiny_llama_step(gpu, ref):
     """benchmark config 1: vocab 512, hidden 128, 2 layers, 4/2 heads x 32, SwiGLU 352, tied, weights N(0,0.02) seed 0,
     4 sequences of 128 tokens, targets shifted by one; forward + backward + AdamW(lr 1e-3, betas 0.9/0.95, wd 0.1)."""

@@ -180,6 +180,53 @@ def test_rank_products(gpu, rows, K, r):
     assert rc != 0 and b"gt_rank_down" in L.lib.gt_last_error(gpu.ctx)
 
 
+def test_held_back_rank_gradient_sums_equal_the_direct_ones(gpu):
+    """gt_rank_grad_slices / gt_rank_grad_parts / gt_rank_slices_group: the partial products of several adapter gradients
+    summed by one launch give, bit for bit, what gt_rank_grad gives each of them (both orientations, store and accumulate,
+    different shapes in one group); shapes that do not go through partial sums report zero slices; malformed groups fail."""
+    import ctypes as C
+    L = mod("lib")
+    lib, c = L.lib, gpu.ctx
+    rs = np.random.RandomState(5)
+    cases = [(2100, 576, 16, 0, 0), (2100, 576, 16, 1, 1), (4096, 1024, 16, 1, 0), (3000, 192, 8, 0, 1), (2500, 320, 20, 0, 0)]
+    parts, nsl, lens, dsts, accs, wants = [], [], [], [], [], []
+    for rows, K, r, tr, acc in cases:
+        h = rs.standard_normal((rows, r)).astype(np.float32)
+        y = rs.standard_normal((rows, K)).astype(np.float32)
+        p0 = rs.standard_normal(r * K).astype(np.float32)
+        bh, by, bd, bw = (gpu.create_state_buffer(a.nbytes) for a in (h, y, p0, p0))
+        gpu.write_state_buffer(bh, h)
+        gpu.write_state_buffer(by, y)
+        gpu.write_state_buffer(bd, p0)
+        gpu.write_state_buffer(bw, p0)
+        L.check(c, lib.gt_rank_grad(c, rows, K, r, bh, by, tr, acc, bw), "gt_rank_grad")
+        wants.append(gpu.read_state_buffer(bw, r * K))
+        ns = C.c_int(-1)
+        L.check(c, lib.gt_rank_grad_slices(c, rows, K, r, by, C.byref(ns)), "gt_rank_grad_slices")
+        assert ns.value >= 2, (rows, K, r, ns.value)
+        bp = gpu.create_state_buffer(ns.value * r * K * 4)
+        L.check(c, lib.gt_rank_grad_parts(c, rows, K, r, bh, by, tr, bp), "gt_rank_grad_parts")
+        parts.append(bp); nsl.append(ns.value); lens.append(r * K); dsts.append(bd); accs.append(acc)
+    n = len(cases)
+    L.check(c, lib.gt_rank_slices_group(c, n, (L.buf * n)(*parts), (C.c_int * n)(*nsl), (C.c_int * n)(*lens), (L.buf * n)(*dsts),
+                                        (C.c_int * n)(*accs)), "gt_rank_slices_group")
+    for i, (rows, K, r, tr, acc) in enumerate(cases):
+        got = gpu.read_state_buffer(dsts[i], r * K)
+        assert got.tobytes() == wants[i].tobytes(), f"held-back sums differ from gt_rank_grad: {cases[i]}"
+    # nothing to hold back: one slice (few rows), or a shape that takes the general GEMM
+    for rows, K, r in ((64, 576, 16), (2100, 100, 16), (2100, 576, 40)):
+        ns = C.c_int(-1)
+        L.check(c, lib.gt_rank_grad_slices(c, rows, K, r, parts[0], C.byref(ns)), "gt_rank_grad_slices")
+        assert ns.value == 0, (rows, K, r, ns.value)
+    assert lib.gt_rank_grad_parts(c, 64, 576, 16, parts[0], parts[0], 0, parts[0]) != 0
+    assert b"single slice" in lib.gt_last_error(c)
+    two = (L.buf * 2)(dsts[0], dsts[0])
+    assert lib.gt_rank_slices_group(c, 2, (L.buf * 2)(parts[0], parts[1]), (C.c_int * 2)(nsl[0], nsl[1]), (C.c_int * 2)(lens[0], lens[1]),
+                                    two, (C.c_int * 2)(0, 0)) != 0
+    assert b"write the same gradient" in lib.gt_last_error(c)
+    L.check(c, lib.gt_rank_slices_group(c, 0, None, None, None, None, None), "empty group")
+
+
 @pytest.mark.parametrize("M,N,K1,K2", [(200, 152, 96, 16), (130, 100, 72, 5), (257, 193, 101, 33), (64, 64, 16, 16), (260, 196, 128, 8),
                                        (132, 100, 64, 32), (300, 576, 192, 24), (200, 152, 96, 40)])
 def test_gemm_pair(gpu, M, N, K1, K2):
