@@ -492,19 +492,20 @@ def run_workload(mods, config, steps, warmup, a, headline):
     return res
 
 
-def naive_host_leg(mods, a, nsteps=3):
+def naive_host_leg(mods, a, nsteps=3, streams=1):
     """What a literal shim over the C ABI gets: the reference's call pattern (one sequence per graph) on ONE stream with
     every host-side hold-back and fusion of HipBackend switched off, so that each autograd op issues its own gt_* call
     in tape order (separate k/v and gate/up products, one dX and one dW launch per linear, unfused residual adds and
     gated activations, separate q and k rotations, add's backward as a launch). Attention still keeps its scores:
-    that is a choice inside the attention entry points, not a host fusion."""
+    that is a choice inside the attention entry points, not a host fusion. streams > 1: the same literal calls with the
+    micro-batches dealt to that many library contexts (the one piece of the host scheduler that needs no knowledge of the graph)."""
     import torch
     ag, hb, arch, optim = mods
     wl = WORKLOADS[3]
     batch = wl["batch"]
     cfg = arch.ModelConfig(**wl["model"])
     model = arch.Model(cfg, synth_weights(arch, cfg))
-    gpu = hb.require_gpu("bench.py", streams=1)
+    gpu = hb.require_gpu("bench.py", streams=streams)
     gpu.batch_linears = gpu.fuse_sibling_dx = gpu.fuse_residual_add = gpu.alias_add_grads = False
     gpu.group_dw = gpu.pair_ropes = gpu.fuse_glu = False
     opt = optim.AdamWHip(gpu, model.params(), lr=1e-3, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0)
@@ -534,7 +535,7 @@ def naive_host_leg(mods, a, nsteps=3):
     finally:
         gpu.uninstall()
         gpu.destroy()
-    return {"graph": f"{batch} graphs of {SEQ} rows per step, one stream, one gt_* call per autograd op (no held-back, batched, grouped or fused launches)",
+    return {"graph": f"{batch} graphs of {SEQ} rows per step, {'one stream' if streams == 1 else f'{streams} streams'}, one gt_* call per autograd op (no held-back, batched, grouped or fused launches)",
             "steps": nsteps, "value": round(nsteps * batch * SEQ / w, 1), "unit": "tokens/s", "ms_per_step": round(1e3 * w / nsteps, 2)}
 
 
@@ -651,6 +652,9 @@ def main():
                 ent["muon_step"] = o["muon"]
             other[f"configs[{ci}]"] = ent
     naive = naive_host_leg(mods, a) if a.naive_host or (a.config == 3 and not a.no_call_pattern and not a.sequential) else None
+    if naive is not None:          # the same literal calls, micro-batches dealt to the backend's streams
+        n4 = naive_host_leg(mods, a, streams=a.streams)
+        naive["with_streams"] = {"streams": a.streams, "value": n4["value"], "unit": "tokens/s", "ms_per_step": n4["ms_per_step"]}
     out = {
         "metric": "train tokens/s (SmolLM2-135M shape, 2048x8); bwd GEMM % FP32 MFMA peak" if a.config == 3 else
                   "train tokens/s (" + wl["name"].split(":")[0] + ")",
