@@ -30,7 +30,7 @@ class Tensor:
     """autograd.ts:20-51. Host arrays are allocated on first touch: an intermediate that lives on
     the device only never pays for a host copy. They are authoritative only after backend.sync()."""
 
-    __slots__ = ("shape", "requires_grad", "_backward", "_prev", "seq", "_data", "_grad", "__weakref__")
+    __slots__ = ("shape", "requires_grad", "_backward", "_prev", "seq", "_data", "_grad", "_dev", "__weakref__")
 
     def __init__(self, data, shape, requires_grad=False):
         global _created
@@ -41,6 +41,7 @@ class Tensor:
                 raise ValueError(f"data length {data.size} != shape {self.shape}")
         self._data = data
         self._grad = None
+        self._dev = None                # a device backend's record for this tensor: (owner key, record)
         self.requires_grad = requires_grad
         self._backward = _noop
         self._prev = []

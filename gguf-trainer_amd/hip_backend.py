@@ -34,6 +34,7 @@ What differs from the reference, on purpose:
 from __future__ import annotations
 
 import ctypes as C
+import gc
 import math
 import weakref
 
@@ -44,6 +45,45 @@ from .autograd import Tensor
 from .lib import NN, NT, TN, HipError, ProfRec, buf as c_buf, check, lib
 
 _ALIGN = 256
+
+
+class _EntryMap:
+    """Tensor -> device record, the WeakMap<Tensor, Entry> of webgpu.ts:322. The record sits in the tensor's own `_dev` slot
+    (a plain attribute read where a WeakKeyDictionary costs a weak reference and a hash per look-up, tens of thousands per
+    step); it dies with the tensor. A tensor already claimed by another live backend falls back to a weak dictionary."""
+    __slots__ = ("_key", "_spill")
+
+    def __init__(self):
+        self._key = object()
+        self._spill = weakref.WeakKeyDictionary()
+
+    def get(self, t, default=None):
+        d = t._dev
+        if d is not None and d[0] is self._key:
+            return d[1]
+        if self._spill:
+            return self._spill.get(t, default)
+        return default
+
+    def __getitem__(self, t):
+        e = self.get(t)
+        if e is None:
+            raise KeyError(t)
+        return e
+
+    def __setitem__(self, t, e):
+        d = t._dev
+        if d is None or d[0] is self._key:
+            t._dev = (self._key, e)
+        else:
+            self._spill[t] = e
+
+    def pop(self, t, default=None):
+        d = t._dev
+        if d is not None and d[0] is self._key:
+            t._dev = None
+            return d[1]
+        return self._spill.pop(t, default)
 
 
 class _Entry:
@@ -107,7 +147,7 @@ class HipBackend:
         self._pools = [dict() for _ in range(self._nstreams)]     # per stream: size class -> free buffers
         self._pool_bytes = 0
         self._state_bytes = 0
-        self._entries: "weakref.WeakKeyDictionary[Tensor, _Entry]" = weakref.WeakKeyDictionary()
+        self._entries = _EntryMap()
         self._externals: "weakref.WeakSet[Tensor]" = weakref.WeakSet()
         self._touched: list = []
         self._touched_ids: set = set()
@@ -161,6 +201,9 @@ class HipBackend:
         self._profiling = False
         self._destroyed = False
         self._explicit_micro_batches = False     # set by next_micro_batch(): boundaries are told, not inferred
+        self.manage_gc = True
+        self._gc_managed = False
+        self._gc_was_enabled = True
 
     # ---- streams ------------------------------------------------------------------------------------------------
     @property
@@ -375,10 +418,26 @@ class HipBackend:
                 check(self._ctx, lib.gt_gemm_sum(self._ctx, NN, acc, rows, ind, n, ks, gs, ws, dx), "linear.dx")
 
     def install(self):
+        """Becomes the ops backend (webgpu.ts:393-399). While installed, and unless manage_gc is off, the interpreter's cyclic
+        garbage collector runs only inside sync(): a step's graph is tens of thousands of tensors and closures that refer to
+        each other, and collections triggered in the middle of recording cost 50 ms of host time per step of eight 2048-row
+        graphs (one in four steps 50 ms more, a full collection), during which the device runs out of queued work. What exists
+        at install time (modules, the model) is frozen out of the collector's sight so that the collection in sync() only
+        walks what a step made."""
         ag.set_ops_backend(self)
+        if self.manage_gc and not self._gc_managed:
+            self._gc_managed = True
+            self._gc_was_enabled = gc.isenabled()
+            gc.freeze()
+            gc.disable()
 
     def uninstall(self):
         ag.set_ops_backend(None)
+        if self._gc_managed:
+            self._gc_managed = False
+            gc.unfreeze()
+            if self._gc_was_enabled:
+                gc.enable()
 
     # ---- raw memory ------------------------------------------------------------------------------------
     def _acquire(self, nbytes: int, stream: int = None) -> int:
@@ -775,6 +834,10 @@ class HipBackend:
         """Wait for the stream; read back `reads` (values) and the accumulated gradients of every
         trainable external tensor touched since the last sync that is not kept on the device; recycle
         all intermediates. The graph is unusable for backward afterwards."""
+        if self._gc_managed:
+            self._flush()
+            self._flush_dx()
+            gc.collect()                # the last step's graph, while the device still has this step's launches to run
         self._join()
         nbytes = 0
         for t in reads:
@@ -829,6 +892,11 @@ class HipBackend:
         self._pend_dw = []
         self._pend_cs = []
         self._pend_rs = []
+        if self._gc_managed:             # destroyed while installed: hand the collector back
+            self._gc_managed = False
+            gc.unfreeze()
+            if self._gc_was_enabled:
+                gc.enable()
         if not self._destroyed:
             self._destroyed = True
             for c in self._ctxs:

@@ -941,6 +941,49 @@ def test_micro_batch_boundaries_told_by_the_trainer(ref):
     assert_close(b1, c1, "told boundaries on four streams vs one stream, dW1", rel_l2=2e-6, max_rel=2e-5)
 
 
+def test_collector_runs_only_at_sync_while_installed(ref):
+    """install() takes the interpreter's cyclic collector out of the recording (disabled, what already exists frozen) and
+    hands it back on uninstall() or on destroy() while installed; sync() collects the previous step's graph; manage_gc =
+    False leaves the collector alone."""
+    import gc
+    import weakref
+    hb, ag, arch = mod("hip_backend"), mod("autograd"), mod("arch")
+    assert gc.isenabled()
+    kw = SMALL["llama"]
+    _, model = build_pair(ref, kw, seed=3, std=0.05)
+    seqs = batches(ref, kw["vocab"], 12, 2, seed=4)
+    be = hb.HipBackend(0, streams=2)
+    try:
+        be.install()
+        assert not gc.isenabled() and gc.get_freeze_count() > 0
+        loss = arch.sequence_loss(model, seqs[0][0], seqs[0][1], 0)
+        ag.backward(loss, 1.0)
+        probe = weakref.ref(loss._prev[0])           # an intermediate of this step's graph (part of a reference cycle)
+        be.sync([loss])
+        assert probe() is not None                  # the graph is alive: the caller holds the loss
+        del loss
+        loss2 = arch.sequence_loss(model, seqs[1][0], seqs[1][1], 0)
+        ag.backward(loss2, 1.0)
+        be.sync([loss2])                            # collects the previous step's graph
+        assert probe() is None
+        be.uninstall()
+        assert gc.isenabled() and gc.get_freeze_count() == 0
+        be.install()
+        assert not gc.isenabled()
+    finally:
+        be.destroy()                                # while installed
+        ag.set_ops_backend(None)
+    assert gc.isenabled() and gc.get_freeze_count() == 0
+    be = hb.HipBackend(0, streams=1)
+    be.manage_gc = False
+    try:
+        be.install()
+        assert gc.isenabled() and gc.get_freeze_count() == 0
+        be.uninstall()
+    finally:
+        be.destroy()
+
+
 def test_grad_fold_sums_in_source_order(gpu):
     """gt_grad_fold: dst (+)= src0 + src1 + ... per tensor in one launch, bit for bit the f32 sums taken in that order;
     absent sources skipped, store and accumulate, sizes that are no multiple of four and an unaligned tensor."""

@@ -136,3 +136,34 @@ def test_window_sampler_injection(ref):
     for step in range(4):
         want = plain.draw(step)[0].tolist()
         assert off.draw(step)[0].tolist() == want and short.draw(step)[0].tolist() == want
+
+
+def test_device_records_ride_on_the_tensor():
+    """HipBackend's tensor -> device record map (webgpu.ts:322's WeakMap): the record sits in the tensor's own slot; two
+    maps (two backends) that meet on one tensor do not see each other's record; pop clears; a record dies with its tensor."""
+    import gc
+    import weakref
+    hb, ag = mod("hip_backend"), mod("autograd")
+    a, b = hb._EntryMap(), hb._EntryMap()
+    t, u = ag.Tensor(None, [2, 3]), ag.Tensor(None, [4])
+    assert a.get(t) is None and a.get(t, 7) == 7
+    with pytest.raises(KeyError):
+        a[t]
+    ea, eb = hb._Entry(24, False), hb._Entry(24, True)
+    a[t] = ea
+    assert a[t] is ea and a.get(t) is ea and b.get(t) is None and a.get(u) is None
+    b[t] = eb                                     # claimed by a: b keeps its record aside
+    assert b[t] is eb and a[t] is ea
+    e2 = hb._Entry(24, False)
+    a[t] = e2                                     # the owner may replace its record
+    assert a[t] is e2 and b[t] is eb
+    assert a.pop(t) is e2 and a.get(t) is None and a.pop(t, 5) == 5 and b[t] is eb
+    assert b.pop(t) is eb and b.get(t) is None
+    class Rec:                                    # (a stand-in that can be weakly referenced)
+        pass
+    rec = Rec()
+    b[u] = rec
+    wr = weakref.ref(rec)
+    del rec, u
+    gc.collect()
+    assert wr() is None
