@@ -250,15 +250,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_gen(AttnP p, const float *__
 int attn_fwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_bwd_mfma32(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
                     float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v,
-                    const float *rot_q, const float *rot_k);
+                    const float *rot_q, const float *rot_k, float *bandp, int band_splits);
 int attn_fwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_fwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf out, gt_buf lse, float *fpart, float *sco);
 int attn_bwd_mfma64(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
                     float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v,
-                    const float *rot_q, const float *rot_k);
+                    const float *rot_q, const float *rot_k, float *bandp, int band_splits);
 int attn_bwd_mfma128(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr, float *part,
                      float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv, int acc_v,
-                     const float *rot_q, const float *rot_k);
+                     const float *rot_q, const float *rot_k, float *bandp, int band_splits);
 static int attn_mfma_supported(int hd) { return hd == 32 || hd == 64 || hd == 128; }
 
 // A launch with fewer 128-row tiles than three per CU is cut further (measured at T = 2048, 9 heads: 1 sequence runs
@@ -332,10 +332,10 @@ static int attn_fwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf
 }
 static int attn_bwd_mfma(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
                          float *part, float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv,
-                         int acc_v, const float *rot_q, const float *rot_k) {
-  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k)
-      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k)
-                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k))
+                         int acc_v, const float *rot_q, const float *rot_k, float *bandp, int band_splits) {
+  if (p.hd == 32 ? attn_bwd_mfma32(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k, bandp, band_splits)
+      : p.hd == 64 ? attn_bwd_mfma64(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k, bandp, band_splits)
+                   : attn_bwd_mfma128(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, sco, dq, acc_q, dk, acc_k, dv, acc_v, rot_q, rot_k, bandp, band_splits))
     return 1;
   if (p.splits > 1 && !dsb) {
     const size_t n4 = (size_t)p.B * p.T * p.Hq * p.hd / 4;
@@ -410,12 +410,16 @@ static int attn_bwd_impl(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int
   size_t ds_floats = (mfma && ctx->opt_attn_keep_ds && T % 128 == 0 && hd >= 64) ? (size_t)rows * T : 0;
   if (ds_floats * sizeof(float) > ((size_t)ctx->opt_attn_ds_limit_mb << 20)) ds_floats = 0;
   const size_t dq_floats = (mfma && p.splits > 1 && !ds_floats) ? (size_t)p.splits * rows * hd : 0;
+  // a small launch of the banded dQ product cuts its K ranges into parts, one plane of dQ's size each (gemm_band_dq_splits)
+  const int band_splits = ds_floats ? gemm_band_dq_splits(ctx, B, T, Hq, window) : 1;
+  const size_t band_floats = band_splits > 1 ? (size_t)band_splits * rows * hd : 0;
   void *ws;
-  if (gt_ws_reserve(ctx, (d_floats + part_floats + dq_floats + ds_floats) * sizeof(float), &ws)) return 1;
+  if (gt_ws_reserve(ctx, (d_floats + part_floats + dq_floats + ds_floats + band_floats) * sizeof(float), &ws)) return 1;
   float *Dr = static_cast<float *>(ws);
   float *part = part_floats ? Dr + d_floats : nullptr;
   float *dqpart = dq_floats ? Dr + d_floats + part_floats : nullptr;
   float *dsb = ds_floats ? Dr + d_floats + part_floats + dq_floats : nullptr;
+  float *bandp = band_floats ? Dr + d_floats + part_floats + dq_floats + ds_floats : nullptr;
   {
     ProfScope ps(ctx, "attention.bwd.D");
     const int G = p.hd / 4;
@@ -443,7 +447,7 @@ static int attn_bwd_impl(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int
     if (rope_table_get(ctx, T, hd, rope.base, rope.pos, &rot)) return 1;
   }
   if (mfma) return attn_bwd_mfma(ctx, p, q, k, v, dout, lse, Dr, part, dqpart, dsb, P<const float>(scores), dq, acc_q, dk, acc_k, dv, acc_v,
-                                 rope.rot_q ? rot : nullptr, rope.rot_k ? rot : nullptr);
+                                 rope.rot_q ? rot : nullptr, rope.rot_k ? rot : nullptr, bandp, band_splits);
   {
     ProfScope ps(ctx, "attention.bwd.dq");
     size_t smem = 4 * (size_t)(2 * hd + WAVE) * sizeof(float);

@@ -820,7 +820,7 @@ int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
 // product dS.K afterwards (5 contractions in all); without it dQ recomputes S and dP in its own kernel (7).
 int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v, gt_buf dout, gt_buf lse, const float *Dr,
                       float *part, float *dqpart, float *dsb, const float *sco, gt_buf dq, int acc_q, gt_buf dk, int acc_k, gt_buf dv,
-                      int acc_v, const float *rot_q, const float *rot_k) {
+                      int acc_v, const float *rot_q, const float *rot_k, float *bandp, int band_splits) {
   GT_REQUIRE(ctx, (q | k | v | dout | dq | dk | dv) % 16 == 0, "attention: buffers must be 16-byte aligned");
   const int group = p.Hq / p.Hkv;
   GT_REQUIRE(ctx, p.splits >= 1 && (p.splits == 1 || dqpart || dsb) && (p.splits * group == 1 || part),
@@ -864,7 +864,7 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
   }
   if (dsb) {
     ProfScope ps(ctx, "attention.bwd.dq");
-    if (gemm_band_dq(ctx, p.B, p.T, p.Hq, p.Hkv, HD, p.window, dsb, P<const float>(k), P<float>(dq), acc_q, rot_q)) return 1;
+    if (gemm_band_dq(ctx, p.B, p.T, p.Hq, p.Hkv, HD, p.window, dsb, P<const float>(k), P<float>(dq), acc_q, rot_q, bandp, band_splits)) return 1;
   }
   return 0;
 }

@@ -35,6 +35,7 @@ struct gt_ctx {
   int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1, opt_gemm_staged = 0;
   int opt_gemm_group = 1;                       // 0: gt_gemm_group launches its products one by one
   int opt_attn_keep_ds = 1, opt_attn_ds_limit_mb = 8192, opt_gemm_sum_min_tiles = -1;
+  int opt_attn_band_splits = -1;       // parts the banded dQ product cuts its K ranges into (-1: chosen from the launch's size)
   bool prof_on = false;
   std::string prof_prefix;
   std::vector<ProfEvent> prof;
@@ -80,8 +81,9 @@ int gemm_scaled_batched(gt_ctx *ctx, int kind, int M, int N, int K, gt_buf A, in
 // gemm.hip: dQ (+)= dS.K per (sequence, head) over each row tile's band of visible keys
 // rot: the rotation table of the rope the query rows went through ([T][hd/2] (cos, sin) pairs), when dQ is wanted with respect
 // to the rows before that rotation (the write-back then applies the rotation's backward), else null
+int gemm_band_dq_splits(gt_ctx *ctx, int B, int T, int Hq, int window);
 int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc,
-                 const float *rot = nullptr);
+                 const float *rot = nullptr, float *parts = nullptr, int splits = 1);
 // embed_rope.hip: the (cos, sin) table of a rotation, built once per (T, hd, base, pos) and kept with the context
 int rope_table_get(gt_ctx *ctx, int T, int hd, double base, int pos, float **out);
 

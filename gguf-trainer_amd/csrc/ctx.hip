@@ -191,6 +191,7 @@ int gt_set_option(gt_ctx *ctx, const char *key, int value) {
   else if (!strcmp(key, "attn.keep_ds")) ctx->opt_attn_keep_ds = value;
   else if (!strcmp(key, "attn.ds_limit_mb")) ctx->opt_attn_ds_limit_mb = value < 0 ? 0 : value;
   else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
+  else if (!strcmp(key, "attn.band_splits")) ctx->opt_attn_band_splits = value;
   else if (!strcmp(key, "prof.sample")) ctx->opt_prof_sample = value >= 1 ? value : 1;
   else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
   else if (!strcmp(key, "gemm.splitk")) ctx->opt_gemm_splitk = value;

@@ -65,6 +65,9 @@ struct GemmArgs {
   // banded batch only: the (cos, sin) table ([M][N/2] pairs) of the rotation the rows of the other operand's source went
   // through; the write-back then applies that rotation's backward to each row of C (pairs (j, j + N/2)). Null: none.
   const float *rope;
+  // banded batch with splits > 1 (small launches): blockIdx.y cuts every row tile's K range into `splits` parts, each written
+  // unrotated and unaccumulated to Pp + blockIdx.y * sP (laid out as C); band_dq_reduce adds them up, rotates and accumulates
+  int64_t sP;
 };
 
 // Which output tile (pm, pn) and which K split or batch member (z) a workgroup works on. Workgroups are handed
@@ -385,6 +388,11 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
     B += (z / a.zdiv) * a.sB + ((z % a.zdiv) / a.zgroup) * a.sB2;
     k0 = a.window > 0 ? (max(0, m0 - a.window + 1) & ~127) : 0;
     kend = min(a.K, m0 + BM);
+    if (a.splits > 1) {                       // this workgroup's share of the row tile's stages (possibly none: it then writes zeros)
+      const int nst = (kend - k0) / BK, per = (nst + a.splits - 1) / a.splits;
+      k0 = min(kend, k0 + (int)blockIdx.y * per * BK);
+      kend = min(kend, k0 + per * BK);
+    }
   } else if (a.splits > 1) { k0 = z * a.kchunk; kend = min(a.K, k0 + a.kchunk); }
   else { A += z * a.sA; B += z * a.sB; }
   // The wavefront's index as a scalar for the loads (which of a stage's loads are its own, and their LDS addresses, are then
@@ -503,7 +511,11 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
   float *C;
   int ldc;
   bool add;
-  if (BAND) { C = a.C + (z / a.zdiv) * a.sC + (z % a.zdiv) * a.sC2; ldc = a.ldc; add = a.acc != 0; }
+  if (BAND) {
+    C = (a.splits > 1 ? a.Pp + (size_t)blockIdx.y * a.sP : a.C) + (z / a.zdiv) * a.sC + (z % a.zdiv) * a.sC2;
+    ldc = a.ldc;
+    add = a.splits > 1 ? false : a.acc != 0;
+  }
   else if (a.splits > 1) { C = a.Pp + (size_t)z * a.M * a.N; ldc = a.N; add = false; }
   else { C = a.C + z * a.sC; ldc = a.ldc; add = a.acc != 0 || a.D != nullptr; }
   const float *Cold = (!BAND && a.D && a.splits == 1) ? a.D + z * a.sD : C;
@@ -513,7 +525,7 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
   // accumulating, one 16-byte load issued before any store) instead of four scalar ones.
   const bool vec_c = (ldc % 4 == 0) && (((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(Cold)) & 15) == 0);
   if constexpr (BAND) {
-    if (a.rope) {
+    if (a.rope && a.splits == 1) {
       // dQ with respect to the rows before their rotation: a pair (j, j + BN/2) of a row sits in two wavefronts' accumulators
       // (WN = 2), so the tile goes through LDS once (the pipeline's buffers are idle now) and every thread then rotates
       // float4 pairs of whole rows: (lo, hi) -> (c lo + s hi, -s lo + c hi), the reference's srcRope backward (wgsl.ts:346-384)
@@ -865,14 +877,58 @@ static int launch_band(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   }
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
-  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>), dim3(zdim, 1, a.nbm * a.nbn), dim3(WM * WN * 64), smem,
+  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>), dim3(zdim, a.splits, a.nbm * a.nbn), dim3(WM * WN * 64), smem,
                      ctx->stream, a);
   GT_LAUNCHED(ctx);
   return 0;
 }
 
+// dQ (+)= sum of the band product's split partials, in split order, rotated back where the rows are wanted before their
+// rotation ((lo, hi) -> (c lo + s hi, -s lo + c hi) per pair (j, j + hd/2), the reference's srcRope backward, wgsl.ts:346-384):
+// one thread per float4 of a row's low half and its partner in the high half. rows = B*T rows of Hq heads.
+__global__ __launch_bounds__(256) void band_dq_reduce(const float *__restrict__ Pp, int splits, int64_t plane, float *dq, int acc,
+                                                      const float *__restrict__ rot, int64_t rows, int T, int Hq, int hd) {
+  const int upr = hd / 8;                                  // float4 units in the low half of a head's row
+  const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (u >= rows * Hq * upr) return;
+  const int c4 = (int)(u % upr);
+  const int64_t rh = u / upr, row = rh / Hq;
+  const size_t lo = (size_t)rh * hd + 4 * c4, hi = lo + hd / 2;
+  v4f a = *reinterpret_cast<const v4f *>(Pp + lo), b = *reinterpret_cast<const v4f *>(Pp + hi);
+  for (int z = 1; z < splits; z++) {
+    a += *reinterpret_cast<const v4f *>(Pp + (size_t)z * plane + lo);
+    b += *reinterpret_cast<const v4f *>(Pp + (size_t)z * plane + hi);
+  }
+  if (rot) {
+    const float *cs = rot + ((size_t)(row % T) * (hd / 2) + 4 * c4) * 2;
+    const v4f c0 = *reinterpret_cast<const v4f *>(cs), c1 = *reinterpret_cast<const v4f *>(cs + 4);
+    const v4f c = {c0[0], c0[2], c1[0], c1[2]}, sn = {c0[1], c0[3], c1[1], c1[3]};
+    const v4f r0 = c * a + sn * b, r1 = -sn * a + c * b;
+    a = r0;
+    b = r1;
+  }
+  if (acc) {
+    a += *reinterpret_cast<const v4f *>(dq + lo);
+    b += *reinterpret_cast<const v4f *>(dq + hi);
+  }
+  *reinterpret_cast<v4f *>(dq + lo) = a;
+  *reinterpret_cast<v4f *>(dq + hi) = b;
+}
+
+// how many parts a small launch of the banded product cuts every row tile's K range into (1: none), so that a single
+// sequence's 16 row tiles per head, whose longest has 16 times the K range of the shortest, become enough workgroups of
+// bounded length to fill the chip; the caller provides that many planes of B*T*Hq*hd floats
+int gemm_band_dq_splits(gt_ctx *ctx, int B, int T, int Hq, int window) {
+  const int64_t tiles = (int64_t)B * Hq * (T / 128);
+  if (ctx->opt_attn_band_splits >= 1) return (int)std::min<int64_t>(std::min(ctx->opt_attn_band_splits, 8), std::max(1, T / 128));
+  // the longest K range of a row tile: the whole sequence, or a window's band (there the tiles are short and alike: no cut)
+  const int kmax = window > 0 ? std::min(T, ((window + 126) & ~127) + 128) : T;
+  if (tiles >= 2 * ctx->num_cu || kmax < 1024) return 1;
+  return (int)std::min<int64_t>(std::min<int64_t>(8, kmax / 256), cdiv(2 * ctx->num_cu, tiles));
+}
+
 int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window, const float *dS, const float *K, float *dQ, int acc,
-                 const float *rot) {
+                 const float *rot, float *parts, int splits) {
   GT_REQUIRE(ctx, T % 128 == 0 && (hd == 64 || hd == 128), "banded dQ product: T %d must be a multiple of 128 and hd %d 64 or 128", T, hd);
   GT_REQUIRE(ctx, ((reinterpret_cast<uintptr_t>(dS) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(dQ)) & 15) == 0,
              "banded dQ product: operands must be 16-byte aligned");
@@ -880,14 +936,21 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.A = dS; a.B = K; a.C = dQ;
   a.M = T; a.N = hd; a.K = T;
   a.lda = T; a.ldb = Hkv * hd; a.ldc = Hq * hd;
-  a.acc = acc; a.kchunk = T; a.splits = 1; a.Pp = nullptr;
+  GT_REQUIRE(ctx, splits >= 1 && (splits == 1 || parts), "banded dQ product: %d splits without a workspace", splits);
+  a.acc = acc; a.kchunk = T; a.splits = splits; a.Pp = parts; a.sP = (int64_t)B * T * Hq * hd;
   a.sA = (int64_t)T * T; a.sB = (int64_t)T * Hkv * hd; a.sC = (int64_t)T * Hq * hd;
   a.zdiv = Hq; a.zgroup = Hq / Hkv; a.window = window; a.sB2 = hd; a.sC2 = hd;
   a.A2 = a.B2 = nullptr; a.K2 = 0; a.lda2 = a.ldb2 = 0; a.nx = 0; a.D = nullptr; a.sD = 0; a.scaled = 0; a.dscale = a.pscale = 1.f;
   a.rope = rot;
   GT_REQUIRE(ctx, !rot || (Hq * hd) % 4 == 0, "banded dQ product: rotated rows need 16-byte aligned output rows");
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
-  return hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26);
+  if (hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26)) return 1;
+  if (splits > 1) {
+    const int64_t rows = (int64_t)B * T, units = rows * Hq * (hd / 8);
+    hipLaunchKernelGGL(band_dq_reduce, dim3((unsigned)cdiv(units, 256)), dim3(256), 0, ctx->stream, parts, splits, a.sP, dQ, acc, rot, rows, T, Hq, hd);
+    GT_LAUNCHED(ctx);
+  }
+  return 0;
 }
 
 // C (+)= sum over i of A_i.B_i with the K segments chained in one loop (NT / NN, every K_i a multiple of 32)

@@ -973,6 +973,50 @@ def test_paired_linear_launches(gpu, ref):
     assert counts == {True: 1, False: 2}, counts
 
 
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 2048, 9, 3, 64, 0), (1, 1024, 4, 2, 128, 0), (2, 1024, 6, 2, 64, 0), (1, 2048, 10, 2, 64, 1500)])
+def test_banded_dq_product_cut_into_parts(gpu, B, T, Hq, Hkv, hd, window):
+    """The banded dQ product of a small launch cuts every row tile's key range into parts (option "attn.band_splits": pinned
+    1, 2, 4, 8 and the library's own choice) whose partial sums one kernel adds up, rotates back and accumulates: the same dq
+    up to the order of the sums, storing and accumulating, with and without the rotation's backward; dk and dv do not change."""
+    lib = mod("lib")
+    L = lib.lib
+    rs = np.random.RandomState(T + hd + window + B)
+    rows = B * T
+    mk = lambda n: rs.standard_normal((rows, n)).astype(np.float32)
+    q, k, v, go, dq0 = mk(Hq * hd), mk(Hkv * hd), mk(Hkv * hd), mk(Hq * hd), mk(Hq * hd)
+    c = gpu.ctx
+
+    def dev(a):
+        b = gpu.create_state_buffer(a.nbytes)
+        gpu.write_state_buffer(b, a)
+        return b
+    bq, bk, bv, bgo = dev(q), dev(k), dev(v), dev(go)
+    bout, blse = gpu.create_state_buffer(q.nbytes), gpu.create_state_buffer(B * Hq * T * 4)
+    bdk, bdv = gpu.create_state_buffer(k.nbytes), gpu.create_state_buffer(v.nbytes)
+    need = C.c_uint64()
+    lib.check(c, L.gt_attn_scores_bytes(c, B, T, Hq, Hkv, hd, window, C.byref(need)), "bytes")
+    bsc = gpu.create_state_buffer(need.value)
+    lib.check(c, L.gt_attn_fwd_scores(c, B, T, Hq, Hkv, hd, window, bq, bk, bv, bout, blse, bsc), "fwd")
+    try:
+        for rot in (0, 1):
+            for acc in (0, 1):
+                ref_out = None
+                for sp in (1, 2, 4, 8, -1):
+                    gpu.set_option("attn.band_splits", sp)
+                    bdq = dev(dq0)
+                    lib.check(c, L.gt_attn_bwd_scores_rope(c, B, T, Hq, Hkv, hd, window, bq, bk, bv, bout, bgo, blse, bsc, 10000.0, 5, rot, 0,
+                                                           bdq, acc, bdk, 0, bdv, 0), "bwd")
+                    got = [gpu.read_state_buffer(b, n).copy() for b, n in ((bdq, q.size), (bdk, k.size), (bdv, v.size))]
+                    gpu.free_state_buffer(bdq)
+                    if ref_out is None:
+                        ref_out = got
+                        continue
+                    assert_close(got[0], ref_out[0], f"dq in {sp} parts, rotation {rot}, acc {acc}", rel_l2=2e-6, max_rel=2e-5)
+                    assert np.array_equal(got[1], ref_out[1]) and np.array_equal(got[2], ref_out[2])
+    finally:
+        gpu.set_option("attn.band_splits", -1)
+
+
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,keep_ds", [(1, 256, 4, 2, 64, 0, 1), (2, 128, 3, 3, 64, 0, 1), (1, 384, 4, 1, 128, 100, 1),
                                                         (2, 256, 6, 2, 64, 70, 0), (1, 128, 2, 2, 128, 0, 0), (8, 256, 9, 3, 64, 0, 1)])
 @pytest.mark.parametrize("acc", [0, 1])
