@@ -34,6 +34,7 @@ struct gt_ctx {
   std::map<RopeKey, float *> rope_tables;
   int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1, opt_gemm_staged = 0;
   int opt_gemm_group = 1;                       // 0: gt_gemm_group launches its products one by one
+  int opt_gemm_split = 0;                       // 1: aligned FP32 products run as six bf16 MFMA products of three-piece operands
   int opt_attn_keep_ds = 1, opt_attn_ds_limit_mb = 8192, opt_gemm_sum_min_tiles = -1;
   int opt_attn_band_splits = -1;       // parts the banded dQ product cuts its K ranges into (-1: chosen from the launch's size)
   bool prof_on = false;
@@ -41,6 +42,7 @@ struct gt_ctx {
   std::vector<ProfEvent> prof;
   unsigned attn_smem_set = 0;                   // head dims whose attention kernels have their LDS size attribute set: bits 32 | 64 | 128 dK/dV, the same << 8 forward
   uint64_t gemm_direct_set = 0;                 // direct-to-LDS GEMM variants whose LDS size attribute is set
+  uint64_t gemm_split_set = 0;                  // the same for the bf16-piece variants
   int opt_prof_sample = 1;                      // events around every n-th launch of a label
   // Pinned host words a kernel writes when it meets an id / target outside its range (it skips that row):
   // [0] = which check (GT_BAD_*), [1] = row, [2] = the value, [3] = the bound. Read after the stream has drained.

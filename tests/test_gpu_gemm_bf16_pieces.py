@@ -1,0 +1,251 @@
+"""The option "gemm.split_bf16": the FP32 products of the path on the bf16 matrix instruction, every operand element cut
+into three bf16 pieces (exact) and six of the nine piece products kept. Same entry points, same tolerances as the FP32
+MFMA kernels: every product kind against float64, the fused forms against their one-by-one counterparts, whole models
+against the oracle (loss 1e-5, gradients 1e-5 relative L2 / 1e-4 max), and its error against float64 next to the
+FP32 kernels' error."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gpu_common import assert_close, mod
+from test_gpu_model import REAL, SMALL, batches, build_pair, compare, hip_step, ref_step
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def pieces(gpu):
+    gpu.set_option("gemm.split_bf16", 1)
+    yield gpu
+    gpu.set_option("gemm.split_bf16", 0)
+    gpu.set_option("gemm.splitk", -1)
+    gpu.set_option("gemm.sum_min_tiles", -1)
+
+
+def labels_of(gpu, run):
+    gpu.start_profile("gemm.")
+    run()
+    return set(gpu.stop_profile())
+
+
+def bufs(gpu, *arrays):
+    out = []
+    for a in arrays:
+        b = gpu.create_state_buffer(a.nbytes)
+        gpu.write_state_buffer(b, a)
+        out.append(b)
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", [(200, 152, 96), (132, 100, 64), (260, 196, 128), (300, 576, 576), (257, 192, 1536), (128, 384, 32),
+                                   (4, 4, 32), (1000, 1536, 64)])
+def test_every_kind_store_accumulate_and_k_split_against_float64(pieces, M, N, K):
+    """NT / NN / TN on both tile shapes (N a multiple of 192 or not), partial tiles on both edges, one stage only (K = 32),
+    store and accumulate, dW cut along K; the profile label says which kernel ran."""
+    gpu = pieces
+    rs = np.random.RandomState(M + N + K)
+    a = rs.standard_normal((M, K)).astype(np.float32)
+    b = rs.standard_normal((N, K)).astype(np.float32)
+    c0 = rs.standard_normal((M, N)).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    da, db, dc = bufs(gpu, a, b, c0)
+    for kind, (A, B) in enumerate([(a, b), (a, np.ascontiguousarray(b.T)), (np.ascontiguousarray(a.T), np.ascontiguousarray(b.T))]):
+        gpu.write_state_buffer(da, A)
+        gpu.write_state_buffer(db, B)
+        for splitk in ((-1, 1, 3) if kind == 2 else (-1,)):
+            for acc in (0, 1):
+                gpu.set_option("gemm.splitk", splitk)
+                gpu.write_state_buffer(dc, c0)
+                seen = labels_of(gpu, lambda: gpu.gemm(kind, acc, M, N, K, da, db, dc))
+                # the direct kernels' condition: whole 16-byte chunks along every operand's contiguous index
+                takes = (kind != 2 or M % 4 == 0) and (kind == 0 or N % 4 == 0)
+                assert any(".bf16x6" in s for s in seen) == takes, seen
+                got = gpu.read_state_buffer(dc, M * N).reshape(M, N)
+                assert_close(got, (want + c0 if acc else want).astype(np.float32), f"kind {kind} splitk {splitk} acc {acc} {M}x{N}x{K}")
+    for h in (da, db, dc):
+        gpu.free_state_buffer(h)
+
+
+@pytest.mark.parametrize("kind,M,N,K", [(0, 70, 83, 75), (1, 64, 64, 100), (2, 96, 66, 64), (0, 1, 5, 3)])
+def test_shapes_the_direct_kernels_do_not_take_stay_on_the_fp32_kernels(pieces, kind, M, N, K):
+    """K not a multiple of 32, or an operand whose contiguous index is not whole 16-byte chunks: the register-staged FP32
+    kernels as before, with the option on."""
+    gpu = pieces
+    rs = np.random.RandomState(K)
+    a = rs.standard_normal((K, M) if kind == 2 else (M, K)).astype(np.float32)
+    b = rs.standard_normal((N, K) if kind == 0 else (K, N)).astype(np.float32)
+    want = (a.T if kind == 2 else a).astype(np.float64) @ (b.T if kind == 0 else b).astype(np.float64)
+    da, db, dc = bufs(gpu, a, b, np.zeros((M, N), np.float32))
+    seen = labels_of(gpu, lambda: gpu.gemm(kind, 0, M, N, K, da, db, dc))
+    assert seen and not any(".bf16x6" in s for s in seen), seen
+    assert_close(gpu.read_state_buffer(dc, M * N).reshape(M, N), want.astype(np.float32), f"fallback kind {kind}")
+    for h in (da, db, dc):
+        gpu.free_state_buffer(h)
+
+
+def test_error_against_float64_next_to_the_fp32_kernels(gpu):
+    """Not reduced precision: over the layer's product shapes the rms error of the piece products against float64 stays
+    within 1.25 x the FP32 MFMA kernels' own (measured 0.9 - 1.2 x: both accumulate in FP32, in a different order)."""
+    rs = np.random.RandomState(7)
+    for kind, M, N, K in [(0, 512, 576, 1536), (1, 512, 1536, 576), (2, 576, 576, 16384), (0, 384, 1536, 576)]:
+        a = rs.standard_normal((K, M) if kind == 2 else (M, K)).astype(np.float32)
+        b = (0.02 * rs.standard_normal((N, K) if kind == 0 else (K, N))).astype(np.float32)
+        want = (a.T if kind == 2 else a).astype(np.float64) @ (b.T if kind == 0 else b).astype(np.float64)
+        da, db, dc = bufs(gpu, a, b, np.zeros((M, N), np.float32))
+        err = []
+        try:
+            for on in (0, 1):
+                gpu.set_option("gemm.split_bf16", on)
+                gpu.gemm(kind, 0, M, N, K, da, db, dc)
+                got = gpu.read_state_buffer(dc, M * N).reshape(M, N).astype(np.float64)
+                err.append(np.sqrt(np.mean((got - want) ** 2)))
+        finally:
+            gpu.set_option("gemm.split_bf16", 0)
+        assert err[1] <= 1.25 * err[0], (kind, M, N, K, err)
+        for h in (da, db, dc):
+            gpu.free_state_buffer(h)
+
+
+@pytest.mark.parametrize("scale_a,scale_b", [(1e-12, 1e-9), (1e12, 1e3), (1e-20, 1e15), (0.0, 1.0)])
+def test_magnitudes_far_from_one(pieces, scale_a, scale_b):
+    """The pieces keep FP32's exponent range: no scaling of the operands is involved. Very small and very large operands give
+    the same relative accuracy; a zero operand gives exact zeros."""
+    gpu = pieces
+    M, N, K = 256, 192, 256
+    rs = np.random.RandomState(3)
+    a = (scale_a * rs.standard_normal((M, K))).astype(np.float32)
+    b = (scale_b * rs.standard_normal((N, K))).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    da, db, dc = bufs(gpu, a, b, np.ones((M, N), np.float32))
+    gpu.gemm(0, 0, M, N, K, da, db, dc)
+    got = gpu.read_state_buffer(dc, M * N).reshape(M, N)
+    if scale_a == 0.0:
+        assert not got.any()
+    else:
+        assert_close(got, want.astype(np.float32), f"scales {scale_a} x {scale_b}")
+    for h in (da, db, dc):
+        gpu.free_state_buffer(h)
+
+
+@pytest.mark.parametrize("kind,M,N,K", [(0, 300, 576, 576), (0, 257, 576, 1536), (1, 130, 96, 64), (2, 96, 64, 2048)])
+@pytest.mark.parametrize("in_place", [False, True])
+def test_product_plus_addend(pieces, kind, M, N, K, in_place):
+    """gt_gemm_add through the piece kernels: bit for bit the product into a buffer plus an elementwise add."""
+    gpu, lib = pieces, mod("lib")
+    rs = np.random.RandomState(M + K)
+    a_ = rs.standard_normal((K, M) if kind == 2 else (M, K)).astype(np.float32)
+    b_ = rs.standard_normal((N, K) if kind == 0 else (K, N)).astype(np.float32)
+    d_ = rs.standard_normal((M, N)).astype(np.float32)
+    da, db, dd, dc, dy = bufs(gpu, a_, b_, d_, d_ if in_place else np.zeros_like(d_), d_)
+    lib.check(gpu.ctx, lib.lib.gt_gemm_add(gpu.ctx, kind, M, N, K, da, db, dc if in_place else dd, dc), "gt_gemm_add")
+    got = gpu.read_state_buffer(dc, M * N).copy()
+    lib.check(gpu.ctx, lib.lib.gt_gemm(gpu.ctx, kind, 0, M, N, K, da, db, dy), "gt_gemm")
+    y = gpu.read_state_buffer(dy, M * N).copy()
+    assert np.array_equal(got, (d_.reshape(-1) + y).astype(np.float32))
+    for h in (da, db, dd, dc, dy):
+        gpu.free_state_buffer(h)
+
+
+def test_batch_of_two_and_scaled_write_back(pieces):
+    """gt_gemm_batched (the gate and up projections as one launch) against float64 per member."""
+    gpu, lib = pieces, mod("lib")
+    M, N, K = 300, 192, 576
+    rs = np.random.RandomState(9)
+    a = rs.standard_normal((M, K)).astype(np.float32)
+    b = rs.standard_normal((2, N, K)).astype(np.float32)
+    da, db, dc = bufs(gpu, a, b, np.zeros((2, M, N), np.float32))
+    lib.check(gpu.ctx, lib.lib.gt_gemm_batched(gpu.ctx, 0, 0, M, N, K, da, 0, db, N * K, dc, M * N, 2), "gt_gemm_batched")
+    got = gpu.read_state_buffer(dc, 2 * M * N).reshape(2, M, N)
+    for i in range(2):
+        assert_close(got[i], (a.astype(np.float64) @ b[i].astype(np.float64).T).astype(np.float32), f"batch member {i}")
+    for h in (da, db, dc):
+        gpu.free_state_buffer(h)
+
+
+@pytest.mark.parametrize("kind,M,N,Ks", [(1, 300, 576, (576, 192, 192)), (1, 257, 576, (1536, 1536)), (1, 128, 640, (640, 128, 128)),
+                                         (0, 200, 192, (64, 96)), (1, 5600, 576, (576, 192, 192))])
+@pytest.mark.parametrize("acc", [0, 1])
+def test_summed_products_in_one_chained_loop(pieces, kind, M, N, Ks, acc):
+    """gt_gemm_sum: the input gradient of sibling projections as one K loop over all their segments."""
+    gpu, lib = pieces, mod("lib")
+    rs = np.random.RandomState(M + sum(Ks))
+    As = [rs.standard_normal((M, K)).astype(np.float32) for K in Ks]
+    Bs = [rs.standard_normal((N, K) if kind == 0 else (K, N)).astype(np.float32) for K in Ks]
+    c0 = rs.standard_normal((M, N)).astype(np.float32)
+    ha, hb = bufs(gpu, *As), bufs(gpu, *Bs)
+    (c,) = bufs(gpu, c0)
+    n = len(Ks)
+    gpu.set_option("gemm.sum_min_tiles", 0)
+    seen = labels_of(gpu, lambda: lib.check(gpu.ctx, lib.lib.gt_gemm_sum(gpu.ctx, kind, acc, M, N, n, (C.c_int * n)(*Ks), (C.c_uint64 * n)(*ha),
+                                                                        (C.c_uint64 * n)(*hb), c), "gt_gemm_sum"))
+    assert len(seen) == 1 and ".bf16x6" in next(iter(seen)), seen
+    want = c0.astype(np.float64) * acc
+    for a_, b_ in zip(As, Bs):
+        want = want + a_.astype(np.float64) @ (b_.T if kind == 0 else b_).astype(np.float64)
+    assert_close(gpu.read_state_buffer(c, M * N).reshape(M, N), want.astype(np.float32), f"sum of {n}")
+    for h in ha + hb + [c]:
+        gpu.free_state_buffer(h)
+
+
+@pytest.mark.parametrize("K,shapes", [(16384, [(576, 1536), (1536, 576), (576, 576), (192, 576)]),
+                                      (2048, [(576, 1536), (1536, 576), (1536, 576), (576, 576), (576, 576), (192, 576), (192, 576), (576, 1536)]),
+                                      (256, [(64, 64), (8, 12)]), (96, [(200, 152), (4, 4), (132, 100)])])
+def test_grouped_weight_gradients(pieces, K, shapes):
+    """gt_gemm_group: the layer's dW products as one launch over all their tiles, K cut into ranges, store and accumulate
+    mixed; each member alone through the same entry point gives the same bits."""
+    gpu, lib = pieces, mod("lib")
+    rs = np.random.RandomState(K + len(shapes))
+    n = len(shapes)
+    As = [rs.standard_normal((K, M)).astype(np.float32) for M, N in shapes]
+    Bs = [rs.standard_normal((K, N)).astype(np.float32) for M, N in shapes]
+    C0 = [rs.standard_normal((M, N)).astype(np.float32) for M, N in shapes]
+    accs = [i % 2 for i in range(n)]
+    da, db, dc = bufs(gpu, *As), bufs(gpu, *Bs), bufs(gpu, *C0)
+    Ms, Ns = (C.c_int * n)(*[m for m, _ in shapes]), (C.c_int * n)(*[n_ for _, n_ in shapes])
+    seen = labels_of(gpu, lambda: lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, n, Ms, Ns, K, (C.c_uint64 * n)(*da), (C.c_uint64 * n)(*db),
+                                                                          (C.c_uint64 * n)(*dc), (C.c_int * n)(*accs)), "gt_gemm_group"))
+    assert any(".bf16x6" in s for s in seen), seen
+    got = [gpu.read_state_buffer(b_, c_.size).copy() for b_, c_ in zip(dc, C0)]
+    for i in range(n):
+        want = As[i].astype(np.float64).T @ Bs[i].astype(np.float64) + (C0[i] if accs[i] else 0)
+        assert_close(got[i], want.astype(np.float32), f"group member {i} {shapes[i]}")
+        gpu.write_state_buffer(dc[i], C0[i])
+        lib.check(gpu.ctx, lib.lib.gt_gemm_group(gpu.ctx, 2, 1, (C.c_int * 1)(shapes[i][0]), (C.c_int * 1)(shapes[i][1]), K, (C.c_uint64 * 1)(da[i]),
+                                                 (C.c_uint64 * 1)(db[i]), (C.c_uint64 * 1)(dc[i]), (C.c_int * 1)(accs[i])), "gt_gemm_group")
+        assert np.array_equal(gpu.read_state_buffer(dc[i], C0[i].size), got[i]), f"member {i} alone vs in the group"
+    for h in da + db + dc:
+        gpu.free_state_buffer(h)
+
+
+@pytest.mark.parametrize("arch_name", ["llama", "qwen3", "gemma3"])
+def test_small_models_against_the_oracle(pieces, ref, arch_name):
+    kw = SMALL[arch_name]
+    rmodel, model = build_pair(ref, kw, seed=1, std=0.1)
+    seqs = batches(ref, kw["vocab"], 19, 2, seed=5, mask_every=5)
+    lh, gh = hip_step(pieces, model, seqs, True, 19)
+    lr, gr = ref_step(ref, rmodel, seqs)
+    compare(lh, gh, lr, gr, f"{arch_name} with bf16 pieces")
+
+
+@pytest.mark.parametrize("name", ["smollm2", "gemma3-window", "qwen3-hd128"])
+@pytest.mark.parametrize("stacked", [False, True])
+def test_real_head_geometry_against_the_oracle(pieces, ref, name, stacked):
+    """Whole graphs at the widths the piece kernels are selected for (576 / 1536 / 640-class rows, 200-token sequences ragged
+    against every tile): loss and every gradient tensor at the tolerances of the FP32 kernels."""
+    kw = REAL[name]
+    rmodel, model = build_pair(ref, kw, seed=11, std=0.05)
+    seqs = batches(ref, kw["vocab"], 200, 2, seed=12, mask_every=7)
+    seen = set()
+    pieces.start_profile("gemm.")
+    lh, gh = hip_step(pieces, model, seqs, stacked, 200)
+    seen = set(pieces.stop_profile())
+    assert any(".bf16x6" in s for s in seen), seen
+    ref.PARALLEL_BWD = True
+    ref.set_threads(min(16, ref.max_threads()))
+    try:
+        lr, gr = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.PARALLEL_BWD = False
+        ref.set_threads(1)
+    compare(lh, gh, lr, gr, f"{name} stacked={stacked} with bf16 pieces")
