@@ -24,6 +24,7 @@ PKG = "gguf-trainer_amd"
 
 PEAK_FP32_MFMA = 157.3e12      # MI355X dense FP32 matrix peak, FLOP/s
 PEAK_HBM = 8.0e12              # B/s
+PEAK_BF16_MFMA = 2500e12       # MI355X dense bf16 matrix peak, FLOP/s (what the bf16-piece leg executes on)
 PROF_SAMPLE = 4                # the timed region brackets about 1 in 4 launches of a GEMM label with HIP events
 # L2-miss traffic per launch (bytes) of the backward GEMM labels that lead the step, from two rocprofv3 --pmc passes over
 # this file made separately (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the factors read off a plain streaming kernel of known
@@ -479,6 +480,33 @@ def run_workload(mods, config, steps, warmup, a, headline):
             res["call_pattern"] = {"graph": f"{batch} graphs of {SEQ} rows per step, one sequence at a time, as src/backend/train-gpu.ts:200-219 calls the backend",
                                    "streams": a.streams, "steps": nseq, "value": round(nseq * batch * SEQ / w1, 1), "unit": "tokens/s",
                                    "ms_per_step": round(1e3 * w1 / nseq, 2)}
+        # The same stacked step with the library's FP32 products on the bf16 matrix instruction ("gemm.split_bf16": three exact
+        # bf16 pieces per operand element, six of the nine piece products, FP32 accumulation; as close to float64 as the FP32
+        # MFMA kernels, tests/test_gpu_gemm_bf16_pieces.py). Outside the headline's timed region; the headline stays on FP32 MFMA.
+        res["bf16_pieces"] = None
+        if headline and not a.sequential and not a.no_bf16_pieces and not any(kv.startswith("gemm.split_bf16") for kv in a.set):
+            nb = max(2, min(6, steps))
+            gpu.set_option("gemm.split_bf16", 1)
+            try:
+                for i in range(2):
+                    step(i % total, False)
+                gpu.sync([])
+                gpu.set_option("prof.sample", PROF_SAMPLE)
+                gpu.start_profile("gemm.")
+                w2 = timed_leg(nb, False, 2)
+                p2 = gpu.stop_profile()
+            finally:
+                gpu.set_option("prof.sample", 1)
+                gpu.set_option("gemm.split_bf16", 0)
+            _, allb2, per2 = gemm_summary(p2, nb)
+            if allb2:
+                allb2["executed_frac_of_bf16_mfma_peak"] = round(6 * allb2["achieved"] * 1e12 / PEAK_BF16_MFMA, 4)
+            res["bf16_pieces"] = {"what": "the headline step with gt_set_option(\"gemm.split_bf16\", 1): every aligned FP32 product as six bf16 MFMA "
+                                          "products of three-piece operands, FP32 accumulate; same entry points, same parity tolerances",
+                                  "steps": nb, "value": round(nb * batch * SEQ / w2, 1), "unit": "tokens/s", "ms_per_step": round(1e3 * w2 / nb, 2),
+                                  "all_bwd_gemms": allb2, "per_kernel": per2,
+                                  "note": "achieved = algorithmic 2MNK FLOP per second; frac is against the FP32 MFMA peak (157.3 TFLOP/s) and can "
+                                          "exceed 1; the kernels execute 6 x that on the bf16 pipes (peak 2500 TFLOP/s)"}
     finally:
         gpu.uninstall()
         ag.set_checkpointing(False)
@@ -568,6 +596,8 @@ def main():
     ap.add_argument("--no-micro", action="store_true", help="skip the isolated-kernel leg (benchmark configs[1] shapes)")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short legs over benchmark configs[2] (gemma3-style, Muon) and configs[4] (Qwen3-0.6B, LoRA)")
+    ap.add_argument("--no-bf16-pieces", action="store_true",
+                    help="skip the short extra leg that reruns the step with the FP32 products on the bf16 matrix instruction")
     ap.add_argument("--naive-host", action="store_true",
                     help="add a leg that runs the reference's call pattern on one stream with every host-side hold-back and fusion off")
     ap.add_argument("--no-pair", action="store_true", help="launch every linear on its own (no batched k/v and gate/up pairs)")
@@ -668,6 +698,7 @@ def main():
         "loss_first": round(losses[0], 4), "loss_last": round(losses[-1], 4),
         "reference_call_pattern": r["call_pattern"],
         "naive_host": naive,
+        "bf16_pieces": r.get("bf16_pieces"),
         "roofline": roof,
         "muon_step": r.get("muon"),
         "kernels": kernels,
