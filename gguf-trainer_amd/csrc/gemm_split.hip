@@ -5,17 +5,17 @@
 
 #define GT_SPLIT_BK 32
 #define GT_SPLIT_NSTG 2
-template <int BM, int BN, int WM, int WN, int KIND, bool MSEG>
+template <int BM, int BN, int WM, int WN, int KIND, bool MSEG, bool SEG2 = false>
 static int launch_split_kind(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   constexpr int smem = GT_SPLIT_NSTG * (BM + BN) * GT_SPLIT_BK * 4;
   if (!(ctx->gemm_split_set & (1ull << slot))) {       // once per context (device): more LDS than a kernel gets by default
-    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, KIND, GT_SPLIT_BK, GT_SPLIT_NSTG, false, false, MSEG, true>),
+    GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, KIND, GT_SPLIT_BK, GT_SPLIT_NSTG, SEG2, false, MSEG, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     ctx->gemm_split_set |= 1ull << slot;
   }
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
-  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, KIND, GT_SPLIT_BK, GT_SPLIT_NSTG, false, false, MSEG, true>), dim3(a.nbm * a.nbn, 1, zdim),
+  hipLaunchKernelGGL((gemm_direct<BM, BN, WM, WN, KIND, GT_SPLIT_BK, GT_SPLIT_NSTG, SEG2, false, MSEG, true>), dim3(a.nbm * a.nbn, 1, zdim),
                      dim3(WM * WN * 64), smem, ctx->stream, a);
   GT_LAUNCHED(ctx);
   return 0;
@@ -33,7 +33,16 @@ static int launch_split(gt_ctx *ctx, int kind, bool wide, GemmArgs &a, int zdim)
   if (!MSEG) return launch_split_kind<128, 128, 2, 2, GT_TN, false>(ctx, a, zdim, s);
   GT_FAIL(ctx, "summed products are NT or NN");
 }
+// two K segments (the second 16 or 32 long, riding in one more stage): NT / NN
+static int launch_split_seg2(gt_ctx *ctx, int kind, bool wide, GemmArgs &a, int zdim) {
+  const int s = 14 + (wide ? 2 : 0) + kind;
+  if (wide) return kind == GT_NT ? launch_split_kind<128, 192, 2, 2, GT_NT, false, true>(ctx, a, zdim, s)
+                                 : launch_split_kind<128, 192, 2, 2, GT_NN, false, true>(ctx, a, zdim, s);
+  return kind == GT_NT ? launch_split_kind<128, 128, 2, 2, GT_NT, false, true>(ctx, a, zdim, s)
+                       : launch_split_kind<128, 128, 2, 2, GT_NN, false, true>(ctx, a, zdim, s);
+}
 int gemm_split_launch(gt_ctx *ctx, int kind, bool wide, bool summed, GemmArgs &a, int zdim) {
+  if (a.K2 > 0) return launch_split_seg2(ctx, kind, wide, a, zdim);
   return summed ? launch_split<true>(ctx, kind, wide, a, zdim) : launch_split<false>(ctx, kind, wide, a, zdim);
 }
 

@@ -447,7 +447,7 @@ __device__ __forceinline__ void split_step(const v4u (&fa)[TM][3], const v4u (&f
 // The work of one workgroup on output tile (pm, pn) and K split or batch member z
 template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2, bool BAND = false, bool MSEG = false, bool SPLIT = false>
 __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm, const int pn, const int z) {
-  static_assert(!SPLIT || (!SEG2 && !BAND), "the bf16-piece path takes plain and summed products");
+  static_assert(!SPLIT || !BAND, "the bf16-piece path takes plain, two-segment and summed products");
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   using TA = DirectTile<BM, KIND != GT_TN, NT, BK>;
@@ -581,6 +581,13 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
         const float *sa = smem + buf * STAGE, *sb = sa + TA::CH * 4;
         RAW(sa, sb, 1)
         split_step<TM, TN>(f0a, f0b, acc, xa, xb, f1a, f1b);
+        if (SEG2 && st == nstage - 1 && a.K2 <= 16) {
+          // a second segment of 16 fills half of its stage: the other half (valid chunks loaded again) is multiplied by zeros
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int p = 0; p < 3; p++) f1b[j][p] = v4u{0, 0, 0, 0};
+        }
         // (after the last stage this prepares a step nobody multiplies, from the other buffer's old contents)
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();

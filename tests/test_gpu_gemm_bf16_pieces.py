@@ -249,3 +249,67 @@ def test_real_head_geometry_against_the_oracle(pieces, ref, name, stacked):
         ref.PARALLEL_BWD = False
         ref.set_threads(1)
     compare(lh, gh, lr, gr, f"{name} stacked={stacked} with bf16 pieces")
+
+
+@pytest.mark.parametrize("M,N,K1,K2", [(200, 152, 96, 16), (300, 576, 576, 16), (257, 192, 1536, 32), (132, 100, 64, 32), (64, 64, 32, 16),
+                                       (260, 196, 128, 8), (300, 576, 192, 24)])
+def test_two_segment_products(pieces, M, N, K1, K2):
+    """gt_gemm_pair (the LoRA linear and its dX): C (+)= A1.B1 + A2.B2 in one K loop. A second segment of 16 or 32 rides in one
+    more stage of the piece kernels (16: the stage's other half is multiplied by zero pieces); 8 and 24 stay on the FP32
+    kernels."""
+    gpu, L = pieces, mod("lib")
+    rs = np.random.RandomState(M + K2)
+    a1, b1 = rs.standard_normal((M, K1)).astype(np.float32), rs.standard_normal((N, K1)).astype(np.float32)
+    a2, b2 = rs.standard_normal((M, K2)).astype(np.float32), rs.standard_normal((N, K2)).astype(np.float32)
+    c0 = rs.standard_normal((M, N)).astype(np.float32)
+    want = a1.astype(np.float64) @ b1.astype(np.float64).T + a2.astype(np.float64) @ b2.astype(np.float64).T
+    h = bufs(gpu, a1, b1, a2, b2, c0)
+    T = lambda x: np.ascontiguousarray(x.T)
+    for kind, ops in enumerate([(a1, b1, a2, b2), (a1, T(b1), a2, T(b2))]):
+        for buf, arr in zip(h, ops):
+            gpu.write_state_buffer(buf, arr)
+        for acc in (0, 1):
+            gpu.write_state_buffer(h[4], c0)
+            seen = labels_of(gpu, lambda: L.check(gpu.ctx, L.lib.gt_gemm_pair(gpu.ctx, kind, acc, M, N, K1, h[0], h[1], K2, h[2], h[3], h[4]), "gt_gemm_pair"))
+            assert any(".bf16x6" in s for s in seen) == (K2 in (16, 32)), seen
+            got = gpu.read_state_buffer(h[4], M * N).reshape(M, N)
+            assert_close(got, (want + c0 if acc else want).astype(np.float32), f"pair kind {kind} acc {acc} {M}x{N}x({K1}+{K2})")
+    for b in h:
+        gpu.free_state_buffer(b)
+
+
+@pytest.mark.parametrize("recompute", [False, True])
+def test_lora_against_the_oracle(pieces, ref, recompute):
+    """Rank-16 adapters on a model of real widths (the two-segment forward and dX, the rank products on their own kernels)."""
+    ag, arch = mod("autograd"), mod("arch")
+    kw = REAL["smollm2"]
+    rmodel, model = build_pair(ref, kw, seed=5, std=0.05)
+    rank, alpha = 16, 16.0
+    rmap, rparams = ref.attach_lora(rmodel, rank, alpha, ref.Mulberry32(11), a_std=0.05)
+    rng = ref.Mulberry32(12)
+    for a, b, _ in rmap.values():
+        b.data[:] = rng.fill_randn([b.size], 0.05)
+    adapters = {}
+    for l, Lr in enumerate(rmodel.layers):
+        for k in ref.MATRIX_KEYS:
+            a, b, _ = rmap[id(Lr[k])]
+            adapters[f"L{l}.{k}"] = (a.data.copy(), b.data.copy())
+    aux = arch.apply_lora(model, rank, alpha, adapters)
+    ref.set_lora_adapters(rmap)
+    seqs = batches(ref, kw["vocab"], 200, 2, seed=8, mask_every=3)
+    ref.PARALLEL_BWD = True
+    ref.set_threads(min(16, ref.max_threads()))
+    try:
+        pieces.start_profile("gemm.")
+        lh, _ = hip_step(pieces, model, seqs, True, 200, recompute=recompute)
+        seen = set(pieces.stop_profile())
+        lr, _ = ref_step(ref, rmodel, seqs)
+    finally:
+        ref.PARALLEL_BWD = False
+        ref.set_threads(1)
+        ref.set_lora_adapters({})
+        arch.clear_lora(model)
+    assert any(".bf16x6" in s for s in seen), seen
+    assert np.all(np.abs(lh - lr) <= 1e-5 * np.abs(lr))
+    for i, (h, r) in enumerate(zip(aux, rparams)):
+        assert_close(h.grad, r.grad, f"lora adapter {i} with bf16 pieces")
