@@ -484,7 +484,7 @@ def run_workload(mods, config, steps, warmup, a, headline):
         # bf16 pieces per operand element, six of the nine piece products, FP32 accumulation; as close to float64 as the FP32
         # MFMA kernels, tests/test_gpu_gemm_bf16_pieces.py). Outside the headline's timed region; the headline stays on FP32 MFMA.
         res["bf16_pieces"] = None
-        if headline and not a.sequential and not a.no_bf16_pieces and not any(kv.startswith("gemm.split_bf16") for kv in a.set):
+        if not a.sequential and not a.no_bf16_pieces and not any(kv.startswith("gemm.split_bf16") for kv in a.set):
             nb = max(2, min(6, steps))
             gpu.set_option("gemm.split_bf16", 1)
             try:
@@ -680,6 +680,8 @@ def main():
                 ent["per_kernel"] = per2
             if o.get("muon"):
                 ent["muon_step"] = o["muon"]
+            if o.get("bf16_pieces"):        # the same workload with "gemm.split_bf16" on (Muon's Newton-Schulz products included)
+                ent["bf16_pieces"] = {k: o["bf16_pieces"][k] for k in ("steps", "value", "unit", "ms_per_step", "all_bwd_gemms")}
             other[f"configs[{ci}]"] = ent
     naive = naive_host_leg(mods, a) if a.naive_host or (a.config == 3 and not a.no_call_pattern and not a.sequential) else None
     if naive is not None:          # the same literal calls, micro-batches dealt to the backend's streams

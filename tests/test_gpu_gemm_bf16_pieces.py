@@ -313,3 +313,21 @@ def test_lora_against_the_oracle(pieces, ref, recompute):
     assert np.all(np.abs(lh - lr) <= 1e-5 * np.abs(lr))
     for i, (h, r) in enumerate(zip(aux, rparams)):
         assert_close(h.grad, r.grad, f"lora adapter {i} with bf16 pieces")
+
+
+@pytest.mark.parametrize("m,n", [(128, 640), (640, 128), (200, 72), (640, 640), (64, 2048)])
+def test_newton_schulz_on_the_piece_kernels(pieces, ref, m, n):
+    """Muon's Newton-Schulz products (batched, with the scaled write-back b A + c A.A and a X + B.X) at the gemma widths."""
+    import test_gpu_optim
+    test_gpu_optim.test_newton_schulz(pieces, ref, m, n)
+
+
+def test_muon_trajectory_on_the_piece_kernels(pieces, ref):
+    import test_gpu_optim
+    test_gpu_optim.test_four_step_trajectory_vs_cpu_trainer(pieces, ref, "muon_wsd")
+
+
+def test_fifty_step_loss_curve_on_the_piece_kernels(pieces, ref):
+    """The 50-step loss curve gate (1e-3 relative) with every aligned product of the tiny model on the piece kernels."""
+    import test_gpu_optim
+    test_gpu_optim.test_fifty_step_loss_curve(pieces, ref)
