@@ -302,6 +302,13 @@ def micro_kernels(gpu, L, reps=10, sustained=30):
     flop = 2.0 * R * H * F
     sus = {"gemm.nn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.NN, 0, R, H, F, dY, W, dX), "dX"), flop),
            "gemm.tn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.TN, 0, F, H, R, dY, X, dW), "dW"), flop)}
+    # the same two products on the bf16-piece kernels ("gemm.split_bf16"), sustained, for the line's bf16_pieces figures
+    gpu.set_option("gemm.split_bf16", 1)
+    try:
+        sus_p = {"gemm.nn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.NN, 0, R, H, F, dY, W, dX), "dX"), flop),
+                 "gemm.tn": sustained_rate(lambda: L.check(c, lib.gt_gemm(c, L.TN, 0, F, H, R, dY, X, dW), "dW"), flop)}
+    finally:
+        gpu.set_option("gemm.split_bf16", 0)
     out = {}
     names = {"gemm.nn": ("dX = dY.W  [16384x576x1536]", "mfma"), "gemm.tn": ("dW = dY^T.X [1536x576x16384]", "mfma"),
              "ce.bwd": ("softmax-CE backward [16384x49152]", "hbm"), "ce": ("CE forward statistics [16384x49152]", "hbm"),
@@ -325,6 +332,9 @@ def micro_kernels(gpu, L, reps=10, sustained=30):
             out[desc]["sustained_frac"] = round(sus[key][1] / PEAK_FP32_MFMA, 4)
             out[desc]["sustained"] = (f"{sustained} launches back to back inside one event pair, after {SETTLE} untimed ones that let the clocks settle "
                                       f"(the reduction pass of a split-K product included)")
+            out[desc]["bf16_pieces_sustained"] = {"us_per_launch": round(1e3 * sus_p[key][0], 1), "achieved": round(sus_p[key][1] / 1e12, 3),
+                                                  "frac_of_fp32_mfma_peak": round(sus_p[key][1] / PEAK_FP32_MFMA, 4),
+                                                  "executed_frac_of_bf16_mfma_peak": round(6 * sus_p[key][1] / PEAK_BF16_MFMA, 4)}
     for key, desc in (("rmsnorm.bwd", "RMSNorm backward [131072x576] (8x the rows, 10 launches back to back)"),
                       ("add", "yardstick out = a + b [131072x576] (8x the rows, 10 launches back to back)")):
         rate = 12.0 * R8 * H / (big[key] * 1e-3)

@@ -331,3 +331,25 @@ def test_fifty_step_loss_curve_on_the_piece_kernels(pieces, ref):
     """The 50-step loss curve gate (1e-3 relative) with every aligned product of the tiny model on the piece kernels."""
     import test_gpu_optim
     test_gpu_optim.test_fifty_step_loss_curve(pieces, ref)
+
+
+def test_recompute_on_and_off_stay_bit_identical(pieces, ref):
+    """The grouped dW products' K split follows K alone on the piece kernels too: with and without recomputed regions the
+    host groups different sets of products, and the gradients may not differ by a bit."""
+    import test_gpu_model
+    test_gpu_model.test_recompute_is_bit_identical_and_matches(pieces, ref, "llama")
+
+
+def test_two_runs_give_the_same_bits(pieces):
+    gpu = pieces
+    rs = np.random.RandomState(1)
+    M, N, K = 640, 576, 4096
+    a, b = rs.standard_normal((K, M)).astype(np.float32), rs.standard_normal((K, N)).astype(np.float32)
+    da, db, dc = bufs(gpu, a, b, np.zeros((M, N), np.float32))
+    runs = []
+    for _ in range(2):
+        gpu.gemm(2, 0, M, N, K, da, db, dc)          # dW with a K split: partials summed in split order
+        runs.append(gpu.read_state_buffer(dc, M * N).copy())
+    assert np.array_equal(runs[0], runs[1])
+    for h in (da, db, dc):
+        gpu.free_state_buffer(h)
