@@ -49,6 +49,7 @@
 #include <algorithm>
 #include <type_traits>
 #include "common.h"
+#include "bf16_pieces.h"
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -181,6 +182,69 @@ __device__ __forceinline__ void t_dot_acc(v16f (&out)[HD / 32], const float *lds
   }
 }
 
+// ---- the forward's contractions on the bf16 matrix instruction (bf16_pieces.h): a lane's 8 consecutive k per MFMA -----------------------
+// this lane's row as pieces: qp[c] = pieces of x[16c + 8g + (0..7)] * mul
+__device__ __forceinline__ void load_row_pieces(v4u (&qp)[HD / 16][3], const float *__restrict__ row, bool valid, int g, float mul) {
+#pragma unroll
+  for (int c = 0; c < HD / 16; c++) {
+    v4f lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+    if (valid) { lo = *reinterpret_cast<const v4f *>(row + 16 * c + 8 * g); hi = *reinterpret_cast<const v4f *>(row + 16 * c + 8 * g + 4); }
+    const float x[8] = {lo[0] * mul, lo[1] * mul, lo[2] * mul, lo[3] * mul, hi[0] * mul, hi[1] * mul, hi[2] * mul, hi[3] * mul};
+    cut8(x, qp[c]);
+  }
+}
+// acc[n] = Tile(32 rows starting at rows + n * 32 * LD) . row^T for N sub-tiles at once: their MFMAs alternate, so that (for N > 1) no MFMA
+// waits for the one before it on the same accumulator
+template <int N>
+__device__ __forceinline__ void rows_dot_pieces(v16f (&acc)[N], const float *rows, const v4u (&qp)[HD / 16][3], int l32, int g) {
+  constexpr int TA[6] = GT_PIECE_TERMS_A, TB[6] = GT_PIECE_TERMS_B;
+#pragma unroll
+  for (int n = 0; n < N; n++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[n][r] = 0.f;
+#pragma unroll
+  for (int c = 0; c < HD / 16; c++) {
+    v4u ka[N][3];
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+      const float *src = rows + (n * 32 + l32) * LD + 16 * c + 8 * g;
+      const v4f lo = *reinterpret_cast<const v4f *>(src), hi = *reinterpret_cast<const v4f *>(src + 4);
+      const float x[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      cut8(x, ka[n]);
+    }
+#pragma unroll
+    for (int t = 0; t < 6; t++)
+#pragma unroll
+      for (int n = 0; n < N; n++)
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, ka[n][TA[t]]), __builtin_bit_cast(v8bf, qp[c][TB[t]]), acc[n], 0, 0, 0);
+  }
+}
+// out[dt] += TileT(cols [col0, col0+32)) . w, w in accumulator order: MFMA j takes w[8j .. 8j+7], the keys 16j + 4g + (0..3) and 16j + 8 + 4g + (0..3)
+template <int LDT>
+__device__ __forceinline__ void t_dot_pieces(v16f (&out)[HD / 32], const float *ldst, int col0, const float (&w)[16], int l32, int g) {
+  constexpr int DT = HD / 32;
+  constexpr int TA[6] = GT_PIECE_TERMS_A, TB[6] = GT_PIECE_TERMS_B;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    v4u pw[3], va[DT][3];
+    const float xw[8] = {w[8 * j], w[8 * j + 1], w[8 * j + 2], w[8 * j + 3], w[8 * j + 4], w[8 * j + 5], w[8 * j + 6], w[8 * j + 7]};
+    cut8(xw, pw);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      const int d = dt * 32 + l32, chunk = (col0 >> 2) + 4 * j + g;
+      const v4f lo = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * (chunk ^ ((d >> 3) & 7)));
+      const v4f hi = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * ((chunk + 2) ^ ((d >> 3) & 7)));
+      const float x[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      cut8(x, va[dt]);
+    }
+#pragma unroll
+    for (int t = 0; t < 6; t++)
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+        out[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, va[dt][TA[t]]), __builtin_bit_cast(v8bf, pw[TB[t]]), out[dt], 0, 0, 0);
+  }
+}
+
 __device__ __forceinline__ void store_row(float *row, const v16f (&acc)[HD / 32], int g, float mul, int add) {
   v4f old[HD / 32][4];
   if (add) {          // every old value first: a load behind a store to the same array would wait for it
@@ -256,7 +320,10 @@ __device__ __forceinline__ void store_grad_row(float *row, const v16f (&acc)[HD 
 // scheduler can run the softmax of one sub-tile, the LDS stores and the loads under the MFMAs of another.
 #define FWD_BUF (KT * LD + HD * (KT + 4))        // floats per buffer: K rows, V transposed
 #define FWD_SMEM (2 * FWD_BUF * sizeof(float))
-template <bool KEEP>
+// PX: both contractions on the bf16 matrix instruction (the query row, the K and V^T tiles and the probabilities as bf16 pieces, cut in
+// registers by every wavefront that reads them). dK/dV stays on the FP32 instruction: its 32-query stages are cut by all four wavefronts,
+// twice (row-major and transposed use), and the piece form measured slower there (739-779 against 668-677 us per launch).
+template <bool KEEP, bool PX = false>
 __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, float *__restrict__ out,
                                                        float *__restrict__ lse, float *__restrict__ fpart, float *sco) {
@@ -278,8 +345,19 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP
   const bool tv = t < p.T;
   const float *kb = k + (size_t)b * p.T * kstr + (size_t)kvh * HD;
   const float *vb = v + (size_t)b * p.T * kstr + (size_t)kvh * HD;
-  float qreg[HD / 2];
-  load_row_regs(qreg, q + ((size_t)b * p.T + (tv ? t : 0)) * qstr + (size_t)h * HD, tv, g, p.c2);
+  float qreg[PX ? 1 : HD / 2];
+  v4u qp[PX ? HD / 16 : 1][3];
+  if constexpr (PX) load_row_pieces(qp, q + ((size_t)b * p.T + (tv ? t : 0)) * qstr + (size_t)h * HD, tv, g, p.c2);
+  else load_row_regs(qreg, q + ((size_t)b * p.T + (tv ? t : 0)) * qstr + (size_t)h * HD, tv, g, p.c2);
+  // the two contractions of a 32-key sub-tile, either way
+  auto scores1 = [&](const float *rows) {
+    if constexpr (PX) { v16f a1[1]; rows_dot_pieces<1>(a1, rows, qp, l32, g); return a1[0]; }
+    else return rows_dot_regs<FWD_NB>(rows, qreg, l32, g);
+  };
+  auto weighted = [&](v16f (&o)[HD / 32], const float *ldst, int col0, const float (&w)[16]) {
+    if constexpr (PX) t_dot_pieces<IO::LDT>(o, ldst, col0, w, l32, g);
+    else t_dot_acc<IO::LDT, FWD_NB>(o, ldst, col0, w, l32, g);
+  };
   const int lo_t = win_lo_m(t, p.window);
   int kt_lo = win_lo_m(qtile * 128, p.window) / KT;
   int kt_hi = min(p.T - 1, qtile * 128 + 127) / KT;
@@ -335,9 +413,13 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP
     float pr[NSUB][16];
     if (plain) {
       float mx = NEG_BIG;
+      v16f sall[NSUB];
+      if constexpr (PX) rows_dot_pieces<NSUB>(sall, sK, qp, l32, g);
 #pragma unroll
       for (int sub = 0; sub < NSUB; sub++) {
-        v16f s = rows_dot_regs<FWD_NB>(sK + sub * 32 * LD, qreg, l32, g);
+        v16f s;
+        if constexpr (PX) s = sall[sub];
+        else s = rows_dot_regs<FWD_NB>(sK + sub * 32 * LD, qreg, l32, g);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           pr[sub][r] = s[r];
@@ -374,7 +456,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP
           IO::store_rows(pt, nxt, tid);
           load_tile(vb, kt + 1);
         }
-        t_dot_acc<IO::LDT, FWD_NB>(oacc, sVt, sub * 32, pr[sub], l32, g);
+        weighted(oacc, sVt, sub * 32, pr[sub]);
       }
     } else {
       IO::store_rows(pt, nxt, tid);
@@ -386,7 +468,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP
         for (int sub = 0; sub < NSUB; sub++) {
           if (!act[sub]) continue;
           const int k0 = kt * KT + sub * 32;
-          v16f s = rows_dot_regs<FWD_NB>(sK + sub * 32 * LD, qreg, l32, g);
+          v16f s = scores1(sK + sub * 32 * LD);
           const bool need_mask = ragged || k0 + 31 > tq0 || k0 < wave_lo_last;
           msk[sub] = need_mask;
           if (need_mask) {
@@ -429,7 +511,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP
             ls += e;
           }
           l += ls;
-          t_dot_acc<IO::LDT, FWD_NB>(oacc, sVt, sub * 32, pr[sub], l32, g);
+          weighted(oacc, sVt, sub * 32, pr[sub]);
         }
       }
     }
@@ -804,6 +886,25 @@ int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
     ctx->attn_smem_set |= HD << 8;
   }
   dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
+#if HD == 64
+  if (ctx->opt_attn_pieces) {          // "attn.split_bf16": the forward of head dim 64 on the bf16 matrix instruction
+    if (!(ctx->attn_smem_set & (1 << 20))) {
+      GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_fwd_mfma_k)<false, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)FWD_SMEM));
+      GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_fwd_mfma_k)<true, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)FWD_SMEM));
+      ctx->attn_smem_set |= 1 << 20;
+    }
+    if (sco)
+      hipLaunchKernelGGL((FN(attn_fwd_mfma_k)<true, true>), grid, dim3(256), FWD_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
+                         P<const float>(v), P<float>(out), P<float>(lse), fpart, sco);
+    else
+      hipLaunchKernelGGL((FN(attn_fwd_mfma_k)<false, true>), grid, dim3(256), FWD_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
+                         P<const float>(v), P<float>(out), P<float>(lse), fpart, sco);
+    GT_LAUNCHED(ctx);
+    return 0;
+  }
+#endif
   if (sco)
     hipLaunchKernelGGL(FN(attn_fwd_mfma_k)<true>, grid, dim3(256), FWD_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k),
                        P<const float>(v), P<float>(out), P<float>(lse), fpart, sco);

@@ -198,6 +198,7 @@ int gt_set_option(gt_ctx *ctx, const char *key, int value) {
   else if (!strcmp(key, "gemm.staged")) ctx->opt_gemm_staged = value;
   else if (!strcmp(key, "gemm.group")) ctx->opt_gemm_group = value;
   else if (!strcmp(key, "gemm.split_bf16")) ctx->opt_gemm_split = value;
+  else if (!strcmp(key, "attn.split_bf16")) ctx->opt_attn_pieces = value;
   else if (!strcmp(key, "gemm.sum_min_tiles")) ctx->opt_gemm_sum_min_tiles = value;
   else GT_FAIL(ctx, "gt_set_option: unknown key '%s'", key);
   return 0;

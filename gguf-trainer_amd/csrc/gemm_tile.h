@@ -354,20 +354,7 @@ struct DirectTile {
 // v_mfma_f32_32x32x2_f32, so the six products per pair cost 3/8 of the FP32 instruction's time, and against float64 the
 // result is as close as the FP32 MFMA's (the accumulation is FP32 either way). Infinities and NaNs come out as NaN
 // (inf - inf in the split).
-typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
-typedef unsigned v2u __attribute__((ext_vector_type(2)));
-typedef unsigned v4u __attribute__((ext_vector_type(4)));
-
-// two consecutive elements' pieces as one register each: (h, m, l) of x0 in the low halves, of x1 in the high halves
-__device__ __forceinline__ void split_pair(float x0, float x1, unsigned &h, unsigned &m, unsigned &l) {
-  const unsigned h0 = __float_as_uint(x0) & 0xFFFF0000u, h1 = __float_as_uint(x1) & 0xFFFF0000u;
-  const float r0 = x0 - __uint_as_float(h0), r1 = x1 - __uint_as_float(h1);
-  const unsigned m0 = __float_as_uint(r0) & 0xFFFF0000u, m1 = __float_as_uint(r1) & 0xFFFF0000u;
-  const float q0 = r0 - __uint_as_float(m0), q1 = r1 - __uint_as_float(m1);
-  h = __builtin_amdgcn_perm(h1, h0, 0x07060302);
-  m = __builtin_amdgcn_perm(m1, m0, 0x07060302);
-  l = __builtin_amdgcn_perm(__float_as_uint(q1), __float_as_uint(q0), 0x07060302);
-}
+#include "bf16_pieces.h"
 
 // The MFMA inputs of one lane from an operand tile as DirectTile leaves it in LDS (FP32): the 8 consecutive k
 // (16c + 8g ...) of `row`, cut into pieces here, in registers, by every wavefront that reads them. The vector work hides

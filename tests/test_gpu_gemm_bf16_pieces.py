@@ -353,3 +353,53 @@ def test_two_runs_give_the_same_bits(pieces):
     assert np.array_equal(runs[0], runs[1])
     for h in (da, db, dc):
         gpu.free_state_buffer(h)
+
+
+# ---- "attn.split_bf16": the attention forward of head dim 64 on the same instruction ------------------------------------------------
+
+@pytest.fixture()
+def attn_pieces(gpu):
+    gpu.set_option("attn.split_bf16", 1)
+    yield gpu
+    gpu.set_option("attn.split_bf16", 0)
+    gpu.set_option("attn.splits", -1)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 700, 4, 2, 64, 0), (2, 333, 6, 2, 64, 300), (1, 1024, 9, 3, 64, 0), (3, 129, 2, 1, 64, 33),
+                                                  (1, 512, 3, 3, 64, 512)])
+@pytest.mark.parametrize("splits", [-1, 1, 5])
+def test_attention_forward_pieces_ragged_windows_gqa_splits(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits):
+    """The head-dim-64 cases of the matrix-core attention tests with the forward on bf16 pieces: ragged T, windows that cut tiles, GQA,
+    stacked sequences, split launches; output and all three gradients (the backward reads the forward's output and statistic)
+    against the oracle at the FP32 kernels' tolerances."""
+    import test_gpu_ops
+    test_gpu_ops.test_attention_mfma_shapes(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 1, 2, 1, 64, 0), (2, 31, 4, 2, 64, 0), (1, 65, 2, 1, 64, 0), (1, 97, 3, 1, 64, 40),
+                                                  (1, 128, 2, 1, 64, 1), (2, 160, 4, 4, 64, 1000)])
+def test_attention_forward_pieces_tile_edges(attn_pieces, ref, B, T, Hq, Hkv, hd, window):
+    import test_gpu_ops
+    test_gpu_ops.test_attention_mfma_tile_edges(attn_pieces, ref, B, T, Hq, Hkv, hd, window)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 640, 2, 2, 64, 129), (1, 256, 3, 1, 64, 1),
+                                                  (1, 1024, 9, 3, 64, 0)])
+@pytest.mark.parametrize("splits,keep_ds", [(1, 1), (3, 1), (1, 0)])
+def test_attention_forward_pieces_kept_scores(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits, keep_ds):
+    """The kept scores the piece forward writes feed the FP32 dK/dV kernel: same output and statistic bit for bit with and without
+    keeping them, gradients to the parity bound, dq of the first sequence against the oracle."""
+    import test_gpu_ops
+    test_gpu_ops.test_attention_kept_scores_equals_recomputed(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits, keep_ds)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,path", [(2, 2048, 9, 3, 64, 0, "kept-scores"), (1, 2048, 10, 2, 64, 512, "kept-scores"),
+                                                       (1, 2048, 9, 3, 64, 0, "recompute")])
+def test_attention_forward_pieces_full_length(attn_pieces, ref, B, T, Hq, Hkv, hd, window, path):
+    import test_gpu_production_shapes
+    test_gpu_production_shapes.test_attention_full_length_vs_oracle(attn_pieces, ref, B, T, Hq, Hkv, hd, window, path)
+
+
+@pytest.mark.parametrize("name", ["smollm2", "gemma3-window"])
+def test_whole_models_with_both_options(pieces, attn_pieces, ref, name):
+    test_real_head_geometry_against_the_oracle(pieces, ref, name, True)
