@@ -182,7 +182,7 @@ __device__ __forceinline__ void t_dot_acc(v16f (&out)[HD / 32], const float *lds
   }
 }
 
-// ---- the forward's contractions on the bf16 matrix instruction (bf16_pieces.h): a lane's 8 consecutive k per MFMA -----------------------
+// ---- attention's contractions on the bf16 matrix instruction (bf16_pieces.h): a lane's 8 consecutive k per MFMA --------------------------
 // this lane's row as pieces: qp[c] = pieces of x[16c + 8g + (0..7)] * mul
 __device__ __forceinline__ void load_row_pieces(v4u (&qp)[HD / 16][3], const float *__restrict__ row, bool valid, int g, float mul) {
 #pragma unroll
@@ -217,6 +217,30 @@ __device__ __forceinline__ void rows_dot_pieces(v16f (&acc)[N], const float *row
 #pragma unroll
       for (int n = 0; n < N; n++)
         acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, ka[n][TA[t]]), __builtin_bit_cast(v8bf, qp[c][TB[t]]), acc[n], 0, 0, 0);
+  }
+}
+// the same with one head-dim block in flight (12 registers fewer; its six MFMAs wait on one another): dK/dV
+template <int LDT>
+__device__ __forceinline__ void t_dot_pieces_lean(v16f (&out)[HD / 32], const float *ldst, int col0, const float (&w)[16], int l32, int g) {
+  constexpr int DT = HD / 32;
+  constexpr int TA[6] = GT_PIECE_TERMS_A, TB[6] = GT_PIECE_TERMS_B;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    v4u pw[3];
+    const float xw[8] = {w[8 * j], w[8 * j + 1], w[8 * j + 2], w[8 * j + 3], w[8 * j + 4], w[8 * j + 5], w[8 * j + 6], w[8 * j + 7]};
+    cut8(xw, pw);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      v4u va[3];
+      const int d = dt * 32 + l32, chunk = (col0 >> 2) + 4 * j + g;
+      const v4f lo = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * (chunk ^ ((d >> 3) & 7)));
+      const v4f hi = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * ((chunk + 2) ^ ((d >> 3) & 7)));
+      const float x[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      cut8(x, va);
+#pragma unroll
+      for (int t = 0; t < 6; t++)
+        out[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, va[TA[t]]), __builtin_bit_cast(v8bf, pw[TB[t]]), out[dt], 0, 0, 0);
+    }
   }
 }
 // out[dt] += TileT(cols [col0, col0+32)) . w, w in accumulator order: MFMA j takes w[8j .. 8j+7], the keys 16j + 4g + (0..3) and 16j + 8 + 4g + (0..3)
@@ -321,8 +345,7 @@ __device__ __forceinline__ void store_grad_row(float *row, const v16f (&acc)[HD 
 #define FWD_BUF (KT * LD + HD * (KT + 4))        // floats per buffer: K rows, V transposed
 #define FWD_SMEM (2 * FWD_BUF * sizeof(float))
 // PX: both contractions on the bf16 matrix instruction (the query row, the K and V^T tiles and the probabilities as bf16 pieces, cut in
-// registers by every wavefront that reads them). dK/dV stays on the FP32 instruction: its 32-query stages are cut by all four wavefronts,
-// twice (row-major and transposed use), and the piece form measured slower there (739-779 against 668-677 us per launch).
+// registers by every wavefront that reads them).
 template <bool KEEP, bool PX = false>
 __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_fwd_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                        const float *__restrict__ v, float *__restrict__ out,
@@ -632,7 +655,12 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 // filled during stage it-1) while stage it computes on the other buffer, the loads of stage it+2 follow, and one barrier
 // ends the stage. None of that depends on the stage's MFMAs, and it is straight-line code, so it runs under them.
 #define DKV_BUF (2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT)        // floats per buffer: sQ, sG, sQt, sGt, lse, D
-template <bool KS, bool DS>
+// PX: the three (four without kept scores) contractions on the bf16 matrix instruction: this lane's key / value row as pieces cut once, the Q
+// and dO tiles (row-major and transposed) and the probabilities / score gradients cut as they are read. The register file is the limit
+// at two wavefronts per SIMD: one head-dim block of the transposed tiles at a time and one accumulator chain per score block keep it at 255-256
+// registers (6 spilled with kept scores and kept dS; 39 with two blocks in flight, which ran slower than the FP32 kernel, as did one
+// wavefront per SIMD without spills).
+template <bool KS, bool DS, bool PX = false>
 __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
                                                            const float *__restrict__ lse, const float *__restrict__ Dr,
@@ -657,9 +685,15 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   const int sk0 = ktile * 128 + wave * 32, s = sk0 + l32;
   const bool sv = s < p.T;
   const size_t koff = ((size_t)b * p.T + (sv ? s : 0)) * kstr + (size_t)kvh * HD;
-  float kreg[KS ? 1 : HD / 2], vreg[HD / 2];
-  if constexpr (!KS) load_row_regs(kreg, k + koff, sv, g, p.c2);
-  load_row_regs(vreg, v + koff, sv, g, 1.0f);
+  float kreg[KS || PX ? 1 : HD / 2], vreg[PX ? 1 : HD / 2];
+  v4u kp[PX && !KS ? HD / 16 : 1][3], vp[PX ? HD / 16 : 1][3];
+  if constexpr (PX) {
+    if constexpr (!KS) load_row_pieces(kp, k + koff, sv, g, p.c2);
+    load_row_pieces(vp, v + koff, sv, g, 1.0f);
+  } else {
+    if constexpr (!KS) load_row_regs(kreg, k + koff, sv, g, p.c2);
+    load_row_regs(vreg, v + koff, sv, g, 1.0f);
+  }
   // queries that can see a key of this workgroup: t in [ktile*128, last key + window - 1]
   const int qt_lo = ktile * (128 / QT);
   // With a dS matrix to fill (dsb: T a multiple of 128), the loop runs on to the end of the last 128-row tile whose
@@ -791,7 +825,10 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
       // at head dim 128 without kept scores both operand rows live in registers (128 of them): four LDS reads in flight
       // instead of eight keep the kernel inside the register file
       constexpr int DKV_NB = (HD >= 128 && !KS) ? 4 : 8;
-      if constexpr (!KS) sc = rows_dot_regs<DKV_NB>(sQ, kreg, l32, g);
+      if constexpr (!KS) {
+        if constexpr (PX) { v16f a1[1]; rows_dot_pieces<1>(a1, sQ, kp, l32, g); sc = a1[0]; }
+        else sc = rows_dot_regs<DKV_NB>(sQ, kreg, l32, g);
+      }
       // The stage as straight-line code. A pair (query tq, key s) is live when s <= tq <= last query that sees s: one
       // unsigned compare per element against this lane's span (computed once per kernel), applied to every tile: a
       // wave-uniform "does this tile need a mask" test would cut the stage into basic blocks, and the scheduler cannot
@@ -800,7 +837,9 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
       // only) between dP and the dS arithmetic: the vector ALU work has independent MFMAs to run under instead of sitting
       // between two dependent blocks, and the group barriers ask for that interleaving (one MFMA, a few vector
       // instructions, and again).
-      v16f dp = rows_dot_regs<DKV_NB>(sG, vreg, l32, g);
+      v16f dp;
+      if constexpr (PX) { v16f a1[1]; rows_dot_pieces<1>(a1, sG, vp, l32, g); dp = a1[0]; }
+      else dp = rows_dot_regs<DKV_NB>(sG, vreg, l32, g);
       float pr[16], ds[16];
       const unsigned rel0 = (unsigned)(t0 + 4 * g - s) + dead;          // query index relative to this lane's key, element (a, j) adds 8a + j
 #pragma unroll
@@ -812,22 +851,27 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
           pr[4 * a + j] = (rel0 + (unsigned)(8 * a + j)) <= span ? e : 0.f;
         }
       }
+      if constexpr (!PX) {
 #pragma unroll
-      for (int i = 0; i < HD / 2; i++) {          // dP with the exponentials
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        for (int i = 0; i < HD / 2; i++) {          // dP with the exponentials
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        }
       }
-      t_dot_acc<IO::LDT, DKV_NB>(vacc, sGt, 0, pr, l32, g);
+      if constexpr (PX) t_dot_pieces_lean<IO::LDT>(vacc, sGt, 0, pr, l32, g);
+      else t_dot_acc<IO::LDT, DKV_NB>(vacc, sGt, 0, pr, l32, g);
 #pragma unroll
       for (int a = 0; a < 4; a++) {
         v4f dv4 = *reinterpret_cast<const v4f *>(sD + 8 * a + 4 * g);
 #pragma unroll
         for (int j = 0; j < 4; j++) ds[4 * a + j] = pr[4 * a + j] * (dp[4 * a + j] - dv4[j]) * p.scale;
       }
+      if constexpr (!PX) {
 #pragma unroll
-      for (int i = 0; i < HD / 2; i++) {          // dV with the dS arithmetic
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        for (int i = 0; i < HD / 2; i++) {          // dV with the dS arithmetic
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        }
       }
       // next stage's tile into the idle buffer (its loads were issued a stage ago), this stage's dS out, the loads of the
       // stage after next: all independent of the dK contraction that follows
@@ -840,7 +884,8 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
         load_q(it + 2);
         load_g(it + 2);
       }
-      t_dot_acc<IO::LDT, DKV_NB>(kacc, sQt, 0, ds, l32, g);
+      if constexpr (PX) t_dot_pieces_lean<IO::LDT>(kacc, sQt, 0, ds, l32, g);
+      else t_dot_acc<IO::LDT, DKV_NB>(kacc, sQt, 0, ds, l32, g);
     }
     stage_end(nxt, it);
     __syncthreads();
@@ -953,6 +998,23 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
       hipLaunchKernelGGL(kern, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k), P<const float>(v),
                          P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco, rot_k);
     };
+#if HD == 64
+    if (ctx->opt_attn_pieces) {          // "attn.split_bf16": dK/dV of head dim 64 on the bf16 matrix instruction
+      if (!(ctx->attn_smem_set & (1 << 21))) {
+        GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false, false, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+        GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false, true, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+        GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, false, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+        GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, true, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+        ctx->attn_smem_set |= 1 << 21;
+      }
+      if (sco) dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false, true>);
+      else dsb ? launch(FN(attn_bwd_dkv_mfma_k)<false, true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<false, false, true>);
+    } else
+#endif
     if (sco) dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false>);
     else dsb ? launch(FN(attn_bwd_dkv_mfma_k)<false, true>) : launch(FN(attn_bwd_dkv_mfma_k)<false, false>);
     GT_LAUNCHED(ctx);

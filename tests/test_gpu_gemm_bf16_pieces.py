@@ -355,7 +355,7 @@ def test_two_runs_give_the_same_bits(pieces):
         gpu.free_state_buffer(h)
 
 
-# ---- "attn.split_bf16": the attention forward of head dim 64 on the same instruction ------------------------------------------------
+# ---- "attn.split_bf16": the attention forward and dK/dV of head dim 64 on the same instruction ------------------------------------
 
 @pytest.fixture()
 def attn_pieces(gpu):
@@ -391,6 +391,23 @@ def test_attention_forward_pieces_kept_scores(attn_pieces, ref, B, T, Hq, Hkv, h
     keeping them, gradients to the parity bound, dq of the first sequence against the oracle."""
     import test_gpu_ops
     test_gpu_ops.test_attention_kept_scores_equals_recomputed(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits, keep_ds)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 512, 2, 1, 64, 127), (1, 768, 2, 1, 64, 300)])
+@pytest.mark.parametrize("acc,splits", [(0, 1), (1, 1), (0, 5), (1, 3)])
+def test_attention_pieces_kept_score_gradients(attn_pieces, ref, B, T, Hq, Hkv, hd, window, acc, splits):
+    """dK/dV on pieces writes the score gradients the banded dQ product reads: against the pair that recomputes them and the oracle.
+    (Window 1, where dq is exactly zero and the two pairs are compared on their rounding residue alone, is left to the FP32 kernels'
+    test: the dQ kernel that recomputes stays on FP32 MFMA, so the residues differ.)"""
+    import test_gpu_ops
+    test_gpu_ops.test_attention_backward_kept_ds_equals_recomputed(attn_pieces, ref, B, T, Hq, Hkv, hd, window, acc, splits)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,keep_ds", [(1, 256, 4, 2, 64, 0, 1), (2, 128, 3, 3, 64, 0, 1), (2, 256, 6, 2, 64, 70, 0), (8, 256, 9, 3, 64, 0, 1)])
+@pytest.mark.parametrize("acc", [0, 1])
+def test_attention_pieces_rotations_in_the_write_backs(attn_pieces, B, T, Hq, Hkv, hd, window, keep_ds, acc):
+    import test_gpu_ops
+    test_gpu_ops.test_attention_backward_with_the_rotations_backward_in_its_write_backs(attn_pieces, B, T, Hq, Hkv, hd, window, keep_ds, acc)
 
 
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,path", [(2, 2048, 9, 3, 64, 0, "kept-scores"), (1, 2048, 10, 2, 64, 512, "kept-scores"),
