@@ -658,8 +658,9 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 // PX: the three (four without kept scores) contractions on the bf16 matrix instruction: this lane's key / value row as pieces cut once, the Q
 // and dO tiles (row-major and transposed) and the probabilities / score gradients cut as they are read. The register file is the limit
 // at two wavefronts per SIMD: one head-dim block of the transposed tiles at a time and one accumulator chain per score block keep it at 255-256
-// registers (6 spilled with kept scores and kept dS; 39 with two blocks in flight, which ran slower than the FP32 kernel, as did one
-// wavefront per SIMD without spills).
+// registers (6 spilled with kept scores and kept dS: 554 us per launch; without the stage of look-ahead for the kept scores nothing
+// spills and it takes 584; 39 spilled with two blocks in flight, which ran slower than the FP32 kernel's 668-679, as did one wavefront
+// per SIMD without spills). Only with kept scores: the key row's pieces for recomputing them do not fit.
 template <bool KS, bool DS, bool PX = false>
 __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
@@ -999,20 +1000,16 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
                          P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco, rot_k);
     };
 #if HD == 64
-    if (ctx->opt_attn_pieces) {          // "attn.split_bf16": dK/dV of head dim 64 on the bf16 matrix instruction
+    if (ctx->opt_attn_pieces && sco) {          // "attn.split_bf16": dK/dV of head dim 64 on the bf16 matrix instruction, where the forward kept
+                                                // its scores (recomputing them needs the key row's pieces too: 34-37 registers spilled)
       if (!(ctx->attn_smem_set & (1 << 21))) {
-        GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false, false, true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
-        GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<false, true, true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
         GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, false, true>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
         GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, true, true>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
         ctx->attn_smem_set |= 1 << 21;
       }
-      if (sco) dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false, true>);
-      else dsb ? launch(FN(attn_bwd_dkv_mfma_k)<false, true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<false, false, true>);
+      dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false, true>);
     } else
 #endif
     if (sco) dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false>);
