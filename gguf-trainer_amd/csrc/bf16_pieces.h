@@ -1,6 +1,7 @@
 // FP32 numbers as bf16 pieces: x = h + m + l exactly, each piece a bf16 (8 significant bits): h = x cut to its upper 16 bits,
 // m = x - h cut likewise, l = the rest. Used by the kernels that run FP32 contractions on v_mfma_f32_32x32x16_bf16
 // (six of the nine piece products; the three smallest, below 2^-24 of the whole, are left out).
+// The pieces keep FP32's exponent range, so nothing is scaled; an x below 2^-110 has lower pieces that are bf16 denormals.
 #pragma once
 #include <hip/hip_runtime.h>
 

@@ -78,7 +78,8 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
  *   "gemm.split_bf16" 1 = every product the LDS-direct kernels take (K a multiple of 32, whole 16-byte chunks along each operand's
  *                  contiguous index; a second segment of 16 or 32) runs on the bf16 matrix instruction: each FP32 element as three
  *                  exact bf16 pieces, six of the nine piece products, FP32 accumulation. As close to float64 as the FP32 MFMA kernels,
- *                  about 1.3 x their rate; not bit-identical to them; inf / NaN operands give NaN. 0 (default) = FP32 MFMA
+ *                  about 1.3 x their rate; not bit-identical to them; inf / NaN operands give NaN, and operands below 2^-110 in
+ *                  magnitude lose their lower pieces (they would be bf16 denormals). 0 (default) = FP32 MFMA
  *   "gemm.sum_min_tiles" gt_gemm_sum chains its products in one loop from this many 128-row output tiles on
  *                  (-1 = one per CU, the default; 0 = always, for tests of the chained kernel on small shapes)
  *   "attn.splits"  -1 = heuristic, n >= 1 = pin the workgroups per attention tile (MFMA kernels, at most 8)
