@@ -201,7 +201,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
   int cfg = 0, splits = 1;
   // "gemm.split_bf16": every product the direct kernels take runs on the bf16 MFMA instead, on 128 x 192 or 128 x 128 tiles
   const bool split = direct_ok && ctx->opt_gemm_split && (K2 == 0 || K2 == 16 || K2 == 32) && !ctx->opt_gemm_staged;
-  const bool wide = N % 192 == 0 && ctx->opt_gemm_split != 3;
+  const bool wide = N % 192 == 0;
   pick_tile(ctx, kind, direct_ok, 1, &M, &N, K, count, K2 > 0, &cfg, &splits, 0, split ? (wide ? 7 : 6) : -1);
   if (!split && ctx->opt_gemm_tile >= 0 && ctx->opt_gemm_tile < NCFG) cfg = ctx->opt_gemm_tile;
   const int bm = kTiles[cfg].bm, bn = kTiles[cfg].bn, bk = kTiles[cfg].bk;
