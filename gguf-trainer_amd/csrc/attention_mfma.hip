@@ -202,6 +202,26 @@ __device__ __forceinline__ void rows_dot_pieces(v16f (&acc)[N], const float *row
   for (int n = 0; n < N; n++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[n][r] = 0.f;
+  if constexpr (N == 1 && HD >= 128) {          // one sub-tile, registers to spare: its six terms alternate between two accumulators
+    v16f other;
+#pragma unroll
+    for (int r = 0; r < 16; r++) other[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < HD / 16; c++) {
+      v4u ka[3];
+      const float *src = rows + l32 * LD + 16 * c + 8 * g;
+      const v4f lo = *reinterpret_cast<const v4f *>(src), hi = *reinterpret_cast<const v4f *>(src + 4);
+      const float x[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      cut8(x, ka);
+#pragma unroll
+      for (int t = 0; t < 6; t += 2) {
+        other = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, ka[TA[t]]), __builtin_bit_cast(v8bf, qp[c][TB[t]]), other, 0, 0, 0);
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, ka[TA[t + 1]]), __builtin_bit_cast(v8bf, qp[c][TB[t + 1]]), acc[0], 0, 0, 0);
+      }
+    }
+    acc[0] += other;
+    return;
+  }
 #pragma unroll
   for (int c = 0; c < HD / 16; c++) {
     v4u ka[N][3];
@@ -932,8 +952,8 @@ int FN(attn_fwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
     ctx->attn_smem_set |= HD << 8;
   }
   dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
-#if HD == 64
-  if (ctx->opt_attn_pieces) {          // "attn.split_bf16": the forward of head dim 64 on the bf16 matrix instruction
+#if HD == 64 || HD == 128
+  if (ctx->opt_attn_pieces) {          // "attn.split_bf16": the forward of head dims 64 and 128 on the bf16 matrix instruction
     if (!(ctx->attn_smem_set & (1 << 20))) {
       GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_fwd_mfma_k)<false, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       (int)FWD_SMEM));

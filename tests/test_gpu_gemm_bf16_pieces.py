@@ -355,7 +355,7 @@ def test_two_runs_give_the_same_bits(pieces):
         gpu.free_state_buffer(h)
 
 
-# ---- "attn.split_bf16": the attention forward and dK/dV of head dim 64 on the same instruction ------------------------------------
+# ---- "attn.split_bf16": the attention forward (head dims 64 and 128) and dK/dV (64) on the same instruction -----------------------
 
 @pytest.fixture()
 def attn_pieces(gpu):
@@ -366,7 +366,7 @@ def attn_pieces(gpu):
 
 
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 700, 4, 2, 64, 0), (2, 333, 6, 2, 64, 300), (1, 1024, 9, 3, 64, 0), (3, 129, 2, 1, 64, 33),
-                                                  (1, 512, 3, 3, 64, 512)])
+                                                  (1, 512, 3, 3, 64, 512), (1, 300, 4, 2, 128, 0), (2, 200, 8, 8, 128, 77), (1, 640, 16, 8, 128, 0)])
 @pytest.mark.parametrize("splits", [-1, 1, 5])
 def test_attention_forward_pieces_ragged_windows_gqa_splits(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits):
     """The head-dim-64 cases of the matrix-core attention tests with the forward on bf16 pieces: ragged T, windows that cut tiles, GQA,
@@ -377,13 +377,14 @@ def test_attention_forward_pieces_ragged_windows_gqa_splits(attn_pieces, ref, B,
 
 
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 1, 2, 1, 64, 0), (2, 31, 4, 2, 64, 0), (1, 65, 2, 1, 64, 0), (1, 97, 3, 1, 64, 40),
-                                                  (1, 128, 2, 1, 64, 1), (2, 160, 4, 4, 64, 1000)])
+                                                  (1, 128, 2, 1, 64, 1), (2, 160, 4, 4, 64, 1000), (1, 127, 2, 2, 128, 0), (1, 129, 2, 1, 128, 128)])
 def test_attention_forward_pieces_tile_edges(attn_pieces, ref, B, T, Hq, Hkv, hd, window):
     import test_gpu_ops
     test_gpu_ops.test_attention_mfma_tile_edges(attn_pieces, ref, B, T, Hq, Hkv, hd, window)
 
 
-@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 640, 2, 2, 64, 129), (1, 1024, 9, 3, 64, 0)])
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 640, 2, 2, 64, 129), (1, 1024, 9, 3, 64, 0),
+                                                  (2, 256, 4, 2, 128, 0), (1, 384, 2, 1, 128, 130)])
 @pytest.mark.parametrize("splits,keep_ds", [(1, 1), (3, 1), (1, 0)])
 def test_attention_forward_pieces_kept_scores(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits, keep_ds):
     """The kept scores the piece forward writes feed the piece dK/dV kernel; without them dK/dV is the FP32 kernel that recomputes.
@@ -411,12 +412,12 @@ def test_attention_pieces_rotations_in_the_write_backs(attn_pieces, B, T, Hq, Hk
 
 
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,path", [(2, 2048, 9, 3, 64, 0, "kept-scores"), (1, 2048, 10, 2, 64, 512, "kept-scores"),
-                                                       (1, 2048, 9, 3, 64, 0, "recompute")])
+                                                       (1, 2048, 9, 3, 64, 0, "recompute"), (1, 2048, 16, 8, 128, 0, "kept-scores")])
 def test_attention_forward_pieces_full_length(attn_pieces, ref, B, T, Hq, Hkv, hd, window, path):
     import test_gpu_production_shapes
     test_gpu_production_shapes.test_attention_full_length_vs_oracle(attn_pieces, ref, B, T, Hq, Hkv, hd, window, path)
 
 
-@pytest.mark.parametrize("name", ["smollm2", "gemma3-window"])
+@pytest.mark.parametrize("name", ["smollm2", "gemma3-window", "qwen3-hd128"])
 def test_whole_models_with_both_options(pieces, attn_pieces, ref, name):
     test_real_head_geometry_against_the_oracle(pieces, ref, name, True)
