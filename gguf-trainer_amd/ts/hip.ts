@@ -1093,9 +1093,16 @@ export async function initHip(device = 0): Promise<HipBackend | null> {
 }
 /** requireGPU analogue: there is no CPU path behind this backend. */
 // deno-lint-ignore require-await
-export async function requireHip(purpose: string, device = 0): Promise<HipBackend> {
+// bf16Pieces: the FP32 products and the attention kernels that have such a form on the bf16 matrix instruction (each FP32 element as three
+// exact bf16 pieces, FP32 accumulation): as close to float64 as the FP32 MFMA kernels, about 1.3 x faster steps, not bit-identical to them.
+export async function requireHip(purpose: string, device = 0, bf16Pieces = false): Promise<HipBackend> {
   try {
-    return new HipBackend(libPath(), device);
+    const hip = new HipBackend(libPath(), device);
+    if (bf16Pieces) {
+      hip.setOption("gemm.split_bf16", 1);
+      hip.setOption("attn.split_bf16", 1);
+    }
+    return hip;
   } catch (e) {
     throw new Error(`${purpose} needs an MI355X and libggufhip.so (GGUFHIP_LIB): ${(e as Error).message}`);
   }

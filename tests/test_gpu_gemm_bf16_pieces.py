@@ -421,3 +421,27 @@ def test_attention_forward_pieces_full_length(attn_pieces, ref, B, T, Hq, Hkv, h
 @pytest.mark.parametrize("name", ["smollm2", "gemma3-window", "qwen3-hd128"])
 def test_whole_models_with_both_options(pieces, attn_pieces, ref, name):
     test_real_head_geometry_against_the_oracle(pieces, ref, name, True)
+
+
+def test_backend_factory_switch(ref):
+    """require_gpu(..., bf16_pieces=True): both options set on every context of the backend; a step on it matches the oracle."""
+    hb = mod("hip_backend")
+    g = hb.require_gpu("the bf16-piece factory test", streams=2, bf16_pieces=True)
+    try:
+        kw = REAL["smollm2"]
+        rmodel, model = build_pair(ref, kw, seed=3, std=0.05)
+        seqs = batches(ref, kw["vocab"], 200, 2, seed=4, mask_every=7)
+        g.start_profile("")
+        lh, gh = hip_step(g, model, seqs, False, 200)          # one sequence per graph: both streams
+        seen = set(g.stop_profile())
+        assert any(".bf16x6" in s for s in seen), seen
+        ref.PARALLEL_BWD = True
+        ref.set_threads(min(16, ref.max_threads()))
+        try:
+            lr, gr = ref_step(ref, rmodel, seqs)
+        finally:
+            ref.PARALLEL_BWD = False
+            ref.set_threads(1)
+        compare(lh, gh, lr, gr, "factory switch")
+    finally:
+        g.destroy()
