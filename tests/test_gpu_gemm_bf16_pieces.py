@@ -86,7 +86,7 @@ def test_shapes_the_direct_kernels_do_not_take_stay_on_the_fp32_kernels(pieces, 
 
 def test_error_against_float64_next_to_the_fp32_kernels(gpu):
     """Not reduced precision: over the layer's product shapes the rms error of the piece products against float64 stays
-    within 1.25 x the FP32 MFMA kernels' own (measured 0.9 - 1.2 x: both accumulate in FP32, in a different order)."""
+    within 1.25 x the FP32 MFMA kernels' own (measured 0.61 - 1.16 x, the same from seed to seed: both accumulate in FP32, in a different order)."""
     rs = np.random.RandomState(7)
     for kind, M, N, K in [(0, 512, 576, 1536), (1, 512, 1536, 576), (2, 576, 576, 16384), (0, 384, 1536, 576)]:
         a = rs.standard_normal((K, M) if kind == 2 else (M, K)).astype(np.float32)
