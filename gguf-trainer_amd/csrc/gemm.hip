@@ -336,7 +336,9 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.rope = rot;
   GT_REQUIRE(ctx, !rot || (Hq * hd) % 4 == 0, "banded dQ product: rotated rows need 16-byte aligned output rows");
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
-  if (hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26)) return 1;
+  if (hd == 64 && ctx->opt_attn_pieces) {          // "attn.split_bf16": the product on the bf16 matrix instruction
+    if (gemm_split_launch_band(ctx, a, B * Hq)) return 1;
+  } else if (hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26)) return 1;
   if (splits > 1) {
     const int64_t rows = (int64_t)B * T, units = rows * Hq * (hd / 8);
     hipLaunchKernelGGL(band_dq_reduce, dim3((unsigned)cdiv(units, 256)), dim3(256), 0, ctx->stream, parts, splits, a.sP, dQ, acc, rot, rows, T, Hq, hd);

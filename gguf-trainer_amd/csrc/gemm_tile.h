@@ -434,7 +434,6 @@ __device__ __forceinline__ void split_step(const v4u (&fa)[TM][3], const v4u (&f
 // The work of one workgroup on output tile (pm, pn) and K split or batch member z
 template <int BM, int BN, int WM, int WN, int KIND, int BK, int NSTG, bool SEG2, bool BAND = false, bool MSEG = false, bool SPLIT = false>
 __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm, const int pn, const int z) {
-  static_assert(!SPLIT || !BAND, "the bf16-piece path takes plain, two-segment and summed products");
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   using TA = DirectTile<BM, KIND != GT_TN, NT, BK>;
@@ -760,3 +759,5 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_group_tn(GemmArgs a, GroupAr
 // argument block carries further K segments (gt_gemm_sum).
 int gemm_split_launch(gt_ctx *ctx, int kind, bool wide, bool summed, GemmArgs &a, int zdim);
 int gemm_split_launch_group(gt_ctx *ctx, bool wide, GemmArgs &a, GroupArgs &g);
+// the banded batch (dQ = dS.K per (sequence, head), head dim 64): 128 x 64 tiles, two wavefronts of 64 x 64
+int gemm_split_launch_band(gt_ctx *ctx, GemmArgs &a, int zdim);

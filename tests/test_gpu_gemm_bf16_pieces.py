@@ -355,7 +355,7 @@ def test_two_runs_give_the_same_bits(pieces):
         gpu.free_state_buffer(h)
 
 
-# ---- "attn.split_bf16": the attention forward (head dims 64 and 128) and dK/dV (64) on the same instruction -----------------------
+# ---- "attn.split_bf16": the attention forward (head dims 64 and 128), dK/dV and the banded dQ product (64) on the same instruction ----
 
 @pytest.fixture()
 def attn_pieces(gpu):
@@ -409,6 +409,16 @@ def test_attention_pieces_kept_score_gradients(attn_pieces, ref, B, T, Hq, Hkv, 
 def test_attention_pieces_rotations_in_the_write_backs(attn_pieces, B, T, Hq, Hkv, hd, window, keep_ds, acc):
     import test_gpu_ops
     test_gpu_ops.test_attention_backward_with_the_rotations_backward_in_its_write_backs(attn_pieces, B, T, Hq, Hkv, hd, window, keep_ds, acc)
+
+
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 2048, 9, 3, 64, 0), (2, 1024, 6, 2, 64, 0), (1, 2048, 10, 2, 64, 1500)])
+def test_attention_pieces_banded_dq_cut_into_parts(attn_pieces, B, T, Hq, Hkv, hd, window):
+    """The banded dQ product on pieces (128 x 64 tiles, two wavefronts of 64 x 64), its key ranges cut into parts for small launches."""
+    import test_gpu_ops
+    try:
+        test_gpu_ops.test_banded_dq_product_cut_into_parts(attn_pieces, B, T, Hq, Hkv, hd, window)
+    finally:
+        attn_pieces.set_option("attn.band_splits", -1)
 
 
 @pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,path", [(2, 2048, 9, 3, 64, 0, "kept-scores"), (1, 2048, 10, 2, 64, 512, "kept-scores"),
