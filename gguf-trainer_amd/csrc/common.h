@@ -34,7 +34,7 @@ struct gt_ctx {
   std::map<RopeKey, float *> rope_tables;
   int opt_attn_generic = 0, opt_gemm_tile = -1, opt_gemm_splitk = -1, opt_attn_splits = -1, opt_gemm_staged = 0;
   int opt_gemm_group = 1;                       // 0: gt_gemm_group launches its products one by one
-  int opt_attn_pieces = 0;                      // 1: attention forward (head dims 64, 128), dK/dV and the banded dQ product (64) on the bf16 matrix instruction too
+  int opt_attn_pieces = 0;                      // 1: attention forward and the banded dQ product (head dims 64, 128) and dK/dV (64) on the bf16 matrix instruction too
   int opt_gemm_split = 0;                       // 1: aligned FP32 products run as six bf16 MFMA products of three-piece operands
   int opt_attn_keep_ds = 1, opt_attn_ds_limit_mb = 8192, opt_gemm_sum_min_tiles = -1;
   int opt_attn_band_splits = -1;       // parts the banded dQ product cuts its K ranges into (-1: chosen from the launch's size)

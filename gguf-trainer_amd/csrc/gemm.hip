@@ -261,7 +261,7 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
 template <int BN>
 static int launch_band(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
   constexpr int BM = 128, BK = 32, NSTG = 3, WM = 2, WN = 2;
-  constexpr int smem = NSTG * (BM + BN) * BK * 4;
+  constexpr int smem = band_lds_bytes<BM, BN, BK, NSTG>();
   if (!(ctx->gemm_direct_set & (1ull << slot))) {
     GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
@@ -336,7 +336,7 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   a.rope = rot;
   GT_REQUIRE(ctx, !rot || (Hq * hd) % 4 == 0, "banded dQ product: rotated rows need 16-byte aligned output rows");
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
-  if (hd == 64 && ctx->opt_attn_pieces) {          // "attn.split_bf16": the product on the bf16 matrix instruction
+  if (ctx->opt_attn_pieces) {          // "attn.split_bf16": the product on the bf16 matrix instruction
     if (gemm_split_launch_band(ctx, a, B * Hq)) return 1;
   } else if (hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26)) return 1;
   if (splits > 1) {

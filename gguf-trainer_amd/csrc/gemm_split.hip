@@ -70,13 +70,14 @@ int gemm_split_launch_group(gt_ctx *ctx, bool wide, GemmArgs &a, GroupArgs &g) {
   return wide ? launch_group_split<128, 192, 2, 2>(ctx, a, g, 12) : launch_group_split<128, 128, 2, 2>(ctx, a, g, 13);
 }
 
-int gemm_split_launch_band(gt_ctx *ctx, GemmArgs &a, int zdim) {
-  constexpr int BM = 128, BN = 64, WM = 2, WN = 1;
-  constexpr int smem = GT_SPLIT_NSTG * (BM + BN) * GT_SPLIT_BK * 4;
-  if (!(ctx->gemm_split_set & (1ull << 18))) {
+template <int HD>
+static int launch_split_band(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
+  constexpr int BM = 128, BN = HD, WM = 2, WN = HD / 64;
+  constexpr int smem = band_lds_bytes<BM, BN, GT_SPLIT_BK, GT_SPLIT_NSTG>();
+  if (!(ctx->gemm_split_set & (1ull << slot))) {
     GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, GT_NN, GT_SPLIT_BK, GT_SPLIT_NSTG, false, true, false, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    ctx->gemm_split_set |= 1ull << 18;
+    ctx->gemm_split_set |= 1ull << slot;
   }
   a.nbm = (int)cdiv(a.M, BM);
   a.nbn = (int)cdiv(a.N, BN);
@@ -84,4 +85,8 @@ int gemm_split_launch_band(gt_ctx *ctx, GemmArgs &a, int zdim) {
                      dim3(WM * WN * 64), smem, ctx->stream, a);
   GT_LAUNCHED(ctx);
   return 0;
+}
+
+int gemm_split_launch_band(gt_ctx *ctx, GemmArgs &a, int zdim) {
+  return a.N == 64 ? launch_split_band<64>(ctx, a, zdim, 18) : launch_split_band<128>(ctx, a, zdim, 19);
 }

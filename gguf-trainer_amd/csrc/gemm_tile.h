@@ -641,7 +641,7 @@ __device__ __forceinline__ void gemm_direct_tile(const GemmArgs &a, const int pm
       // dQ with respect to the rows before their rotation: a pair (j, j + BN/2) of a row sits in two wavefronts' accumulators
       // (WN = 2), so the tile goes through LDS once (the pipeline's buffers are idle now) and every thread then rotates
       // float4 pairs of whole rows: (lo, hi) -> (c lo + s hi, -s lo + c hi), the reference's srcRope backward (wgsl.ts:346-384)
-      static_assert(!BAND || NSTG * (BM + BN) * BK >= BM * (BN + 4), "the tile must fit the pipeline's LDS");
+      // (the launchers size the dynamic LDS for the larger of the pipeline and this tile: band_lds_bytes)
       constexpr int LDS_C = BN + 4;            // = 4 mod 32 words: 8 lanes of a b128 access cover all banks
       __syncthreads();                         // everybody is done reading the last stage
 #pragma unroll
@@ -754,6 +754,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_group_tn(GemmArgs a, GroupAr
   a.Pp += (size_t)a.splits * p.e0;
   gemm_direct_tile<BM, BN, WM, WN, GT_TN, BK, NSTG, false, false, false, SPLIT>(a, lp / p.nbn, lp % p.nbn, z);
 }
+
+// dynamic LDS of a banded launch: the pipeline's stages, or the BM x (BN + 4) tile its rotating write-back passes through LDS
+template <int BM, int BN, int BK, int NSTG>
+constexpr int band_lds_bytes() {
+  return 4 * (NSTG * (BM + BN) * BK > BM * (BN + 4) ? NSTG * (BM + BN) * BK : BM * (BN + 4));
+}
+
 
 // gemm_split.hip: the bf16-piece instantiations. wide: 128 x 192 tiles (N a multiple of 192), else 128 x 128; summed: the
 // argument block carries further K segments (gt_gemm_sum).

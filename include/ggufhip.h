@@ -87,8 +87,8 @@ int gt_resident_bytes(gt_ctx *ctx, uint64_t *bytes);                  /* live gt
  *                  banded product over them (T a multiple of 128, hd 64 or 128); 0 = dQ always
  *                  recomputes the scores in its own kernel
  *   "attn.ds_limit_mb" largest dS workspace taken for that, in MiB (default 8192; B*Hq*T*T*4 bytes are needed)
- *   "attn.split_bf16" 1 = the attention forward (head dims 64 and 128), and at head dim 64 the dK/dV kernel (where the forward kept its
- *                  scores) and the banded dQ product, run their contractions the same way (rows, tiles, probabilities and score gradients
+ *   "attn.split_bf16" 1 = the attention forward and the banded dQ product (head dims 64 and 128), and at head dim 64 the dK/dV kernel (where
+ *                  the forward kept its scores), run their contractions the same way (rows, tiles, probabilities and score gradients
  *                  as bf16 pieces); everything else in attention stays on FP32 MFMA. 0 (default) = FP32 MFMA
  *   "attn.band_splits" -1 = heuristic, n >= 1 = pin the parts that banded product cuts each row tile's key range into (at most
  *                  8; launches with fewer row tiles than two per CU are cut so that a single sequence fills the chip)

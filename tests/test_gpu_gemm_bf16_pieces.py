@@ -355,7 +355,7 @@ def test_two_runs_give_the_same_bits(pieces):
         gpu.free_state_buffer(h)
 
 
-# ---- "attn.split_bf16": the attention forward (head dims 64 and 128), dK/dV and the banded dQ product (64) on the same instruction ----
+# ---- "attn.split_bf16": the attention forward (head dims 64 and 128), dK/dV (64) and the banded dQ product on the same instruction ----
 
 @pytest.fixture()
 def attn_pieces(gpu):
@@ -394,7 +394,8 @@ def test_attention_forward_pieces_kept_scores(attn_pieces, ref, B, T, Hq, Hkv, h
     test_gpu_ops.test_attention_kept_scores_equals_recomputed(attn_pieces, ref, B, T, Hq, Hkv, hd, window, splits, keep_ds)
 
 
-@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 512, 2, 1, 64, 127), (1, 768, 2, 1, 64, 300)])
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 256, 4, 2, 64, 0), (2, 384, 6, 2, 64, 100), (1, 512, 2, 1, 64, 127), (1, 768, 2, 1, 64, 300),
+                                                  (2, 256, 4, 2, 128, 0), (1, 384, 2, 1, 128, 130)])
 @pytest.mark.parametrize("acc,splits", [(0, 1), (1, 1), (0, 5), (1, 3)])
 def test_attention_pieces_kept_score_gradients(attn_pieces, ref, B, T, Hq, Hkv, hd, window, acc, splits):
     """dK/dV on pieces writes the score gradients the banded dQ product reads: against the pair that recomputes them and the oracle.
@@ -404,16 +405,17 @@ def test_attention_pieces_kept_score_gradients(attn_pieces, ref, B, T, Hq, Hkv, 
     test_gpu_ops.test_attention_backward_kept_ds_equals_recomputed(attn_pieces, ref, B, T, Hq, Hkv, hd, window, acc, splits)
 
 
-@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,keep_ds", [(1, 256, 4, 2, 64, 0, 1), (2, 128, 3, 3, 64, 0, 1), (2, 256, 6, 2, 64, 70, 0), (8, 256, 9, 3, 64, 0, 1)])
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window,keep_ds", [(1, 256, 4, 2, 64, 0, 1), (2, 128, 3, 3, 64, 0, 1), (2, 256, 6, 2, 64, 70, 0), (8, 256, 9, 3, 64, 0, 1),
+                                                          (1, 256, 4, 2, 128, 0, 1), (2, 256, 2, 1, 128, 70, 1)])
 @pytest.mark.parametrize("acc", [0, 1])
 def test_attention_pieces_rotations_in_the_write_backs(attn_pieces, B, T, Hq, Hkv, hd, window, keep_ds, acc):
     import test_gpu_ops
     test_gpu_ops.test_attention_backward_with_the_rotations_backward_in_its_write_backs(attn_pieces, B, T, Hq, Hkv, hd, window, keep_ds, acc)
 
 
-@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 2048, 9, 3, 64, 0), (2, 1024, 6, 2, 64, 0), (1, 2048, 10, 2, 64, 1500)])
+@pytest.mark.parametrize("B,T,Hq,Hkv,hd,window", [(1, 2048, 9, 3, 64, 0), (2, 1024, 6, 2, 64, 0), (1, 2048, 10, 2, 64, 1500), (1, 1024, 4, 2, 128, 0)])
 def test_attention_pieces_banded_dq_cut_into_parts(attn_pieces, B, T, Hq, Hkv, hd, window):
-    """The banded dQ product on pieces (128 x 64 tiles, two wavefronts of 64 x 64), its key ranges cut into parts for small launches."""
+    """The banded dQ product on pieces (128 x hd tiles, wavefronts of 64 x 64), its key ranges cut into parts for small launches."""
     import test_gpu_ops
     try:
         test_gpu_ops.test_banded_dq_product_cut_into_parts(attn_pieces, B, T, Hq, Hkv, hd, window)
