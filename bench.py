@@ -497,7 +497,7 @@ def run_workload(mods, config, steps, warmup, a, headline):
         if not a.sequential and not a.no_bf16_pieces and not any(kv.startswith("gemm.split_bf16") for kv in a.set):
             nb = max(2, min(6, steps))
             gpu.set_option("gemm.split_bf16", 1)
-            gpu.set_option("attn.split_bf16", 1)       # and the attention forward (head dims 64, 128), dK/dV and the banded dQ product (64)
+            gpu.set_option("attn.split_bf16", 1)       # and the attention forward and banded dQ product (head dims 64, 128) and dK/dV (64)
             try:
                 for i in range(2):
                     step(i % total, False)
@@ -519,7 +519,7 @@ def run_workload(mods, config, steps, warmup, a, headline):
             if allb2:
                 allb2["executed_frac_of_bf16_mfma_peak"] = round(6 * allb2["achieved"] * 1e12 / PEAK_BF16_MFMA, 4)
             res["bf16_pieces"] = {"what": "the same step with gt_set_option(\"gemm.split_bf16\", 1) and (\"attn.split_bf16\", 1): every aligned FP32 product, "
-                                          "and the attention forward (head dims 64, 128), dK/dV and the banded dQ product (64), as six bf16 MFMA products of three-piece operands, FP32 accumulate; "
+                                          "and the attention forward and banded dQ product (head dims 64, 128) and dK/dV (64), as six bf16 MFMA products of three-piece operands, FP32 accumulate; "
                                           "same entry points, same parity tolerances",
                                   "steps": nb, "value": round(nb * batch * SEQ / w2, 1), "unit": "tokens/s", "ms_per_step": round(1e3 * w2 / nb, 2),
                                   "all_bwd_gemms": allb2, "per_kernel": per2,
