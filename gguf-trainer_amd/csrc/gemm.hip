@@ -258,9 +258,11 @@ static int gemm_impl(gt_ctx *ctx, int kind, int acc, int M, int N, int K, gt_buf
 // (sequence, head): one banded NN product per pair, all in one launch. dS holds B*Hq [T][T] matrices in blocks
 // [row tile of 128][key step of 32][128 rows][32 keys] (what one pipeline stage loads is one contiguous 16 KB block)
 // whose blocks inside each row tile's band are all written (zeros where a pair is masked); T is a multiple of 128.
-template <int BN>
+// Head dim 128 runs two pipeline stages, not three: 98 KB of LDS left one workgroup per CU, 68 KB lets two stay (341 -> 318 us
+// per launch at 4 x 2048 tokens of 16 heads).
+template <int BN, int NSTG = 3>
 static int launch_band(gt_ctx *ctx, GemmArgs &a, int zdim, int slot) {
-  constexpr int BM = 128, BK = 32, NSTG = 3, WM = 2, WN = 2;
+  constexpr int BM = 128, BK = 32, WM = 2, WN = 2;
   constexpr int smem = band_lds_bytes<BM, BN, BK, NSTG>();
   if (!(ctx->gemm_direct_set & (1ull << slot))) {
     GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct<BM, BN, WM, WN, GT_NN, BK, NSTG, false, true>),
@@ -338,7 +340,7 @@ int gemm_band_dq(gt_ctx *ctx, int B, int T, int Hq, int Hkv, int hd, int window,
   GT_REQUIRE(ctx, T / 128 <= 65535, "banded dQ product: %d row tiles exceed the grid", T / 128);
   if (ctx->opt_attn_pieces) {          // "attn.split_bf16": the product on the bf16 matrix instruction
     if (gemm_split_launch_band(ctx, a, B * Hq)) return 1;
-  } else if (hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128>(ctx, a, B * Hq, 26)) return 1;
+  } else if (hd == 64 ? launch_band<64>(ctx, a, B * Hq, 25) : launch_band<128, 2>(ctx, a, B * Hq, 26)) return 1;
   if (splits > 1) {
     const int64_t rows = (int64_t)B * T, units = rows * Hq * (hd / 8);
     hipLaunchKernelGGL(band_dq_reduce, dim3((unsigned)cdiv(units, 256)), dim3(256), 0, ctx->stream, parts, splits, a.sP, dQ, acc, rot, rows, T, Hq, hd);
