@@ -239,30 +239,6 @@ __device__ __forceinline__ void rows_dot_pieces(v16f (&acc)[N], const float *row
         acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, ka[n][TA[t]]), __builtin_bit_cast(v8bf, qp[c][TB[t]]), acc[n], 0, 0, 0);
   }
 }
-// the same with one head-dim block in flight (12 registers fewer; its six MFMAs wait on one another): dK/dV
-template <int LDT>
-__device__ __forceinline__ void t_dot_pieces_lean(v16f (&out)[HD / 32], const float *ldst, int col0, const float (&w)[16], int l32, int g) {
-  constexpr int DT = HD / 32;
-  constexpr int TA[6] = GT_PIECE_TERMS_A, TB[6] = GT_PIECE_TERMS_B;
-#pragma unroll
-  for (int j = 0; j < 2; j++) {
-    v4u pw[3];
-    const float xw[8] = {w[8 * j], w[8 * j + 1], w[8 * j + 2], w[8 * j + 3], w[8 * j + 4], w[8 * j + 5], w[8 * j + 6], w[8 * j + 7]};
-    cut8(xw, pw);
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++) {
-      v4u va[3];
-      const int d = dt * 32 + l32, chunk = (col0 >> 2) + 4 * j + g;
-      const v4f lo = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * (chunk ^ ((d >> 3) & 7)));
-      const v4f hi = *reinterpret_cast<const v4f *>(ldst + d * LDT + 4 * ((chunk + 2) ^ ((d >> 3) & 7)));
-      const float x[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      cut8(x, va);
-#pragma unroll
-      for (int t = 0; t < 6; t++)
-        out[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, va[TA[t]]), __builtin_bit_cast(v8bf, pw[TB[t]]), out[dt], 0, 0, 0);
-    }
-  }
-}
 // out[dt] += TileT(cols [col0, col0+32)) . w, w in accumulator order: MFMA j takes w[8j .. 8j+7], the keys 16j + 4g + (0..3) and 16j + 8 + 4g + (0..3)
 template <int LDT>
 __device__ __forceinline__ void t_dot_pieces(v16f (&out)[HD / 32], const float *ldst, int col0, const float (&w)[16], int l32, int g) {
@@ -286,6 +262,111 @@ __device__ __forceinline__ void t_dot_pieces(v16f (&out)[HD / 32], const float *
 #pragma unroll
       for (int dt = 0; dt < DT; dt++)
         out[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, va[dt][TA[t]]), __builtin_bit_cast(v8bf, pw[TB[t]]), out[dt], 0, 0, 0);
+  }
+}
+
+// ---- dK/dV on pieces: the query-side tiles cut ONCE per workgroup, as they are stored, into planes of bf16 pairs ----
+// A thread stores columns d = 4 (tid % 8) + (0..3) and d + 32 of row tid / 8 of a 32 x 64 tile; cutting (row, d) and (row, d + 32)
+// together gives one word per piece (h, m or l): the low and the high half. Row-major planes [piece][row][32 words] keep those words:
+// they feed the contraction over the head dim, whose k-slots then run d, d + 32, d + 1, d + 33, ... (the other operand, this lane's own
+// row, is cut in the same order). Transposed planes [piece][d = 0..63][16 words] feed the contractions over the rows and hold two ROWS
+// of one column to a word (see pl_store_t). In both, 16-byte chunks of a plane row are XOR-swizzled so that the b128 reads of 8
+// consecutive lanes cover all banks.
+#define PL_PLANE 1024                                   // words per plane
+#define PL_GR 0                                          // dO, row-major
+#define PL_GT (3 * PL_PLANE)                             // dO, transposed
+#define PL_QT (6 * PL_PLANE)                             // Q, transposed
+#define PL_L (9 * PL_PLANE)                              // lse, then D
+#define PL_BUF (9 * PL_PLANE + 2 * 32)                   // words per buffer
+// this thread's share of a tile: row tid / 8, columns 4 (tid % 8) + (0..3) in x0 and 32 more in x1, cut into words w[piece][e]
+__device__ __forceinline__ void pl_cut_unit(const v4f &x0, const v4f &x1, unsigned (&w)[3][4]) {
+#pragma unroll
+  for (int e = 0; e < 4; e++) split_pair(x0[e], x1[e], w[0][e], w[1][e], w[2][e]);
+}
+__device__ __forceinline__ void pl_store_rows(const unsigned (&w)[3][4], unsigned *planes, int tid) {
+  const int row = tid / 8, c = tid % 8;
+#pragma unroll
+  for (int pc = 0; pc < 3; pc++)
+    *reinterpret_cast<v4u *>(planes + pc * PL_PLANE + row * 32 + 4 * (c ^ (row & 7))) = v4u{w[pc][0], w[pc][1], w[pc][2], w[pc][3]};
+}
+// transposed planes: word (d, pair of rows) = the pieces of (row, d) and (row + 1, d), row even. The thread of the even row and the
+// thread of the odd row (8 lanes apart in a DPP row) exchange their words; the even one then writes the word of column d, the odd
+// one that of column d + 32. Words of a 64-byte plane row are ordered so that the 8 k-slots of a lane are one 16-byte chunk; chunks are
+// XOR-swizzled within a row (reads conflict-free; a wavefront's stores, 8 columns 4 apart of 8 rows, meet four by four: telling them apart
+// by one more address bit costs the two registers the kernel does not have).
+__device__ __forceinline__ int pl_swz_t(int d) { return ((d >> 1) & 3) ^ ((d >> 3) & 3); }
+__device__ __forceinline__ void pl_store_t(const unsigned (&w)[3][4], unsigned *planes, int tid) {
+  const int row = tid / 8, c = tid % 8, odd = row & 1, pr = row >> 1;
+  const unsigned sel = odd ? 0x03020706u : 0x05040100u;
+  const int pos = (pr & 9) | ((pr & 4) >> 1) | ((pr & 2) << 1);          // pair 8j + 4i + 2g + s sits at word 8j + 4g + 2i + s
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const int d = 32 * odd + 4 * c + e, at = d * 16 + 4 * ((pos >> 2) ^ pl_swz_t(d)) + (pos & 3);
+#pragma unroll
+    for (int pc = 0; pc < 3; pc++) {
+      const unsigned other = (unsigned)__builtin_amdgcn_mov_dpp((int)w[pc][e], 0x128, 0xf, 0xf, true);          // row_ror:8: the partner's word
+      planes[pc * PL_PLANE + at] = __builtin_amdgcn_perm(other, w[pc][e], sel);
+    }
+  }
+}
+// this lane's row in the planes' k-slot order: vp[c][piece] word e = pieces of (x[8c + 4g + e], x[32 + 8c + 4g + e]) * mul
+__device__ __forceinline__ void pl_load_row(v4u (&vp)[4][3], const float *__restrict__ row, bool valid, int g, float mul) {
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    v4f lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+    if (valid) { lo = *reinterpret_cast<const v4f *>(row + 8 * c + 4 * g); hi = *reinterpret_cast<const v4f *>(row + 32 + 8 * c + 4 * g); }
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      unsigned h, m, l;
+      split_pair(lo[e] * mul, hi[e] * mul, h, m, l);
+      vp[c][0][e] = h; vp[c][1][e] = m; vp[c][2][e] = l;
+    }
+  }
+}
+// Tile(32 rows, row-major planes) . row^T: four steps of 16 k-slots, six piece products each, no vector work at all
+__device__ __forceinline__ v16f pl_rows_dot(const unsigned *planes, const v4u (&vp)[4][3], int l32, int g) {
+  constexpr int TA[6] = GT_PIECE_TERMS_A, TB[6] = GT_PIECE_TERMS_B;
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  v4u a[2][3];
+  auto fetch = [&](int c) {
+#pragma unroll
+    for (int pc = 0; pc < 3; pc++) a[c & 1][pc] = *reinterpret_cast<const v4u *>(planes + pc * PL_PLANE + l32 * 32 + 4 * ((2 * c + g) ^ (l32 & 7)));
+  };
+  fetch(0);
+#pragma unroll
+  for (int c = 0; c < 4; c++) {          // the next step's operand is asked for before this step's MFMAs, and no further ahead
+    if (c < 3) fetch(c + 1);
+#pragma unroll
+    for (int t = 0; t < 6; t++)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a[c & 1][TA[t]]), __builtin_bit_cast(v8bf, vp[c][TB[t]]), acc, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  return acc;
+}
+// out[dt] += TileT(transposed planes) . w, w in accumulator order (MFMA j takes w[8j .. 8j+7]: rows 16j + 4g + (0..3) and 16j + 8 + 4g + (0..3))
+__device__ __forceinline__ void pl_t_dot(v16f (&out)[HD / 32], const unsigned *planes, const float (&w)[16], int l32, int g) {
+  constexpr int TA[6] = GT_PIECE_TERMS_A, TB[6] = GT_PIECE_TERMS_B;
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    v4u pw[3];
+    const float xw[8] = {w[8 * j], w[8 * j + 1], w[8 * j + 2], w[8 * j + 3], w[8 * j + 4], w[8 * j + 5], w[8 * j + 6], w[8 * j + 7]};
+    cut8(xw, pw);
+    v4u va[HD / 32][3];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+      for (int pc = 0; pc < 3; pc++) {
+        const int d = 32 * dt + l32;
+        va[dt][pc] = *reinterpret_cast<const v4u *>(planes + pc * PL_PLANE + d * 16 + 4 * ((2 * j + g) ^ pl_swz_t(d)));
+      }
+#pragma unroll
+    for (int t = 0; t < 6; t++)          // the blocks' chains alternate
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; dt++)
+        out[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, va[dt][TA[t]]), __builtin_bit_cast(v8bf, pw[TB[t]]), out[dt], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -675,12 +756,15 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 // filled during stage it-1) while stage it computes on the other buffer, the loads of stage it+2 follow, and one barrier
 // ends the stage. None of that depends on the stage's MFMAs, and it is straight-line code, so it runs under them.
 #define DKV_BUF (2 * QT * LD + 2 * HD * (QT + 4) + 2 * QT)        // floats per buffer: sQ, sG, sQt, sGt, lse, D
-// PX: the three (four without kept scores) contractions on the bf16 matrix instruction: this lane's key / value row as pieces cut once, the Q
-// and dO tiles (row-major and transposed) and the probabilities / score gradients cut as they are read. The register file is the limit
-// at two wavefronts per SIMD: one head-dim block of the transposed tiles at a time and one accumulator chain per score block keep it at 255-256
-// registers (6 spilled with kept scores and kept dS: 554 us per launch; without the stage of look-ahead for the kept scores nothing
-// spills and it takes 584; 39 spilled with two blocks in flight, which ran slower than the FP32 kernel's 668-679, as did one wavefront
-// per SIMD without spills). Only with kept scores: the key row's pieces for recomputing them do not fit.
+// PX (head dim 64, kept scores): the three contractions on the bf16 matrix instruction. The Q and dO tiles are the same for the four
+// wavefronts of a workgroup, so they are cut into pieces ONCE, by the threads that store them (each thread holds columns d and d + 32
+// of one row, whose pieces pair up into words), into three kinds of planes: dO row-major for dP = dO.V^T (this lane's value row is cut
+// once per kernel in the same k-slot order), dO and Q transposed, two rows to a word, for dV += P^T.dO and dK += dS^T.Q: the
+// contractions read their tile operand as ready MFMA registers, one b128 per piece, and only the probabilities and score gradients are
+// cut as they are made. 7 vector instructions per MFMA where every wavefront cutting every tile it read took 12.7; on one box 522-529 us
+// per launch against 580-594. The register file is what is left as the limit at two wavefronts per SIMD (256, five of them in scratch):
+// the kept scores of a stage are asked for at its top, not a stage ahead (16 registers: with them 13 spill and the launch takes 589),
+// and scheduling barriers keep the operand fetches from being issued all at once. 2 x 37 KB of LDS.
 template <bool KS, bool DS, bool PX = false>
 __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(AttnP p, const float *__restrict__ q, const float *__restrict__ k,
                                                            const float *__restrict__ v, const float *__restrict__ go,
@@ -707,11 +791,10 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   const bool sv = s < p.T;
   const size_t koff = ((size_t)b * p.T + (sv ? s : 0)) * kstr + (size_t)kvh * HD;
   float kreg[KS || PX ? 1 : HD / 2], vreg[PX ? 1 : HD / 2];
-  v4u kp[PX && !KS ? HD / 16 : 1][3], vp[PX ? HD / 16 : 1][3];
-  if constexpr (PX) {
-    if constexpr (!KS) load_row_pieces(kp, k + koff, sv, g, p.c2);
-    load_row_pieces(vp, v + koff, sv, g, 1.0f);
-  } else {
+  static_assert(!PX || (KS && HD == 64), "dK/dV on pieces: kept scores and head dim 64 only");
+  v4u vp[PX ? 4 : 1][3];
+  if constexpr (PX) pl_load_row(vp, v + koff, sv, g, 1.0f);
+  else {
     if constexpr (!KS) load_row_regs(kreg, k + koff, sv, g, p.c2);
     load_row_regs(vreg, v + koff, sv, g, 1.0f);
   }
@@ -752,7 +835,10 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   // row statistics of a stage: threads 0..31 fetch lse, 32..63 fetch D (the other threads fetch the same words again: no branch)
   const float *statp = ((tid & QT) ? Dr : lse) + ((size_t)b * p.Hq + h) * p.T;
   unsigned qoffs[IO::PER];
-  IO::offsets(qoffs, qstr, tid);
+  if constexpr (PX) {          // row tid / 8: columns 4 (tid % 8) + (0..3), and 32 further on in the second unit
+    qoffs[0] = (unsigned)(((tid / 8) * qstr + 4 * (tid % 8)) * sizeof(float));
+    qoffs[IO::PER - 1] = qoffs[0] + 32 * (unsigned)sizeof(float);
+  } else IO::offsets(qoffs, qstr, tid);
   // Stage indices past the end are clamped to the last stage: its tile is loaded, and written to the idle buffer, again,
   // which nobody reads; the loop body has no test for "is there a next stage".
   // With kept scores T is a multiple of 128 and no tile is short: telling the loads so takes their clamp arithmetic out of the
@@ -760,13 +846,13 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   constexpr bool WHOLE = KS && HD >= 128;
   auto load_q = [&](int it) {
     const int qt = qt_lo + min(it, niter - 1);
-    IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, WHOLE ? QT : p.T - qt * QT, tid);
+    IO::load(pq, qb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, WHOLE || PX ? QT : p.T - qt * QT, tid);
   };
   auto load_g = [&](int it) {          // dO and the row statistics
     const int qt = qt_lo + min(it, niter - 1);
     if constexpr (ONE_SET) IO::load(pq, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, p.T - qt * QT, tid);
-    else IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, WHOLE ? QT : p.T - qt * QT, tid);
-    pstat = statp[WHOLE ? qt * QT + (tid % QT) : min(qt * QT + (tid % QT), p.T - 1)];
+    else IO::load(pg, gb + (size_t)qt * QT * qstr, qoffs, (unsigned)qstr, WHOLE || PX ? QT : p.T - qt * QT, tid);
+    pstat = statp[WHOLE || PX ? qt * QT + (tid % QT) : min(qt * QT + (tid % QT), p.T - 1)];
   };
   auto load_scores = [&](int it) {          // blocks the forward has not written hold anything: their stage is skipped
     const int qt = qt_lo + min(it, niter - 1);
@@ -774,10 +860,24 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
     for (int a = 0; a < 4; a++) psc[a] = *reinterpret_cast<const v4f *>(scw + (size_t)qt * 1024 + 8 * a);
   };
   auto store_q = [&](float *buf) {
+    if constexpr (PX) {
+      unsigned w[3][4];
+      pl_cut_unit(pq[0], pq[IO::PER - 1], w);
+      pl_store_t(w, reinterpret_cast<unsigned *>(buf) + PL_QT, tid);
+      return;
+    }
     if (!KS) IO::store_rows(pq, buf, tid);
     IO::store_t(pq, buf + O_QT, tid);
   };
   auto store_g = [&](float *buf) {
+    if constexpr (PX) {          // one cut serves both layouts
+      unsigned w[3][4];
+      pl_cut_unit(pg[0], pg[IO::PER - 1], w);
+      pl_store_rows(w, reinterpret_cast<unsigned *>(buf) + PL_GR, tid);
+      pl_store_t(w, reinterpret_cast<unsigned *>(buf) + PL_GT, tid);
+      if (tid < 2 * QT) buf[PL_L + tid] = pstat;
+      return;
+    }
     if constexpr (ONE_SET) {
       IO::store_rows(pq, buf + O_G, tid);
       IO::store_t(pq, buf + O_GT, tid);
@@ -808,7 +908,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
       load_q(it_lo + 1);
     } else {
       load_g(it_lo);
-      if (KS) load_scores(it_lo);
+      if (KS && !PX) load_scores(it_lo);
       store_q(dkv_smem);
       store_g(dkv_smem);
       load_q(it_lo + 1);
@@ -817,14 +917,17 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
     __syncthreads();
   }
   for (int it = it_lo; it < niter; it++) {
-    const float *cur = dkv_smem + ((it - it_lo) & 1) * DKV_BUF;
-    float *nxt = dkv_smem + (((it - it_lo) & 1) ^ 1) * DKV_BUF;
-    const float *sQ = cur, *sG = cur + O_G, *sQt = cur + O_QT, *sGt = cur + O_GT, *sL = cur + O_L, *sD = cur + O_D;
+    constexpr int BUF = PX ? PL_BUF : DKV_BUF;
+    const float *cur = dkv_smem + ((it - it_lo) & 1) * BUF;
+    float *nxt = dkv_smem + (((it - it_lo) & 1) ^ 1) * BUF;
+    const float *sQ = cur, *sG = cur + O_G, *sQt = cur + O_QT, *sGt = cur + O_GT, *sL = cur + (PX ? PL_L : O_L), *sD = cur + (PX ? PL_L + QT : O_D);
+    const unsigned *pl = reinterpret_cast<const unsigned *>(cur);
     v16f sc;
     if (KS) {            // out of the prefetch registers, which the next stage's scores then fill
+      if constexpr (PX) load_scores(it);          // (on pieces there are no registers for a stage of look-ahead: asked for here, first used after the dP contraction)
 #pragma unroll
       for (int r = 0; r < 16; r++) sc[r] = psc[r / 4][r % 4];
-      load_scores(it + 1);
+      if constexpr (!PX) load_scores(it + 1);
     }
     const int t0 = (qt_lo + it) * QT;
     // this lane's column of the dS block of (query stage, keys of this wavefront): rows t0 + 8a + 4g + j. The matrix of a
@@ -847,8 +950,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
       // instead of eight keep the kernel inside the register file
       constexpr int DKV_NB = (HD >= 128 && !KS) ? 4 : 8;
       if constexpr (!KS) {
-        if constexpr (PX) { v16f a1[1]; rows_dot_pieces<1>(a1, sQ, kp, l32, g); sc = a1[0]; }
-        else sc = rows_dot_regs<DKV_NB>(sQ, kreg, l32, g);
+        sc = rows_dot_regs<DKV_NB>(sQ, kreg, l32, g);
       }
       // The stage as straight-line code. A pair (query tq, key s) is live when s <= tq <= last query that sees s: one
       // unsigned compare per element against this lane's span (computed once per kernel), applied to every tile: a
@@ -859,7 +961,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
       // between two dependent blocks, and the group barriers ask for that interleaving (one MFMA, a few vector
       // instructions, and again).
       v16f dp;
-      if constexpr (PX) { v16f a1[1]; rows_dot_pieces<1>(a1, sG, vp, l32, g); dp = a1[0]; }
+      if constexpr (PX) dp = pl_rows_dot(pl + PL_GR, vp, l32, g);
       else dp = rows_dot_regs<DKV_NB>(sG, vreg, l32, g);
       float pr[16], ds[16];
       const unsigned rel0 = (unsigned)(t0 + 4 * g - s) + dead;          // query index relative to this lane's key, element (a, j) adds 8a + j
@@ -879,7 +981,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
           __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
         }
       }
-      if constexpr (PX) t_dot_pieces_lean<IO::LDT>(vacc, sGt, 0, pr, l32, g);
+      if constexpr (PX) pl_t_dot(vacc, pl + PL_GT, pr, l32, g);
       else t_dot_acc<IO::LDT, DKV_NB>(vacc, sGt, 0, pr, l32, g);
 #pragma unroll
       for (int a = 0; a < 4; a++) {
@@ -905,7 +1007,7 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
         load_q(it + 2);
         load_g(it + 2);
       }
-      if constexpr (PX) t_dot_pieces_lean<IO::LDT>(kacc, sQt, 0, ds, l32, g);
+      if constexpr (PX) pl_t_dot(kacc, pl + PL_QT, ds, l32, g);
       else t_dot_acc<IO::LDT, DKV_NB>(kacc, sQt, 0, ds, l32, g);
     }
     stage_end(nxt, it);
@@ -1015,8 +1117,9 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
   {
     ProfScope ps(ctx, "attention.bwd.dkv");
     dim3 grid((unsigned)(cdiv(p.T, 128) * p.Hq * p.B * p.splits));
+    size_t smem = DKV_SMEM;
     auto launch = [&](auto kern) {
-      hipLaunchKernelGGL(kern, grid, dim3(256), DKV_SMEM, ctx->stream, p, P<const float>(q), P<const float>(k), P<const float>(v),
+      hipLaunchKernelGGL(kern, grid, dim3(256), smem, ctx->stream, p, P<const float>(q), P<const float>(k), P<const float>(v),
                          P<const float>(dout), P<const float>(lse), Dr, P<float>(dk), acc_k, P<float>(dv), acc_v, part, dsb, sco, rot_k);
     };
 #if HD == 64
@@ -1024,11 +1127,12 @@ int FN(attn_bwd_mfma)(gt_ctx *ctx, const AttnP &p, gt_buf q, gt_buf k, gt_buf v,
                                                 // its scores (recomputing them needs the key row's pieces too: 34-37 registers spilled)
       if (!(ctx->attn_smem_set & (1 << 21))) {
         GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, false, true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * PL_BUF * sizeof(unsigned))));
         GT_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(FN(attn_bwd_dkv_mfma_k)<true, true, true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)DKV_SMEM));
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * PL_BUF * sizeof(unsigned))));
         ctx->attn_smem_set |= 1 << 21;
       }
+      smem = 2 * PL_BUF * sizeof(unsigned);
       dsb ? launch(FN(attn_bwd_dkv_mfma_k)<true, true, true>) : launch(FN(attn_bwd_dkv_mfma_k)<true, false, true>);
     } else
 #endif
