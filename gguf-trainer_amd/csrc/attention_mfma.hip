@@ -762,7 +762,7 @@ __global__ __launch_bounds__(256) void FN(attn_bwd_dq_mfma_k)(AttnP p, const flo
 // once per kernel in the same k-slot order), dO and Q transposed, two rows to a word, for dV += P^T.dO and dK += dS^T.Q: the
 // contractions read their tile operand as ready MFMA registers, one b128 per piece, and only the probabilities and score gradients are
 // cut as they are made. 7 vector instructions per MFMA where every wavefront cutting every tile it read took 12.7; on one box 522-529 us
-// per launch against 580-594. The register file is what is left as the limit at two wavefronts per SIMD (256, five of them in scratch):
+// per launch against 580-594. The register file is what is left as the limit at two wavefronts per SIMD (255 of 256, nothing in scratch):
 // the kept scores of a stage are asked for at its top, not a stage ahead (16 registers: with them 13 spill and the launch takes 589),
 // and scheduling barriers keep the operand fetches from being issued all at once. 2 x 37 KB of LDS.
 template <bool KS, bool DS, bool PX = false>
@@ -774,7 +774,9 @@ __global__ __launch_bounds__(256, WAVES_PER_SIMD) void FN(attn_bwd_dkv_mfma_k)(A
   using IO = TileIO<QT>;
   extern __shared__ __attribute__((aligned(16))) float dkv_smem[];      // 2 x 35 KB at hd 64, 2 x 69 KB at hd 128
   constexpr int O_G = QT * LD, O_QT = 2 * QT * LD, O_GT = O_QT + HD * IO::LDT, O_L = O_GT + HD * IO::LDT, O_D = O_L + QT;
-  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, g = lane / 32, l32 = lane % 32;
+  // the wavefront's number as a scalar: what follows from it (its keys' offsets, its blocks of the kept scores and of dS) then stays in scalar
+  // registers, five vector registers fewer in a kernel that is short of them (the forward got slower by the same change and keeps tid / 64)
+  const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64), g = lane / 32, l32 = lane % 32;
   // 1-D grid, key tile slowest: the first key tiles are seen by the most queries and go first. One workgroup
   // per QUERY head: with a kv group larger than one, each head's dK/dV goes to its own slice of the workspace
   // and attn_group_sum adds the slices in head order (a fixed order, so still deterministic); splitting by

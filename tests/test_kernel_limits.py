@@ -20,9 +20,8 @@ READELF = shutil.which("llvm-readelf") or "/opt/rocm/llvm/bin/llvm-readelf"
 
 LDS_STATIC_LIMIT = 64 * 1024          # beyond this a kernel must take dynamic LDS and raise its attribute
 REGS_PER_LANE = 512                   # unified VGPR + AGPR file of a gfx950 wavefront at one wave per SIMD
-# kernel name fragment -> bytes of scratch it may use. One does: dK/dV of head dim 64 on bf16 pieces with kept scores and kept dS keeps five
-# registers in scratch at two wavefronts per SIMD
-SPILL_ALLOWED = {"attn_bwd_dkv_mfma_k64ILb1ELb1ELb1E": 20}
+# kernel name fragment -> bytes of scratch it may use: none does (a scratch access waits for every load in flight, a kernel's prefetches included)
+SPILL_ALLOWED = {}
 
 
 def code_objects(blob):
